@@ -1,0 +1,178 @@
+/*
+ * pto_hip.h — C ABI of the MI355X (gfx950) execution path for PyPTO's paged-attention
+ * decode and FFN tile programs.
+ *
+ * The library behind this header (libpto_hip.so) replaces, for those programs, what the
+ * reference reaches through its device runtime: kernel code produced by the PTO codegen
+ * plus the task-graph scheduler that launches it.  The boundary is kept in the shape the
+ * reference's own launcher uses, so a binding on the reference side is a thin stub:
+ *
+ *   Worker.init / register / run / close         python/pypto/runtime/device_runner.py:821-842
+ *   Worker.malloc / free / copy_to / copy_from   python/pypto/runtime/runtime_base.py:106-118
+ *   TaskArgs: all tensors first, then u64 scalars python/pypto/runtime/runner.py:906-956
+ *   kernel_entry(int64_t* args) + ChipTensor     python/pypto/backend/pto_backend.py:538-645,898-915
+ *   benchmark(): register once, launch N rounds  python/pypto/runtime/bench.py:1251-1267
+ *
+ * Conventions
+ *   - every function returns a PtoHipStatus; pto_hip_last_error() gives the message of the
+ *     last failure on the calling thread (the reference raises ValueError / RuntimeError,
+ *     python/bindings/modules/error.cpp:60-78; PTO_HIP_ERR_INVALID_VALUE maps to ValueError,
+ *     everything else to RuntimeError).
+ *   - tensors are device memory unless stated; pointers are plain addresses; `stream` is a
+ *     hipStream_t passed as void* (NULL = the device's default stream).  Launches are
+ *     asynchronous on that stream.
+ *   - no function takes or returns a torch type.
+ */
+#ifndef PTO_HIP_H_
+#define PTO_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PTO_HIP_API __attribute__((visibility("default")))
+
+typedef enum PtoHipStatus {
+  PTO_HIP_OK = 0,
+  PTO_HIP_ERR_INVALID_VALUE = 1,   /* bad argument: shape, dtype, null pointer  (ValueError)  */
+  PTO_HIP_ERR_RUNTIME = 2,         /* a HIP call failed                          (RuntimeError) */
+  PTO_HIP_ERR_NOT_INITIALIZED = 3, /* pto_hip_init not called / already closed   (RuntimeError) */
+  PTO_HIP_ERR_UNSUPPORTED = 4,     /* valid request this build has no kernel for (RuntimeError) */
+  PTO_HIP_ERR_NOT_FOUND = 5        /* unknown program name or callable id        (ValueError)  */
+} PtoHipStatus;
+
+/* Element type codes: the values of DataType::k*Code, include/pypto/core/dtype.h:48-96. */
+typedef enum PtoHipDataType {
+  PTO_HIP_INT8 = 0x11,
+  PTO_HIP_INT32 = 0x13,
+  PTO_HIP_INT64 = 0x14,
+  PTO_HIP_FP8E4M3FN = 0x31,
+  PTO_HIP_FP16 = 0x33,
+  PTO_HIP_FP32 = 0x34,
+  PTO_HIP_BF16 = 0x40
+} PtoHipDataType;
+
+#define PTO_HIP_MAX_DIMS 5
+
+/* Tensor descriptor as generated kernels see it: `buffer.addr`, `start_offset` (in elements),
+ * `shapes[]`, `ndims`  (python/pypto/backend/pto_backend.py:578-606).  `dtype` is this
+ * library's addition; the reference carries the type in the generated code instead. */
+typedef struct PtoHipBuffer {
+  uint64_t addr; /* base address (device; host allowed only where a program says so) */
+  uint64_t size; /* bytes */
+} PtoHipBuffer;
+
+typedef struct PtoHipChipTensor {
+  PtoHipBuffer buffer;
+  uint64_t start_offset;
+  uint32_t shapes[PTO_HIP_MAX_DIMS];
+  uint32_t ndims;
+  uint32_t dtype; /* PtoHipDataType */
+  uint32_t reserved;
+} PtoHipChipTensor;
+
+typedef struct PtoHipDeviceInfo {
+  int32_t device_id;
+  int32_t compute_units;
+  int32_t wavefront_size;
+  int32_t lds_bytes_per_cu;
+  int64_t hbm_bytes;
+  char arch[32]; /* "gfx950" */
+} PtoHipDeviceInfo;
+
+/* ---- lifecycle: Worker.init / close (device_runner.py:821-842) -------------------------
+ * One device per process.  init may be called again for the same device (each call must be
+ * matched by a close; the last close releases the library's device memory). */
+PTO_HIP_API int pto_hip_init(int device_id);
+PTO_HIP_API int pto_hip_close(void);
+PTO_HIP_API const char* pto_hip_last_error(void);
+PTO_HIP_API int pto_hip_device_info(PtoHipDeviceInfo* info);
+
+/* ---- memory: Worker.malloc / free / copy_to / copy_from (runtime_base.py:106-118) ------- */
+PTO_HIP_API int pto_hip_malloc(size_t nbytes, uint64_t* dev_ptr);
+PTO_HIP_API int pto_hip_free(uint64_t dev_ptr);
+PTO_HIP_API int pto_hip_copy_to(uint64_t dst_dev_ptr, const void* src_host_ptr, size_t nbytes);
+PTO_HIP_API int pto_hip_copy_from(void* dst_host_ptr, uint64_t src_dev_ptr, size_t nbytes);
+PTO_HIP_API int pto_hip_sync(void* stream);
+
+/* ---- programs: Worker.register / run (device_runner.py:839-840) -------------------------
+ * A program is addressed by the name of the reference tile program it stands for.  Tensor
+ * order and meaning follow that program's orchestration signature; all tensors come first,
+ * then the scalars as raw 64-bit patterns (floats bit-cast, runner.py:948-953).
+ *
+ *  "paged_attention"   examples/models/04_paged_attention.py:272-288
+ *      tensors: query[B*Hq,D] bf16|fp16, key_cache[pool*Hkv*bs,D], value_cache (same),
+ *               block_table[B*max_blocks] i32, context_lens[B] i32, out[B*Hq,D] fp32,
+ *               config[7] i64 = {B,Hq,Hkv,D,bs,max_blocks,scale_bits}  (HOST or device memory)
+ *               [, k_scale[pool,Hkv] fp32, v_scale[pool,Hkv] fp32]  when the caches are FP8E4M3FN
+ *      cache row of (block p, kv head h, token t) = (p*Hkv + h)*bs + t
+ *  "paged_gather"      src/ir/op/tensor_ops/paged_gather.cpp:74-199
+ *      tensors: src[rows,hidden], indices[n] i32, block_table[nblk] i32, out[n,size]
+ *      scalars: block_size, col_offset
+ *  "rms_norm"          examples/intermediate/03_normalization.py:33-65
+ *      tensors: x[T,H], gamma[1,H] fp32, out[T,H] (dtype of x or fp32);  scalars: eps (f32 bits)
+ *  "ffn_swiglu"        examples/models/01_ffn.py:111-131
+ *      tensors: hidden_states[T,H], gate_proj_weight[H,I], up_proj_weight[H,I],
+ *               down_proj_weight[I,H], output[T,H] (fp32 or dtype of x)
+ *  "ffn_block"         tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:155-187
+ *      tensors: x[T,H], gamma[1,H] fp32, w_gate[H,I], w_up[H,I], w_down[I,H], out[T,H]
+ *      scalars: eps (f32 bits)
+ */
+PTO_HIP_API int pto_hip_register(const char* program_name, int* callable_id);
+PTO_HIP_API int pto_hip_unregister(int callable_id);
+PTO_HIP_API int pto_hip_run(int callable_id, const PtoHipChipTensor* tensors, int n_tensors,
+                            const uint64_t* scalars, int n_scalars, void* stream);
+
+/* Packed form of the generated-kernel ABI: args[0..n_tensors) are PtoHipChipTensor*,
+ * args[n_tensors..n_tensors+n_scalars) raw u64 scalars (pto_backend.py:898-915). */
+PTO_HIP_API int pto_hip_kernel_entry(int callable_id, int64_t* args, int n_tensors, int n_scalars,
+                                     void* stream);
+
+/* Register-once, launch-many timing (runtime/bench.py:1251-1267).  `tensors` holds
+ * n_sets * n_tensors descriptors; round r uses set r % n_sets, so a caller can rotate
+ * through several copies of the operands to keep the working set out of the last-level
+ * cache.  Timed with HIP events on `stream` around `rounds` back-to-back launches;
+ * *avg_us is the mean time per launch in microseconds. */
+PTO_HIP_API int pto_hip_benchmark(int callable_id, const PtoHipChipTensor* tensors, int n_sets,
+                                  int n_tensors, const uint64_t* scalars, int n_scalars,
+                                  int rounds, int warmup, void* stream, float* avg_us);
+
+/* ---- typed entry points (what pto_hip_run dispatches to) ------------------------------- */
+
+/* Paged-attention decode.  config is HOST memory; kv_dtype/q_dtype are PtoHipDataType;
+ * k_scale/v_scale are NULL unless kv_dtype == PTO_HIP_FP8E4M3FN. */
+PTO_HIP_API int pto_hip_paged_attention(const void* query, const void* key_cache,
+                                        const void* value_cache, const int32_t* block_table,
+                                        const int32_t* context_lens, float* out,
+                                        const int64_t* config, int q_dtype, int kv_dtype,
+                                        const float* k_scale, const float* v_scale, void* stream);
+
+PTO_HIP_API int pto_hip_paged_gather(const void* src, const int32_t* indices,
+                                     const int32_t* block_table, void* out, int64_t n_indices,
+                                     int64_t src_rows, int64_t src_hidden, int64_t table_len,
+                                     int64_t block_size, int64_t col_offset, int64_t size,
+                                     int elem_bytes, void* stream);
+
+PTO_HIP_API int pto_hip_rms_norm(const void* x, const float* gamma, void* out, int64_t rows,
+                                 int64_t hidden, float eps, int x_dtype, int out_dtype,
+                                 void* stream);
+
+/* out = (silu(x Wg) * (x Wu)) Wd ; gamma != NULL adds the RMSNorm prologue (ffn_block). */
+PTO_HIP_API int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void* w_gate,
+                                   const void* w_up, const void* w_down, void* out,
+                                   int64_t tokens, int64_t hidden, int64_t intermediate,
+                                   float eps, int dtype, int out_dtype, void* stream);
+
+/* ---- tuning knobs (integers by name; unknown names are PTO_HIP_ERR_NOT_FOUND) ------------
+ *  "attn_tokens_per_partition"  0 = choose from the device's CU count (default)
+ */
+PTO_HIP_API int pto_hip_set_option(const char* name, int64_t value);
+PTO_HIP_API int pto_hip_get_option(const char* name, int64_t* value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PTO_HIP_H_ */

@@ -1,0 +1,47 @@
+"""CPU oracle for the paged-attention / FFN hot path.
+
+TEST INFRASTRUCTURE ONLY.  Everything under ``oracle/`` is a CPU restatement
+(plain torch on the host) of the torch golden functions that the reference
+keeps next to its tile programs.  It is the checker the HIP path is compared
+with; nothing in the product package imports it.  Allowed importers: the
+``tests/`` tree, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py``.
+
+Pinning status (what fixes each function independently of its own formula):
+
+* ``paged_gather``            — pinned: closed-form row-id known-answer case of
+                                 the reference's own test plus permutation
+                                 invariants (tests/test_oracle_attention.py).
+* ``paged_attention_golden``  — pinned: fp64 brute-force loops on tiny shapes,
+                                 ``torch.nn.functional.scaled_dot_product_attention``
+                                 on gathered dense K/V, softmax invariants
+                                 (uniform scores -> mean of V, dominant score ->
+                                 that V row), partition independence.
+* ``ffn_swiglu`` / ``ffn_block`` — pinned: ``torch.nn.functional.silu`` form in
+                                 fp64, committed seeded fixture.
+* ``rms_norm``                — pinned: ``torch.nn.functional.rms_norm``.
+* ``rope_rotate_half``        — pinned: complex-rotation closed form, position-0
+                                 identity, norm preservation, relative-position
+                                 property.
+* fp8-e4m3 KV and W8A16       — the reference has no such path; pinned by
+                                 closed forms only (exhaustive 256-code table,
+                                 integer matmul identity).
+"""
+
+from .attention import (  # noqa: F401
+    decode_config,
+    dequant_kv_fp8,
+    paged_attention_dense,
+    paged_attention_golden,
+    paged_attention_grouped_golden,
+    paged_gather,
+    quantize_kv_fp8,
+)
+from .ffn import ffn_block, ffn_swiglu, rms_norm, swiglu  # noqa: F401
+from .layer import (  # noqa: F401
+    decoder_layer_decode,
+    quantize_w8,
+    rope_cos_sin,
+    rope_rotate_half,
+    w8a16_matmul,
+)

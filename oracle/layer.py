@@ -1,0 +1,120 @@
+"""CPU oracle: RoPE, W8A16 projections and one decoder-layer decode step.
+
+TEST INFRASTRUCTURE ONLY — see ``oracle/__init__.py``.
+
+* RoPE rotate-half                 tests/st/examples/03_llm_models/test_llama_7b_mini_1h.py:83-96,146-161
+                                   examples/models/qwen3_jit/kernels/attention.py:52-102 (decode form:
+                                   position = seq_len - 1, K/V row written into the cache)
+* layer composition                test_llama_7b_mini_1h.py:119-198,
+                                   tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:255-287
+* W8A16 (int8 weights, per-output-channel fp32 scale): the reference has no
+  such path; closed form ``w_q = clamp(round(w / s), -127, 127)``,
+  ``s = amax_col / 127``, ``y = (x @ w_q) * s``.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .attention import encode_scale, paged_attention_golden
+from .ffn import rms_norm, swiglu
+
+
+def rope_cos_sin(max_pos: int, head_dim: int, theta: float = 10000.0):
+    """cos/sin tables [max_pos, head_dim/2]: angle = pos * theta^(-2i/head_dim).
+
+    test_llama_7b_mini_1h.py:83-96 (theta 1e4 there).
+    """
+    half = head_dim // 2
+    freqs = torch.arange(half).float()
+    inv = 1.0 / (theta ** (2 * freqs / head_dim))
+    angles = torch.arange(max_pos).float().unsqueeze(1) * inv.unsqueeze(0)
+    return torch.cos(angles), torch.sin(angles)
+
+
+def rope_rotate_half(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """``lo' = lo*cos - hi*sin ; hi' = hi*cos + lo*sin`` on the last dim (fp32).
+
+    test_llama_7b_mini_1h.py:146-161.  ``cos``/``sin`` broadcast against
+    ``x[..., :half]``.
+    """
+    half = x.shape[-1] // 2
+    xf = x.float()
+    lo, hi = xf[..., :half], xf[..., half:]
+    return torch.cat([lo * cos - hi * sin, hi * cos + lo * sin], dim=-1)
+
+
+def quantize_w8(w: torch.Tensor):
+    """Per-output-channel symmetric int8: returns (w_q int8 [in,out], scale fp32 [out])."""
+    wf = w.float()
+    amax = wf.abs().amax(dim=0)
+    scale = torch.where(amax > 0, amax / 127.0, torch.ones_like(amax))
+    w_q = torch.clamp(torch.round(wf / scale), -127, 127).to(torch.int8)
+    return w_q, scale.contiguous()
+
+
+def w8a16_matmul(x: torch.Tensor, w_q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """``(x @ w_q) * scale`` with fp32 accumulation -> fp32."""
+    return torch.matmul(x.float(), w_q.float()) * scale.float().reshape(1, -1)
+
+
+def decoder_layer_decode(
+    hidden, seq_lens, block_table, key_cache, value_cache,
+    rope_cos, rope_sin, gamma_in, gamma_post,
+    wqkv_q, wqkv_s, wo_q, wo_s, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s,
+    *, num_heads: int, kv_head_num: int, head_dim: int, block_size: int,
+    max_num_blocks_per_req: int, eps: float = 1e-6,
+):
+    """One LLaMA-style decoder layer, one new token per sequence.
+
+    RMSNorm -> QKV projection -> RoPE at ``pos = seq_len - 1`` -> K/V row written
+    into the paged cache (attention.py:52-80 of the qwen3_jit kernels) -> paged
+    attention over ``seq_len`` tokens -> o_proj + residual -> RMSNorm -> SwiGLU FFN
+    + residual (test_qwen3_decode_scope3_mixed.py:255-287).  Activations are
+    rounded to the activation dtype wherever the model path casts.
+
+    Returns (out [B, H] act dtype, key_cache, value_cache) — caches are updated copies.
+    """
+    act = hidden.dtype
+    b, h = hidden.shape
+    hq, kv, d, bs = num_heads, kv_head_num, head_dim, block_size
+    key_cache = key_cache.clone()
+    value_cache = value_cache.clone()
+
+    normed = rms_norm(hidden, gamma_in, eps, out_dtype=act)
+    qkv = w8a16_matmul(normed, wqkv_q, wqkv_s)  # [B, (Hq+2Hkv)*D] fp32
+    q = qkv[:, : hq * d].reshape(b, hq, d)
+    k = qkv[:, hq * d : (hq + kv) * d].reshape(b, kv, d)
+    v = qkv[:, (hq + kv) * d :].reshape(b, kv, d)
+
+    pos = (seq_lens.long() - 1)
+    cos = rope_cos[pos].unsqueeze(1)  # [B, 1, D/2]
+    sin = rope_sin[pos].unsqueeze(1)
+    q = rope_rotate_half(q, cos, sin).to(act)
+    k = rope_rotate_half(k, cos, sin).to(act)
+    v = v.to(act)
+
+    table = block_table.reshape(b, max_num_blocks_per_req).long()
+    for bi in range(b):
+        p = int(pos[bi])
+        blk = int(table[bi, p // bs])
+        for hh in range(kv):
+            row = (blk * kv + hh) * bs + p % bs
+            key_cache[row] = k[bi, hh]
+            value_cache[row] = v[bi, hh]
+
+    config = torch.tensor(
+        [b, hq, kv, d, bs, max_num_blocks_per_req, encode_scale(1.0 / (d ** 0.5))], dtype=torch.int64
+    )
+    attn = paged_attention_golden(
+        q.reshape(b * hq, d), key_cache, value_cache, block_table, seq_lens, config
+    ).reshape(b, hq * d).to(act)
+
+    resid1 = w8a16_matmul(attn, wo_q, wo_s) + hidden.float()
+    normed2 = rms_norm(resid1, gamma_post, eps, out_dtype=act)
+    gate = w8a16_matmul(normed2, wg_q, wg_s)
+    up = w8a16_matmul(normed2, wu_q, wu_s)
+    mlp = swiglu(gate, up).to(act)
+    down = w8a16_matmul(mlp, wd_q, wd_s)
+    out = (down + resid1).to(act)
+    return out, key_cache, value_cache

@@ -1,0 +1,108 @@
+"""ctypes binding of libpto_hip.so — the only way this package reaches the GPU.
+
+There is no CPU fallback: if the shared library is missing or a call fails, an exception is
+raised.  Status codes map to the exception classes the reference raises through its
+bindings (python/bindings/modules/error.cpp:60-78).
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libpto_hip.so"
+
+OK, ERR_INVALID_VALUE, ERR_RUNTIME, ERR_NOT_INITIALIZED, ERR_UNSUPPORTED, ERR_NOT_FOUND = range(6)
+MAX_DIMS = 5
+
+# Every symbol include/pto_hip.h declares.
+EXPORTS = (
+    "pto_hip_init", "pto_hip_close", "pto_hip_last_error", "pto_hip_device_info",
+    "pto_hip_malloc", "pto_hip_free", "pto_hip_copy_to", "pto_hip_copy_from", "pto_hip_sync",
+    "pto_hip_register", "pto_hip_unregister", "pto_hip_run", "pto_hip_kernel_entry",
+    "pto_hip_benchmark", "pto_hip_paged_attention", "pto_hip_paged_gather", "pto_hip_rms_norm",
+    "pto_hip_ffn_swiglu", "pto_hip_set_option", "pto_hip_get_option",
+)
+
+
+class Buffer(C.Structure):
+    _fields_ = [("addr", C.c_uint64), ("size", C.c_uint64)]
+
+
+class ChipTensor(C.Structure):
+    _fields_ = [
+        ("buffer", Buffer),
+        ("start_offset", C.c_uint64),
+        ("shapes", C.c_uint32 * MAX_DIMS),
+        ("ndims", C.c_uint32),
+        ("dtype", C.c_uint32),
+        ("reserved", C.c_uint32),
+    ]
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [
+        ("device_id", C.c_int32),
+        ("compute_units", C.c_int32),
+        ("wavefront_size", C.c_int32),
+        ("lds_bytes_per_cu", C.c_int32),
+        ("hbm_bytes", C.c_int64),
+        ("arch", C.c_char * 32),
+    ]
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load libpto_hip.so (once) and declare the prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise RuntimeError(
+            f"{LIB_PATH} is not built. Build it with `python -m pypto_amd.build`; "
+            "this package has no other execution path."
+        )
+    lib = C.CDLL(str(LIB_PATH))
+    vp, u64, i64 = C.c_void_p, C.c_uint64, C.c_int64
+    lib.pto_hip_last_error.restype = C.c_char_p
+    lib.pto_hip_last_error.argtypes = []
+    protos = {
+        "pto_hip_init": [C.c_int],
+        "pto_hip_close": [],
+        "pto_hip_device_info": [C.POINTER(DeviceInfo)],
+        "pto_hip_malloc": [C.c_size_t, C.POINTER(u64)],
+        "pto_hip_free": [u64],
+        "pto_hip_copy_to": [u64, vp, C.c_size_t],
+        "pto_hip_copy_from": [vp, u64, C.c_size_t],
+        "pto_hip_sync": [vp],
+        "pto_hip_register": [C.c_char_p, C.POINTER(C.c_int)],
+        "pto_hip_unregister": [C.c_int],
+        "pto_hip_run": [C.c_int, C.POINTER(ChipTensor), C.c_int, C.POINTER(u64), C.c_int, vp],
+        "pto_hip_kernel_entry": [C.c_int, C.POINTER(i64), C.c_int, C.c_int, vp],
+        "pto_hip_benchmark": [C.c_int, C.POINTER(ChipTensor), C.c_int, C.c_int, C.POINTER(u64),
+                              C.c_int, C.c_int, C.c_int, vp, C.POINTER(C.c_float)],
+        "pto_hip_paged_attention": [vp, vp, vp, vp, vp, vp, C.POINTER(i64), C.c_int, C.c_int, vp, vp, vp],
+        "pto_hip_paged_gather": [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, C.c_int, vp],
+        "pto_hip_rms_norm": [vp, vp, vp, i64, i64, C.c_float, C.c_int, C.c_int, vp],
+        "pto_hip_ffn_swiglu": [vp, vp, vp, vp, vp, vp, i64, i64, i64, C.c_float, C.c_int, C.c_int, vp],
+        "pto_hip_set_option": [C.c_char_p, i64],
+        "pto_hip_get_option": [C.c_char_p, C.POINTER(i64)],
+    }
+    for name, argtypes in protos.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = C.c_int
+    _lib = lib
+    return lib
+
+
+def check(status: int) -> None:
+    """Raise the exception the reference would raise for this status."""
+    if status == OK:
+        return
+    msg = load().pto_hip_last_error().decode("utf-8", "replace")
+    if status in (ERR_INVALID_VALUE, ERR_NOT_FOUND):
+        raise ValueError(msg)
+    raise RuntimeError(msg)

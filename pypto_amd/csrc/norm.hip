@@ -1,0 +1,98 @@
+// RMSNorm: y = x * rsqrt(mean(x^2) + eps) * gamma, fp32 statistics, one workgroup per row.
+//
+// Reference tile programs: examples/intermediate/03_normalization.py:33-65 (sqrt + divide),
+// examples/models/qwen3_jit/kernels/rmsnorm.py:26-53 (two-pass chunked, cast to bf16);
+// golden tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:278-280.
+// Two passes over the row (the second one hits in cache), reduced with wave shuffles + LDS,
+// scaled and written in the output type.
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+template <typename T>
+__device__ __forceinline__ float to_f32(T v);
+template <>
+__device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ float to_f32<__bf16>(__bf16 v) { return (float)v; }
+template <>
+__device__ __forceinline__ float to_f32<_Float16>(_Float16 v) { return (float)v; }
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(kThreads) void rms_norm_kernel(const TI* __restrict__ x,
+                                                            const float* __restrict__ gamma,
+                                                            TO* __restrict__ out, int64_t hidden,
+                                                            float eps) {
+  const int64_t row = blockIdx.x;
+  const TI* xr = x + row * hidden;
+  TO* orow = out + row * hidden;
+  float ss = 0.f;
+  for (int64_t i = threadIdx.x; i < hidden; i += kThreads) {
+    const float v = to_f32<TI>(xr[i]);
+    ss += v * v;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+  __shared__ float wsum[kThreads / 64];
+  if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int w = 0; w < kThreads / 64; ++w) tot += wsum[w];
+  const float inv = rsqrtf(tot / (float)hidden + eps);
+  for (int64_t i = threadIdx.x; i < hidden; i += kThreads) {
+    float y = to_f32<TI>(xr[i]) * inv;
+    if (gamma) y *= gamma[i];
+    orow[i] = (TO)y;
+  }
+}
+
+template <typename TI>
+int launch_out(const void* x, const float* gamma, void* out, int64_t rows, int64_t hidden, float eps,
+               int out_dtype, hipStream_t st) {
+  dim3 grid((unsigned)rows), block(kThreads);
+  switch (out_dtype) {
+    case PTO_HIP_FP32:
+      hipLaunchKernelGGL((rms_norm_kernel<TI, float>), grid, block, 0, st, (const TI*)x, gamma,
+                         (float*)out, hidden, eps);
+      break;
+    case PTO_HIP_BF16:
+      hipLaunchKernelGGL((rms_norm_kernel<TI, __bf16>), grid, block, 0, st, (const TI*)x, gamma,
+                         (__bf16*)out, hidden, eps);
+      break;
+    case PTO_HIP_FP16:
+      hipLaunchKernelGGL((rms_norm_kernel<TI, _Float16>), grid, block, 0, st, (const TI*)x, gamma,
+                         (_Float16*)out, hidden, eps);
+      break;
+    default:
+      return pto_hip::fail(PTO_HIP_ERR_INVALID_VALUE, "rms_norm: out dtype %s not in {FP32, BF16, FP16}",
+                           pto_hip::dtype_name(out_dtype));
+  }
+  PTO_CHECK_HIP(hipGetLastError());
+  return PTO_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" int pto_hip_rms_norm(const void* x, const float* gamma, void* out, int64_t rows,
+                                int64_t hidden, float eps, int x_dtype, int out_dtype, void* stream) {
+  using namespace pto_hip;
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(rows >= 0 && hidden > 0, "rms_norm: bad shape [%lld, %lld]", (long long)rows, (long long)hidden);
+  PTO_CHECK_ARG(rows < (1ll << 31), "rms_norm: too many rows");
+  if (rows == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(x && out, "rms_norm: null tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+  switch (x_dtype) {
+    case PTO_HIP_FP32: return launch_out<float>(x, gamma, out, rows, hidden, eps, out_dtype, st);
+    case PTO_HIP_BF16: return launch_out<__bf16>(x, gamma, out, rows, hidden, eps, out_dtype, st);
+    case PTO_HIP_FP16: return launch_out<_Float16>(x, gamma, out, rows, hidden, eps, out_dtype, st);
+    default:
+      return fail(PTO_HIP_ERR_INVALID_VALUE, "rms_norm: x dtype %s not in {FP32, BF16, FP16}",
+                  dtype_name(x_dtype));
+  }
+}

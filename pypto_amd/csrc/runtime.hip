@@ -1,0 +1,477 @@
+// Host launcher of libpto_hip: lifecycle, device memory, the program registry and the
+// tensors-first / scalars-after dispatch that stands in for the reference's
+// Worker.register / Worker.run (python/pypto/runtime/device_runner.py:821-842) and for the
+// generated orchestration entry that unpacks ChipTensor arguments
+// (python/pypto/backend/pto_backend.py:538-645).  Work is issued on a HIP stream in program
+// order; there is no task graph and no scheduler thread.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+#include "common.h"
+
+namespace pto_hip {
+
+std::string& last_error() {
+  static thread_local std::string msg;
+  return msg;
+}
+
+int fail(int status, const char* fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  last_error() = buf;
+  return status;
+}
+
+Context& ctx() {
+  static Context c;
+  return c;
+}
+
+int workspace(size_t bytes, void** ptr) {
+  Context& c = ctx();
+  if (bytes > c.workspace_bytes) {
+    // Work queued on any stream may still read the old buffer.
+    PTO_CHECK_HIP(hipDeviceSynchronize());
+    if (c.workspace) PTO_CHECK_HIP(hipFree(c.workspace));
+    c.workspace = nullptr;
+    c.workspace_bytes = 0;
+    size_t want = bytes + bytes / 4;
+    PTO_CHECK_HIP(hipMalloc(&c.workspace, want));
+    c.workspace_bytes = want;
+  }
+  *ptr = c.workspace;
+  return PTO_HIP_OK;
+}
+
+namespace {
+
+enum ProgramKind {
+  kPagedAttention = 0,
+  kPagedGather,
+  kRmsNorm,
+  kFfnSwiglu,
+  kFfnBlock,
+  kNumPrograms
+};
+
+const char* const kProgramNames[kNumPrograms] = {"paged_attention", "paged_gather", "rms_norm",
+                                                 "ffn_swiglu", "ffn_block"};
+
+std::mutex g_mu;
+std::vector<int> g_callables;  // callable id -> ProgramKind, -1 once unregistered
+
+inline const void* tptr(const PtoHipChipTensor& t) {
+  return reinterpret_cast<const void*>(t.buffer.addr + t.start_offset * (uint64_t)dtype_bytes(t.dtype));
+}
+inline void* tptr_mut(const PtoHipChipTensor& t) { return const_cast<void*>(tptr(t)); }
+
+inline int64_t numel(const PtoHipChipTensor& t) {
+  int64_t n = 1;
+  for (uint32_t i = 0; i < t.ndims; ++i) n *= t.shapes[i];
+  return n;
+}
+
+inline float scalar_f32(uint64_t bits) {
+  uint32_t lo = (uint32_t)(bits & 0xFFFFFFFFu);
+  float f;
+  std::memcpy(&f, &lo, 4);
+  return f;
+}
+
+int check_tensor(const char* prog, const char* name, const PtoHipChipTensor& t, int ndims_min,
+                 int ndims_max) {
+  PTO_CHECK_ARG(t.ndims >= (uint32_t)ndims_min && t.ndims <= (uint32_t)ndims_max &&
+                    t.ndims <= PTO_HIP_MAX_DIMS,
+                "%s: tensor '%s' has %u dims, expected %d..%d", prog, name, t.ndims, ndims_min,
+                ndims_max);
+  PTO_CHECK_ARG(dtype_bytes(t.dtype) != 0, "%s: tensor '%s' has unknown dtype code 0x%x", prog,
+                name, t.dtype);
+  PTO_CHECK_ARG(t.buffer.addr != 0 || numel(t) == 0, "%s: tensor '%s' has a null buffer", prog,
+                name);
+  return PTO_HIP_OK;
+}
+
+// Reads the 7-slot int64 config wherever it lives.  The reference's orchestration reads it
+// with tensor.read on a host-visible buffer; a device-resident config costs one blocking copy.
+int read_config(const PtoHipChipTensor& t, hipStream_t stream, int64_t out[7]) {
+  PTO_CHECK_ARG(t.dtype == PTO_HIP_INT64 && numel(t) == 7,
+                "paged_attention: config must be INT64[7], got %s[%lld]", dtype_name(t.dtype),
+                (long long)numel(t));
+  const void* src = tptr(t);
+  hipPointerAttribute_t attr;
+  hipError_t e = hipPointerGetAttributes(&attr, src);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();  // plain host memory: not an error for us
+    std::memcpy(out, src, 7 * sizeof(int64_t));
+    return PTO_HIP_OK;
+  }
+  if (attr.type == hipMemoryTypeDevice) {
+    PTO_CHECK_HIP(hipMemcpyAsync(out, src, 7 * sizeof(int64_t), hipMemcpyDeviceToHost, stream));
+    PTO_CHECK_HIP(hipStreamSynchronize(stream));
+  } else {
+    std::memcpy(out, src, 7 * sizeof(int64_t));
+  }
+  return PTO_HIP_OK;
+}
+
+int run_paged_attention(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns,
+                        hipStream_t stream) {
+  PTO_CHECK_ARG(nt == 7 || nt == 9, "paged_attention: expected 7 tensors (9 with FP8 scales), got %d", nt);
+  PTO_CHECK_ARG(ns == 0, "paged_attention: expected no scalars, got %d", ns);
+  static const char* names[9] = {"query", "key_cache", "value_cache", "block_table", "context_lens",
+                                 "out", "config", "k_scale", "v_scale"};
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor("paged_attention", names[i], t[i], 1, 2);
+    if (rc) return rc;
+  }
+  int64_t cfg[7];
+  int rc = read_config(t[6], stream, cfg);
+  if (rc) return rc;
+  const int64_t batch = cfg[0], hq = cfg[1], hkv = cfg[2], d = cfg[3], bs = cfg[4], mb = cfg[5];
+  PTO_CHECK_ARG(batch >= 0 && hq > 0 && hkv > 0 && d > 0 && bs > 0 && mb > 0,
+                "paged_attention: config holds a non-positive dimension");
+  PTO_CHECK_ARG(t[3].dtype == PTO_HIP_INT32 && t[4].dtype == PTO_HIP_INT32,
+                "paged_attention: block_table and context_lens must be INT32");
+  PTO_CHECK_ARG(t[5].dtype == PTO_HIP_FP32, "paged_attention: out must be FP32, got %s",
+                dtype_name(t[5].dtype));
+  PTO_CHECK_ARG(numel(t[0]) == batch * hq * d, "paged_attention: query has %lld elements, config says %lld",
+                (long long)numel(t[0]), (long long)(batch * hq * d));
+  PTO_CHECK_ARG(numel(t[5]) == batch * hq * d, "paged_attention: out has %lld elements, config says %lld",
+                (long long)numel(t[5]), (long long)(batch * hq * d));
+  PTO_CHECK_ARG(numel(t[3]) >= batch * mb, "paged_attention: block_table has %lld entries, needs %lld",
+                (long long)numel(t[3]), (long long)(batch * mb));
+  PTO_CHECK_ARG(numel(t[4]) >= batch, "paged_attention: context_lens has %lld entries, needs %lld",
+                (long long)numel(t[4]), (long long)batch);
+  PTO_CHECK_ARG(numel(t[1]) % (hkv * bs * d) == 0 && numel(t[1]) == numel(t[2]) &&
+                    t[1].dtype == t[2].dtype,
+                "paged_attention: key/value cache must be equal-shaped [pool*Hkv*bs, D]");
+  const float* ks = nullptr;
+  const float* vs = nullptr;
+  if (t[1].dtype == PTO_HIP_FP8E4M3FN) {
+    PTO_CHECK_ARG(nt == 9, "paged_attention: FP8E4M3FN cache needs k_scale and v_scale tensors");
+    const int64_t pool = numel(t[1]) / (hkv * bs * d);
+    PTO_CHECK_ARG(t[7].dtype == PTO_HIP_FP32 && t[8].dtype == PTO_HIP_FP32 &&
+                      numel(t[7]) == pool * hkv && numel(t[8]) == pool * hkv,
+                  "paged_attention: k_scale/v_scale must be FP32[pool_blocks, Hkv]");
+    ks = reinterpret_cast<const float*>(tptr(t[7]));
+    vs = reinterpret_cast<const float*>(tptr(t[8]));
+  }
+  return pto_hip_paged_attention(tptr(t[0]), tptr(t[1]), tptr(t[2]),
+                                 reinterpret_cast<const int32_t*>(tptr(t[3])),
+                                 reinterpret_cast<const int32_t*>(tptr(t[4])),
+                                 reinterpret_cast<float*>(tptr_mut(t[5])), cfg, (int)t[0].dtype,
+                                 (int)t[1].dtype, ks, vs, stream);
+}
+
+int run_paged_gather(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns,
+                     hipStream_t stream) {
+  PTO_CHECK_ARG(nt == 4 && ns == 2,
+                "paged_gather: expected 4 tensors + 2 scalars (block_size, col_offset), got %d + %d",
+                nt, ns);
+  static const char* names[4] = {"src", "indices", "block_table", "out"};
+  for (int i = 0; i < 4; ++i) {
+    int rc = check_tensor("paged_gather", names[i], t[i], 1, 2);
+    if (rc) return rc;
+  }
+  PTO_CHECK_ARG(t[0].ndims == 2 && t[3].ndims == 2, "paged_gather: src and out must be 2-D");
+  PTO_CHECK_ARG(t[1].dtype == PTO_HIP_INT32 && t[2].dtype == PTO_HIP_INT32,
+                "paged_gather: indices and block_table must be INT32");
+  PTO_CHECK_ARG(t[0].dtype == t[3].dtype, "paged_gather: out dtype %s differs from src dtype %s",
+                dtype_name(t[3].dtype), dtype_name(t[0].dtype));
+  PTO_CHECK_ARG(t[3].shapes[0] == numel(t[1]), "paged_gather: out has %u rows for %lld indices",
+                t[3].shapes[0], (long long)numel(t[1]));
+  return pto_hip_paged_gather(tptr(t[0]), reinterpret_cast<const int32_t*>(tptr(t[1])),
+                              reinterpret_cast<const int32_t*>(tptr(t[2])), tptr_mut(t[3]),
+                              numel(t[1]), t[0].shapes[0], t[0].shapes[1], numel(t[2]),
+                              (int64_t)s[0], (int64_t)s[1], t[3].shapes[1],
+                              dtype_bytes(t[0].dtype), stream);
+}
+
+int run_rms_norm(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream) {
+  PTO_CHECK_ARG(nt == 3 && ns == 1, "rms_norm: expected 3 tensors + 1 scalar (eps), got %d + %d", nt, ns);
+  static const char* names[3] = {"x", "gamma", "out"};
+  for (int i = 0; i < 3; ++i) {
+    int rc = check_tensor("rms_norm", names[i], t[i], 1, 2);
+    if (rc) return rc;
+  }
+  PTO_CHECK_ARG(t[0].ndims == 2, "rms_norm: x must be 2-D");
+  const int64_t rows = t[0].shapes[0], hidden = t[0].shapes[1];
+  PTO_CHECK_ARG(t[1].dtype == PTO_HIP_FP32 && numel(t[1]) == hidden,
+                "rms_norm: gamma must be FP32 with %lld elements", (long long)hidden);
+  PTO_CHECK_ARG(numel(t[2]) == rows * hidden, "rms_norm: out shape differs from x");
+  return pto_hip_rms_norm(tptr(t[0]), reinterpret_cast<const float*>(tptr(t[1])), tptr_mut(t[2]),
+                          rows, hidden, scalar_f32(s[0]), (int)t[0].dtype, (int)t[2].dtype, stream);
+}
+
+int run_ffn(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream,
+            bool with_norm) {
+  const char* prog = with_norm ? "ffn_block" : "ffn_swiglu";
+  const int want_t = with_norm ? 6 : 5, want_s = with_norm ? 1 : 0;
+  PTO_CHECK_ARG(nt == want_t && ns == want_s, "%s: expected %d tensors + %d scalars, got %d + %d",
+                prog, want_t, want_s, nt, ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor(prog, "operand", t[i], 2, 2);
+    if (rc) return rc;
+  }
+  const PtoHipChipTensor& x = t[0];
+  const int w0 = with_norm ? 2 : 1;
+  const PtoHipChipTensor &wg = t[w0], &wu = t[w0 + 1], &wd = t[w0 + 2], &out = t[w0 + 3];
+  const int64_t tokens = x.shapes[0], hidden = x.shapes[1], inter = wg.shapes[1];
+  PTO_CHECK_ARG(wg.shapes[0] == hidden && wu.shapes[0] == hidden && wu.shapes[1] == inter &&
+                    wd.shapes[0] == inter && wd.shapes[1] == hidden,
+                "%s: weight shapes must be gate/up [H,I] and down [I,H] with H=%lld", prog,
+                (long long)hidden);
+  PTO_CHECK_ARG(wg.dtype == x.dtype && wu.dtype == x.dtype && wd.dtype == x.dtype,
+                "%s: weights must have the dtype of x (%s)", prog, dtype_name(x.dtype));
+  PTO_CHECK_ARG(out.shapes[0] == tokens && out.shapes[1] == hidden, "%s: out must be [T,H]", prog);
+  const float* gamma = nullptr;
+  float eps = 0.f;
+  if (with_norm) {
+    PTO_CHECK_ARG(t[1].dtype == PTO_HIP_FP32 && numel(t[1]) == hidden,
+                  "%s: gamma must be FP32 with %lld elements", prog, (long long)hidden);
+    gamma = reinterpret_cast<const float*>(tptr(t[1]));
+    eps = scalar_f32(s[0]);
+  }
+  return pto_hip_ffn_swiglu(tptr(x), gamma, tptr(wg), tptr(wu), tptr(wd), tptr_mut(out), tokens,
+                            hidden, inter, eps, (int)x.dtype, (int)out.dtype, stream);
+}
+
+int dispatch(int kind, const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns,
+             hipStream_t stream) {
+  switch (kind) {
+    case kPagedAttention: return run_paged_attention(t, nt, s, ns, stream);
+    case kPagedGather: return run_paged_gather(t, nt, s, ns, stream);
+    case kRmsNorm: return run_rms_norm(t, nt, s, ns, stream);
+    case kFfnSwiglu: return run_ffn(t, nt, s, ns, stream, false);
+    case kFfnBlock: return run_ffn(t, nt, s, ns, stream, true);
+    default: return fail(PTO_HIP_ERR_NOT_FOUND, "unknown program kind %d", kind);
+  }
+}
+
+int lookup(int callable_id, int* kind) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (callable_id < 0 || (size_t)callable_id >= g_callables.size() || g_callables[callable_id] < 0)
+    return fail(PTO_HIP_ERR_NOT_FOUND, "callable id %d is not registered", callable_id);
+  *kind = g_callables[callable_id];
+  return PTO_HIP_OK;
+}
+
+}  // namespace
+}  // namespace pto_hip
+
+using namespace pto_hip;
+
+extern "C" {
+
+const char* pto_hip_last_error(void) { return last_error().c_str(); }
+
+int pto_hip_init(int device_id) {
+  Context& c = ctx();
+  int n = 0;
+  PTO_CHECK_HIP(hipGetDeviceCount(&n));
+  PTO_CHECK_ARG(device_id >= 0 && device_id < n, "device_id %d out of range: %d device(s) visible",
+                device_id, n);
+  if (c.initialized && c.device != device_id)
+    return fail(PTO_HIP_ERR_INVALID_VALUE,
+                "already initialised on device %d; close before binding device %d", c.device,
+                device_id);
+  PTO_CHECK_HIP(hipSetDevice(device_id));
+  hipDeviceProp_t prop;
+  PTO_CHECK_HIP(hipGetDeviceProperties(&prop, device_id));
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(PTO_HIP_ERR_UNSUPPORTED, "device %d is %s; this library is built for gfx950 only",
+                device_id, prop.gcnArchName);
+  c.device = device_id;
+  c.num_cu = prop.multiProcessorCount;
+  if (!c.flags) PTO_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&c.flags), 256));
+  c.initialized = true;
+  ++c.refcount;
+  return PTO_HIP_OK;
+}
+
+int pto_hip_close(void) {
+  Context& c = ctx();
+  if (!c.initialized) return PTO_HIP_OK;
+  if (--c.refcount > 0) return PTO_HIP_OK;  // another worker still holds the device
+  c.refcount = 0;
+  PTO_CHECK_HIP(hipDeviceSynchronize());
+  if (c.workspace) PTO_CHECK_HIP(hipFree(c.workspace));
+  c.workspace = nullptr;
+  c.workspace_bytes = 0;
+  if (c.flags) PTO_CHECK_HIP(hipFree(c.flags));
+  c.flags = nullptr;
+  c.initialized = false;
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_callables.clear();
+  }
+  return PTO_HIP_OK;
+}
+
+int pto_hip_device_info(PtoHipDeviceInfo* info) {
+  Context& c = ctx();
+  if (!c.initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(info != nullptr, "device_info: null output");
+  hipDeviceProp_t prop;
+  PTO_CHECK_HIP(hipGetDeviceProperties(&prop, c.device));
+  std::memset(info, 0, sizeof(*info));
+  info->device_id = c.device;
+  info->compute_units = prop.multiProcessorCount;
+  info->wavefront_size = prop.warpSize;
+  info->lds_bytes_per_cu = (int32_t)prop.maxSharedMemoryPerMultiProcessor;
+  info->hbm_bytes = (int64_t)prop.totalGlobalMem;
+  std::strncpy(info->arch, prop.gcnArchName, sizeof(info->arch) - 1);
+  for (char* ch = info->arch; *ch; ++ch)
+    if (*ch == ':') { *ch = 0; break; }
+  return PTO_HIP_OK;
+}
+
+int pto_hip_malloc(size_t nbytes, uint64_t* dev_ptr) {
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(dev_ptr != nullptr, "malloc: null output");
+  void* p = nullptr;
+  if (nbytes > 0) PTO_CHECK_HIP(hipMalloc(&p, nbytes));
+  *dev_ptr = reinterpret_cast<uint64_t>(p);
+  return PTO_HIP_OK;
+}
+
+int pto_hip_free(uint64_t dev_ptr) {
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  if (dev_ptr) PTO_CHECK_HIP(hipFree(reinterpret_cast<void*>(dev_ptr)));
+  return PTO_HIP_OK;
+}
+
+int pto_hip_copy_to(uint64_t dst_dev_ptr, const void* src_host_ptr, size_t nbytes) {
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  if (nbytes == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(dst_dev_ptr && src_host_ptr, "copy_to: null pointer");
+  PTO_CHECK_HIP(hipMemcpy(reinterpret_cast<void*>(dst_dev_ptr), src_host_ptr, nbytes, hipMemcpyHostToDevice));
+  return PTO_HIP_OK;
+}
+
+int pto_hip_copy_from(void* dst_host_ptr, uint64_t src_dev_ptr, size_t nbytes) {
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  if (nbytes == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(dst_host_ptr && src_dev_ptr, "copy_from: null pointer");
+  PTO_CHECK_HIP(hipMemcpy(dst_host_ptr, reinterpret_cast<const void*>(src_dev_ptr), nbytes, hipMemcpyDeviceToHost));
+  return PTO_HIP_OK;
+}
+
+int pto_hip_sync(void* stream) {
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
+  return PTO_HIP_OK;
+}
+
+int pto_hip_register(const char* program_name, int* callable_id) {
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(program_name && callable_id, "register: null argument");
+  for (int k = 0; k < kNumPrograms; ++k) {
+    if (std::strcmp(program_name, kProgramNames[k]) == 0) {
+      std::lock_guard<std::mutex> lk(g_mu);
+      g_callables.push_back(k);
+      *callable_id = (int)g_callables.size() - 1;
+      return PTO_HIP_OK;
+    }
+  }
+  return fail(PTO_HIP_ERR_NOT_FOUND, "no HIP program named '%s'", program_name);
+}
+
+int pto_hip_unregister(int callable_id) {
+  int kind;
+  int rc = lookup(callable_id, &kind);
+  if (rc) return rc;
+  std::lock_guard<std::mutex> lk(g_mu);
+  g_callables[callable_id] = -1;
+  return PTO_HIP_OK;
+}
+
+int pto_hip_run(int callable_id, const PtoHipChipTensor* tensors, int n_tensors,
+                const uint64_t* scalars, int n_scalars, void* stream) {
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  int kind;
+  int rc = lookup(callable_id, &kind);
+  if (rc) return rc;
+  PTO_CHECK_ARG(n_tensors >= 0 && n_scalars >= 0 && (tensors || n_tensors == 0) &&
+                    (scalars || n_scalars == 0),
+                "run: bad argument arrays");
+  return dispatch(kind, tensors, n_tensors, scalars, n_scalars, (hipStream_t)stream);
+}
+
+int pto_hip_kernel_entry(int callable_id, int64_t* args, int n_tensors, int n_scalars, void* stream) {
+  PTO_CHECK_ARG(args || (n_tensors + n_scalars) == 0, "kernel_entry: null args");
+  PTO_CHECK_ARG(n_tensors >= 0 && n_tensors <= 64 && n_scalars >= 0 && n_scalars <= 64,
+                "kernel_entry: argument counts out of range");
+  PtoHipChipTensor t[64];
+  uint64_t s[64];
+  for (int i = 0; i < n_tensors; ++i) {
+    PTO_CHECK_ARG(args[i] != 0, "kernel_entry: tensor argument %d is null", i);
+    t[i] = *reinterpret_cast<const PtoHipChipTensor*>(args[i]);
+  }
+  for (int i = 0; i < n_scalars; ++i) s[i] = (uint64_t)args[n_tensors + i];
+  return pto_hip_run(callable_id, t, n_tensors, s, n_scalars, stream);
+}
+
+int pto_hip_benchmark(int callable_id, const PtoHipChipTensor* tensors, int n_sets, int n_tensors,
+                      const uint64_t* scalars, int n_scalars, int rounds, int warmup, void* stream,
+                      float* avg_us) {
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(n_sets >= 1 && rounds >= 1 && warmup >= 0 && avg_us, "benchmark: bad arguments");
+  hipStream_t st = (hipStream_t)stream;
+  for (int r = 0; r < warmup; ++r) {
+    int rc = pto_hip_run(callable_id, tensors + (size_t)(r % n_sets) * n_tensors, n_tensors, scalars,
+                         n_scalars, stream);
+    if (rc) return rc;
+  }
+  hipEvent_t e0, e1;
+  PTO_CHECK_HIP(hipEventCreate(&e0));
+  PTO_CHECK_HIP(hipEventCreate(&e1));
+  PTO_CHECK_HIP(hipStreamSynchronize(st));
+  PTO_CHECK_HIP(hipEventRecord(e0, st));
+  int rc = PTO_HIP_OK;
+  for (int r = 0; r < rounds && rc == PTO_HIP_OK; ++r)
+    rc = pto_hip_run(callable_id, tensors + (size_t)(r % n_sets) * n_tensors, n_tensors, scalars,
+                     n_scalars, stream);
+  hipError_t e = hipEventRecord(e1, st);
+  if (e == hipSuccess) e = hipEventSynchronize(e1);
+  float ms = 0.f;
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc) return rc;
+  if (e != hipSuccess) return fail(PTO_HIP_ERR_RUNTIME, "benchmark timing failed: %s", hipGetErrorString(e));
+  *avg_us = ms * 1000.f / (float)rounds;
+  return PTO_HIP_OK;
+}
+
+int pto_hip_set_option(const char* name, int64_t value) {
+  PTO_CHECK_ARG(name != nullptr, "set_option: null name");
+  Context& c = ctx();
+  if (!std::strcmp(name, "attn_tokens_per_partition")) {
+    PTO_CHECK_ARG(value >= 0, "attn_tokens_per_partition must be >= 0");
+    c.attn_tokens_per_partition = value;
+  } else if (!std::strcmp(name, "gemm_variant")) {
+    c.gemm_variant = value;
+  } else {
+    return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
+  }
+  return PTO_HIP_OK;
+}
+
+int pto_hip_get_option(const char* name, int64_t* value) {
+  PTO_CHECK_ARG(name && value, "get_option: null argument");
+  Context& c = ctx();
+  if (!std::strcmp(name, "attn_tokens_per_partition")) *value = c.attn_tokens_per_partition;
+  else if (!std::strcmp(name, "gemm_variant")) *value = c.gemm_variant;
+  else return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
+  return PTO_HIP_OK;
+}
+
+}  // extern "C"

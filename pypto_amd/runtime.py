@@ -1,0 +1,527 @@
+"""Run-side API of the MI355X path, in the shape of ``pypto.runtime``.
+
+Mirrors, for the HIP target, the reference's run-side surface so that a test written for the
+reference reads the same here:
+
+* ``RunConfig``          python/pypto/runtime/runner.py:155-384  (platform whitelist, rtol/atol)
+* ``DeviceTensor``       python/pypto/runtime/device_tensor.py:43-110
+* ``ChipWorker``         python/pypto/runtime/worker.py:118-673  (init/close, malloc/free,
+                         copy_to/copy_from, alloc_tensor/free_tensor, run, register)
+* ``RegistrationHandle`` python/pypto/runtime/worker.py:675-773
+* ``run``                python/pypto/runtime/runner.py:628-682
+* ``benchmark``          python/pypto/runtime/bench.py:1267
+* ``validate_golden``    python/pypto/runtime/device_runner.py:850-899
+
+Everything executes through libpto_hip.so (``pypto_amd._lib``); there is no CPU path.
+Host tensors must be CPU and contiguous (runner.py:930-939); outputs are written back in
+place into the caller's tensors and nothing is returned (device_runner.py:751-755).
+"""
+
+from __future__ import annotations
+
+import contextvars
+import ctypes as C
+import struct
+from dataclasses import dataclass
+from typing import Any, Sequence
+
+import torch
+
+from . import _lib
+
+PLATFORMS = ("mi355x",)
+
+# torch dtype -> DataType code (include/pypto/core/dtype.h:48-96)
+_DTYPE_CODES = {
+    torch.int8: 0x11,
+    torch.int32: 0x13,
+    torch.int64: 0x14,
+    torch.float8_e4m3fn: 0x31,
+    torch.float16: 0x33,
+    torch.float32: 0x34,
+    torch.bfloat16: 0x40,
+}
+
+IN, OUT, INOUT = "IN", "OUT", "INOUT"
+HOST = "HOST"  # read on the host by the launcher; never copied to the device
+
+
+@dataclass(frozen=True)
+class HipProgram:
+    """A tile program the HIP target has a kernel for, with its tensor signature.
+
+    The counterpart of a ``CompiledProgram`` whose manifest lists per-tensor IN/OUT/INOUT
+    directions (python/pypto/backend/pto_backend.py:933-1045).
+    """
+
+    name: str
+    signature: tuple[str, ...]
+    optional: int = 0  # trailing tensors that may be omitted
+    scalars: tuple[str, ...] = ()
+
+    def __call__(self, *args: Any, config: "RunConfig | None" = None) -> None:
+        run(self, *args, config=config)
+
+
+paged_attention = HipProgram("paged_attention", (IN, IN, IN, IN, IN, OUT, HOST, IN, IN), optional=2)
+paged_gather = HipProgram("paged_gather", (IN, IN, IN, OUT), scalars=("block_size", "col_offset"))
+rms_norm = HipProgram("rms_norm", (IN, IN, OUT), scalars=("eps",))
+ffn_swiglu = HipProgram("ffn_swiglu", (IN, IN, IN, IN, OUT))
+ffn_block = HipProgram("ffn_block", (IN, IN, IN, IN, IN, OUT), scalars=("eps",))
+
+PROGRAMS = {p.name: p for p in (paged_attention, paged_gather, rms_norm, ffn_swiglu, ffn_block)}
+
+
+@dataclass
+class RunConfig:
+    """Configuration of one run (subset of runner.py:155-365 that applies to the HIP target)."""
+
+    platform: str = "mi355x"
+    device_id: int = 0
+    rtol: float = 1e-5
+    atol: float = 1e-5
+
+    def __post_init__(self) -> None:
+        if self.platform not in PLATFORMS:
+            raise ValueError(f"Invalid platform {self.platform!r}. Expected 'mi355x'.")
+        if isinstance(self.device_id, bool) or not isinstance(self.device_id, int) or self.device_id < 0:
+            raise ValueError(f"device_id must be a non-negative int, got {self.device_id!r}")
+
+
+class DeviceTensor:
+    """Handle to a buffer already resident on a worker (device_tensor.py:43-110)."""
+
+    def __init__(self, data_ptr: int, shape: Sequence[int], dtype: torch.dtype) -> None:
+        if isinstance(data_ptr, bool) or not isinstance(data_ptr, int) or data_ptr <= 0:
+            raise ValueError(f"DeviceTensor.data_ptr must be a positive int, got {data_ptr!r}")
+        raw_shape = tuple(shape)
+        for d in raw_shape:
+            if isinstance(d, bool) or not isinstance(d, int):
+                raise TypeError(f"DeviceTensor.shape must contain ints, got {raw_shape!r}")
+        if not raw_shape:
+            raise ValueError("DeviceTensor.shape must be non-empty")
+        if any(d <= 0 for d in raw_shape):
+            raise ValueError(f"DeviceTensor.shape must be all positive, got {raw_shape}")
+        if not isinstance(dtype, torch.dtype):
+            raise TypeError(f"DeviceTensor.dtype must be torch.dtype, got {type(dtype).__name__}")
+        self.data_ptr = data_ptr
+        self.shape = raw_shape
+        self.dtype = dtype
+
+    @property
+    def nbytes(self) -> int:
+        n = torch.tensor([], dtype=self.dtype).element_size()
+        for d in self.shape:
+            n *= d
+        return n
+
+    def __repr__(self) -> str:
+        return f"DeviceTensor(data_ptr=0x{self.data_ptr:x}, shape={self.shape}, dtype={self.dtype})"
+
+
+def scalar_to_uint64(value: Any) -> int:
+    """Raw 64-bit pattern of a scalar argument; floats travel as fp32 bits (runner.py:948-953)."""
+    if isinstance(value, bool):
+        return int(value)
+    if isinstance(value, int):
+        return value & 0xFFFFFFFFFFFFFFFF
+    if isinstance(value, float):
+        return struct.unpack("I", struct.pack("f", value))[0]
+    raise TypeError(f"unsupported scalar type {type(value).__name__}")
+
+
+def _dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODES[dtype]
+    except KeyError:
+        raise ValueError(f"dtype {dtype} has no DataType code on the HIP target") from None
+
+
+def _descriptor(ptr: int, shape: Sequence[int], dtype: torch.dtype, nbytes: int) -> _lib.ChipTensor:
+    if len(shape) > _lib.MAX_DIMS:
+        raise ValueError(f"tensors of more than {_lib.MAX_DIMS} dims are not supported, got {tuple(shape)}")
+    t = _lib.ChipTensor()
+    t.buffer.addr = ptr
+    t.buffer.size = nbytes
+    t.start_offset = 0
+    for i, d in enumerate(shape):
+        t.shapes[i] = d
+    t.ndims = len(shape)
+    t.dtype = _dtype_code(dtype)
+    return t
+
+
+_active_worker: contextvars.ContextVar["ChipWorker | None"] = contextvars.ContextVar(
+    "pypto_amd_active_worker", default=None
+)
+
+
+class ChipWorker:
+    """Single-GPU execution handle bound to one ``(platform, device_id)`` (worker.py:118-673).
+
+    Inside ``with ChipWorker(...)`` the module-level :func:`run` reuses this worker instead of
+    creating a one-shot one.
+    """
+
+    def __init__(self, config: RunConfig | None = None, *, level: int = 2, auto_init: bool = True) -> None:
+        if level != 2:
+            raise ValueError(
+                f"ChipWorker only supports level=2; got level={level}. "
+                f"L3+ runtimes go through DistributedWorker."
+            )
+        self._config = config or RunConfig()
+        self._lib = _lib.load()
+        self._initialized = False
+        self._owned: dict[int, int] = {}  # device ptr -> nbytes (alloc_tensor / malloc)
+        self._handles: list[RegistrationHandle] = []
+        self._token = None
+        if auto_init:
+            self.init()
+
+    # ---- lifecycle -------------------------------------------------------------------
+    def init(self) -> None:
+        if self._initialized:
+            return
+        _lib.check(self._lib.pto_hip_init(self._config.device_id))
+        self._initialized = True
+
+    def close(self) -> None:
+        if not self._initialized:
+            return
+        for h in self._handles:
+            h._mark_closed()
+        self._handles.clear()
+        for ptr in list(self._owned):
+            _lib.check(self._lib.pto_hip_free(ptr))
+        self._owned.clear()
+        _lib.check(self._lib.pto_hip_close())
+        self._initialized = False
+
+    def __enter__(self) -> "ChipWorker":
+        self.init()
+        self._token = _active_worker.set(self)
+        return self
+
+    def __exit__(self, *_exc: Any) -> None:
+        if self._token is not None:
+            _active_worker.reset(self._token)
+            self._token = None
+        self.close()
+
+    @staticmethod
+    def current() -> "ChipWorker | None":
+        return _active_worker.get()
+
+    @property
+    def initialized(self) -> bool:
+        return self._initialized
+
+    @property
+    def platform(self) -> str:
+        return self._config.platform
+
+    @property
+    def device_id(self) -> int:
+        return self._config.device_id
+
+    @property
+    def level(self) -> int:
+        return 2
+
+    def _require_ready(self, op: str) -> None:
+        if not self._initialized:
+            raise RuntimeError(f"ChipWorker.{op}() called on a worker that is not initialized")
+
+    def device_info(self) -> dict:
+        self._require_ready("device_info")
+        info = _lib.DeviceInfo()
+        _lib.check(self._lib.pto_hip_device_info(C.byref(info)))
+        return {
+            "device_id": info.device_id,
+            "compute_units": info.compute_units,
+            "wavefront_size": info.wavefront_size,
+            "lds_bytes_per_cu": info.lds_bytes_per_cu,
+            "hbm_bytes": info.hbm_bytes,
+            "arch": info.arch.decode(),
+        }
+
+    def set_option(self, name: str, value: int) -> None:
+        _lib.check(self._lib.pto_hip_set_option(name.encode(), int(value)))
+
+    # ---- raw memory (runtime_base.py:106-118) -------------------------------------------
+    def malloc(self, nbytes: int) -> int:
+        self._require_ready("malloc")
+        ptr = C.c_uint64(0)
+        _lib.check(self._lib.pto_hip_malloc(int(nbytes), C.byref(ptr)))
+        self._owned[ptr.value] = int(nbytes)
+        return ptr.value
+
+    def free(self, ptr: int) -> None:
+        self._require_ready("free")
+        if ptr not in self._owned:
+            raise ValueError(f"pointer 0x{ptr:x} was not allocated by this worker")
+        _lib.check(self._lib.pto_hip_free(ptr))
+        del self._owned[ptr]
+
+    def copy_to(self, dst_dev_ptr: int, src_host_ptr: int, nbytes: int) -> None:
+        self._require_ready("copy_to")
+        _lib.check(self._lib.pto_hip_copy_to(dst_dev_ptr, src_host_ptr, int(nbytes)))
+
+    def copy_from(self, dst_host_ptr: int, src_dev_ptr: int, nbytes: int) -> None:
+        self._require_ready("copy_from")
+        _lib.check(self._lib.pto_hip_copy_from(dst_host_ptr, src_dev_ptr, int(nbytes)))
+
+    def sync(self, stream: int = 0) -> None:
+        self._require_ready("sync")
+        _lib.check(self._lib.pto_hip_sync(stream))
+
+    # ---- resident tensors (runtime_base.py:228-314) -------------------------------------
+    def alloc_tensor(self, shape: Sequence[int], dtype: torch.dtype, *, init: torch.Tensor | None = None) -> DeviceTensor:
+        self._require_ready("alloc_tensor")
+        shape = tuple(int(d) for d in shape)
+        nbytes = torch.tensor([], dtype=dtype).element_size()
+        for d in shape:
+            nbytes *= d
+        ptr = self.malloc(nbytes)
+        t = DeviceTensor(ptr, shape, dtype)
+        if init is not None:
+            _check_host_tensor(init, "init")
+            if tuple(init.shape) != shape or init.dtype != dtype:
+                raise ValueError(f"init has shape {tuple(init.shape)}/{init.dtype}, expected {shape}/{dtype}")
+            self.copy_to(ptr, init.data_ptr(), nbytes)
+        return t
+
+    def free_tensor(self, t: DeviceTensor) -> None:
+        self.free(t.data_ptr)
+
+    def to_host(self, t: DeviceTensor) -> torch.Tensor:
+        out = torch.empty(t.shape, dtype=t.dtype)
+        self.copy_from(out.data_ptr(), t.data_ptr, t.nbytes)
+        return out
+
+    # ---- dispatch -------------------------------------------------------------------
+    def register(self, program: HipProgram) -> "RegistrationHandle":
+        self._require_ready("register")
+        if not isinstance(program, HipProgram):
+            raise TypeError(f"register() expects a HipProgram, got {type(program).__name__}")
+        cid = C.c_int(-1)
+        _lib.check(self._lib.pto_hip_register(program.name.encode(), C.byref(cid)))
+        h = RegistrationHandle(self, cid.value, program)
+        self._handles.append(h)
+        return h
+
+    def run(self, program: HipProgram, *args: Any, config: RunConfig | None = None, stream: int = 0) -> None:
+        with self.register(program) as h:
+            h(*args, config=config, stream=stream)
+
+    def _dispatch(self, cid: int, program: HipProgram, args: Sequence[Any], stream: int) -> None:
+        tensors, scalars = _split_args(program, args)
+        staged: list[tuple[torch.Tensor, int, int]] = []  # (host tensor, dev ptr, nbytes) to copy back
+        temps: list[int] = []
+        descs = (_lib.ChipTensor * len(tensors))()
+        try:
+            for i, (arg, direction) in enumerate(zip(tensors, program.signature)):
+                if isinstance(arg, DeviceTensor):
+                    descs[i] = _descriptor(arg.data_ptr, arg.shape, arg.dtype, arg.nbytes)
+                elif isinstance(arg, torch.Tensor) and arg.is_cuda:
+                    if not arg.is_contiguous():
+                        raise ValueError(f"tensor argument {i} must be contiguous")
+                    nbytes = arg.numel() * arg.element_size()
+                    descs[i] = _descriptor(arg.data_ptr() or 1, tuple(arg.shape), arg.dtype, nbytes)
+                elif isinstance(arg, torch.Tensor):
+                    _check_host_tensor(arg, f"argument {i}")
+                    nbytes = arg.numel() * arg.element_size()
+                    if direction == HOST:
+                        descs[i] = _descriptor(arg.data_ptr(), tuple(arg.shape), arg.dtype, nbytes)
+                        continue
+                    ptr = self.malloc(max(nbytes, 1))
+                    temps.append(ptr)
+                    if direction in (IN, INOUT) and nbytes:
+                        self.copy_to(ptr, arg.data_ptr(), nbytes)
+                    if direction in (OUT, INOUT):
+                        staged.append((arg, ptr, nbytes))
+                    descs[i] = _descriptor(ptr, tuple(arg.shape), arg.dtype, nbytes)
+                else:
+                    raise TypeError(
+                        f"tensor argument {i} must be a torch.Tensor or DeviceTensor, got {type(arg).__name__}"
+                    )
+            sc = (C.c_uint64 * max(len(scalars), 1))(*[scalar_to_uint64(s) for s in scalars])
+            _lib.check(self._lib.pto_hip_run(cid, descs, len(tensors), sc, len(scalars), stream))
+            if staged or temps:
+                self.sync(stream)
+            for host, ptr, nbytes in staged:
+                if nbytes:
+                    self.copy_from(host.data_ptr(), ptr, nbytes)
+        finally:
+            for ptr in temps:
+                self.free(ptr)
+
+
+class RegistrationHandle:
+    """A program registered once on a worker, callable many times (worker.py:675-773)."""
+
+    def __init__(self, worker: ChipWorker, cid: int, program: HipProgram) -> None:
+        self._worker = worker
+        self._cid = cid
+        self._program = program
+        self._closed = False
+
+    @property
+    def cid(self) -> int:
+        return self._cid
+
+    @property
+    def compiled(self) -> HipProgram:
+        return self._program
+
+    @property
+    def closed(self) -> bool:
+        return self._closed
+
+    def __call__(self, *args: Any, config: RunConfig | None = None, stream: int = 0) -> None:
+        if self._closed:
+            raise RuntimeError("RegistrationHandle is closed")
+        self._worker._dispatch(self._cid, self._program, args, stream)
+
+    def unregister(self) -> None:
+        if self._closed:
+            return
+        _lib.check(self._worker._lib.pto_hip_unregister(self._cid))
+        self._closed = True
+
+    def _mark_closed(self) -> None:
+        self._closed = True
+
+    def __enter__(self) -> "RegistrationHandle":
+        return self
+
+    def __exit__(self, *_exc: Any) -> None:
+        self.unregister()
+
+
+def _check_host_tensor(t: torch.Tensor, what: str) -> None:
+    if t.device.type != "cpu":
+        raise ValueError(f"{what} must be a CPU tensor, got device {t.device}")
+    if not t.is_contiguous():
+        raise ValueError(f"{what} must be contiguous")
+
+
+def _split_args(program: HipProgram, args: Sequence[Any]) -> tuple[list[Any], list[Any]]:
+    n_t_max = len(program.signature)
+    n_t_min = n_t_max - program.optional
+    n_s = len(program.scalars)
+    n = len(args)
+    if not (n_t_min + n_s <= n <= n_t_max + n_s):
+        raise ValueError(
+            f"{program.name} takes {n_t_min}..{n_t_max} tensors followed by {n_s} scalar(s) "
+            f"{program.scalars}, got {n} argument(s)"
+        )
+    n_t = n - n_s
+    return list(args[:n_t]), list(args[n_t:])
+
+
+def run(program: HipProgram, *tensors: Any, config: RunConfig | None = None) -> HipProgram:
+    """Execute *program* with *tensors* (then scalars) on the device; outputs are updated in place.
+
+    Counterpart of ``pypto.runtime.run`` (runner.py:628-682).  Reuses the worker of an
+    enclosing ``with ChipWorker(...)``; otherwise opens a one-shot worker.
+    """
+    if isinstance(program, str):
+        program = PROGRAMS[program]
+    config = config or RunConfig()
+    worker = ChipWorker.current()
+    if worker is not None and worker.initialized and worker.device_id == config.device_id:
+        worker.run(program, *tensors, config=config)
+    else:
+        w = ChipWorker(config)
+        try:
+            w.run(program, *tensors, config=config)
+        finally:
+            w.close()
+    return program
+
+
+@dataclass
+class BenchmarkStats:
+    rounds: int
+    warmup: int
+    device_wall_us: float  # mean device time per launch
+
+    @property
+    def avg_us(self) -> float:
+        return self.device_wall_us
+
+
+def benchmark(
+    handle: RegistrationHandle,
+    arg_sets: Sequence[Sequence[Any]],
+    *,
+    rounds: int = 100,
+    warmup: int = 3,
+    stream: int = 0,
+) -> BenchmarkStats:
+    """Register-once, launch-many timing with HIP events (bench.py:1251-1267).
+
+    ``arg_sets`` holds one or more complete argument lists of device-resident tensors; the
+    rounds cycle through them so a caller can keep the working set larger than the
+    last-level cache.
+    """
+    if rounds <= 0:
+        raise ValueError(f"rounds must be positive, got {rounds}")
+    program = handle.compiled
+    worker = handle._worker
+    flat: list[_lib.ChipTensor] = []
+    scalars: list[Any] = []
+    n_t = None
+    for args in arg_sets:
+        tensors, scalars = _split_args(program, args)
+        if n_t is None:
+            n_t = len(tensors)
+        elif n_t != len(tensors):
+            raise ValueError("all argument sets must have the same number of tensors")
+        for i, (arg, direction) in enumerate(zip(tensors, program.signature)):
+            if isinstance(arg, DeviceTensor):
+                flat.append(_descriptor(arg.data_ptr, arg.shape, arg.dtype, arg.nbytes))
+            elif isinstance(arg, torch.Tensor) and (arg.is_cuda or direction == HOST):
+                flat.append(_descriptor(arg.data_ptr(), tuple(arg.shape), arg.dtype, arg.numel() * arg.element_size()))
+            else:
+                raise ValueError("benchmark() needs device-resident tensors (DeviceTensor or CUDA torch tensors)")
+    descs = (_lib.ChipTensor * len(flat))(*flat)
+    sc = (C.c_uint64 * max(len(scalars), 1))(*[scalar_to_uint64(s) for s in scalars])
+    avg = C.c_float(0.0)
+    _lib.check(
+        worker._lib.pto_hip_benchmark(
+            handle.cid, descs, len(arg_sets), n_t, sc, len(scalars), rounds, warmup, stream, C.byref(avg)
+        )
+    )
+    return BenchmarkStats(rounds=rounds, warmup=warmup, device_wall_us=float(avg.value))
+
+
+def validate_golden(
+    outputs: dict[str, torch.Tensor],
+    golden: dict[str, torch.Tensor],
+    rtol: float = 1e-5,
+    atol: float = 1e-5,
+) -> None:
+    """``torch.isclose`` comparison where NaN in the golden marks a don't-care element.
+
+    Same contract as device_runner.py:850-899.
+    """
+    for name, actual_tensor in outputs.items():
+        actual = actual_tensor.cpu()
+        expected = golden[name].cpu()
+        care = ~torch.isnan(expected)
+        close = torch.isclose(actual, expected, rtol=rtol, atol=atol) | ~care
+        if not bool(close.all()):
+            bad = torch.where(~close.flatten())[0]
+            fa, fe = actual.flatten(), expected.flatten()
+            n_show = min(20, bad.numel())
+            lines = [f"    [{i.item()}] actual={fa[i].item()}, expected={fe[i].item()}" for i in bad[:n_show]]
+            n_dc = int((~care).sum().item())
+            skipped = f" ({n_dc} don't-care skipped)" if n_dc else ""
+            raise AssertionError(
+                f"Output '{name}' does not match golden.\n"
+                f"Mismatched elements: {bad.numel()}/{actual.numel()}{skipped}\n"
+                f"rtol={rtol}, atol={atol}\n"
+                f"First {n_show} mismatches:\n" + "\n".join(lines)
+            )

@@ -1,0 +1,213 @@
+"""Seeded synthetic inputs for the benchmark configurations of the hot path.
+
+Input distributions follow the reference's ``build_tensors`` where it has one
+(examples/models/04_paged_attention.py:544-577: q/K/V ``randn`` bf16, int32 block table and
+context lengths, 7-slot int64 config with the scale as fp32 bits) with the deviations the
+benchmark configurations ask for: a block table that is a seeded random *permutation* of the
+physical blocks, per-sequence context lengths drawn uniformly, and KV heads > 1 laid out as
+``[block][kv_head][token][dim]``.
+
+All builders are deterministic for a given ``seed`` and ``device``.  Nothing here computes an
+expected result.
+"""
+
+from __future__ import annotations
+
+import math
+import struct
+from dataclasses import dataclass
+
+import torch
+
+FP8_E4M3_MAX = 448.0
+
+
+def scale_bits(scale: float) -> int:
+    return struct.unpack("I", struct.pack("f", float(scale)))[0]
+
+
+@dataclass
+class AttentionInputs:
+    query: torch.Tensor
+    key_cache: torch.Tensor
+    value_cache: torch.Tensor
+    block_table: torch.Tensor
+    context_lens: torch.Tensor
+    out: torch.Tensor
+    config: torch.Tensor  # int64[7], always on the host
+    k_scale: torch.Tensor | None = None
+    v_scale: torch.Tensor | None = None
+
+    def args(self) -> tuple:
+        base = (self.query, self.key_cache, self.value_cache, self.block_table, self.context_lens,
+                self.out, self.config)
+        if self.k_scale is not None:
+            return base + (self.k_scale, self.v_scale)
+        return base
+
+    def kv_bytes(self) -> int:
+        """Algorithmic K+V bytes one decode pass must read: sum(ctx) * Hkv * D * 2 * elem."""
+        cfg = self.config.tolist()
+        hkv, d = cfg[2], cfg[3]
+        return int(self.context_lens.sum().item()) * hkv * d * 2 * self.key_cache.element_size()
+
+    def algorithmic_bytes(self) -> int:
+        """K/V rows + scales + query + output + block table + context lengths."""
+        cfg = self.config.tolist()
+        b, hq, hkv, d, bs = cfg[0], cfg[1], cfg[2], cfg[3], cfg[4]
+        ctx = self.context_lens.to("cpu", torch.int64)
+        blocks = int(((ctx + bs - 1) // bs).sum().item())
+        n = self.kv_bytes()
+        if self.k_scale is not None:
+            n += blocks * hkv * 2 * 4
+        n += b * hq * d * self.query.element_size()
+        n += b * hq * d * 4
+        n += blocks * 4 + b * 4
+        return n
+
+
+def _quantize_fp8(cache: torch.Tensor, pool_blocks: int, hkv: int, bs: int):
+    """e4m3 codes + one fp32 scale per (block, KV head): scale = amax/448, RNE cast."""
+    d = cache.shape[1]
+    x = cache.float().reshape(pool_blocks, hkv, bs * d)
+    amax = x.abs().amax(dim=-1)
+    scale = torch.where(amax > 0, amax / FP8_E4M3_MAX, torch.ones_like(amax))
+    codes = (x / scale.unsqueeze(-1)).to(torch.float8_e4m3fn).reshape(-1, d)
+    return codes, scale.contiguous()
+
+
+def paged_attention_inputs(
+    *,
+    batch: int,
+    num_heads: int,
+    kv_head_num: int,
+    head_dim: int = 128,
+    block_size: int = 128,
+    ctx_range: tuple[int, int] = (512, 4096),
+    pool_blocks: int | None = None,
+    max_num_blocks_per_req: int | None = None,
+    dtype: torch.dtype = torch.bfloat16,
+    fp8_kv: bool = False,
+    scale: float | None = None,
+    seed: int = 0,
+    device: str | torch.device = "cpu",
+    context_lens: list[int] | None = None,
+) -> AttentionInputs:
+    """Build one paged-attention decode problem.
+
+    The block table is the first ``sum(ceil(ctx_b / bs))`` entries of a seeded permutation of
+    the pool's physical block ids, laid out row-major per sequence and padded with 0.
+    """
+    dev = torch.device(device)
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    if context_lens is None:
+        lo, hi = ctx_range
+        ctx = torch.randint(lo, hi + 1, (batch,), generator=g, dtype=torch.int64)
+    else:
+        ctx = torch.tensor(context_lens, dtype=torch.int64)
+        assert ctx.numel() == batch
+    nblk = (ctx + block_size - 1) // block_size
+    if max_num_blocks_per_req is None:
+        top = max(int(ctx_range[1]), int(ctx.max().item()) if batch else 0, 1)
+        max_num_blocks_per_req = (top + block_size - 1) // block_size
+    total = int(nblk.sum().item())
+    if pool_blocks is None:
+        pool_blocks = max(total, 1)
+    assert total <= pool_blocks, f"pool of {pool_blocks} blocks cannot hold {total}"
+    perm = torch.randperm(pool_blocks, generator=g)[:total].to(torch.int32)
+    table = torch.zeros((batch, max_num_blocks_per_req), dtype=torch.int32)
+    off = 0
+    for b in range(batch):
+        n = int(nblk[b])
+        table[b, :n] = perm[off : off + n]
+        off += n
+
+    gd = torch.Generator(device=dev).manual_seed(seed + 1)
+    rows = pool_blocks * kv_head_num * block_size
+    query = torch.randn((batch * num_heads, head_dim), generator=gd, device=dev, dtype=torch.float32).to(dtype)
+    key_cache = torch.randn((rows, head_dim), generator=gd, device=dev, dtype=dtype)
+    value_cache = torch.randn((rows, head_dim), generator=gd, device=dev, dtype=dtype)
+    k_scale = v_scale = None
+    if fp8_kv:
+        key_cache, k_scale = _quantize_fp8(key_cache, pool_blocks, kv_head_num, block_size)
+        value_cache, v_scale = _quantize_fp8(value_cache, pool_blocks, kv_head_num, block_size)
+    if scale is None:
+        scale = 1.0 / math.sqrt(head_dim)
+    config = torch.tensor(
+        [batch, num_heads, kv_head_num, head_dim, block_size, max_num_blocks_per_req, scale_bits(scale)],
+        dtype=torch.int64,
+    )
+    return AttentionInputs(
+        query=query,
+        key_cache=key_cache,
+        value_cache=value_cache,
+        block_table=table.flatten().contiguous().to(dev),
+        context_lens=ctx.to(torch.int32).to(dev),
+        out=torch.zeros((batch * num_heads, head_dim), dtype=torch.float32, device=dev),
+        config=config,
+        k_scale=k_scale,
+        v_scale=v_scale,
+    )
+
+
+def attention_small(seed: int = 0, device="cpu", **over) -> AttentionInputs:
+    """Paged-attention decode, small: B16 Hq32 Hkv8 D128 bs128, ctx~U[512,4096], pool 1024, bf16."""
+    kw = dict(batch=16, num_heads=32, kv_head_num=8, head_dim=128, block_size=128,
+              ctx_range=(512, 4096), pool_blocks=1024, dtype=torch.bfloat16, seed=seed, device=device)
+    kw.update(over)
+    return paged_attention_inputs(**kw)
+
+
+def attention_long_fp8(seed: int = 0, device="cpu", **over) -> AttentionInputs:
+    """Paged-attention decode, long context, e4m3 KV: B64 Hq64 Hkv8 D128 bs128, ctx~U[8192,32768]."""
+    kw = dict(batch=64, num_heads=64, kv_head_num=8, head_dim=128, block_size=128,
+              ctx_range=(8192, 32768), pool_blocks=None, dtype=torch.bfloat16, fp8_kv=True,
+              seed=seed, device=device)
+    kw.update(over)
+    return paged_attention_inputs(**kw)
+
+
+@dataclass
+class FfnInputs:
+    x: torch.Tensor
+    gamma: torch.Tensor | None
+    w_gate: torch.Tensor
+    w_up: torch.Tensor
+    w_down: torch.Tensor
+    out: torch.Tensor
+    eps: float = 1e-6
+
+    def flops(self) -> int:
+        t, h = self.x.shape
+        i = self.w_gate.shape[1]
+        return 6 * t * h * i
+
+
+def ffn_inputs(*, tokens: int, hidden: int, intermediate: int, dtype=torch.bfloat16, with_norm: bool = True,
+               out_dtype=torch.float32, seed: int = 0, device="cpu") -> FfnInputs:
+    """x ~ N(0,1); weights ~ N(0,0.02) stored [in, out]; gamma ~ N(1,0.02) fp32."""
+    dev = torch.device(device)
+    g = torch.Generator(device=dev).manual_seed(seed)
+
+    def rn(shape, std=1.0, mean=0.0):
+        return torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * std + mean
+
+    x = rn((tokens, hidden)).to(dtype)
+    w_gate = rn((hidden, intermediate), 0.02).to(dtype)
+    w_up = rn((hidden, intermediate), 0.02).to(dtype)
+    w_down = rn((intermediate, hidden), 0.02).to(dtype)
+    gamma = rn((1, hidden), 0.02, 1.0) if with_norm else None
+    out = torch.zeros((tokens, hidden), dtype=out_dtype, device=dev)
+    return FfnInputs(x, gamma, w_gate, w_up, w_down, out)
+
+
+def ffn_tiny(seed: int = 0, device="cpu") -> FfnInputs:
+    """FFN tile program of the reference's example at x[128,512] fp16, I=1024, no norm."""
+    return ffn_inputs(tokens=128, hidden=512, intermediate=1024, dtype=torch.float16, with_norm=False,
+                      seed=seed, device=device)
+
+
+def ffn_llama7b(seed: int = 0, device="cpu") -> FfnInputs:
+    """FFN at LLaMA-7B shape: T2048 H4096 I11008 bf16 with RMSNorm prologue."""
+    return ffn_inputs(tokens=2048, hidden=4096, intermediate=11008, dtype=torch.bfloat16, with_norm=True,
+                      seed=seed, device=device)

@@ -1,0 +1,135 @@
+"""GPU parity: paged-attention decode through the C ABI vs the CPU oracle.
+
+Tolerances: the task's bar is max-abs 1e-2 and rel 2e-2 against the torch golden
+(the reference itself checks rtol=atol=2e-2, examples/models/04_paged_attention.py:648).
+"""
+
+import pytest
+import torch
+
+import oracle
+from pypto_amd import workloads
+from pypto_amd.runtime import paged_attention, validate_golden
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 1e-2, 2e-2
+
+
+def _run(worker, inp, tpp=0):
+    worker.set_option("attn_tokens_per_partition", tpp)
+    dev = [t.cuda() if isinstance(t, torch.Tensor) and i != 6 else t for i, t in enumerate(inp.args())]
+    dev[5].fill_(float("nan"))
+    torch.cuda.synchronize()
+    with worker.register(paged_attention) as h:
+        h(*dev)
+    worker.sync()
+    worker.set_option("attn_tokens_per_partition", 0)
+    return dev[5].cpu()
+
+
+def _golden(inp):
+    return oracle.paged_attention_golden(inp.query, inp.key_cache, inp.value_cache, inp.block_table,
+                                         inp.context_lens, inp.config, inp.k_scale, inp.v_scale)
+
+
+def _check(out, ref):
+    err = (out - ref).abs().max().item()
+    print(f"max_abs_err={err:.3e}", flush=True)
+    assert torch.isfinite(out).all()
+    validate_golden({"out": out}, {"out": ref}, rtol=RTOL, atol=ATOL)
+    assert err <= ATOL + RTOL * ref.abs().max().item()
+
+
+@pytest.mark.parametrize("tpp", [0, 128, 512, 4096])
+def test_small_config_matches_golden(worker, tpp):
+    """B16 Hq32 Hkv8 D128 bs128, ctx~U[512,4096], permutation table (reduced pool)."""
+    inp = workloads.attention_small(seed=0, pool_blocks=None)
+    out = _run(worker, inp, tpp)
+    _check(out, _golden(inp))
+
+
+@pytest.mark.parametrize(
+    "batch,hq,hkv,d,bs,ctxs",
+    [
+        (1, 16, 1, 128, 128, [200]),                 # torch-codegen test shape: B1 H16 D128 ctx200
+        (4, 16, 1, 128, 128, [1, 127, 128, 129]),    # block edges
+        (3, 16, 1, 128, 64, [1000, 64, 65]),         # block 64, unaligned ctx 1000
+        (2, 16, 1, 256, 64, [513, 100]),             # head_dim 256
+        (5, 8, 2, 128, 16, [0, 5, 16, 17, 333]),     # empty sequence, tiny blocks
+        (2, 64, 1, 128, 128, [700, 300]),            # group of 64 query heads on one KV head
+        (2, 24, 8, 128, 128, [257, 31]),             # group of 3 (padded MFMA columns)
+    ],
+)
+def test_shapes_and_edges(worker, batch, hq, hkv, d, bs, ctxs):
+    inp = workloads.paged_attention_inputs(batch=batch, num_heads=hq, kv_head_num=hkv, head_dim=d,
+                                           block_size=bs, context_lens=ctxs, ctx_range=(1, max(max(ctxs), 1)),
+                                           seed=7)
+    ref = _golden(inp)
+    for tpp in (0, 32, 256):
+        out = _run(worker, inp, tpp)
+        _check(out, ref)
+    if 0 in ctxs:
+        rows = hq
+        i = ctxs.index(0)
+        assert (out[i * rows:(i + 1) * rows] == 0).all()
+
+
+def test_fp16_cache(worker):
+    inp = workloads.paged_attention_inputs(batch=3, num_heads=16, kv_head_num=4, context_lens=[300, 17, 129],
+                                           ctx_range=(1, 300), dtype=torch.float16, seed=3)
+    _check(_run(worker, inp), _golden(inp))
+
+
+def test_duplicate_table_entries(worker):
+    """The reference draws the table with replacement (04_paged_attention.py:568-570)."""
+    inp = workloads.paged_attention_inputs(batch=4, num_heads=16, kv_head_num=1, context_lens=[512] * 4,
+                                           ctx_range=(1, 512), pool_blocks=16, seed=5)
+    g = torch.Generator().manual_seed(11)
+    inp.block_table = torch.randint(0, 16, inp.block_table.shape, generator=g, dtype=torch.int32)
+    _check(_run(worker, inp), _golden(inp))
+
+
+def test_block_permutation_invariance_is_bit_exact(worker):
+    """Moving physical blocks and permuting the table consistently must not change one bit."""
+    inp = workloads.paged_attention_inputs(batch=4, num_heads=32, kv_head_num=8, context_lens=[640, 129, 1024, 77],
+                                           ctx_range=(1, 1024), pool_blocks=64, seed=9)
+    out_a = _run(worker, inp, 128)
+    g = torch.Generator().manual_seed(123)
+    perm = torch.randperm(64, generator=g)          # new position of old block p is perm[p]
+    rows = 8 * 128
+    kc = inp.key_cache.reshape(64, rows, 128)
+    vc = inp.value_cache.reshape(64, rows, 128)
+    kc2, vc2 = torch.empty_like(kc), torch.empty_like(vc)
+    kc2[perm] = kc
+    vc2[perm] = vc
+    inp.key_cache = kc2.reshape(-1, 128)
+    inp.value_cache = vc2.reshape(-1, 128)
+    inp.block_table = perm[inp.block_table.long()].to(torch.int32)
+    out_b = _run(worker, inp, 128)
+    assert torch.equal(out_a, out_b)
+
+
+def test_uniform_scores_give_mean_of_values(worker):
+    """q = 0 makes every score equal: the output is the mean of the valid V rows."""
+    inp = workloads.paged_attention_inputs(batch=2, num_heads=16, kv_head_num=2, context_lens=[300, 64],
+                                           ctx_range=(1, 300), seed=2)
+    inp.query.zero_()
+    out = _run(worker, inp).reshape(2, 2, 8, 128)
+    bs, table = 128, inp.block_table.reshape(2, -1)
+    vc = inp.value_cache.float().reshape(-1, 2, bs, 128)
+    for b, n in enumerate([300, 64]):
+        for h in range(2):
+            rows = torch.cat([vc[table[b, i], h] for i in range((n + bs - 1) // bs)])[:n]
+            assert torch.allclose(out[b, h, 0], rows.mean(0), atol=2e-3, rtol=1e-2)
+
+
+def test_full_size_small_config_properties(worker):
+    """Full pool of 1024 blocks: partition-count independence and golden parity."""
+    inp = workloads.attention_small(seed=0)
+    ref = _golden(inp)
+    outs = [_run(worker, inp, tpp) for tpp in (0, 128, 1024)]
+    for o in outs:
+        _check(o, ref)
+    assert (outs[0] - outs[1]).abs().max() < 2e-3
+    assert (outs[0] - outs[2]).abs().max() < 2e-3

@@ -1,0 +1,88 @@
+"""GPU parity: RMSNorm and the SwiGLU FFN through the C ABI vs the CPU oracle."""
+
+import pytest
+import torch
+
+import oracle
+from pypto_amd import workloads
+from pypto_amd.runtime import ffn_block, ffn_swiglu, rms_norm, validate_golden
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,hidden", [(5, 64), (32, 4096), (3, 1000)])
+def test_rms_norm(worker, dtype, rows, hidden):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((rows, hidden), generator=g).to(dtype)
+    gamma = 1 + 0.02 * torch.randn((1, hidden), generator=g)
+    out = torch.zeros_like(x)
+    with worker.register(rms_norm) as h:
+        h(x, gamma, out, 1e-6)
+    ref = oracle.rms_norm(x, gamma, 1e-6, out_dtype=dtype)
+    # one ulp of the output type: the kernel's rsqrt and torch's differ in the last fp32 bit
+    tol = {torch.float32: 2e-6, torch.bfloat16: 8e-3, torch.float16: 1e-3}[dtype]
+    validate_golden({"out": out.float()}, {"out": ref.float()}, rtol=tol, atol=tol)
+
+
+def test_ffn_reference_example_fp32(worker):
+    """The reference's own case: 64x64 fp32, seed 0, rtol=atol=3e-3 (examples/models/01_ffn.py:155-179)."""
+    torch.manual_seed(0)
+    x = torch.randn(64, 64)
+    wg = torch.randn(64, 64)
+    wu = torch.randn(64, 64)
+    wd = torch.randn(64, 64)
+    out = torch.zeros(64, 64)
+    with worker.register(ffn_swiglu) as h:
+        h(x, wg, wu, wd, out)
+    gate, up = x @ wg, x @ wu
+    expected = (gate * torch.sigmoid(gate) * up) @ wd
+    assert torch.allclose(out, expected, rtol=3e-3, atol=3e-3)
+    assert torch.allclose(out, oracle.ffn_swiglu(x, wg, wu, wd), rtol=3e-3, atol=3e-3)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+def test_ffn_tiny_fp16(worker, variant):
+    """x[128,512] fp16, I=1024, weights N(0,0.02), seed 0; max-abs 1e-2 / rel 2e-2."""
+    inp = workloads.ffn_tiny(seed=0)
+    worker.set_option("gemm_variant", variant)
+    with worker.register(ffn_swiglu) as h:
+        h(inp.x, inp.w_gate, inp.w_up, inp.w_down, inp.out)
+    worker.set_option("gemm_variant", 0)
+    ref = oracle.ffn_swiglu(inp.x, inp.w_gate, inp.w_up, inp.w_down, h_dtype=torch.float16)
+    print("max_abs_err", (inp.out - ref).abs().max().item(), "ref_max", ref.abs().max().item(), flush=True)
+    validate_golden({"out": inp.out}, {"out": ref}, rtol=2e-2, atol=1e-3)
+    ref32 = oracle.ffn_swiglu(inp.x, inp.w_gate, inp.w_up, inp.w_down)
+    validate_golden({"out": inp.out}, {"out": ref32}, rtol=2e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("t,h,i", [(256, 512, 1024), (100, 264, 520), (512, 1024, 2816)])
+def test_ffn_block_bf16(worker, variant, t, h, i):
+    """RMSNorm prologue + SwiGLU FFN, bf16, incl. shapes that are not tile multiples."""
+    inp = workloads.ffn_inputs(tokens=t, hidden=h, intermediate=i, seed=1)
+    worker.set_option("gemm_variant", variant)
+    with worker.register(ffn_block) as hd:
+        hd(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, inp.out, inp.eps)
+    worker.set_option("gemm_variant", 0)
+    ref = oracle.ffn_block(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, inp.eps)
+    print("max_abs_err", (inp.out - ref).abs().max().item(), "ref_max", ref.abs().max().item(), flush=True)
+    validate_golden({"out": inp.out}, {"out": ref}, rtol=2e-2, atol=1e-2)
+
+
+def test_ffn_llama7b_linearity_and_sample(worker):
+    """Full LLaMA-7B shape: sampled rows vs the oracle, and linearity in W_down."""
+    inp = workloads.ffn_llama7b(seed=0, device="cuda")
+    with worker.register(ffn_block) as hd:
+        hd(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, inp.out, inp.eps)
+        worker.sync()
+        out1 = inp.out.clone()
+        rows = torch.tensor([0, 1, 777, 2047])
+        ref = oracle.ffn_block(inp.x[rows].cpu(), inp.gamma.cpu(), inp.w_gate.cpu(), inp.w_up.cpu(),
+                               inp.w_down.cpu(), inp.eps)
+        validate_golden({"out": out1[rows].cpu()}, {"out": ref}, rtol=2e-2, atol=1e-2)
+        # out is linear in W_down: doubling it (exact in bf16) doubles the output exactly.
+        wd2 = (inp.w_down.float() * 2).to(torch.bfloat16)
+        hd(inp.x, inp.gamma, inp.w_gate, inp.w_up, wd2, inp.out, inp.eps)
+        worker.sync()
+        assert torch.equal(inp.out, out1 * 2)
