@@ -37,6 +37,14 @@ FLAGS = [
 ]
 
 
+# Per-file additions.  The attention kernels keep their MFMA accumulators in architectural VGPRs
+# (they are rescaled by VALU code every chunk); the GEMM keeps the default AGPR form.
+EXTRA_FLAGS = {
+    "paged_attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "paged_attention_fp8.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+
+
 def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
@@ -52,7 +60,7 @@ def _compile(src: Path, force: bool) -> Path:
     obj = OBJ_DIR / (src.stem + ".o")
     headers = list(CSRC.glob("*.h")) + list(INCLUDE.glob("*.h"))
     if force or _stale(obj, [src] + headers):
-        cmd = [HIPCC, *FLAGS, "-c", str(src), "-o", str(obj)]
+        cmd = [HIPCC, *FLAGS, *EXTRA_FLAGS.get(src.name, []), "-c", str(src), "-o", str(obj)]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed for {src.name}:\n{r.stderr}")

@@ -40,10 +40,15 @@ struct Context {
   // Grow-only device scratch for partial results (attention partitions, FFN intermediates).
   void* workspace = nullptr;
   size_t workspace_bytes = 0;
+  // Zero-initialised arrival counters for kernels whose last workgroup merges partial results;
+  // every such kernel leaves them zero again.
+  int* counters = nullptr;
+  size_t counters_len = 0;
   // 256 bytes of device flags written by kernels that report bad indices to the host.
   int* flags = nullptr;
   // options
   int64_t attn_tokens_per_partition = 0;
+  int64_t attn_waves_per_cu = 0;
   int64_t gemm_variant = 0;
 };
 
@@ -51,6 +56,8 @@ Context& ctx();
 // Returns a workspace of at least `bytes` (reallocates if too small; stream-ordered callers
 // must not hold an older pointer across a growing call).
 int workspace(size_t bytes, void** ptr);
+// Returns `n` zeroed int counters (grown on demand; same caveat as workspace()).
+int counters(size_t n, int** ptr);
 
 inline int dtype_bytes(int dt) {
   switch (dt) {

@@ -37,7 +37,7 @@ struct AttnParams {
   float* out;
   float* part_o;   // [B*Hq, n_part, D]
   float* part_ml;  // [B*Hq, n_part, 2]  (running max in log2 units, row sum)
-  int hq, hkv, group, gtiles, bs, max_blocks, tpp, n_part;
+  int batch, hq, hkv, group, gtiles, bs, max_blocks, tpp, n_part;
   float scale_log2e;
 };
 
@@ -72,31 +72,52 @@ __device__ __forceinline__ uint32_t round_pack(float a, float b, float& ra, floa
   }
 }
 
-// One chunk of K and V as loaded from the cache (16-bit elements, head_dim D).
 template <int D>
-struct KVChunk {
-  u32x4 k[2][D / 32];     // [tile][k-step]   lane (r, j): token r, elements (s*4+j)*8..+8
-  u32x4 v[D / 128][8];    // [d-set][e]       lane (c, j): token t(j,e), elements (set*16+c)*8..+8
+__device__ __forceinline__ void store_rows(float* o, const f32x4 (&acc)[D / 128][8], int j, float mul) {
+  // acc[set][i][r] = O[g][d], d = set*128 + (j*4 + r)*8 + i
+#pragma unroll
+  for (int set = 0; set < D / 128; ++set)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float4 lo = {acc[set][0][r] * mul, acc[set][1][r] * mul, acc[set][2][r] * mul, acc[set][3][r] * mul};
+      float4 hi = {acc[set][4][r] * mul, acc[set][5][r] * mul, acc[set][6][r] * mul, acc[set][7][r] * mul};
+      float4* dst = reinterpret_cast<float4*>(o + set * 128 + (j * 4 + r) * 8);
+      dst[0] = lo;
+      dst[1] = hi;
+    }
+}
+
+// Lane roles inside a chunk (c = lane % 16, j = lane / 16):
+//   K fragment [tile][s]: token tile*16 + c, head-dim elements (s*4 + j)*8 .. +8
+//   V fragment [set][e] : token (e/4)*16 + j*4 + e%4, head-dim elements (set*16 + c)*8 .. +8
+// so that the 8 probabilities a lane holds after QK^T (two accumulator tiles, rows j*4 .. j*4+3)
+// are, in order, the k-values of the lane's V fragments.
+template <int D>
+struct KFrag {
+  u32x4 t[2][D / 32];
+};
+template <int D>
+struct VFrag {
+  u32x4 t[D / 128][8];
 };
 
 template <int D>
-__device__ __forceinline__ void load_chunk(KVChunk<D>& kv, const uint16_t* kbase0,
-                                           const uint16_t* kbase1, const uint16_t* vbase0,
-                                           const uint16_t* vbase1, int c, int j) {
+__device__ __forceinline__ void load_k(KFrag<D>& k, const char* base0, const char* base1, uint32_t koff) {
 #pragma unroll
   for (int s = 0; s < D / 32; ++s) {
-    kv.k[0][s] = *reinterpret_cast<const u32x4*>(kbase0 + c * D + (s * 4 + j) * 8);
-    kv.k[1][s] = *reinterpret_cast<const u32x4*>(kbase1 + c * D + (s * 4 + j) * 8);
+    k.t[0][s] = *reinterpret_cast<const u32x4*>(base0 + koff + s * 64);
+    k.t[1][s] = *reinterpret_cast<const u32x4*>(base1 + koff + s * 64);
   }
+}
+
+template <int D>
+__device__ __forceinline__ void load_v(VFrag<D>& v, const char* base0, const char* base1, uint32_t voff) {
 #pragma unroll
-  for (int set = 0; set < D / 128; ++set) {
+  for (int set = 0; set < D / 128; ++set)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const uint16_t* vb = (e < 4) ? vbase0 : vbase1;
-      kv.v[set][e] =
-          *reinterpret_cast<const u32x4*>(vb + (j * 4 + (e & 3)) * D + (set * 16 + c) * 8);
-    }
-  }
+    for (int e = 0; e < 8; ++e)
+      v.t[set][e] = *reinterpret_cast<const u32x4*>((e < 4 ? base0 : base1) + voff + set * 256 +
+                                                    (e & 3) * (D * 2));
 }
 
 template <int D, bool BF16>
@@ -104,10 +125,16 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   const int lane = threadIdx.x;
   const int c = lane & 15;   // MFMA row / column index of this lane
   const int j = lane >> 4;   // MFMA k-group of this lane
-  const int part = blockIdx.x;
-  const int h = blockIdx.y / p.gtiles;
-  const int gt = blockIdx.y % p.gtiles;
-  const int b = blockIdx.z;
+  // Linear workgroup id -> (partition, sequence, KV head, query tile) with the partition index
+  // slowest.  Workgroups go to the 8 XCDs round-robin by id, so each XCD sees every partition
+  // index equally often (late partitions exist only for long sequences) and the mostly-empty
+  // tail of the grid is dispatched last.
+  const int pairs = p.batch * p.hkv * p.gtiles;
+  const int part = blockIdx.x / pairs;
+  const int pair = blockIdx.x % pairs;
+  const int b = pair / (p.hkv * p.gtiles);
+  const int h = (pair / p.gtiles) % p.hkv;
+  const int gt = pair % p.gtiles;
 
   int ctx = p.ctx_lens[b];
   const int max_ctx = p.max_blocks * p.bs;
@@ -139,17 +166,19 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
     }
   }
 
-  const uint16_t* kc = reinterpret_cast<const uint16_t*>(p.kc);
-  const uint16_t* vc = reinterpret_cast<const uint16_t*>(p.vc);
+  const char* kc = reinterpret_cast<const char*>(p.kc);
+  const char* vc = reinterpret_cast<const char*>(p.vc);
   const int32_t* table = p.block_table + (size_t)b * p.max_blocks;
+  const uint32_t koff = (uint32_t)(c * D + j * 8) * 2;        // byte offset of this lane in a K tile
+  const uint32_t voff = (uint32_t)(j * 4 * D + c * 8) * 2;    // ... in a V tile
 
-  // Row offset (in elements) of the 16-token tile that starts at logical token `tok`.
+  // Byte offset of the 16-token tile starting at logical token `tok` (wave-uniform).
   auto tile_offset = [&](int tok) -> size_t {
-    // A tile past the end is never used; point it at the first tile so the load stays in
-    // bounds even when the block table holds nothing for that logical block.
+    // A tile past the end is never used; point it at the partition's first tile so the load
+    // stays in bounds even when the block table holds nothing for that logical block.
     if (tok >= tok_end) tok = tok_begin;
     const int blk = table[tok / p.bs];
-    return ((size_t)(blk * p.hkv + h) * p.bs + (tok % p.bs)) * D;
+    return ((size_t)(blk * p.hkv + h) * p.bs + (tok % p.bs)) * (D * 2);
   };
 
   f32x4 acc[D / 128][8];
@@ -160,43 +189,39 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   float m_run = kMinMax;
   float l_run = 0.f;
 
-  KVChunk<D> cur;
-  {
-    const size_t o0 = tile_offset(tok_begin), o1 = tile_offset(tok_begin + 16);
-    load_chunk<D>(cur, kc + o0, kc + o1, vc + o0, vc + o1, c, j);
-  }
+  // Software pipeline: K of chunk n+1 is requested as soon as QK^T of chunk n has consumed
+  // the K registers, V of chunk n at the top of iteration n.  All loads are unconditional (the
+  // look-ahead past the last chunk re-reads the first tile, a cache hit) so that the number of
+  // requests in flight at each wait is known at compile time.
+  KFrag<D> kf;
+  VFrag<D> vf;
+  size_t o0 = tile_offset(tok_begin), o1 = tile_offset(tok_begin + 16);
+  load_k<D>(kf, kc + o0, kc + o1, koff);
 
   for (int tok = tok_begin; tok < tok_end; tok += kChunk) {
-    KVChunk<D> nxt;
-    const bool has_next = tok + kChunk < tok_end;
-    if (has_next) {
-      const size_t o0 = tile_offset(tok + kChunk), o1 = tile_offset(tok + kChunk + 16);
-      load_chunk<D>(nxt, kc + o0, kc + o1, vc + o0, vc + o1, c, j);
-    }
+    load_v<D>(vf, vc + o0, vc + o1, voff);
+    o0 = tile_offset(tok + kChunk);
+    o1 = tile_offset(tok + kChunk + 16);
 
     // ---- S^T = K Q^T : two 16x16 tiles, rows = tokens, columns = query heads ----
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < D / 32; ++s) {
-      s0 = mfma16<BF16>(cur.k[0][s], qf[s], s0);
-      s1 = mfma16<BF16>(cur.k[1][s], qf[s], s1);
+      s0 = mfma16<BF16>(kf.t[0][s], qf[s], s0);
+      s1 = mfma16<BF16>(kf.t[1][s], qf[s], s1);
     }
+    load_k<D>(kf, kc + o0, kc + o1, koff);
+
     float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sv[e] *= p.scale_log2e;
     const bool partial = tok + kChunk > tok_end;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int t = tok + (e >> 2) * 16 + j * 4 + (e & 3);
-      sv[e] = (t < tok_end) ? sv[e] * p.scale_log2e : -INFINITY;
-    }
     if (partial) {
-      // Rows past the end may hold anything; keep them out of the PV product.
 #pragma unroll
-      for (int set = 0; set < D / 128; ++set)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int t = tok + (e >> 2) * 16 + j * 4 + (e & 3);
-          if (t >= tok_end) cur.v[set][e] = u32x4{0u, 0u, 0u, 0u};
-        }
+      for (int e = 0; e < 8; ++e) {
+        const int t = tok + (e >> 2) * 16 + j * 4 + (e & 3);
+        if (t >= tok_end) sv[e] = -INFINITY;
+      }
     }
 
     // ---- online softmax (column-wise: every lane of a column agrees on the maximum) ----
@@ -204,23 +229,38 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
                      fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
     mx = fmaxf(mx, __shfl_xor(mx, 16));
     mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-    m_run = m_new;
+    if (__builtin_amdgcn_ballot_w64(mx > m_run) != 0) {
+      // Some column's maximum grew: rescale the running sum and the accumulators.
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int set = 0; set < D / 128; ++set)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[set][i] *= alpha;
+    }
     u32x4 pf;
     float psum = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; e += 2) {
       float ra, rb;
-      pf[e >> 1] = round_pack<BF16>(__builtin_amdgcn_exp2f(sv[e] - m_new),
-                                    __builtin_amdgcn_exp2f(sv[e + 1] - m_new), ra, rb);
+      pf[e >> 1] = round_pack<BF16>(__builtin_amdgcn_exp2f(sv[e] - m_run),
+                                    __builtin_amdgcn_exp2f(sv[e + 1] - m_run), ra, rb);
       psum += ra + rb;
     }
-    l_run = l_run * alpha + psum;
+    l_run += psum;
+
+    if (partial) {
+      // Rows past the end may hold anything; keep them out of the PV product.
 #pragma unroll
-    for (int set = 0; set < D / 128; ++set)
+      for (int set = 0; set < D / 128; ++set)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[set][i] *= alpha;
+        for (int e = 0; e < 8; ++e) {
+          const int t = tok + (e >> 2) * 16 + j * 4 + (e & 3);
+          if (t >= tok_end) vf.t[set][e] = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
 
     // ---- O^T += V^T P^T : transpose each lane's 8 tokens x 8 elements, then 8 MFMAs ----
 #pragma unroll
@@ -231,12 +271,10 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
         u32x4 vt;
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)
-          vt[kk] = __builtin_amdgcn_perm(cur.v[set][2 * kk + 1][i >> 1],
-                                         cur.v[set][2 * kk][i >> 1], sel);
+          vt[kk] = __builtin_amdgcn_perm(vf.t[set][2 * kk + 1][i >> 1], vf.t[set][2 * kk][i >> 1], sel);
         acc[set][i] = mfma16<BF16>(vt, pf, acc[set][i]);
       }
     }
-    if (has_next) cur = nxt;
   }
 
   // Row sum over the four k-groups of a column.
@@ -244,35 +282,11 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   l_run += __shfl_xor(l_run, 32);
 
   if (!g_valid) return;
-  // acc[set][i][r] = O[g][d], d = set*128 + (j*4 + r)*8 + i
   if (p.n_part == 1) {
-    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
-    float* o = p.out + (size_t)hq_row * D;
-#pragma unroll
-    for (int set = 0; set < D / 128; ++set)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float4 lo = {acc[set][0][r] * inv, acc[set][1][r] * inv, acc[set][2][r] * inv,
-                     acc[set][3][r] * inv};
-        float4 hi = {acc[set][4][r] * inv, acc[set][5][r] * inv, acc[set][6][r] * inv,
-                     acc[set][7][r] * inv};
-        float4* dst = reinterpret_cast<float4*>(o + set * 128 + (j * 4 + r) * 8);
-        dst[0] = lo;
-        dst[1] = hi;
-      }
+    store_rows<D>(p.out + (size_t)hq_row * D, acc, j, l_run > 0.f ? 1.f / l_run : 0.f);
   } else {
     const size_t slot = (size_t)hq_row * p.n_part + part;
-    float* o = p.part_o + slot * D;
-#pragma unroll
-    for (int set = 0; set < D / 128; ++set)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float4 lo = {acc[set][0][r], acc[set][1][r], acc[set][2][r], acc[set][3][r]};
-        float4 hi = {acc[set][4][r], acc[set][5][r], acc[set][6][r], acc[set][7][r]};
-        float4* dst = reinterpret_cast<float4*>(o + set * 128 + (j * 4 + r) * 8);
-        dst[0] = lo;
-        dst[1] = hi;
-      }
+    store_rows<D>(p.part_o + slot * D, acc, j, 1.f);
     if (j == 0) {
       p.part_ml[slot * 2 + 0] = m_run;
       p.part_ml[slot * 2 + 1] = l_run;
@@ -282,38 +296,72 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
 
 // Merge of the per-partition (m, l, o): the online-update algebra of
 // examples/models/04_paged_attention.py:186-215 applied across partitions, then o / l.
+// One wavefront per output row; partitions are read four at a time so that their loads overlap.
 template <int D>
-__global__ __launch_bounds__(D) void attn_reduce_kernel(AttnParams p) {
-  const int row = blockIdx.x;  // b*Hq + query head
+__global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // b*Hq + query head
+  if (row >= p.batch * p.hq) return;
   const int b = row / p.hq;
-  const int d = threadIdx.x;
   int ctx = p.ctx_lens[b];
   const int max_ctx = p.max_blocks * p.bs;
   ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
   const int np = (ctx + p.tpp - 1) / p.tpp;
   const float* ml = p.part_ml + (size_t)row * p.n_part * 2;
   const float* po = p.part_o + (size_t)row * p.n_part * D;
+  // lane i holds (m, l) of partitions i, i+64, ...
   float m = kMinMax;
-  for (int i = 0; i < np; ++i) m = fmaxf(m, ml[2 * i]);
-  float l = 0.f, o = 0.f;
-  for (int i = 0; i < np; ++i) {
-    const float w = __builtin_amdgcn_exp2f(ml[2 * i] - m);
-    l += w * ml[2 * i + 1];
-    o += w * po[(size_t)i * D + d];
+  for (int i = lane; i < np; i += 64) m = fmaxf(m, ml[2 * i]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  float l = 0.f;
+  for (int i = lane; i < np; i += 64) l += __builtin_amdgcn_exp2f(ml[2 * i] - m) * ml[2 * i + 1];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off);
+  float o[D / 64];
+#pragma unroll
+  for (int k = 0; k < D / 64; ++k) o[k] = 0.f;
+  int i = 0;
+  for (; i + 4 <= np; i += 4) {
+    float w[4], v[4][D / 64];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      w[u] = ml[2 * (i + u)];
+#pragma unroll
+      for (int k = 0; k < D / 64; ++k) v[u][k] = po[(size_t)(i + u) * D + k * 64 + lane];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float wgt = __builtin_amdgcn_exp2f(w[u] - m);
+#pragma unroll
+      for (int k = 0; k < D / 64; ++k) o[k] += wgt * v[u][k];
+    }
   }
-  p.out[(size_t)row * D + d] = l > 0.f ? o / l : 0.f;
+  for (; i < np; ++i) {
+    const float wgt = __builtin_amdgcn_exp2f(ml[2 * i] - m);
+#pragma unroll
+    for (int k = 0; k < D / 64; ++k) o[k] += wgt * po[(size_t)i * D + k * 64 + lane];
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+  for (int k = 0; k < D / 64; ++k) p.out[(size_t)row * D + k * 64 + lane] = o[k] * inv;
 }
 
 template <int D>
 int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
-  dim3 grid(p.n_part, p.hkv * p.gtiles, batch);
+  dim3 grid((unsigned)(p.n_part * p.hkv * p.gtiles * batch));
+  // Unused dynamic LDS caps the wavefronts resident per CU so that the dispatcher spreads the
+  // grid over all CUs instead of filling some to their register limit.
+  const int64_t cap = pto_hip::ctx().attn_waves_per_cu;
+  const size_t lds = cap > 0 ? (size_t)(163840 / cap) / 1024 * 1024 : 0;
   if (bf16)
-    hipLaunchKernelGGL((attn_partition_kernel<D, true>), grid, dim3(64), 0, stream, p);
+    hipLaunchKernelGGL((attn_partition_kernel<D, true>), grid, dim3(64), lds, stream, p);
   else
-    hipLaunchKernelGGL((attn_partition_kernel<D, false>), grid, dim3(64), 0, stream, p);
+    hipLaunchKernelGGL((attn_partition_kernel<D, false>), grid, dim3(64), lds, stream, p);
   PTO_CHECK_HIP(hipGetLastError());
   if (p.n_part > 1) {
-    hipLaunchKernelGGL((attn_reduce_kernel<D>), dim3(batch * p.hq), dim3(D), 0, stream, p);
+    hipLaunchKernelGGL((attn_reduce_kernel<D>), dim3((unsigned)((batch * p.hq + 3) / 4)), dim3(256), 0,
+                       stream, p);
     PTO_CHECK_HIP(hipGetLastError());
   }
   return PTO_HIP_OK;
@@ -375,6 +423,7 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
   p.block_table = block_table;
   p.ctx_lens = context_lens;
   p.out = out;
+  p.batch = (int)batch;
   p.hq = (int)hq;
   p.hkv = (int)hkv;
   p.group = (int)(hq / hkv);
@@ -383,23 +432,30 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
   p.max_blocks = (int)max_blocks;
   p.scale_log2e = scale * kLog2e;
 
-  // Context partitions: enough wavefronts to fill every SIMD twice over, each partition a
-  // whole number of 32-token chunks (and of KV blocks when blocks are at least that big).
   const int64_t max_ctx = max_blocks * bs;
+  const bool bf16 = q_dtype == PTO_HIP_BF16;
+
+  // Context partitions: about one wavefront per SIMD when every sequence is at its maximum
+  // length (measured best for short launches, where the spread of finishing times matters more
+  // than occupancy), but never more than 2048 tokens per partition so long contexts still
+  // bring several wavefronts per SIMD.  Each partition is a whole number of 32-token chunks (and
+  // of KV blocks when blocks are at least that big).
   const int64_t align = bs >= kChunk ? bs : kChunk;
   int64_t tpp = cx.attn_tokens_per_partition;
   if (tpp <= 0) {
     const int64_t units = batch * hkv * p.gtiles;
-    const int64_t slots = (int64_t)cx.num_cu * 8;
+    const int64_t slots = (int64_t)cx.num_cu * 4;
     int64_t want = (slots + units - 1) / units;
     if (want < 1) want = 1;
     tpp = (max_ctx + want - 1) / want;
+    if (tpp > 2048) tpp = 2048;
   }
   tpp = (tpp + align - 1) / align * align;
   if (tpp > max_ctx) tpp = (max_ctx + align - 1) / align * align;
   p.tpp = (int)tpp;
   p.n_part = (int)((max_ctx + tpp - 1) / tpp);
-  PTO_CHECK_ARG(hkv * p.gtiles <= 65535, "paged_attention: too many KV heads (%lld)", (long long)hkv);
+  PTO_CHECK_ARG((int64_t)p.n_part * batch * hkv * p.gtiles < (1ll << 31),
+                "paged_attention: batch x heads x partitions exceeds the grid limit");
 
   if (p.n_part > 1) {
     const size_t rows = (size_t)batch * hq;
@@ -411,7 +467,6 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
     p.part_o = reinterpret_cast<float*>(ws);
     p.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + o_bytes);
   }
-  const bool bf16 = q_dtype == PTO_HIP_BF16;
   if (d == 128) return launch<128>(p, (int)batch, bf16, (hipStream_t)stream);
   return launch<256>(p, (int)batch, bf16, (hipStream_t)stream);
 }

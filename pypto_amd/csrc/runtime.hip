@@ -50,6 +50,22 @@ int workspace(size_t bytes, void** ptr) {
   return PTO_HIP_OK;
 }
 
+int counters(size_t n, int** ptr) {
+  Context& c = ctx();
+  if (n > c.counters_len) {
+    PTO_CHECK_HIP(hipDeviceSynchronize());
+    if (c.counters) PTO_CHECK_HIP(hipFree(c.counters));
+    c.counters = nullptr;
+    c.counters_len = 0;
+    size_t want = n + n / 2 + 1024;
+    PTO_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&c.counters), want * sizeof(int)));
+    PTO_CHECK_HIP(hipMemset(c.counters, 0, want * sizeof(int)));
+    c.counters_len = want;
+  }
+  *ptr = c.counters;
+  return PTO_HIP_OK;
+}
+
 namespace {
 
 enum ProgramKind {
@@ -307,6 +323,9 @@ int pto_hip_close(void) {
   c.workspace_bytes = 0;
   if (c.flags) PTO_CHECK_HIP(hipFree(c.flags));
   c.flags = nullptr;
+  if (c.counters) PTO_CHECK_HIP(hipFree(c.counters));
+  c.counters = nullptr;
+  c.counters_len = 0;
   c.initialized = false;
   {
     std::lock_guard<std::mutex> lk(g_mu);
@@ -459,6 +478,10 @@ int pto_hip_set_option(const char* name, int64_t value) {
     c.attn_tokens_per_partition = value;
   } else if (!std::strcmp(name, "gemm_variant")) {
     c.gemm_variant = value;
+  } else if (!std::strcmp(name, "attn_waves_per_cu")) {
+    PTO_CHECK_ARG(value >= 0 && value <= 16, "attn_waves_per_cu must be in [0, 16]");
+    c.attn_waves_per_cu = value;
+
   } else {
     return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
   }
@@ -470,6 +493,7 @@ int pto_hip_get_option(const char* name, int64_t* value) {
   Context& c = ctx();
   if (!std::strcmp(name, "attn_tokens_per_partition")) *value = c.attn_tokens_per_partition;
   else if (!std::strcmp(name, "gemm_variant")) *value = c.gemm_variant;
+  else if (!std::strcmp(name, "attn_waves_per_cu")) *value = c.attn_waves_per_cu;
   else return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
   return PTO_HIP_OK;
 }

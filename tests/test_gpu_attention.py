@@ -17,6 +17,7 @@ ATOL, RTOL = 1e-2, 2e-2
 
 
 def _run(worker, inp, tpp=0):
+    """tpp = tokens per context partition; 0 lets the library choose."""
     worker.set_option("attn_tokens_per_partition", tpp)
     dev = [t.cuda() if isinstance(t, torch.Tensor) and i != 6 else t for i, t in enumerate(inp.args())]
     dev[5].fill_(float("nan"))
@@ -115,7 +116,7 @@ def test_uniform_scores_give_mean_of_values(worker):
     inp = workloads.paged_attention_inputs(batch=2, num_heads=16, kv_head_num=2, context_lens=[300, 64],
                                            ctx_range=(1, 300), seed=2)
     inp.query.zero_()
-    out = _run(worker, inp).reshape(2, 2, 8, 128)
+    out = _run(worker, inp, 128).reshape(2, 2, 8, 128)
     bs, table = 128, inp.block_table.reshape(2, -1)
     vc = inp.value_cache.float().reshape(-1, 2, bs, 128)
     for b, n in enumerate([300, 64]):
