@@ -1,0 +1,161 @@
+#!/usr/bin/env python3
+"""One-GPU benchmark of the paged-attention / FFN hot path on MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one paged-attention decode pass over one batch of the "small" configuration
+(batch 16, 32 query heads, 8 KV heads, head_dim 128, block 128, context ~U[512,4096], bf16 KV in
+a pool of 1024 blocks, permutation block table).  The step rotates through several identical KV
+pools so the working set stays larger than the 256 MB last-level cache.  The printed JSON line
+carries the whole-step throughput (`value`), the roofline of the dominant kernel, the FFN block
+at LLaMA-7B shape as a second measurement, and the CPU oracle timed on this machine's host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+KV_POOLS = 4                   # 4 x 537 MB of K+V, cycled
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument("--no-ffn", action="store_true", help="skip the FFN measurement")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path, run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from pypto_amd import workloads
+    from pypto_amd.runtime import ChipWorker, RunConfig, benchmark, ffn_block, paged_attention
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+
+    worker = ChipWorker(RunConfig(platform="mi355x", device_id=0))
+    info = worker.device_info()
+
+    # ---- paged-attention decode, small configuration ------------------------------------
+    pools = [workloads.attention_small(seed=0, device="cuda") for _ in range(KV_POOLS)]
+    torch.cuda.synchronize()
+    step_bytes = pools[0].algorithmic_bytes()
+    arg_sets = [p.args() for p in pools]
+    handle = worker.register(paged_attention)
+
+    benchmark(handle, arg_sets, rounds=max(args.warmup, 1), warmup=0)  # untimed warm-up steps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    stats = benchmark(handle, arg_sets, rounds=args.steps, warmup=0)   # exactly K timed steps
+    torch.cuda.synchronize()
+    wall_s = time.perf_counter() - t0
+    ms_per_step = wall_s * 1e3 / args.steps
+    value = step_bytes / (wall_s / args.steps) / 1e9
+    step_us_events = stats.device_wall_us
+
+    # Dominant kernel alone (streaming kernel, partials left unmerged), HIP events on its stream.
+    worker.set_option("attn_skip_merge", 1)
+    benchmark(handle, arg_sets, rounds=10, warmup=0)
+    kstats = benchmark(handle, arg_sets, rounds=args.steps, warmup=0)
+    worker.set_option("attn_skip_merge", 0)
+    kernel_us = kstats.device_wall_us
+    achieved = step_bytes / kernel_us / 1e3  # GB/s
+
+    result = {
+        "metric": "paged-attn decode HBM GB/s + FFN TFLOP/s, % of MI355X roofline, 1 GPU",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "paged-attention decode small: B16 Hq32 Hkv8 D128 bs128 ctx~U[512,4096] bf16 KV, "
+                        "pool 1024 blocks, permutation table, scale 1/sqrt(128), fp32 softmax",
+            "kv_pools_rotated": KV_POOLS,
+            "algorithmic_bytes_per_step": step_bytes,
+            "step_us_hip_events": round(step_us_events, 2),
+            "device": info["arch"],
+            "compute_units": info["compute_units"],
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "attn_partition_kernel<128, true>",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "kernel_us": round(kernel_us, 2),
+            "traffic": None,
+        },
+    }
+    handle.unregister()
+
+    # ---- FFN block at LLaMA-7B shape (second half of the metric) ------------------------------
+    if not args.no_ffn:
+        f = workloads.ffn_llama7b(seed=0, device="cuda")
+        torch.cuda.synchronize()
+        with worker.register(ffn_block) as fh:
+            fargs = [(f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.out, f.eps)]
+            benchmark(fh, fargs, rounds=3, warmup=0)
+            fstats = benchmark(fh, fargs, rounds=20, warmup=0)
+        tflops = f.flops() / fstats.device_wall_us / 1e6
+        result["ffn"] = {
+            "workload": "FFN LLaMA-7B: T2048 H4096 I11008 bf16, RMSNorm prologue, SwiGLU, fp32 accumulate",
+            "flops_per_step": f.flops(),
+            "us_per_step": round(fstats.device_wall_us, 1),
+            "achieved": round(tflops, 1),
+            "peak": MFMA_BF16_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+            "bound": "mfma",
+        }
+        del f
+
+    # ---- CPU baseline: the oracle on this machine's host cores --------------------------------
+    if not args.no_cpu_baseline:
+        import oracle
+
+        p = pools[0]
+        host = [t.cpu() for t in (p.query, p.key_cache, p.value_cache, p.block_table, p.context_lens, p.config)]
+        times = []
+        oracle.paged_attention_golden(*host)  # warm-up
+        for _ in range(3):
+            t0 = time.perf_counter()
+            oracle.paged_attention_golden(*host)
+            times.append(time.perf_counter() - t0)
+        med = statistics.median(times)
+        result["cpu_baseline"] = {
+            "value": round(step_bytes / med / 1e9, 3),
+            "unit": "GB/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": "one full step of the same workload (torch block-loop golden), median of 3 after 1 warm-up; "
+                      f"{med * 1e3:.1f} ms per step, os.cpu_count()={os.cpu_count()}",
+        }
+
+    worker.close()
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

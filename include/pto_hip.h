@@ -168,6 +168,10 @@ PTO_HIP_API int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void
 
 /* ---- tuning knobs (integers by name; unknown names are PTO_HIP_ERR_NOT_FOUND) ------------
  *  "attn_tokens_per_partition"  0 = choose from the device's CU count (default)
+ *  "attn_waves_per_cu"          cap on resident attention wavefronts per CU, 0 = none (default)
+ *  "attn_skip_merge"            1 = launch only the streaming attention kernel and leave the
+ *                               partition partials unmerged (kernel timing aid; output invalid)
+ *  "gemm_variant"               FFN GEMM tiling: 0 = default choice, 1..2 = fixed alternatives
  */
 PTO_HIP_API int pto_hip_set_option(const char* name, int64_t value);
 PTO_HIP_API int pto_hip_get_option(const char* name, int64_t* value);

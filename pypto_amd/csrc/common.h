@@ -49,6 +49,7 @@ struct Context {
   // options
   int64_t attn_tokens_per_partition = 0;
   int64_t attn_waves_per_cu = 0;
+  int64_t attn_skip_merge = 0;
   int64_t gemm_variant = 0;
 };
 

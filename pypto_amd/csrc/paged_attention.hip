@@ -359,7 +359,9 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   else
     hipLaunchKernelGGL((attn_partition_kernel<D, false>), grid, dim3(64), lds, stream, p);
   PTO_CHECK_HIP(hipGetLastError());
-  if (p.n_part > 1) {
+  // "attn_skip_merge" leaves the partials unmerged: a timing aid that isolates the streaming
+  // kernel; results are not valid in that mode.
+  if (p.n_part > 1 && !pto_hip::ctx().attn_skip_merge) {
     hipLaunchKernelGGL((attn_reduce_kernel<D>), dim3((unsigned)((batch * p.hq + 3) / 4)), dim3(256), 0,
                        stream, p);
     PTO_CHECK_HIP(hipGetLastError());

@@ -478,6 +478,8 @@ int pto_hip_set_option(const char* name, int64_t value) {
     c.attn_tokens_per_partition = value;
   } else if (!std::strcmp(name, "gemm_variant")) {
     c.gemm_variant = value;
+  } else if (!std::strcmp(name, "attn_skip_merge")) {
+    c.attn_skip_merge = value != 0;
   } else if (!std::strcmp(name, "attn_waves_per_cu")) {
     PTO_CHECK_ARG(value >= 0 && value <= 16, "attn_waves_per_cu must be in [0, 16]");
     c.attn_waves_per_cu = value;
@@ -494,6 +496,7 @@ int pto_hip_get_option(const char* name, int64_t* value) {
   if (!std::strcmp(name, "attn_tokens_per_partition")) *value = c.attn_tokens_per_partition;
   else if (!std::strcmp(name, "gemm_variant")) *value = c.gemm_variant;
   else if (!std::strcmp(name, "attn_waves_per_cu")) *value = c.attn_waves_per_cu;
+  else if (!std::strcmp(name, "attn_skip_merge")) *value = c.attn_skip_merge;
   else return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
   return PTO_HIP_OK;
 }
