@@ -1,0 +1,93 @@
+"""Pins the FFN / RMSNorm / RoPE / W8A16 oracle functions against library routines and closed forms."""
+
+import math
+
+import pytest
+import torch
+
+import oracle
+
+
+def test_rms_norm_matches_library():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(7, 96, generator=g)
+    gamma = 1 + 0.1 * torch.randn(1, 96, generator=g)
+    ref = torch.nn.functional.rms_norm(x, (96,), gamma.reshape(-1), eps=1e-6)
+    assert torch.allclose(oracle.rms_norm(x, gamma, 1e-6), ref, atol=1e-6, rtol=1e-6)
+    # closed form on a constant row: x / sqrt(x^2 + eps)
+    row = torch.full((1, 16), 3.0)
+    assert torch.allclose(oracle.rms_norm(row, None, 1e-5), row / math.sqrt(9 + 1e-5))
+    # sqrt-then-divide form of the teaching example is the same function
+    y = x / torch.sqrt((x ** 2).mean(-1, keepdim=True) + 1e-5) * gamma
+    assert torch.allclose(oracle.rms_norm(x, gamma, 1e-5), y, atol=1e-6)
+    assert oracle.rms_norm(x.to(torch.bfloat16), gamma, 1e-6, out_dtype=torch.bfloat16).dtype == torch.bfloat16
+
+
+def test_ffn_reference_example_formula():
+    """examples/models/01_ffn.py:155-179: seed 0, 64x64 fp32, silu form == sigmoid form."""
+    torch.manual_seed(0)
+    x, wg, wu, wd = (torch.randn(64, 64) for _ in range(4))
+    gate, up = x @ wg, x @ wu
+    expected = (gate * torch.sigmoid(gate) * up) @ wd
+    out = oracle.ffn_swiglu(x, wg, wu, wd)
+    assert torch.allclose(out, expected, rtol=3e-3, atol=3e-3)
+    lib = (torch.nn.functional.silu(x.double() @ wg.double()) * (x.double() @ wu.double())) @ wd.double()
+    assert torch.allclose(out.double(), lib, rtol=1e-4, atol=1e-3)
+    # swapping gate and up, or dropping the activation, must be visible
+    assert not torch.allclose(oracle.ffn_swiglu(x, wu, wg, wd), expected, rtol=3e-3, atol=3e-3)
+
+
+def test_ffn_block_model_form():
+    """test_qwen3_decode_scope3_mixed.py:276-287: normed and h rounded to bf16."""
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(9, 64, generator=g).to(torch.bfloat16)
+    gamma = 1 + 0.02 * torch.randn(1, 64, generator=g)
+    wg, wu = (0.1 * torch.randn(64, 96, generator=g)).to(torch.bfloat16), (0.1 * torch.randn(64, 96, generator=g)).to(torch.bfloat16)
+    wd = (0.1 * torch.randn(96, 64, generator=g)).to(torch.bfloat16)
+    variance = x.float().pow(2).mean(dim=-1, keepdim=True)
+    normed = (x.float() * torch.rsqrt(variance + 1e-6) * gamma).bfloat16()
+    gate = normed.float() @ wg.float()
+    up = normed.float() @ wu.float()
+    mlp = (gate * torch.sigmoid(gate) * up).bfloat16()
+    expected = mlp.float() @ wd.float()
+    assert torch.equal(oracle.ffn_block(x, gamma, wg, wu, wd, 1e-6), expected)
+    resid = torch.randn(9, 64, generator=g)
+    assert torch.equal(oracle.ffn_block(x, gamma, wg, wu, wd, 1e-6, residual=resid), expected + resid)
+
+
+def test_rope_closed_forms():
+    cos, sin = oracle.rope_cos_sin(64, 32, theta=5e5)
+    assert cos.shape == (64, 16)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(5, 32, generator=g)
+    # position 0 is the identity
+    assert torch.allclose(oracle.rope_rotate_half(x, cos[0], sin[0]), x)
+    # complex-rotation closed form: (lo + i hi) * exp(i * pos * theta_k)
+    pos = 13
+    y = oracle.rope_rotate_half(x, cos[pos], sin[pos])
+    inv = 5e5 ** (-torch.arange(16).double() * 2 / 32)
+    z = torch.complex(x[:, :16].double(), x[:, 16:].double()) * torch.exp(1j * pos * inv)
+    assert torch.allclose(y[:, :16].double(), z.real, atol=1e-5) and torch.allclose(y[:, 16:].double(), z.imag, atol=1e-5)
+    # per-pair norm is preserved
+    assert torch.allclose(y[:, :16] ** 2 + y[:, 16:] ** 2, x[:, :16] ** 2 + x[:, 16:] ** 2, atol=1e-5)
+    # relative-position property: <rope(q, m), rope(k, n)> depends on m - n only
+    q, k = torch.randn(32, generator=g), torch.randn(32, generator=g)
+    d1 = oracle.rope_rotate_half(q, cos[20], sin[20]) @ oracle.rope_rotate_half(k, cos[17], sin[17])
+    d2 = oracle.rope_rotate_half(q, cos[9], sin[9]) @ oracle.rope_rotate_half(k, cos[6], sin[6])
+    assert d1.item() == pytest.approx(d2.item(), abs=1e-4)
+
+
+def test_w8a16_closed_form():
+    g = torch.Generator().manual_seed(3)
+    w = 0.02 * torch.randn(48, 24, generator=g)
+    wq, s = oracle.quantize_w8(w)
+    assert wq.dtype == torch.int8 and s.shape == (24,)
+    assert int(wq.abs().max()) == 127 and (wq.abs().amax(0) == 127).all()
+    assert torch.allclose(s, w.abs().amax(0) / 127)
+    assert ((wq.float() * s - w).abs() <= s / 2 + 1e-9).all()
+    x = torch.randn(5, 48, generator=g).to(torch.bfloat16)
+    y = oracle.w8a16_matmul(x, wq, s)
+    # integer identity: (x @ wq) * s, computed in float64
+    ref = (x.double() @ wq.double()) * s.double()
+    assert torch.allclose(y.double(), ref, atol=1e-5, rtol=1e-5)
+    assert torch.allclose(y, x.float() @ w, atol=2e-2)
