@@ -115,7 +115,7 @@ def main() -> int:
         torch.cuda.synchronize()
         with worker.register(ffn_block) as fh:
             fargs = [(f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.out, f.eps)]
-            benchmark(fh, fargs, rounds=3, warmup=0)
+            benchmark(fh, fargs, rounds=10, warmup=0)
             fstats = benchmark(fh, fargs, rounds=20, warmup=0)
         tflops = f.flops() / fstats.device_wall_us / 1e6
         result["ffn"] = {

@@ -9,9 +9,10 @@
 // One MFMA GEMM kernel serves both matmuls:
 //   * block tile (64*MT) x 256 x 64, four wavefronts, each owning (32*MT) x 128 of the tile as
 //     MT x 4 accumulators of v_mfma_f32_32x32x16;
-//   * A goes HBM -> VGPR -> LDS as 16-byte chunks; B ([K, N], N contiguous) is transposed 8x8
-//     in registers with v_perm_b32 on its way to LDS so both operands are read back k-contiguous
-//     with ds_read_b128 from rows padded to 144 bytes (conflict-free);
+//   * both operands go HBM -> VGPR -> LDS as coalesced 16-byte chunks in their memory layout:
+//     A rows ([M, K], k contiguous) are read back with ds_read_b128; B rows ([K, N], n
+//     contiguous) are read back with the transposing ds_read_b64_tr_b16, which hands every
+//     lane the k-values of its column;
 //   * in the gate/up pass the 256 LDS columns are 128 gate + 128 up columns of the same output
 //     range, so SiLU(gate) * up is applied on the accumulators and only h is written;
 //   * workgroup ids are remapped so that the ids sharing an XCD (id mod 8) work on neighbouring
@@ -26,10 +27,13 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4s lds_v4s;
 
 constexpr int BK = 64;        // k extent of one LDS tile
 constexpr int LDK = BK + 8;   // padded LDS row, in 16-bit elements (144 bytes)
 constexpr int BN = 256;       // LDS columns per tile
+constexpr int LDN = BN + 32;  // padded LDS row of the B tile, in elements (576 bytes)
 constexpr int kXcds = 8;
 
 struct GemmParams {
@@ -40,6 +44,7 @@ struct GemmParams {
   int64_t lda, ldb, ldc;
   int m, n, k;
   int tiles_m, tiles_n;
+  int splits, k_per_split;  // split-K: fp32 output accumulated with atomics into zeroed memory
 };
 
 template <bool BF16>
@@ -67,60 +72,81 @@ __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
   return base + local;
 }
 
-template <int MT, int NBUF, bool DUAL, bool BF16, typename OutT>
+// EDGE = false assumes m, n, k are multiples of the tile; EDGE = true clamps every address into
+// the operands (so all loads stay unconditional) and zeroes the A chunks that lie past k.
+template <int MT, int NBUF, bool DUAL, bool BF16, bool EDGE, typename OutT>
 __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   constexpr int BM = 64 * MT;
   constexpr int A_ELEMS = BM * LDK;
-  constexpr int B_ELEMS = BN * LDK;
+  constexpr int B_ELEMS = BK * LDN;
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-  uint16_t* sa = smem;                      // [NBUF][BM][LDK]
-  uint16_t* sb = smem + NBUF * A_ELEMS;     // [NBUF][BN][LDK]  (n-major, k contiguous)
+  uint16_t* sa = smem;                      // [NBUF][BM][LDK]  rows = m, k contiguous
+  uint16_t* sb = smem + NBUF * A_ELEMS;     // [NBUF][BK][LDN]  rows = k, n contiguous (as in memory)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave & 1, wn = wave >> 1;
 
-  const int tile = xcd_remap(blockIdx.x, p.tiles_m * p.tiles_n);
+  const int ntiles = p.tiles_m * p.tiles_n;
+  const int logical = xcd_remap(blockIdx.x, ntiles * p.splits);
+  const int split = logical / ntiles, tile = logical % ntiles;
   const int tm = tile % p.tiles_m, tn = tile / p.tiles_m;
+  const int k_begin = split * p.k_per_split;
+  const int klen = min(p.k, k_begin + p.k_per_split) - k_begin;  // this workgroup's k extent
   const int m0 = tm * BM;
   const int n0 = tn * (DUAL ? BN / 2 : BN);
 
   // ---- global -> register staging ---------------------------------------------------
   // A: thread owns 16-byte chunk (tid % 8) of rows tid/8 + 32*i.
   const int a_chunk = tid & 7, a_row = tid >> 3;
-  // B: thread owns an 8(k) x 8(n) unit: k rows (tid%8)*8.., LDS columns (tid/8)*8..
-  const int b_kb = tid & 7, b_nb = tid >> 3;
+  // B: thread owns 16-byte chunk (tid % 32) of k rows tid/32 + 8*i; in the gate/up pass chunks
+  // 0..15 come from the gate weights and 16..31 from the up weights (same output columns).
+  const int b_chunk = tid & 31, b_row = tid >> 5;
   const uint16_t* bsrc;
-  int b_col;  // global column of the unit
+  int b_col;  // global column of the chunk
   if (DUAL) {
-    bsrc = (b_nb < 16) ? p.b0 : p.b1;
-    b_col = n0 + (b_nb & 15) * 8;
+    bsrc = (b_chunk < 16) ? p.b0 : p.b1;
+    b_col = n0 + (b_chunk & 15) * 8;
   } else {
     bsrc = p.b0;
-    b_col = n0 + b_nb * 8;
+    b_col = n0 + b_chunk * 8;
   }
-  const bool b_col_ok = b_col < p.n;
+  if (EDGE) b_col = min(b_col, p.n - 8);
+  const uint16_t* a_ptr[2 * MT];
+#pragma unroll
+  for (int i = 0; i < 2 * MT; ++i) {
+    int r = m0 + a_row + 32 * i;
+    if (EDGE) r = min(r, p.m - 1);
+    a_ptr[i] = p.a + (int64_t)r * p.lda + k_begin + a_chunk * 8;
+  }
+  const uint16_t* b_ptr = bsrc + (int64_t)(k_begin + b_row) * p.ldb + b_col;
 
   u32x4 ra[2 * MT];
   u32x4 rb[8];
+  auto load_a = [&](int k0, int i) {
+    if constexpr (EDGE) {
+      const int ka = min(k0 + a_chunk * 8, klen - 8) - a_chunk * 8;  // clamped tile origin for A
+      const bool a_ok = k0 + a_chunk * 8 < klen;
+      u32x4 v = *reinterpret_cast<const u32x4*>(a_ptr[i] + ka);
+      u32x4 z = {0u, 0u, 0u, 0u};
+      ra[i] = a_ok ? v : z;
+    } else {
+      ra[i] = *reinterpret_cast<const u32x4*>(a_ptr[i] + k0);
+    }
+  };
+  auto load_b = [&](int k0, int i) {
+    if constexpr (EDGE) {
+      const int kk = min(k0 + b_row + 8 * i, klen - 1) - b_row;
+      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)kk * p.ldb);
+    } else {
+      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)(k0 + 8 * i) * p.ldb);
+    }
+  };
   auto load_tile = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 2 * MT; ++i) {
-      const int r = m0 + a_row + 32 * i;
-      const int kk = k0 + a_chunk * 8;
-      u32x4 z = {0u, 0u, 0u, 0u};
-      ra[i] = (r < p.m && kk < p.k)
-                  ? *reinterpret_cast<const u32x4*>(p.a + (int64_t)r * p.lda + kk)
-                  : z;
-    }
+    for (int i = 0; i < 2 * MT; ++i) load_a(k0, i);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int kk = k0 + b_kb * 8 + e;
-      u32x4 z = {0u, 0u, 0u, 0u};
-      rb[e] = (b_col_ok && kk < p.k)
-                  ? *reinterpret_cast<const u32x4*>(bsrc + (int64_t)kk * p.ldb + b_col)
-                  : z;
-    }
+    for (int i = 0; i < 8; ++i) load_b(k0, i);
   };
   auto store_tile = [&](int buf) {
     uint16_t* da = sa + buf * A_ELEMS;
@@ -129,14 +155,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
       *reinterpret_cast<u32x4*>(da + (a_row + 32 * i) * LDK + a_chunk * 8) = ra[i];
     uint16_t* db = sb + buf * B_ELEMS;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
-      u32x4 t;
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk)
-        t[kk] = __builtin_amdgcn_perm(rb[2 * kk + 1][i >> 1], rb[2 * kk][i >> 1], sel);
-      *reinterpret_cast<u32x4*>(db + (b_nb * 8 + i) * LDK + b_kb * 8) = t;
-    }
+    for (int i = 0; i < 8; ++i)
+      *reinterpret_cast<u32x4*>(db + (b_row + 8 * i) * LDN + b_chunk * 8) = rb[i];
   };
 
   f32x16 acc[MT][4];
@@ -147,52 +167,81 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][jn][r] = 0.f;
 
-  // LDS row of this lane's operand fragments.
-  const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
-  int b_rows[4];
+  // Operand fragments of v_mfma_f32_32x32x16: lane l holds row/column l%32, k = 8*(l/32)..+8.
+  //  A: one 16-byte read from its m-row.
+  //  B: two transposing reads.  In each group of 16 lanes, lane s supplies the address of 4
+  //     consecutive n of k-row s/4 (columns (s%4)*4..); the hardware hands lane c of the group
+  //     the four k-values of column c.  Lanes 16..31 take the next 16 columns, lanes 32..63 the
+  //     next 8 k-rows.
+  const int a_frag = (wm * MT * 32 + (lane & 31)) * LDK + (lane >> 5) * 8;
+  const int grp = lane >> 4, sub = lane & 15;
+  int b_frag[4];
 #pragma unroll
-  for (int jn = 0; jn < 4; ++jn)
-    b_rows[jn] = DUAL ? ((jn >> 1) * (BN / 2) + wn * 64 + (jn & 1) * 32) : (wn * 128 + jn * 32);
+  for (int jn = 0; jn < 4; ++jn) {
+    const int col = DUAL ? ((jn >> 1) * (BN / 2) + wn * 64 + (jn & 1) * 32) : (wn * 128 + jn * 32);
+    b_frag[jn] = ((grp >> 1) * 8 + (sub >> 2)) * LDN + col + (grp & 1) * 16 + (sub & 3) * 4;
+  }
 
-  auto compute = [&](int buf) {
-    const uint16_t* ca = sa + buf * A_ELEMS + (wm * MT * 32 + frag_row) * LDK + frag_k;
-    const uint16_t* cb = sb + buf * B_ELEMS + frag_row * LDK + frag_k;
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      u32x4 fa[MT], fb[4];
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-        fa[i] = *reinterpret_cast<const u32x4*>(ca + i * 32 * LDK + ks * 16);
-#pragma unroll
-      for (int jn = 0; jn < 4; ++jn)
-        fb[jn] = *reinterpret_cast<const u32x4*>(cb + b_rows[jn] * LDK + ks * 16);
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int jn = 0; jn < 4; ++jn) acc[i][jn] = mfma32<BF16>(fa[i], fb[jn], acc[i][jn]);
+  // One LDS read of the fragment set for k-step `ks` of buffer `buf`: r < MT reads A fragment r,
+  // the rest read half (4 k-rows) of a B fragment.
+  u32x4 fa[2][MT], fb[2][4];
+  auto read_one = [&](int buf, int ks, int set, int r) {
+    if (r < MT) {
+      fa[set][r] = *reinterpret_cast<const u32x4*>(sa + buf * A_ELEMS + a_frag + ks * 16 + r * 32 * LDK);
+    } else {
+      const int jn = (r - MT) >> 1, half = (r - MT) & 1;
+      const uint16_t* src = sb + buf * B_ELEMS + (ks * 16 + half * 4) * LDN + b_frag[jn];
+      const uint2 v = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)src));
+      fb[set][jn][half * 2 + 0] = v.x;
+      fb[set][jn][half * 2 + 1] = v.y;
     }
   };
+  constexpr int kReads = MT + 8;                              // LDS reads per k-step
+  constexpr int kSlots = MT * 4;                              // MFMAs per k-step
+  constexpr int kReadsPerSlot = (kReads + kSlots - 1) / kSlots;
+  constexpr int kSteps = BK / 16;
 
-  const int nk = (p.k + BK - 1) / BK;
+  // Main loop, one iteration per k-tile.  Registers ra/rb hold tile kt+1 on entry.  The MFMAs of
+  // k-step ks are interleaved with the LDS reads of the fragments for ks+1 and, in turn, with
+  // the LDS writes of tile kt+1 (k-steps 0-1) and the global loads of tile kt+2 (k-steps 2-3),
+  // so each MFMA issues next to at most a few memory instructions.  sched_barrier pins that
+  // order.  All loads are unconditional (past the end they re-read the last tile, a cache hit)
+  // so the number of requests outstanding at each wait is known at compile time.
+  const int nk = (klen + BK - 1) / BK;
   load_tile(0);
-  if constexpr (NBUF == 2) {
-    store_tile(0);
+  store_tile(0);
+  load_tile(min(1, nk - 1) * BK);
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < kReads; ++r) read_one(0, 0, 0, r);
+
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    const int k_next = min(kt + 2, nk - 1) * BK;
+    uint16_t* da = sa + (buf ^ 1) * A_ELEMS;
+    uint16_t* db = sb + (buf ^ 1) * B_ELEMS;
+#pragma unroll
+    for (int ks = 0; ks < kSteps; ++ks) {
+#pragma unroll
+      for (int q = 0; q < kSlots; ++q) {
+        const int i = q / 4, jn = q % 4;
+        acc[i][jn] = mfma32<BF16>(fa[ks & 1][i], fb[ks & 1][jn], acc[i][jn]);
+        if (ks + 1 < kSteps) {
+#pragma unroll
+          for (int r = q * kReadsPerSlot; r < (q + 1) * kReadsPerSlot; ++r)
+            if (r < kReads) read_one(buf, ks + 1, (ks + 1) & 1, r);
+        }
+        if (ks == 0 && q < 2 * MT)
+          *reinterpret_cast<u32x4*>(da + (a_row + 32 * q) * LDK + a_chunk * 8) = ra[q];
+        if (ks == 1 && q < 8) *reinterpret_cast<u32x4*>(db + (b_row + 8 * q) * LDN + b_chunk * 8) = rb[q];
+        if (ks == 2 && q < 2 * MT) load_a(k_next, q);
+        if (ks == 3 && q < 8) load_b(k_next, q);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
     __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-      const int buf = kt & 1;
-      if (kt + 1 < nk) load_tile((kt + 1) * BK);
-      compute(buf);
-      if (kt + 1 < nk) store_tile(buf ^ 1);
-      __syncthreads();
-    }
-  } else {
-    for (int kt = 0; kt < nk; ++kt) {
-      store_tile(0);
-      __syncthreads();
-      if (kt + 1 < nk) load_tile((kt + 1) * BK);
-      compute(0);
-      __syncthreads();
-    }
+#pragma unroll
+    for (int r = 0; r < kReads; ++r) read_one(buf ^ 1, 0, 0, r);
   }
 
   // ---- epilogue ------------------------------------------------------------------------
@@ -216,40 +265,78 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 #pragma unroll
         for (int jn = 0; jn < 4; ++jn) {
           const int col = n0 + wn * 128 + jn * 32 + (lane & 31);
-          if (col < p.n) store_out<OutT>(c + (int64_t)row * p.ldc + col, acc[i][jn][r]);
+          if (col < p.n) {
+            if (p.splits > 1)
+              unsafeAtomicAdd(reinterpret_cast<float*>(p.c) + (int64_t)row * p.ldc + col, acc[i][jn][r]);
+            else
+              store_out<OutT>(c + (int64_t)row * p.ldc + col, acc[i][jn][r]);
+          }
         }
       }
     }
   }
 }
 
-template <int MT, int NBUF, bool DUAL, bool BF16, typename OutT>
-int launch_gemm(GemmParams p, hipStream_t st) {
+
+template <int MT, int NBUF, bool DUAL, bool BF16, bool EDGE, typename OutT>
+int launch_gemm_e(GemmParams p, hipStream_t st) {
   constexpr int BM = 64 * MT;
   p.tiles_m = (p.m + BM - 1) / BM;
   const int bn_out = DUAL ? BN / 2 : BN;
   p.tiles_n = (p.n + bn_out - 1) / bn_out;
-  const size_t smem = (size_t)NBUF * (BM + BN) * LDK * sizeof(uint16_t);
-  auto kern = gemm_kernel<MT, NBUF, DUAL, BF16, OutT>;
+  const size_t smem = (size_t)NBUF * (BM * LDK + BK * LDN) * sizeof(uint16_t);
+  auto kern = gemm_kernel<MT, NBUF, DUAL, BF16, EDGE, OutT>;
   static bool attr_set = false;  // per instantiation
   if (!attr_set) {
     PTO_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(256), smem, st, p);
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(256), smem, st, p);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
 }
 
+template <int MT, int NBUF, bool DUAL, bool BF16, typename OutT>
+int launch_gemm(GemmParams p, hipStream_t st) {
+  constexpr int BM_ = 64 * MT;
+  const bool edge = p.m % BM_ != 0 || p.n % (DUAL ? BN / 2 : BN) != 0 || p.k % BK != 0 ||
+                    (p.splits > 1 && p.k_per_split % BK != 0);
+  return edge ? launch_gemm_e<MT, NBUF, DUAL, BF16, true, OutT>(p, st)
+              : launch_gemm_e<MT, NBUF, DUAL, BF16, false, OutT>(p, st);
+}
+
+__global__ __launch_bounds__(256) void zero_kernel(float4* p, size_t n4) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256)
+    p[i] = float4{0.f, 0.f, 0.f, 0.f};
+}
+
 template <bool DUAL, bool BF16, typename OutT>
-int launch_variant(const GemmParams& p, hipStream_t st) {
+int launch_variant(GemmParams p, hipStream_t st) {
   const int64_t variant = pto_hip::ctx().gemm_variant;
-  // variant 0: 256x256 tile, double-buffered LDS, one workgroup per CU (default)
-  // variant 1: 128x256 tile, single LDS buffer, two workgroups per CU
-  // variant 2: 128x256 tile, double-buffered
-  if (variant == 1 || (variant == 0 && p.m <= 128)) return launch_gemm<2, 1, DUAL, BF16, OutT>(p, st);
-  if (variant == 2) return launch_gemm<2, 2, DUAL, BF16, OutT>(p, st);
+  p.splits = 1;
+  p.k_per_split = p.k;
+  // variant 1: 256x256 tile; variant 2: 128x256 tile; variant 3: 256x256 tile, k split in two.
+  // variant 0 prefers the large tile; when that leaves CUs without a workgroup it splits k in
+  // two for a contiguous fp32 output (sum of two terms: the result does not depend on which
+  // half arrives first) and otherwise falls back to the smaller tile.
+  const int64_t big_tiles = (int64_t)((p.m + 255) / 256) * ((p.n + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256));
+  const bool can_split = !DUAL && sizeof(OutT) == 4 && p.ldc == p.n && ((int64_t)p.m * p.n) % 4 == 0 &&
+                         p.k >= 4 * BK;
+  bool split = variant == 3 && can_split;
+  bool small = variant == 2;
+  if (variant == 0 && big_tiles < pto_hip::ctx().num_cu) {
+    if (can_split && big_tiles * 2 >= pto_hip::ctx().num_cu / 2) split = true;
+    else small = true;
+  }
+  if (small) return launch_gemm<2, 2, DUAL, BF16, OutT>(p, st);
+  if (split) {
+    p.splits = 2;
+    p.k_per_split = ((p.k + 2 * BK - 1) / (2 * BK)) * BK;
+    const size_t n4 = (size_t)p.m * p.n / 4;
+    hipLaunchKernelGGL(zero_kernel, dim3(1024), dim3(256), 0, st, reinterpret_cast<float4*>(p.c), n4);
+    PTO_CHECK_HIP(hipGetLastError());
+  }
   return launch_gemm<4, 2, DUAL, BF16, OutT>(p, st);
 }
 

@@ -51,6 +51,57 @@ __global__ __launch_bounds__(kThreads) void rms_norm_kernel(const TI* __restrict
   }
 }
 
+// 16-bit rows whose length is a multiple of 8 and at most 8 * kThreads * kVecPerThread: each
+// thread keeps its 16-byte chunks in registers, so the row is read from memory once.
+constexpr int kVecPerThread = 4;
+template <typename T>
+__global__ __launch_bounds__(kThreads) void rms_norm_vec_kernel(const T* __restrict__ x,
+                                                                const float* __restrict__ gamma,
+                                                                T* __restrict__ out, int64_t hidden,
+                                                                float eps) {
+  typedef __attribute__((__vector_size__(8 * sizeof(T)))) T vec8;
+  const int64_t row = blockIdx.x;
+  const vec8* xr = reinterpret_cast<const vec8*>(x + row * hidden);
+  vec8* orow = reinterpret_cast<vec8*>(out + row * hidden);
+  const int nvec = (int)(hidden / 8);
+  vec8 v[kVecPerThread];
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < kVecPerThread; ++u) {
+    const int i = threadIdx.x + u * kThreads;
+    if (i < nvec) {
+      v[u] = xr[i];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float f = (float)v[u][e];
+        ss += f * f;
+      }
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+  __shared__ float wsum[kThreads / 64];
+  if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int w = 0; w < kThreads / 64; ++w) tot += wsum[w];
+  const float inv = rsqrtf(tot / (float)hidden + eps);
+#pragma unroll
+  for (int u = 0; u < kVecPerThread; ++u) {
+    const int i = threadIdx.x + u * kThreads;
+    if (i < nvec) {
+      vec8 o;
+      const float4 g0 = gamma ? reinterpret_cast<const float4*>(gamma)[2 * i] : float4{1.f, 1.f, 1.f, 1.f};
+      const float4 g1 = gamma ? reinterpret_cast<const float4*>(gamma)[2 * i + 1] : float4{1.f, 1.f, 1.f, 1.f};
+      const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = (T)((float)v[u][e] * inv * g[e]);
+      orow[i] = o;
+    }
+  }
+}
+
 template <typename TI>
 int launch_out(const void* x, const float* gamma, void* out, int64_t rows, int64_t hidden, float eps,
                int out_dtype, hipStream_t st) {
@@ -87,6 +138,20 @@ extern "C" int pto_hip_rms_norm(const void* x, const float* gamma, void* out, in
   if (rows == 0) return PTO_HIP_OK;
   PTO_CHECK_ARG(x && out, "rms_norm: null tensor pointer");
   hipStream_t st = (hipStream_t)stream;
+  const bool vec_ok = x_dtype == out_dtype && (x_dtype == PTO_HIP_BF16 || x_dtype == PTO_HIP_FP16) &&
+                      hidden % 8 == 0 && hidden <= 8 * kThreads * kVecPerThread &&
+                      ((uintptr_t)x | (uintptr_t)out | (uintptr_t)gamma) % 16 == 0;
+  if (vec_ok) {
+    dim3 grid((unsigned)rows), block(kThreads);
+    if (x_dtype == PTO_HIP_BF16)
+      hipLaunchKernelGGL(rms_norm_vec_kernel<__bf16>, grid, block, 0, st, (const __bf16*)x, gamma,
+                         (__bf16*)out, hidden, eps);
+    else
+      hipLaunchKernelGGL(rms_norm_vec_kernel<_Float16>, grid, block, 0, st, (const _Float16*)x, gamma,
+                         (_Float16*)out, hidden, eps);
+    PTO_CHECK_HIP(hipGetLastError());
+    return PTO_HIP_OK;
+  }
   switch (x_dtype) {
     case PTO_HIP_FP32: return launch_out<float>(x, gamma, out, rows, hidden, eps, out_dtype, st);
     case PTO_HIP_BF16: return launch_out<__bf16>(x, gamma, out, rows, hidden, eps, out_dtype, st);
