@@ -15,6 +15,8 @@
 //   * the query group of a KV head (padded to 16 rows) stays in registers as B operand.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -37,6 +39,8 @@ struct AttnParams {
   float* out;
   float* part_o;   // [B*Hq, n_part, D]
   float* part_ml;  // [B*Hq, n_part, 2]  (running max in log2 units, row sum)
+  const float* k_scale;  // [pool_blocks, Hkv] for an e4m3 cache, else null
+  const float* v_scale;
   int batch, hq, hkv, group, gtiles, bs, max_blocks, tpp, n_part;
   float scale_log2e;
 };
@@ -92,35 +96,54 @@ __device__ __forceinline__ void store_rows(float* o, const f32x4 (&acc)[D / 128]
 //   V fragment [set][e] : token (e/4)*16 + j*4 + e%4, head-dim elements (set*16 + c)*8 .. +8
 // so that the 8 probabilities a lane holds after QK^T (two accumulator tiles, rows j*4 .. j*4+3)
 // are, in order, the k-values of the lane's V fragments.
-template <int D>
+// With an e4m3 cache a 16-byte K load holds 16 elements, i.e. the operands of two MFMA k-steps:
+//   K fragment [tile][s2]: token tile*16 + c, elements (s2*4 + j)*16 .. +16  (steps 2*s2, 2*s2+1)
+//   V fragment [set][e]  : 8 bytes, token as above, elements (set*16 + c)*8 .. +8
+// Codes are widened to bf16 exactly (scale 1); the per-(block, head) scales are applied to the
+// scores and to the accumulators in fp32.
+template <int D, bool FP8>
 struct KFrag {
-  u32x4 t[2][D / 32];
+  u32x4 t[2][FP8 ? D / 64 : D / 32];
 };
-template <int D>
+template <int D, bool FP8>
 struct VFrag {
-  u32x4 t[D / 128][8];
+  typename std::conditional<FP8, uint2, u32x4>::type t[D / 128][8];
 };
 
-template <int D>
-__device__ __forceinline__ void load_k(KFrag<D>& k, const char* base0, const char* base1, uint32_t koff) {
+template <int D, bool FP8>
+__device__ __forceinline__ void load_k(KFrag<D, FP8>& k, const char* base0, const char* base1, uint32_t koff) {
 #pragma unroll
-  for (int s = 0; s < D / 32; ++s) {
+  for (int s = 0; s < (FP8 ? D / 64 : D / 32); ++s) {
     k.t[0][s] = *reinterpret_cast<const u32x4*>(base0 + koff + s * 64);
     k.t[1][s] = *reinterpret_cast<const u32x4*>(base1 + koff + s * 64);
   }
 }
 
-template <int D>
-__device__ __forceinline__ void load_v(VFrag<D>& v, const char* base0, const char* base1, uint32_t voff) {
+template <int D, bool FP8>
+__device__ __forceinline__ void load_v(VFrag<D, FP8>& v, const char* base0, const char* base1, uint32_t voff) {
+  constexpr int kRow = FP8 ? D : D * 2;        // bytes per token row
+  constexpr int kSet = FP8 ? 128 : 256;        // bytes per 128-element set
+  typedef typename std::conditional<FP8, uint2, u32x4>::type vec_t;
 #pragma unroll
   for (int set = 0; set < D / 128; ++set)
 #pragma unroll
     for (int e = 0; e < 8; ++e)
-      v.t[set][e] = *reinterpret_cast<const u32x4*>((e < 4 ? base0 : base1) + voff + set * 256 +
-                                                    (e & 3) * (D * 2));
+      v.t[set][e] = *reinterpret_cast<const vec_t*>((e < 4 ? base0 : base1) + voff + set * kSet + (e & 3) * kRow);
 }
 
-template <int D, bool BF16>
+// Two e4m3 codes (low or high half of a dword) -> two packed bf16, exact.
+__device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w, bool hi) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const bf16x2 r = hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true)
+                      : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
+  return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ u32x4 fp8x8_to_bf16x8(uint32_t w0, uint32_t w1) {
+  return u32x4{fp8x2_to_bf16x2(w0, false), fp8x2_to_bf16x2(w0, true), fp8x2_to_bf16x2(w1, false),
+               fp8x2_to_bf16x2(w1, true)};
+}
+
+template <int D, bool BF16, bool FP8>
 __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   const int lane = threadIdx.x;
   const int c = lane & 15;   // MFMA row / column index of this lane
@@ -155,30 +178,34 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
     return;
   }
 
-  // Query fragments (B operand): column = query head, k-group j holds elements (s*4+j)*8..+8.
+  // Query fragments (B operand): column = query head; k-group j of step s holds the elements
+  // its K fragment holds: (s*4+j)*8..+8, or for an e4m3 cache ((s/2)*4+j)*16 + (s%2)*8..+8.
   u32x4 qf[D / 32];
   {
     const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + (size_t)hq_row * D;
 #pragma unroll
     for (int s = 0; s < D / 32; ++s) {
       u32x4 z = {0u, 0u, 0u, 0u};
-      qf[s] = g_valid ? *reinterpret_cast<const u32x4*>(qrow + (s * 4 + j) * 8) : z;
+      const int el = FP8 ? ((s >> 1) * 4 + j) * 16 + (s & 1) * 8 : (s * 4 + j) * 8;
+      qf[s] = g_valid ? *reinterpret_cast<const u32x4*>(qrow + el) : z;
     }
   }
 
   const char* kc = reinterpret_cast<const char*>(p.kc);
   const char* vc = reinterpret_cast<const char*>(p.vc);
   const int32_t* table = p.block_table + (size_t)b * p.max_blocks;
-  const uint32_t koff = (uint32_t)(c * D + j * 8) * 2;        // byte offset of this lane in a K tile
-  const uint32_t voff = (uint32_t)(j * 4 * D + c * 8) * 2;    // ... in a V tile
+  constexpr int kEsz = FP8 ? 1 : 2;                                // bytes per cache element
+  const uint32_t koff = (uint32_t)(c * D * kEsz + j * 16);             // byte offset of this lane in a K tile
+  const uint32_t voff = (uint32_t)(j * 4 * D * kEsz + c * 8 * kEsz);   // ... in a V tile
 
   // Byte offset of the 16-token tile starting at logical token `tok` (wave-uniform).
+  int blk_of_tile = 0;  // physical block of the tile last looked up
   auto tile_offset = [&](int tok) -> size_t {
     // A tile past the end is never used; point it at the partition's first tile so the load
     // stays in bounds even when the block table holds nothing for that logical block.
     if (tok >= tok_end) tok = tok_begin;
-    const int blk = table[tok / p.bs];
-    return ((size_t)(blk * p.hkv + h) * p.bs + (tok % p.bs)) * (D * 2);
+    blk_of_tile = table[tok / p.bs];
+    return ((size_t)(blk_of_tile * p.hkv + h) * p.bs + (tok % p.bs)) * (D * kEsz);
   };
 
   f32x4 acc[D / 128][8];
@@ -193,28 +220,52 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   // the K registers, V of chunk n at the top of iteration n.  All loads are unconditional (the
   // look-ahead past the last chunk re-reads the first tile, a cache hit) so that the number of
   // requests in flight at each wait is known at compile time.
-  KFrag<D> kf;
-  VFrag<D> vf;
-  size_t o0 = tile_offset(tok_begin), o1 = tile_offset(tok_begin + 16);
-  load_k<D>(kf, kc + o0, kc + o1, koff);
+  KFrag<D, FP8> kf;
+  VFrag<D, FP8> vf;
+  size_t o0 = tile_offset(tok_begin + 16), o1 = o0;
+  o1 = o0;
+  o0 = tile_offset(tok_begin);
+  // e4m3 cache: a chunk lies inside one block (block_size is a multiple of 32), whose two scales
+  // apply to the whole chunk.  The accumulators are kept in units of the current block's V
+  // scale, v_unit; they are converted when the block changes and once more at the end.
+  float k_mul = p.scale_log2e, v_unit = 1.f, v_next = 1.f, k_next = p.scale_log2e;
+  if constexpr (FP8) {
+    k_mul = p.scale_log2e * p.k_scale[blk_of_tile * p.hkv + h];
+    v_unit = p.v_scale[blk_of_tile * p.hkv + h];
+  }
+  load_k<D, FP8>(kf, kc + o0, kc + o1, koff);
 
   for (int tok = tok_begin; tok < tok_end; tok += kChunk) {
-    load_v<D>(vf, vc + o0, vc + o1, voff);
-    o0 = tile_offset(tok + kChunk);
+    load_v<D, FP8>(vf, vc + o0, vc + o1, voff);
     o1 = tile_offset(tok + kChunk + 16);
+    o0 = tile_offset(tok + kChunk);
+    if constexpr (FP8) {
+      k_next = p.scale_log2e * p.k_scale[blk_of_tile * p.hkv + h];
+      v_next = p.v_scale[blk_of_tile * p.hkv + h];
+    }
 
     // ---- S^T = K Q^T : two 16x16 tiles, rows = tokens, columns = query heads ----
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (FP8) {
 #pragma unroll
-    for (int s = 0; s < D / 32; ++s) {
-      s0 = mfma16<BF16>(kf.t[0][s], qf[s], s0);
-      s1 = mfma16<BF16>(kf.t[1][s], qf[s], s1);
+      for (int s2 = 0; s2 < D / 64; ++s2) {
+        s0 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[0][s2][0], kf.t[0][s2][1]), qf[2 * s2], s0);
+        s1 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[1][s2][0], kf.t[1][s2][1]), qf[2 * s2], s1);
+        s0 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[0][s2][2], kf.t[0][s2][3]), qf[2 * s2 + 1], s0);
+        s1 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[1][s2][2], kf.t[1][s2][3]), qf[2 * s2 + 1], s1);
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < D / 32; ++s) {
+        s0 = mfma16<BF16>(kf.t[0][s], qf[s], s0);
+        s1 = mfma16<BF16>(kf.t[1][s], qf[s], s1);
+      }
     }
-    load_k<D>(kf, kc + o0, kc + o1, koff);
+    load_k<D, FP8>(kf, kc + o0, kc + o1, koff);
 
     float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
 #pragma unroll
-    for (int e = 0; e < 8; ++e) sv[e] *= p.scale_log2e;
+    for (int e = 0; e < 8; ++e) sv[e] *= k_mul;
     const bool partial = tok + kChunk > tok_end;
     if (partial) {
 #pragma unroll
@@ -258,22 +309,40 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int t = tok + (e >> 2) * 16 + j * 4 + (e & 3);
-          if (t >= tok_end) vf.t[set][e] = u32x4{0u, 0u, 0u, 0u};
+          if (t >= tok_end) vf.t[set][e] = typename std::conditional<FP8, uint2, u32x4>::type{};
         }
     }
 
     // ---- O^T += V^T P^T : transpose each lane's 8 tokens x 8 elements, then 8 MFMAs ----
 #pragma unroll
     for (int set = 0; set < D / 128; ++set) {
+      u32x4 vw[8];  // the lane's 8 tokens x 8 elements as 16-bit values
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if constexpr (FP8) vw[e] = fp8x8_to_bf16x8(vf.t[set][e].x, vf.t[set][e].y);
+        else vw[e] = vf.t[set][e];
+      }
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
         u32x4 vt;
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)
-          vt[kk] = __builtin_amdgcn_perm(vf.t[set][2 * kk + 1][i >> 1], vf.t[set][2 * kk][i >> 1], sel);
+          vt[kk] = __builtin_amdgcn_perm(vw[2 * kk + 1][i >> 1], vw[2 * kk][i >> 1], sel);
         acc[set][i] = mfma16<BF16>(vt, pf, acc[set][i]);
       }
+    }
+    if constexpr (FP8) {
+      // Next chunk may belong to another block: re-express the accumulators in its V scale.
+      if (v_next != v_unit) {
+        const float r = v_unit / v_next;
+#pragma unroll
+        for (int set = 0; set < D / 128; ++set)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[set][i] *= r;
+        v_unit = v_next;
+      }
+      k_mul = k_next;
     }
   }
 
@@ -283,10 +352,10 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
 
   if (!g_valid) return;
   if (p.n_part == 1) {
-    store_rows<D>(p.out + (size_t)hq_row * D, acc, j, l_run > 0.f ? 1.f / l_run : 0.f);
+    store_rows<D>(p.out + (size_t)hq_row * D, acc, j, l_run > 0.f ? v_unit / l_run : 0.f);
   } else {
     const size_t slot = (size_t)hq_row * p.n_part + part;
-    store_rows<D>(p.part_o + slot * D, acc, j, 1.f);
+    store_rows<D>(p.part_o + slot * D, acc, j, v_unit);
     if (j == 0) {
       p.part_ml[slot * 2 + 0] = m_run;
       p.part_ml[slot * 2 + 1] = l_run;
@@ -347,7 +416,7 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
   for (int k = 0; k < D / 64; ++k) p.out[(size_t)row * D + k * 64 + lane] = o[k] * inv;
 }
 
-template <int D>
+template <int D, bool FP8>
 int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   dim3 grid((unsigned)(p.n_part * p.hkv * p.gtiles * batch));
   // Unused dynamic LDS caps the wavefronts resident per CU so that the dispatcher spreads the
@@ -355,9 +424,11 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   const int64_t cap = pto_hip::ctx().attn_waves_per_cu;
   const size_t lds = cap > 0 ? (size_t)(163840 / cap) / 1024 * 1024 : 0;
   if (bf16)
-    hipLaunchKernelGGL((attn_partition_kernel<D, true>), grid, dim3(64), lds, stream, p);
+    hipLaunchKernelGGL((attn_partition_kernel<D, true, FP8>), grid, dim3(64), lds, stream, p);
+  else if constexpr (!FP8)
+    hipLaunchKernelGGL((attn_partition_kernel<D, false, false>), grid, dim3(64), lds, stream, p);
   else
-    hipLaunchKernelGGL((attn_partition_kernel<D, false>), grid, dim3(64), lds, stream, p);
+    return pto_hip::fail(PTO_HIP_ERR_UNSUPPORTED, "paged_attention: an FP8E4M3FN cache needs a BF16 query");
   PTO_CHECK_HIP(hipGetLastError());
   // "attn_skip_merge" leaves the partials unmerged: a timing aid that isolates the streaming
   // kernel; results are not valid in that mode.
@@ -370,13 +441,6 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
 }
 
 }  // namespace
-
-namespace pto_hip {
-int paged_attention_fp8(const void* query, const void* key_cache, const void* value_cache,
-                        const int32_t* block_table, const int32_t* context_lens, float* out,
-                        const int64_t* config, int q_dtype, const float* k_scale,
-                        const float* v_scale, hipStream_t stream);
-}
 
 extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
                                        const void* value_cache, const int32_t* block_table,
@@ -406,14 +470,16 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
                 "paged_attention: max_num_blocks_per_req %lld out of range", (long long)max_blocks);
   PTO_CHECK_ARG(q_dtype == PTO_HIP_BF16 || q_dtype == PTO_HIP_FP16,
                 "paged_attention: query dtype must be BF16 or FP16, got %s", dtype_name(q_dtype));
-  if (kv_dtype == PTO_HIP_FP8E4M3FN) {
+  const bool fp8 = kv_dtype == PTO_HIP_FP8E4M3FN;
+  if (fp8) {
     PTO_CHECK_ARG(k_scale && v_scale, "paged_attention: FP8E4M3FN cache needs k_scale and v_scale");
-    return paged_attention_fp8(query, key_cache, value_cache, block_table, context_lens, out,
-                               config, q_dtype, k_scale, v_scale, (hipStream_t)stream);
+    PTO_CHECK_ARG(bs % 32 == 0, "paged_attention: FP8E4M3FN cache needs block_size %% 32 == 0, got %lld",
+                  (long long)bs);
+  } else {
+    PTO_CHECK_ARG(kv_dtype == q_dtype,
+                  "paged_attention: cache dtype %s must match query dtype %s (or be FP8E4M3FN)",
+                  dtype_name(kv_dtype), dtype_name(q_dtype));
   }
-  PTO_CHECK_ARG(kv_dtype == q_dtype,
-                "paged_attention: cache dtype %s must match query dtype %s (or be FP8E4M3FN)",
-                dtype_name(kv_dtype), dtype_name(q_dtype));
   if (d != 128 && d != 256)
     return fail(PTO_HIP_ERR_UNSUPPORTED, "paged_attention: head_dim %lld not built (128, 256)",
                 (long long)d);
@@ -425,6 +491,8 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
   p.block_table = block_table;
   p.ctx_lens = context_lens;
   p.out = out;
+  p.k_scale = k_scale;
+  p.v_scale = v_scale;
   p.batch = (int)batch;
   p.hq = (int)hq;
   p.hkv = (int)hkv;
@@ -469,6 +537,10 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
     p.part_o = reinterpret_cast<float*>(ws);
     p.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + o_bytes);
   }
-  if (d == 128) return launch<128>(p, (int)batch, bf16, (hipStream_t)stream);
-  return launch<256>(p, (int)batch, bf16, (hipStream_t)stream);
+  if (fp8) {
+    if (d == 128) return launch<128, true>(p, (int)batch, bf16, (hipStream_t)stream);
+    return launch<256, true>(p, (int)batch, bf16, (hipStream_t)stream);
+  }
+  if (d == 128) return launch<128, false>(p, (int)batch, bf16, (hipStream_t)stream);
+  return launch<256, false>(p, (int)batch, bf16, (hipStream_t)stream);
 }

@@ -134,3 +134,56 @@ def test_full_size_small_config_properties(worker):
         _check(o, ref)
     assert (outs[0] - outs[1]).abs().max() < 2e-3
     assert (outs[0] - outs[2]).abs().max() < 2e-3
+
+
+# ---- e4m3 KV cache with one fp32 scale per (block, KV head) -------------------------------
+
+@pytest.mark.parametrize(
+    "batch,hq,hkv,bs,ctxs",
+    [
+        (3, 16, 2, 128, [300, 17, 129]),
+        (2, 64, 8, 128, [1500, 640]),        # group of 8, several blocks per partition
+        (4, 8, 8, 32, [1, 32, 33, 200]),     # one query head per KV head, small blocks
+        (2, 32, 2, 64, [0, 777]),            # empty sequence
+    ],
+)
+def test_fp8_cache_matches_golden(worker, batch, hq, hkv, bs, ctxs):
+    inp = workloads.paged_attention_inputs(batch=batch, num_heads=hq, kv_head_num=hkv, block_size=bs,
+                                           context_lens=ctxs, ctx_range=(1, max(ctxs)), fp8_kv=True, seed=11)
+    assert inp.key_cache.dtype == torch.float8_e4m3fn
+    ref = _golden(inp)
+    for tpp in (0, 64, 512):
+        _check(_run(worker, inp, tpp), ref)
+
+
+def test_fp8_quantiser_agrees_with_oracle():
+    """The input builder's quantiser and the oracle's are the same function of the data."""
+    g = torch.Generator().manual_seed(0)
+    cache = torch.randn(4 * 2 * 32, 128, generator=g).to(torch.bfloat16)
+    a, sa = workloads._quantize_fp8(cache, 4, 2, 32)
+    b, sb = oracle.quantize_kv_fp8(cache, 4, 2, 32)
+    assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)) and torch.equal(sa, sb)
+
+
+def test_fp8_scale_plumbing(worker):
+    """Doubling every V scale doubles the output; a K scale change acts like a softmax scale change."""
+    inp = workloads.paged_attention_inputs(batch=2, num_heads=16, kv_head_num=2, block_size=64,
+                                           context_lens=[200, 64], ctx_range=(1, 200), fp8_kv=True, seed=12)
+    base = _run(worker, inp)
+    inp.v_scale = inp.v_scale * 2
+    assert torch.allclose(_run(worker, inp), base * 2, rtol=1e-6, atol=1e-7)
+    inp.v_scale = inp.v_scale / 2
+    inp.k_scale = inp.k_scale * 0.5
+    half_k = _run(worker, inp)
+    inp.k_scale = inp.k_scale * 2
+    cfg = inp.config.clone()
+    cfg[6] = workloads.scale_bits(0.5 / 128 ** 0.5)
+    inp.config = cfg
+    assert torch.allclose(_run(worker, inp), half_k, rtol=1e-5, atol=1e-6)
+
+
+def test_fp8_rejects_small_blocks(worker):
+    inp = workloads.paged_attention_inputs(batch=1, num_heads=8, kv_head_num=1, block_size=16,
+                                           context_lens=[40], ctx_range=(1, 40), fp8_kv=True, seed=13)
+    with pytest.raises(ValueError, match="block_size % 32"):
+        _run(worker, inp)
