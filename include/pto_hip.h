@@ -120,6 +120,19 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *  "ffn_block"         tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:155-187
  *      tensors: x[T,H], gamma[1,H] fp32, w_gate[H,I], w_up[H,I], w_down[I,H], out[T,H]
  *      scalars: eps (f32 bits)
+ *  "w8a16_matmul"      examples/models/qwen3_jit/kernels/projection.py:145-177 with int8 weights
+ *      tensors: x[M,K], w_q[K,N] i8, w_scale[N] fp32, [residual[M,N],] out[M,N]
+ *  "w8a16_swiglu"      examples/models/qwen3_jit/kernels/mlp.py:22-61 with int8 weights
+ *      tensors: x[M,K], wg_q[K,N] i8, wg_scale[N], wu_q[K,N] i8, wu_scale[N], out[M,N]
+ *  "rope_kv_cache_update"  examples/models/qwen3_jit/kernels/attention.py:39-102
+ *      tensors: qkv[B,(Hq+2Hkv)*D] fp32, seq_lens[B] i32, rope_cos[max_pos,D/2], rope_sin,
+ *               block_table[B*max_blocks] i32, key_cache (INOUT), value_cache (INOUT), q_out[B*Hq,D]
+ *      scalars: num_heads, kv_head_num, head_dim, block_size
+ *  "decoder_layer_decode"  examples/models/qwen3_jit/qwen3_decode.py:47-113
+ *      tensors: hidden_states[B,H], seq_lens, block_table, key_cache (INOUT), value_cache (INOUT),
+ *               rope_cos, rope_sin, gamma_in[H], gamma_post[H], wqkv_q, wqkv_s, wo_q, wo_s, wg_q, wg_s,
+ *               wu_q, wu_s, wd_q, wd_s, out[B,H]
+ *      scalars: num_heads, kv_head_num, head_dim, block_size, eps (f32 bits)
  */
 PTO_HIP_API int pto_hip_register(const char* program_name, int* callable_id);
 PTO_HIP_API int pto_hip_unregister(int callable_id);
@@ -165,6 +178,63 @@ PTO_HIP_API int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void
                                    const void* w_up, const void* w_down, void* out,
                                    int64_t tokens, int64_t hidden, int64_t intermediate,
                                    float eps, int dtype, int out_dtype, void* stream);
+
+/* W8A16 decode projection (no counterpart in the reference, which has no quantised weights; the
+ * contract is its projection kernel's, examples/models/qwen3_jit/kernels/projection.py:145-177,
+ * x @ W with W [in, out]):  out[M<=32, N] = (x[M,K] @ w_q[K,N]) * w_scale[N] (+ residual[M,N]).
+ * x is BF16/FP16, w_q INT8, accumulation fp32; residual may be NULL. */
+PTO_HIP_API int pto_hip_w8a16_matmul(const void* x, const void* w_q, const float* w_scale,
+                                     const void* residual, void* out, int64_t m, int64_t k, int64_t n,
+                                     int x_dtype, int res_dtype, int out_dtype, void* stream);
+
+/* out[M,N] = SiLU((x @ wg_q) * wg_scale) * ((x @ wu_q) * wu_scale): the gate/up half of the
+ * FFN with int8 weights (examples/models/qwen3_jit/kernels/mlp.py:22-61). */
+PTO_HIP_API int pto_hip_w8a16_swiglu(const void* x, const void* wg_q, const float* wg_scale,
+                                     const void* wu_q, const float* wu_scale, void* out, int64_t m,
+                                     int64_t k, int64_t n, int x_dtype, int out_dtype, void* stream);
+
+/* RoPE at pos = seq_len - 1, K/V rows appended to the paged cache, rotated Q cast to `dtype`
+ * (examples/models/qwen3_jit/kernels/attention.py:39-102).  qkv is FP32 [B, (Hq+2Hkv)*D] laid out
+ * q heads, then k heads, then v heads; rope_cos/rope_sin are FP32 [max_pos, D/2].  A position
+ * outside the tables is skipped and reported by the next pto_hip_sync. */
+PTO_HIP_API int pto_hip_rope_kv_cache_update(const float* qkv, const int32_t* seq_lens,
+                                             const float* rope_cos, const float* rope_sin,
+                                             const int32_t* block_table, void* key_cache,
+                                             void* value_cache, void* q_out, int64_t batch,
+                                             int64_t num_heads, int64_t kv_head_num, int64_t head_dim,
+                                             int64_t block_size, int64_t max_num_blocks_per_req,
+                                             int64_t max_pos, int64_t pool_rows, int dtype, void* stream);
+
+/* One decoder layer, one new token per sequence (examples/models/qwen3_jit/qwen3_decode.py:47-113):
+ * RMSNorm -> QKV -> RoPE + K/V append -> paged attention -> o_proj + residual -> RMSNorm ->
+ * SwiGLU FFN + residual.  Projection weights are INT8 [in, out] with FP32 per-output scales. */
+typedef struct PtoHipDecoderLayerArgs {
+  const void* hidden_states;  /* [B, H] dtype */
+  const int32_t* seq_lens;    /* [B] context length including the new token */
+  const int32_t* block_table; /* [B, max_num_blocks_per_req] */
+  void* key_cache;            /* [pool_rows, D] dtype, updated in place */
+  void* value_cache;
+  const float* rope_cos;      /* [max_pos, D/2] */
+  const float* rope_sin;
+  const float* gamma_in;      /* [H] */
+  const float* gamma_post;    /* [H] */
+  const void* wqkv_q;         /* [H, (Hq+2Hkv)*D] int8 */
+  const float* wqkv_s;
+  const void* wo_q;           /* [Hq*D, H] */
+  const float* wo_s;
+  const void* wg_q;           /* [H, I] */
+  const float* wg_s;
+  const void* wu_q;           /* [H, I] */
+  const float* wu_s;
+  const void* wd_q;           /* [I, H] */
+  const float* wd_s;
+  void* out;                  /* [B, H] dtype */
+  int64_t batch, hidden, num_heads, kv_head_num, head_dim, intermediate;
+  int64_t block_size, max_num_blocks_per_req, max_pos, pool_rows;
+  float eps;
+  int32_t dtype;              /* PTO_HIP_BF16 or PTO_HIP_FP16 */
+} PtoHipDecoderLayerArgs;
+PTO_HIP_API int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* args, void* stream);
 
 /* ---- tuning knobs (integers by name; unknown names are PTO_HIP_ERR_NOT_FOUND) ------------
  *  "attn_tokens_per_partition"  0 = choose from the device's CU count (default)

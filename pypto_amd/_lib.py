@@ -22,6 +22,8 @@ EXPORTS = (
     "pto_hip_register", "pto_hip_unregister", "pto_hip_run", "pto_hip_kernel_entry",
     "pto_hip_benchmark", "pto_hip_paged_attention", "pto_hip_paged_gather", "pto_hip_rms_norm",
     "pto_hip_ffn_swiglu", "pto_hip_set_option", "pto_hip_get_option",
+    "pto_hip_w8a16_matmul", "pto_hip_w8a16_swiglu", "pto_hip_rope_kv_cache_update",
+    "pto_hip_decoder_layer_decode",
 )
 
 
@@ -87,6 +89,11 @@ def load() -> C.CDLL:
         "pto_hip_paged_gather": [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, C.c_int, vp],
         "pto_hip_rms_norm": [vp, vp, vp, i64, i64, C.c_float, C.c_int, C.c_int, vp],
         "pto_hip_ffn_swiglu": [vp, vp, vp, vp, vp, vp, i64, i64, i64, C.c_float, C.c_int, C.c_int, vp],
+        "pto_hip_w8a16_matmul": [vp, vp, vp, vp, vp, i64, i64, i64, C.c_int, C.c_int, C.c_int, vp],
+        "pto_hip_w8a16_swiglu": [vp, vp, vp, vp, vp, vp, i64, i64, i64, C.c_int, C.c_int, vp],
+        "pto_hip_rope_kv_cache_update": [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64,
+                                         C.c_int, vp],
+        "pto_hip_decoder_layer_decode": [vp, vp],
         "pto_hip_set_option": [C.c_char_p, i64],
         "pto_hip_get_option": [C.c_char_p, C.POINTER(i64)],
     }

@@ -44,6 +44,9 @@ struct Context {
   // every such kernel leaves them zero again.
   int* counters = nullptr;
   size_t counters_len = 0;
+  // Intermediates of the composed decoder layer (grow-only).
+  void* layer_ws = nullptr;
+  size_t layer_ws_bytes = 0;
   // 256 bytes of device flags written by kernels that report bad indices to the host.
   int* flags = nullptr;
   // options

@@ -54,7 +54,10 @@ int counters(size_t n, int** ptr) {
   Context& c = ctx();
   if (n > c.counters_len) {
     PTO_CHECK_HIP(hipDeviceSynchronize());
-    if (c.counters) PTO_CHECK_HIP(hipFree(c.counters));
+    if (c.layer_ws) PTO_CHECK_HIP(hipFree(c.layer_ws));
+  c.layer_ws = nullptr;
+  c.layer_ws_bytes = 0;
+  if (c.counters) PTO_CHECK_HIP(hipFree(c.counters));
     c.counters = nullptr;
     c.counters_len = 0;
     size_t want = n + n / 2 + 1024;
@@ -74,11 +77,16 @@ enum ProgramKind {
   kRmsNorm,
   kFfnSwiglu,
   kFfnBlock,
+  kW8a16Matmul,
+  kW8a16Swiglu,
+  kRopeKvCacheUpdate,
+  kDecoderLayerDecode,
   kNumPrograms
 };
 
-const char* const kProgramNames[kNumPrograms] = {"paged_attention", "paged_gather", "rms_norm",
-                                                 "ffn_swiglu", "ffn_block"};
+const char* const kProgramNames[kNumPrograms] = {
+    "paged_attention", "paged_gather",  "rms_norm",           "ffn_swiglu",          "ffn_block",
+    "w8a16_matmul",    "w8a16_swiglu",  "rope_kv_cache_update", "decoder_layer_decode"};
 
 std::mutex g_mu;
 std::vector<int> g_callables;  // callable id -> ProgramKind, -1 once unregistered
@@ -259,6 +267,143 @@ int run_ffn(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStr
                             hidden, inter, eps, (int)x.dtype, (int)out.dtype, stream);
 }
 
+int run_w8a16_matmul(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
+  PTO_CHECK_ARG((nt == 4 || nt == 5) && ns == 0,
+                "w8a16_matmul: expected x, w_q, w_scale, [residual,] out and no scalars, got %d + %d", nt, ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor("w8a16_matmul", "operand", t[i], 1, 2);
+    if (rc) return rc;
+  }
+  const PtoHipChipTensor &x = t[0], &wq = t[1], &ws = t[2], &out = t[nt - 1];
+  PTO_CHECK_ARG(x.ndims == 2 && wq.ndims == 2 && out.ndims == 2, "w8a16_matmul: x, w_q and out must be 2-D");
+  const int64_t m = x.shapes[0], k = x.shapes[1], n = wq.shapes[1];
+  PTO_CHECK_ARG(wq.dtype == PTO_HIP_INT8 && wq.shapes[0] == k, "w8a16_matmul: w_q must be INT8 [K=%lld, N]", (long long)k);
+  PTO_CHECK_ARG(ws.dtype == PTO_HIP_FP32 && numel(ws) == n, "w8a16_matmul: w_scale must be FP32 [N=%lld]", (long long)n);
+  PTO_CHECK_ARG(out.shapes[0] == m && out.shapes[1] == n, "w8a16_matmul: out must be [M, N]");
+  const void* res = nullptr;
+  int res_dt = 0;
+  if (nt == 5) {
+    PTO_CHECK_ARG(numel(t[3]) == m * n, "w8a16_matmul: residual must be [M, N]");
+    res = tptr(t[3]);
+    res_dt = (int)t[3].dtype;
+    PTO_CHECK_ARG(res_dt == PTO_HIP_FP32 || res_dt == PTO_HIP_BF16 || res_dt == PTO_HIP_FP16,
+                  "w8a16_matmul: residual dtype %s not in {FP32, BF16, FP16}", dtype_name(res_dt));
+  }
+  return pto_hip_w8a16_matmul(tptr(x), tptr(wq), reinterpret_cast<const float*>(tptr(ws)), res, tptr_mut(out), m, k,
+                              n, (int)x.dtype, res_dt, (int)out.dtype, stream);
+}
+
+int run_w8a16_swiglu(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
+  PTO_CHECK_ARG(nt == 6 && ns == 0, "w8a16_swiglu: expected x, wg_q, wg_scale, wu_q, wu_scale, out, got %d + %d", nt, ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor("w8a16_swiglu", "operand", t[i], 1, 2);
+    if (rc) return rc;
+  }
+  const PtoHipChipTensor& x = t[0];
+  PTO_CHECK_ARG(x.ndims == 2 && t[1].ndims == 2 && t[3].ndims == 2 && t[5].ndims == 2, "w8a16_swiglu: matrices must be 2-D");
+  const int64_t m = x.shapes[0], k = x.shapes[1], n = t[1].shapes[1];
+  PTO_CHECK_ARG(t[1].dtype == PTO_HIP_INT8 && t[3].dtype == PTO_HIP_INT8 && t[1].shapes[0] == k &&
+                    t[3].shapes[0] == k && t[3].shapes[1] == n,
+                "w8a16_swiglu: weights must be INT8 [K, N]");
+  PTO_CHECK_ARG(t[2].dtype == PTO_HIP_FP32 && t[4].dtype == PTO_HIP_FP32 && numel(t[2]) == n && numel(t[4]) == n,
+                "w8a16_swiglu: scales must be FP32 [N]");
+  PTO_CHECK_ARG(t[5].shapes[0] == m && t[5].shapes[1] == n, "w8a16_swiglu: out must be [M, N]");
+  return pto_hip_w8a16_swiglu(tptr(x), tptr(t[1]), reinterpret_cast<const float*>(tptr(t[2])), tptr(t[3]),
+                              reinterpret_cast<const float*>(tptr(t[4])), tptr_mut(t[5]), m, k, n, (int)x.dtype,
+                              (int)t[5].dtype, stream);
+}
+
+int run_rope_kv(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream) {
+  PTO_CHECK_ARG(nt == 8 && ns == 4,
+                "rope_kv_cache_update: expected qkv, seq_lens, rope_cos, rope_sin, block_table, key_cache, "
+                "value_cache, q_out + scalars num_heads, kv_head_num, head_dim, block_size; got %d + %d", nt, ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor("rope_kv_cache_update", "operand", t[i], 1, 2);
+    if (rc) return rc;
+  }
+  const int64_t hq = (int64_t)s[0], hkv = (int64_t)s[1], d = (int64_t)s[2], bs = (int64_t)s[3];
+  PTO_CHECK_ARG(hq > 0 && hkv > 0 && d > 0 && bs > 0, "rope_kv_cache_update: non-positive scalar");
+  const int64_t batch = numel(t[1]);
+  PTO_CHECK_ARG(t[0].dtype == PTO_HIP_FP32 && numel(t[0]) == batch * (hq + 2 * hkv) * d,
+                "rope_kv_cache_update: qkv must be FP32 [B, (Hq+2Hkv)*D]");
+  PTO_CHECK_ARG(t[1].dtype == PTO_HIP_INT32 && t[4].dtype == PTO_HIP_INT32,
+                "rope_kv_cache_update: seq_lens and block_table must be INT32");
+  PTO_CHECK_ARG(t[2].dtype == PTO_HIP_FP32 && t[3].dtype == PTO_HIP_FP32 && numel(t[2]) == numel(t[3]) &&
+                    numel(t[2]) % (d / 2) == 0,
+                "rope_kv_cache_update: rope_cos/rope_sin must be FP32 [max_pos, D/2]");
+  PTO_CHECK_ARG(batch > 0 ? numel(t[4]) % batch == 0 : true, "rope_kv_cache_update: block_table must be [B, max_blocks]");
+  PTO_CHECK_ARG(t[5].dtype == t[6].dtype && t[5].dtype == t[7].dtype && numel(t[5]) == numel(t[6]) &&
+                    numel(t[5]) % d == 0 && numel(t[7]) == batch * hq * d,
+                "rope_kv_cache_update: caches and q_out must share a dtype; caches [rows, D], q_out [B*Hq, D]");
+  return pto_hip_rope_kv_cache_update(reinterpret_cast<const float*>(tptr(t[0])),
+                                      reinterpret_cast<const int32_t*>(tptr(t[1])),
+                                      reinterpret_cast<const float*>(tptr(t[2])),
+                                      reinterpret_cast<const float*>(tptr(t[3])),
+                                      reinterpret_cast<const int32_t*>(tptr(t[4])), tptr_mut(t[5]), tptr_mut(t[6]),
+                                      tptr_mut(t[7]), batch, hq, hkv, d, bs, batch ? numel(t[4]) / batch : 1,
+                                      numel(t[2]) / (d / 2), numel(t[5]) / d, (int)t[5].dtype, stream);
+}
+
+int run_decoder_layer(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream) {
+  PTO_CHECK_ARG(nt == 20 && ns == 5,
+                "decoder_layer_decode: expected 20 tensors + scalars num_heads, kv_head_num, head_dim, "
+                "block_size, eps; got %d + %d", nt, ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor("decoder_layer_decode", "operand", t[i], 1, 2);
+    if (rc) return rc;
+  }
+  PtoHipDecoderLayerArgs a{};
+  a.hidden_states = tptr(t[0]);
+  a.seq_lens = reinterpret_cast<const int32_t*>(tptr(t[1]));
+  a.block_table = reinterpret_cast<const int32_t*>(tptr(t[2]));
+  a.key_cache = tptr_mut(t[3]);
+  a.value_cache = tptr_mut(t[4]);
+  a.rope_cos = reinterpret_cast<const float*>(tptr(t[5]));
+  a.rope_sin = reinterpret_cast<const float*>(tptr(t[6]));
+  a.gamma_in = reinterpret_cast<const float*>(tptr(t[7]));
+  a.gamma_post = reinterpret_cast<const float*>(tptr(t[8]));
+  a.wqkv_q = tptr(t[9]);
+  a.wqkv_s = reinterpret_cast<const float*>(tptr(t[10]));
+  a.wo_q = tptr(t[11]);
+  a.wo_s = reinterpret_cast<const float*>(tptr(t[12]));
+  a.wg_q = tptr(t[13]);
+  a.wg_s = reinterpret_cast<const float*>(tptr(t[14]));
+  a.wu_q = tptr(t[15]);
+  a.wu_s = reinterpret_cast<const float*>(tptr(t[16]));
+  a.wd_q = tptr(t[17]);
+  a.wd_s = reinterpret_cast<const float*>(tptr(t[18]));
+  a.out = tptr_mut(t[19]);
+  PTO_CHECK_ARG(t[0].ndims == 2, "decoder_layer_decode: hidden_states must be [B, H]");
+  a.batch = t[0].shapes[0];
+  a.hidden = t[0].shapes[1];
+  a.num_heads = (int64_t)s[0];
+  a.kv_head_num = (int64_t)s[1];
+  a.head_dim = (int64_t)s[2];
+  a.block_size = (int64_t)s[3];
+  a.eps = scalar_f32(s[4]);
+  PTO_CHECK_ARG(a.num_heads > 0 && a.kv_head_num > 0 && a.head_dim > 1 && a.block_size > 0,
+                "decoder_layer_decode: non-positive scalar");
+  PTO_CHECK_ARG(t[13].ndims == 2, "decoder_layer_decode: w_gate must be [H, I]");
+  a.intermediate = t[13].shapes[1];
+  a.max_num_blocks_per_req = a.batch ? numel(t[2]) / a.batch : 1;
+  a.max_pos = numel(t[5]) / (a.head_dim / 2);
+  a.pool_rows = numel(t[3]) / a.head_dim;
+  a.dtype = (int)t[0].dtype;
+  const int64_t qkv_n = (a.num_heads + 2 * a.kv_head_num) * a.head_dim;
+  PTO_CHECK_ARG(t[3].dtype == t[0].dtype && t[4].dtype == t[0].dtype && t[19].dtype == t[0].dtype,
+                "decoder_layer_decode: caches and out must have the activation dtype");
+  PTO_CHECK_ARG(t[9].dtype == PTO_HIP_INT8 && numel(t[9]) == a.hidden * qkv_n && numel(t[10]) == qkv_n &&
+                    numel(t[11]) == a.num_heads * a.head_dim * a.hidden && numel(t[12]) == a.hidden &&
+                    numel(t[13]) == a.hidden * a.intermediate && numel(t[15]) == numel(t[13]) &&
+                    numel(t[17]) == numel(t[13]) && numel(t[14]) == a.intermediate &&
+                    numel(t[16]) == a.intermediate && numel(t[18]) == a.hidden,
+                "decoder_layer_decode: weight or scale shapes do not match the model dimensions");
+  PTO_CHECK_ARG(numel(t[7]) == a.hidden && numel(t[8]) == a.hidden && numel(t[1]) == a.batch &&
+                    numel(t[19]) == a.batch * a.hidden,
+                "decoder_layer_decode: gamma, seq_lens or out shape mismatch");
+  return pto_hip_decoder_layer_decode(&a, stream);
+}
+
 int dispatch(int kind, const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns,
              hipStream_t stream) {
   switch (kind) {
@@ -267,6 +412,10 @@ int dispatch(int kind, const PtoHipChipTensor* t, int nt, const uint64_t* s, int
     case kRmsNorm: return run_rms_norm(t, nt, s, ns, stream);
     case kFfnSwiglu: return run_ffn(t, nt, s, ns, stream, false);
     case kFfnBlock: return run_ffn(t, nt, s, ns, stream, true);
+    case kW8a16Matmul: return run_w8a16_matmul(t, nt, s, ns, stream);
+    case kW8a16Swiglu: return run_w8a16_swiglu(t, nt, s, ns, stream);
+    case kRopeKvCacheUpdate: return run_rope_kv(t, nt, s, ns, stream);
+    case kDecoderLayerDecode: return run_decoder_layer(t, nt, s, ns, stream);
     default: return fail(PTO_HIP_ERR_NOT_FOUND, "unknown program kind %d", kind);
   }
 }
@@ -306,7 +455,10 @@ int pto_hip_init(int device_id) {
                 device_id, prop.gcnArchName);
   c.device = device_id;
   c.num_cu = prop.multiProcessorCount;
-  if (!c.flags) PTO_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&c.flags), 256));
+  if (!c.flags) {
+    PTO_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&c.flags), 256));
+    PTO_CHECK_HIP(hipMemset(c.flags, 0, 256));
+  }
   c.initialized = true;
   ++c.refcount;
   return PTO_HIP_OK;
@@ -323,6 +475,9 @@ int pto_hip_close(void) {
   c.workspace_bytes = 0;
   if (c.flags) PTO_CHECK_HIP(hipFree(c.flags));
   c.flags = nullptr;
+  if (c.layer_ws) PTO_CHECK_HIP(hipFree(c.layer_ws));
+  c.layer_ws = nullptr;
+  c.layer_ws_bytes = 0;
   if (c.counters) PTO_CHECK_HIP(hipFree(c.counters));
   c.counters = nullptr;
   c.counters_len = 0;
@@ -386,6 +541,14 @@ int pto_hip_copy_from(void* dst_host_ptr, uint64_t src_dev_ptr, size_t nbytes) {
 int pto_hip_sync(void* stream) {
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
+  // Device-side argument errors of launches that do not block are reported here.
+  int flags[2] = {0, 0};
+  PTO_CHECK_HIP(hipMemcpy(flags, ctx().flags, sizeof(flags), hipMemcpyDeviceToHost));
+  if (flags[1]) {
+    PTO_CHECK_HIP(hipMemset(ctx().flags + 1, 0, sizeof(int)));
+    return fail(PTO_HIP_ERR_INVALID_VALUE,
+                "rope_kv_cache_update: a decode position lies outside the rope table, the block table or the cache");
+  }
   return PTO_HIP_OK;
 }
 

@@ -211,3 +211,102 @@ def ffn_llama7b(seed: int = 0, device="cpu") -> FfnInputs:
     """FFN at LLaMA-7B shape: T2048 H4096 I11008 bf16 with RMSNorm prologue."""
     return ffn_inputs(tokens=2048, hidden=4096, intermediate=11008, dtype=torch.bfloat16, with_norm=True,
                       seed=seed, device=device)
+
+
+def quantize_w8(w: torch.Tensor):
+    """Per-output-channel symmetric int8 of a [in, out] weight: (codes int8, scale fp32 [out])."""
+    wf = w.float()
+    amax = wf.abs().amax(dim=0)
+    scale = torch.where(amax > 0, amax / 127.0, torch.ones_like(amax))
+    codes = torch.clamp(torch.round(wf / scale), -127, 127).to(torch.int8)
+    return codes.contiguous(), scale.contiguous()
+
+
+def rope_tables(max_pos: int, head_dim: int, theta: float = 5e5, device="cpu"):
+    """cos/sin [max_pos, head_dim/2] fp32: angle = pos * theta^(-2i/head_dim)."""
+    half = head_dim // 2
+    inv = 1.0 / (theta ** (2 * torch.arange(half, dtype=torch.float32, device=device) / head_dim))
+    ang = torch.arange(max_pos, dtype=torch.float32, device=device).unsqueeze(1) * inv.unsqueeze(0)
+    return torch.cos(ang).contiguous(), torch.sin(ang).contiguous()
+
+
+@dataclass
+class DecoderLayerInputs:
+    hidden: torch.Tensor
+    seq_lens: torch.Tensor
+    block_table: torch.Tensor
+    key_cache: torch.Tensor
+    value_cache: torch.Tensor
+    rope_cos: torch.Tensor
+    rope_sin: torch.Tensor
+    gamma_in: torch.Tensor
+    gamma_post: torch.Tensor
+    weights: dict  # name -> (codes int8 [in,out], scale fp32 [out]) for qkv, o, gate, up, down
+    out: torch.Tensor
+    num_heads: int
+    kv_head_num: int
+    head_dim: int
+    block_size: int
+    max_num_blocks_per_req: int
+    eps: float = 1e-6
+
+    def args(self) -> tuple:
+        w = self.weights
+        return (self.hidden, self.seq_lens, self.block_table, self.key_cache, self.value_cache, self.rope_cos,
+                self.rope_sin, self.gamma_in, self.gamma_post, *w["qkv"], *w["o"], *w["gate"], *w["up"], *w["down"],
+                self.out, self.num_heads, self.kv_head_num, self.head_dim, self.block_size, self.eps)
+
+    def algorithmic_bytes(self) -> int:
+        """int8 weights + the K/V rows attention reads (the HBM-bound part of the step)."""
+        wbytes = sum(c.numel() for c, _ in self.weights.values())
+        kv = int(self.seq_lens.sum().item()) * self.kv_head_num * self.head_dim * 2 * self.key_cache.element_size()
+        return wbytes + kv
+
+
+def decoder_layer_inputs(*, batch=32, hidden=4096, num_heads=32, kv_head_num=8, head_dim=128,
+                         intermediate=14336, context=4096, block_size=128, theta=5e5,
+                         dtype=torch.bfloat16, seed=0, device="cpu", context_lens=None) -> DecoderLayerInputs:
+    """One decode step of a LLaMA-style layer: int8 weights from N(0,0.02), bf16 activations and KV."""
+    dev = torch.device(device)
+    g = torch.Generator(device=dev).manual_seed(seed)
+
+    def rn(shape, std=1.0, mean=0.0):
+        return torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * std + mean
+
+    if context_lens is None:
+        context_lens = [context] * batch
+    ctx = torch.tensor(context_lens, dtype=torch.int64)
+    max_blocks = (max(int(ctx.max()), 1) + block_size - 1) // block_size
+    nblk = (ctx + block_size - 1) // block_size
+    total = max(int(nblk.sum()), 1)
+    gc = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(total, generator=gc).to(torch.int32)
+    table = torch.zeros((batch, max_blocks), dtype=torch.int32)
+    off = 0
+    for b in range(batch):
+        n = int(nblk[b])
+        table[b, :n] = perm[off:off + n]
+        off += n
+    rows = total * kv_head_num * block_size
+    qkv_n = (num_heads + 2 * kv_head_num) * head_dim
+    weights = {
+        "qkv": quantize_w8(rn((hidden, qkv_n), 0.02)),
+        "o": quantize_w8(rn((num_heads * head_dim, hidden), 0.02)),
+        "gate": quantize_w8(rn((hidden, intermediate), 0.02)),
+        "up": quantize_w8(rn((hidden, intermediate), 0.02)),
+        "down": quantize_w8(rn((intermediate, hidden), 0.02)),
+    }
+    cos, sin = rope_tables(max_blocks * block_size, head_dim, theta, device=dev)
+    return DecoderLayerInputs(
+        hidden=rn((batch, hidden)).to(dtype),
+        seq_lens=ctx.to(torch.int32).to(dev),
+        block_table=table.flatten().contiguous().to(dev),
+        key_cache=rn((rows, head_dim)).to(dtype),
+        value_cache=rn((rows, head_dim)).to(dtype),
+        rope_cos=cos, rope_sin=sin,
+        gamma_in=rn((hidden,), 0.02, 1.0), gamma_post=rn((hidden,), 0.02, 1.0),
+        weights=weights,
+        out=torch.zeros((batch, hidden), dtype=dtype, device=dev),
+        num_heads=num_heads, kv_head_num=kv_head_num, head_dim=head_dim, block_size=block_size,
+        max_num_blocks_per_req=max_blocks,
+    )

@@ -1,0 +1,133 @@
+"""GPU parity: W8A16 projections, RoPE + KV append, and one decoder-layer decode step vs the oracle."""
+
+import pytest
+import torch
+
+import oracle
+from pypto_amd import workloads
+from pypto_amd.runtime import (decoder_layer_decode, rope_kv_cache_update, validate_golden, w8a16_matmul,
+                               w8a16_matmul_residual, w8a16_swiglu)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,n", [(32, 4096, 6144), (5, 256, 264), (1, 1024, 8), (32, 14336, 4096)])
+def test_w8a16_matmul(worker, dtype, m, k, n):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(m, k, generator=g).to(dtype)
+    wq, s = workloads.quantize_w8(0.02 * torch.randn(k, n, generator=g))
+    out = torch.zeros(m, n)
+    with worker.register(w8a16_matmul) as h:
+        h(x, wq, s, out)
+    ref = oracle.w8a16_matmul(x, wq, s)
+    # exact products, fp32 accumulation in a different order: relative 1e-5 of the row scale
+    validate_golden({"out": out}, {"out": ref}, rtol=1e-4, atol=1e-4 * float(ref.abs().max()))
+    res = torch.randn(m, n, generator=g)
+    out16 = torch.zeros(m, n, dtype=dtype)
+    with worker.register(w8a16_matmul_residual) as h:
+        h(x, wq, s, res, out16)
+    validate_golden({"out": out16.float()}, {"out": (ref + res).to(dtype).float()}, rtol=1e-2, atol=1e-2)
+
+
+def test_w8a16_quantiser_matches_oracle():
+    g = torch.Generator().manual_seed(1)
+    w = 0.02 * torch.randn(64, 48, generator=g)
+    a, sa = workloads.quantize_w8(w)
+    b, sb = oracle.quantize_w8(w)
+    assert torch.equal(a, b) and torch.equal(sa, sb)
+
+
+def test_w8a16_swiglu(worker):
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(32, 512, generator=g).to(torch.bfloat16)
+    wg, sg = workloads.quantize_w8(0.05 * torch.randn(512, 1024, generator=g))
+    wu, su = workloads.quantize_w8(0.05 * torch.randn(512, 1024, generator=g))
+    out = torch.zeros(32, 1024, dtype=torch.bfloat16)
+    with worker.register(w8a16_swiglu) as h:
+        h(x, wg, sg, wu, su, out)
+    ref = oracle.swiglu(oracle.w8a16_matmul(x, wg, sg), oracle.w8a16_matmul(x, wu, su)).to(torch.bfloat16)
+    validate_golden({"out": out.float()}, {"out": ref.float()}, rtol=1e-2, atol=1e-3)
+
+
+def test_w8a16_argument_rules(worker):
+    x = torch.zeros(33, 64, dtype=torch.bfloat16)
+    wq = torch.zeros(64, 64, dtype=torch.int8)
+    s = torch.ones(64)
+    with pytest.raises(ValueError, match="at most 32"):
+        with worker.register(w8a16_matmul) as h:
+            h(x, wq, s, torch.zeros(33, 64))
+
+
+def test_rope_kv_cache_update(worker):
+    b, hq, hkv, d, bs = 3, 8, 2, 128, 16
+    seq = [17, 1, 40]
+    inp = workloads.decoder_layer_inputs(batch=b, hidden=256, num_heads=hq, kv_head_num=hkv, head_dim=d,
+                                         intermediate=512, block_size=bs, context_lens=seq, seed=3)
+    g = torch.Generator().manual_seed(4)
+    qkv = torch.randn(b, (hq + 2 * hkv) * d, generator=g)
+    kc, vc = inp.key_cache.clone(), inp.value_cache.clone()
+    q_out = torch.zeros(b * hq, d, dtype=torch.bfloat16)
+    with worker.register(rope_kv_cache_update) as h:
+        h(qkv, inp.seq_lens, inp.rope_cos, inp.rope_sin, inp.block_table, kc, vc, q_out, hq, hkv, d, bs)
+    pos = torch.tensor(seq) - 1
+    cos, sin = inp.rope_cos[pos].unsqueeze(1), inp.rope_sin[pos].unsqueeze(1)
+    q = oracle.rope_rotate_half(qkv[:, :hq * d].reshape(b, hq, d), cos, sin).to(torch.bfloat16)
+    k = oracle.rope_rotate_half(qkv[:, hq * d:(hq + hkv) * d].reshape(b, hkv, d), cos, sin).to(torch.bfloat16)
+    v = qkv[:, (hq + hkv) * d:].reshape(b, hkv, d).to(torch.bfloat16)
+    assert torch.allclose(q_out.float(), q.reshape(-1, d).float(), atol=2e-2, rtol=1e-2)
+    table = inp.block_table.reshape(b, -1)
+    touched = set()
+    for bi in range(b):
+        p = int(pos[bi])
+        for hh in range(hkv):
+            row = (int(table[bi, p // bs]) * hkv + hh) * bs + p % bs
+            touched.add(row)
+            assert torch.allclose(kc[row].float(), k[bi, hh].float(), atol=2e-2, rtol=1e-2)
+            assert torch.equal(vc[row], v[bi, hh])
+    keep = torch.ones(kc.shape[0], dtype=torch.bool)
+    keep[list(touched)] = False
+    assert torch.equal(kc[keep], inp.key_cache[keep]) and torch.equal(vc[keep], inp.value_cache[keep])
+
+
+def test_rope_position_out_of_range_is_reported(worker):
+    inp = workloads.decoder_layer_inputs(batch=1, hidden=256, num_heads=2, kv_head_num=1, head_dim=128,
+                                         intermediate=512, block_size=16, context_lens=[16], seed=5)
+    qkv = torch.zeros(1, 4 * 128)
+    bad = torch.tensor([500], dtype=torch.int32)  # beyond the rope table and the block table
+    q_out = torch.zeros(2, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="decode position"):
+        with worker.register(rope_kv_cache_update) as h:
+            h(qkv, bad, inp.rope_cos, inp.rope_sin, inp.block_table, inp.key_cache.clone(), inp.value_cache.clone(),
+              q_out, 2, 1, 128, 16)
+
+
+def _oracle_layer(inp):
+    w = inp.weights
+    return oracle.decoder_layer_decode(
+        inp.hidden, inp.seq_lens, inp.block_table, inp.key_cache, inp.value_cache, inp.rope_cos, inp.rope_sin,
+        inp.gamma_in, inp.gamma_post, *w["qkv"], *w["o"], *w["gate"], *w["up"], *w["down"],
+        num_heads=inp.num_heads, kv_head_num=inp.kv_head_num, head_dim=inp.head_dim, block_size=inp.block_size,
+        max_num_blocks_per_req=inp.max_num_blocks_per_req, eps=inp.eps)
+
+
+@pytest.mark.parametrize("batch,ctxs", [(4, [100, 1, 257, 33]), (32, None)])
+def test_decoder_layer_decode(worker, batch, ctxs):
+    """Reduced model (H1024, Hq8, Hkv2, D128, I2816), same pipeline as the full configuration."""
+    if ctxs is None:
+        g = torch.Generator().manual_seed(9)
+        ctxs = torch.randint(1, 600, (batch,), generator=g).tolist()
+    inp = workloads.decoder_layer_inputs(batch=batch, hidden=1024, num_heads=8, kv_head_num=2, head_dim=128,
+                                         intermediate=2816, block_size=128, context_lens=ctxs, seed=6)
+    ref_out, ref_k, ref_v = _oracle_layer(inp)
+    kc0, vc0 = inp.key_cache.clone(), inp.value_cache.clone()
+    with worker.register(decoder_layer_decode) as h:
+        h(*inp.args())
+    err = (inp.out.float() - ref_out.float()).abs().max().item()
+    print("max_abs_err", err, "ref_max", ref_out.float().abs().max().item(), flush=True)
+    validate_golden({"out": inp.out.float()}, {"out": ref_out.float()}, rtol=2e-2, atol=2e-2)
+    # the appended K/V rows (bf16 roundings of fp32 values that differ in the last bit) and nothing else changed
+    assert torch.allclose(inp.key_cache.float(), ref_k.float(), atol=2e-2, rtol=1e-2)
+    assert torch.allclose(inp.value_cache.float(), ref_v.float(), atol=2e-2, rtol=1e-2)
+    changed = (inp.key_cache != kc0).any(dim=1).sum().item()
+    assert changed <= batch * 2
