@@ -32,6 +32,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--no-ffn", action="store_true", help="skip the FFN measurement")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy, a known-size reference for HBM byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path, run with --gpus 1", file=sys.stderr)
@@ -151,6 +153,13 @@ def main() -> int:
             "sample": "one full step of the same workload (torch block-loop golden), median of 3 after 1 warm-up; "
                       f"{med * 1e3:.1f} ms per step, os.cpu_count()={os.cpu_count()}",
         }
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        result["config"]["calibration_copy_bytes"] = 1 << 30
 
     worker.close()
     print(json.dumps(result))
