@@ -52,6 +52,7 @@ struct Context {
   // options
   int64_t attn_tokens_per_partition = 0;
   int64_t attn_waves_per_cu = 0;
+  int64_t attn_variant = 0;  // 0 streaming form (head_dim 128), 1 partition grid
   int64_t attn_skip_merge = 0;
   int64_t gemm_variant = 0;
 };

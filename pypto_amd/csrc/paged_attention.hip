@@ -42,6 +42,7 @@ struct AttnParams {
   const float* k_scale;  // [pool_blocks, Hkv] for an e4m3 cache, else null
   const float* v_scale;
   int batch, hq, hkv, group, gtiles, bs, max_blocks, tpp, n_part;
+  int n_wg;  // streaming form: resident workgroups (one per CU)
   float scale_log2e;
 };
 
@@ -110,12 +111,51 @@ struct VFrag {
   typename std::conditional<FP8, uint2, u32x4>::type t[D / 128][8];
 };
 
+// K tiles are fetched with fully coalesced 16-byte loads (a wavefront reads 1 KB of consecutive
+// rows per instruction), parked in a per-wavefront LDS buffer with rows padded by 16 bytes, and
+// read back in the MFMA operand layout (lane = token).  Loading them from memory directly in
+// that layout makes every lane of a load touch a different cache line: 64 L1 tag look-ups per
+// instruction instead of 16, which - not HBM - then bounds the kernel.
 template <int D, bool FP8>
-__device__ __forceinline__ void load_k(KFrag<D, FP8>& k, const char* base0, const char* base1, uint32_t koff) {
+struct KStage {
+  static constexpr int kRowBytes = FP8 ? D : 2 * D;
+  static constexpr int kPitch = kRowBytes + 16;
+  static constexpr int kTileBytes = 16 * kPitch;
+  static constexpr int kBytes = 2 * kTileBytes;           // LDS bytes per wavefront
+  static constexpr int kLoads = 16 * kRowBytes / 1024;    // 16-byte loads per lane and tile
+};
+
+template <int D, bool FP8>
+__device__ __forceinline__ void load_k(KFrag<D, FP8>& k, const char* base0, const char* base1, int lane) {
 #pragma unroll
-  for (int s = 0; s < (FP8 ? D / 64 : D / 32); ++s) {
-    k.t[0][s] = *reinterpret_cast<const u32x4*>(base0 + koff + s * 64);
-    k.t[1][s] = *reinterpret_cast<const u32x4*>(base1 + koff + s * 64);
+  for (int s = 0; s < KStage<D, FP8>::kLoads; ++s) {
+    k.t[0][s] = *reinterpret_cast<const u32x4*>(base0 + s * 1024 + lane * 16);
+    k.t[1][s] = *reinterpret_cast<const u32x4*>(base1 + s * 1024 + lane * 16);
+  }
+}
+
+// Registers (memory order) -> LDS.
+template <int D, bool FP8>
+__device__ __forceinline__ void stage_k(const KFrag<D, FP8>& k, char* kbuf, int lane) {
+  typedef KStage<D, FP8> S;
+#pragma unroll
+  for (int s = 0; s < S::kLoads; ++s) {
+    const int off = s * 1024 + lane * 16;
+    const int dst = (off / S::kRowBytes) * S::kPitch + off % S::kRowBytes;
+    *reinterpret_cast<u32x4*>(kbuf + dst) = k.t[0][s];
+    *reinterpret_cast<u32x4*>(kbuf + S::kTileBytes + dst) = k.t[1][s];
+  }
+}
+
+// LDS -> registers in operand order: lane (c, j), step s holds 16 bytes at row c, byte (s*4+j)*16.
+template <int D, bool FP8>
+__device__ __forceinline__ void fetch_k(KFrag<D, FP8>& k, const char* kbuf, int c, int j) {
+  typedef KStage<D, FP8> S;
+#pragma unroll
+  for (int s = 0; s < S::kLoads; ++s) {
+    const int src = c * S::kPitch + (s * 4 + j) * 16;
+    k.t[0][s] = *reinterpret_cast<const u32x4*>(kbuf + src);
+    k.t[1][s] = *reinterpret_cast<const u32x4*>(kbuf + S::kTileBytes + src);
   }
 }
 
@@ -143,41 +183,16 @@ __device__ __forceinline__ u32x4 fp8x8_to_bf16x8(uint32_t w0, uint32_t w1) {
                fp8x2_to_bf16x2(w1, true)};
 }
 
+// Attention of one query group (16 padded columns) over the chunks tok_first, tok_first +
+// tok_step, ... < tok_end of one (sequence, KV head): on return acc holds O^T in units of v_unit,
+// m_run the running maximum (log2 units) and l_run the row sum, both per column and already
+// summed over the wavefront.  tok_first must be a multiple of 32 below tok_end.
 template <int D, bool BF16, bool FP8>
-__global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
-  const int lane = threadIdx.x;
-  const int c = lane & 15;   // MFMA row / column index of this lane
-  const int j = lane >> 4;   // MFMA k-group of this lane
-  // Linear workgroup id -> (partition, sequence, KV head, query tile) with the partition index
-  // slowest.  Workgroups go to the 8 XCDs round-robin by id, so each XCD sees every partition
-  // index equally often (late partitions exist only for long sequences) and the mostly-empty
-  // tail of the grid is dispatched last.
-  const int pairs = p.batch * p.hkv * p.gtiles;
-  const int part = blockIdx.x / pairs;
-  const int pair = blockIdx.x % pairs;
-  const int b = pair / (p.hkv * p.gtiles);
-  const int h = (pair / p.gtiles) % p.hkv;
-  const int gt = pair % p.gtiles;
-
-  int ctx = p.ctx_lens[b];
-  const int max_ctx = p.max_blocks * p.bs;
-  ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
-  const int tok_begin = part * p.tpp;
-  const int tok_end = min(ctx, tok_begin + p.tpp);
-  const int g = gt * 16 + c;               // query head within the KV group
-  const bool g_valid = g < p.group;
-  const int hq_row = b * p.hq + h * p.group + g;
-
-  if (tok_begin >= tok_end) {
-    // Nothing to read.  An empty sequence yields zeros (09_paged_attention_spmd.py:647-651).
-    if (p.n_part == 1 && g_valid) {
-      float* o = p.out + (size_t)hq_row * D;
-#pragma unroll
-      for (int i = 0; i < D / 4; ++i) o[j * (D / 4) + i] = 0.f;
-    }
-    return;
-  }
-
+__device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, int hq_row, bool g_valid,
+                                             int tok_first, int tok_end, int tok_step, int c, int j,
+                                             char* kbuf, int first_window, f32x4 (&acc)[D / 128][8],
+                                             float& m_run, float& l_run, float& v_unit) {
+  const int lane = j * 16 + c;
   // Query fragments (B operand): column = query head; k-group j of step s holds the elements
   // its K fragment holds: (s*4+j)*8..+8, or for an e4m3 cache ((s/2)*4+j)*16 + (s%2)*8..+8.
   u32x4 qf[D / 32];
@@ -195,26 +210,47 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   const char* vc = reinterpret_cast<const char*>(p.vc);
   const int32_t* table = p.block_table + (size_t)b * p.max_blocks;
   constexpr int kEsz = FP8 ? 1 : 2;                                // bytes per cache element
-  const uint32_t koff = (uint32_t)(c * D * kEsz + j * 16);             // byte offset of this lane in a K tile
   const uint32_t voff = (uint32_t)(j * 4 * D * kEsz + c * 8 * kEsz);   // ... in a V tile
 
-  // Byte offset of the 16-token tile starting at logical token `tok` (wave-uniform).
-  int blk_of_tile = 0;  // physical block of the tile last looked up
-  auto tile_offset = [&](int tok) -> size_t {
-    // A tile past the end is never used; point it at the partition's first tile so the load
-    // stays in bounds even when the block table holds nothing for that logical block.
-    if (tok >= tok_end) tok = tok_begin;
-    blk_of_tile = table[tok / p.bs];
-    return ((size_t)(blk_of_tile * p.hkv + h) * p.bs + (tok % p.bs)) * (D * kEsz);
+  // Block-table window: lane i holds the physical block (and, for an e4m3 cache, the two scales)
+  // of logical block win_base + i, fetched with one vector load per 64 blocks so that the
+  // per-chunk look-ups below are register reads, not memory round trips on the load path.
+  int win_base = 0, win_blk = 0;
+  float win_ks = 1.f, win_vs = 1.f;
+  auto load_window = [&](int first_block, bool preloaded) {
+    win_base = first_block;
+    const int idx = min(first_block + lane, p.max_blocks - 1);
+    win_blk = preloaded ? first_window : table[idx];
+    if constexpr (FP8) {
+      // table entries past the end of the range may hold anything: do not dereference them
+      const bool ok = (first_block + lane) * p.bs < tok_end;
+      win_ks = ok ? p.k_scale[(size_t)win_blk * p.hkv + h] : 1.f;
+      win_vs = ok ? p.v_scale[(size_t)win_blk * p.hkv + h] : 1.f;
+    }
   };
+  load_window(tok_first / p.bs, true);
 
-  f32x4 acc[D / 128][8];
+  // Byte offset of the 16-token tile starting at logical token `tok` (wave-uniform).
+  int slot_of_tile = 0;  // window slot of the tile last looked up
+  auto tile_offset = [&](int tok) -> size_t {
+    // A tile past the end is never used; point it at the range's first tile so the load stays
+    // in bounds even when the block table holds nothing for that logical block.
+    if (tok >= tok_end) tok = tok_first;
+    const int lb = tok / p.bs;
+    if (lb < win_base || lb >= win_base + 64) load_window(lb, false);
+    slot_of_tile = lb - win_base;
+    const int blk = __builtin_amdgcn_readlane(win_blk, slot_of_tile);
+    return ((size_t)(blk * p.hkv + h) * p.bs + (tok % p.bs)) * (D * kEsz);
+  };
+  auto scale_k = [&]() { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, win_ks), slot_of_tile)); };
+  auto scale_v = [&]() { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, win_vs), slot_of_tile)); };
+
 #pragma unroll
   for (int set = 0; set < D / 128; ++set)
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[set][i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = kMinMax;
-  float l_run = 0.f;
+  m_run = kMinMax;
+  l_run = 0.f;
 
   // Software pipeline: K of chunk n+1 is requested as soon as QK^T of chunk n has consumed
   // the K registers, V of chunk n at the top of iteration n.  All loads are unconditional (the
@@ -222,30 +258,33 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   // requests in flight at each wait is known at compile time.
   KFrag<D, FP8> kf;
   VFrag<D, FP8> vf;
-  size_t o0 = tile_offset(tok_begin + 16), o1 = o0;
+  size_t o0 = tile_offset(tok_first + 16), o1 = o0;
   o1 = o0;
-  o0 = tile_offset(tok_begin);
+  o0 = tile_offset(tok_first);
   // e4m3 cache: a chunk lies inside one block (block_size is a multiple of 32), whose two scales
   // apply to the whole chunk.  The accumulators are kept in units of the current block's V
   // scale, v_unit; they are converted when the block changes and once more at the end.
-  float k_mul = p.scale_log2e, v_unit = 1.f, v_next = 1.f, k_next = p.scale_log2e;
+  float k_mul = p.scale_log2e, v_next = 1.f, k_next = p.scale_log2e;
+  v_unit = 1.f;
   if constexpr (FP8) {
-    k_mul = p.scale_log2e * p.k_scale[blk_of_tile * p.hkv + h];
-    v_unit = p.v_scale[blk_of_tile * p.hkv + h];
+    k_mul = p.scale_log2e * scale_k();
+    v_unit = scale_v();
   }
-  load_k<D, FP8>(kf, kc + o0, kc + o1, koff);
+  load_k<D, FP8>(kf, kc + o0, kc + o1, lane);
+  load_v<D, FP8>(vf, vc + o0, vc + o1, voff);
+  stage_k<D, FP8>(kf, kbuf, lane);
 
-  for (int tok = tok_begin; tok < tok_end; tok += kChunk) {
-    load_v<D, FP8>(vf, vc + o0, vc + o1, voff);
-    o1 = tile_offset(tok + kChunk + 16);
-    o0 = tile_offset(tok + kChunk);
+  for (int tok = tok_first; tok < tok_end; tok += tok_step) {
+    o1 = tile_offset(tok + tok_step + 16);
+    o0 = tile_offset(tok + tok_step);
     if constexpr (FP8) {
-      k_next = p.scale_log2e * p.k_scale[blk_of_tile * p.hkv + h];
-      v_next = p.v_scale[blk_of_tile * p.hkv + h];
+      k_next = p.scale_log2e * scale_k();
+      v_next = scale_v();
     }
 
     // ---- S^T = K Q^T : two 16x16 tiles, rows = tokens, columns = query heads ----
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    fetch_k<D, FP8>(kf, kbuf, c, j);
     if constexpr (FP8) {
 #pragma unroll
       for (int s2 = 0; s2 < D / 64; ++s2) {
@@ -261,7 +300,7 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
         s1 = mfma16<BF16>(kf.t[1][s], qf[s], s1);
       }
     }
-    load_k<D, FP8>(kf, kc + o0, kc + o1, koff);
+    load_k<D, FP8>(kf, kc + o0, kc + o1, lane);  // next chunk, into the registers QK^T just released
 
     float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
 #pragma unroll
@@ -344,11 +383,59 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
       }
       k_mul = k_next;
     }
+    load_v<D, FP8>(vf, vc + o0, vc + o1, voff);  // next chunk, into the registers PV just released
+    stage_k<D, FP8>(kf, kbuf, lane);
   }
 
   // Row sum over the four k-groups of a column.
   l_run += __shfl_xor(l_run, 16);
   l_run += __shfl_xor(l_run, 32);
+}
+
+template <int D, bool BF16, bool FP8>
+__global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
+  const int lane = threadIdx.x;
+  const int c = lane & 15;   // MFMA row / column index of this lane
+  const int j = lane >> 4;   // MFMA k-group of this lane
+  // Linear workgroup id -> (partition, sequence, KV head, query tile) with the partition index
+  // slowest.  Workgroups go to the 8 XCDs round-robin by id, so each XCD sees every partition
+  // index equally often (late partitions exist only for long sequences) and the mostly-empty
+  // tail of the grid is dispatched last.
+  const int pairs = p.batch * p.hkv * p.gtiles;
+  const int part = blockIdx.x / pairs;
+  const int pair = blockIdx.x % pairs;
+  const int b = pair / (p.hkv * p.gtiles);
+  const int h = (pair / p.gtiles) % p.hkv;
+  const int gt = pair % p.gtiles;
+
+  // The first block-table window is requested before the context length is known: its address
+  // depends only on the workgroup id, so the two loads overlap instead of forming a chain.
+  const int first_window =
+      p.block_table[(size_t)b * p.max_blocks + min(part * p.tpp / p.bs + lane, p.max_blocks - 1)];
+  int ctx = p.ctx_lens[b];
+  const int max_ctx = p.max_blocks * p.bs;
+  ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
+  const int tok_begin = part * p.tpp;
+  const int tok_end = min(ctx, tok_begin + p.tpp);
+  const int g = gt * 16 + c;               // query head within the KV group
+  const bool g_valid = g < p.group;
+  const int hq_row = b * p.hq + h * p.group + g;
+
+  if (tok_begin >= tok_end) {
+    // Nothing to read.  An empty sequence yields zeros (09_paged_attention_spmd.py:647-651).
+    if (p.n_part == 1 && g_valid) {
+      float* o = p.out + (size_t)hq_row * D;
+#pragma unroll
+      for (int i = 0; i < D / 4; ++i) o[j * (D / 4) + i] = 0.f;
+    }
+    return;
+  }
+
+  __shared__ __attribute__((aligned(16))) char k_lds[KStage<D, FP8>::kBytes];
+  f32x4 acc[D / 128][8];
+  float m_run, l_run, v_unit;
+  attend_range<D, BF16, FP8>(p, b, h, hq_row, g_valid, tok_begin, tok_end, kChunk, c, j, k_lds, first_window, acc,
+                             m_run, l_run, v_unit);
 
   if (!g_valid) return;
   if (p.n_part == 1) {
@@ -416,6 +503,95 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
   for (int k = 0; k < D / 64; ++k) p.out[(size_t)row * D + k * 64 + lane] = o[k] * inv;
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Balanced form of the partition kernel.  Under HBM saturation every CU gets about the same
+// share of the bandwidth, so the launch lasts as long as the CU with the most bytes to fetch;
+// the hardware dispatcher, left alone, parks between 2 and 12 single-wavefront workgroups on a
+// CU.  Here one workgroup of kBalWaves wavefronts is pinned to each CU (its LDS use allows only
+// one) and the non-empty (sequence, KV head, query tile, partition) items, enumerated densely,
+// are dealt round-robin: item i goes to workgroup i mod n_wg.  Every CU then fetches the same
+// number of partitions, give or take one.  Partials and their merge are those of the
+// partition-grid kernel.
+// ---------------------------------------------------------------------------------------------
+template <int D, bool BF16, bool FP8, int kBalWaves>
+__global__ __launch_bounds__(kBalWaves * 64) void attn_balanced_kernel(AttnParams p) {
+  __shared__ __attribute__((aligned(16))) char k_lds[kBalWaves][KStage<D, FP8>::kBytes];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, j = lane >> 4;
+  const int hg_count = p.hkv * p.gtiles;
+  const int max_ctx = p.max_blocks * p.bs;
+  const int n_workers = p.n_wg * kBalWaves;
+
+  if (p.n_part == 1) {
+    // No merge kernel runs: rows of empty sequences are zeroed here
+    // (09_paged_attention_spmd.py:647-651).
+    for (int row = blockIdx.x * kBalWaves + wave; row < p.batch * p.hq; row += n_workers) {
+      if (p.ctx_lens[row / p.hq] <= 0)
+        for (int d = lane; d < D; d += 64) p.out[(size_t)row * D + d] = 0.f;
+    }
+  }
+
+  // Items of this wavefront: blockIdx.x + n_wg * (wave + kBalWaves * k), k = 0, 1, ...
+  for (int item = blockIdx.x + p.n_wg * wave;; item += p.n_wg * kBalWaves) {
+    // Locate the item: sequence b holds items [A_b, A_b + np_b * hg_count), np_b = ceil(ctx_b / tpp).
+    int base = 0, fb = -1, foff = 0, fnp = 1;
+    for (int b0 = 0; b0 < p.batch; b0 += 64) {
+      int ctx = (b0 + lane < p.batch) ? p.ctx_lens[b0 + lane] : 0;
+      ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
+      const int n = (ctx + p.tpp - 1) / p.tpp * hg_count;
+      int incl = n;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
+      }
+      const int lo = base + incl - n;
+      const unsigned long long hit = __ballot(n > 0 && lo <= item && item < lo + n);
+      if (hit) {
+        const int src = __ffsll((long long)hit) - 1;
+        fb = b0 + src;
+        foff = item - __shfl(lo, src);
+        fnp = __shfl(n, src) / hg_count;
+        break;
+      }
+      base += __shfl(incl, 63);
+    }
+    if (fb < 0) break;  // past the last item (uniform over the wavefront)
+    const int b = __builtin_amdgcn_readfirstlane(fb);
+    const int np = __builtin_amdgcn_readfirstlane(fnp);
+    const int off = __builtin_amdgcn_readfirstlane(foff);
+    const int hg = off / np, part = off % np;
+    const int h = hg / p.gtiles, gt = hg % p.gtiles;
+    int ctx = p.ctx_lens[b];
+    ctx = ctx > max_ctx ? max_ctx : ctx;
+    const int tok_begin = part * p.tpp;
+    const int tok_end = min(ctx, tok_begin + p.tpp);
+    const int g = gt * 16 + c;
+    const bool g_valid = g < p.group;
+    const int hq_row = b * p.hq + h * p.group + g;
+
+    f32x4 acc[D / 128][8];
+    float m_run, l_run, v_unit;
+    const int first_window =
+        p.block_table[(size_t)b * p.max_blocks + min(tok_begin / p.bs + lane, p.max_blocks - 1)];
+    attend_range<D, BF16, FP8>(p, b, h, hq_row, g_valid, tok_begin, tok_end, kChunk, c, j, k_lds[wave],
+                               first_window, acc, m_run, l_run, v_unit);
+    if (g_valid) {
+      if (p.n_part == 1) {
+        store_rows<D>(p.out + (size_t)hq_row * D, acc, j, l_run > 0.f ? v_unit / l_run : 0.f);
+      } else {
+        const size_t slot = (size_t)hq_row * p.n_part + part;
+        store_rows<D>(p.part_o + slot * D, acc, j, v_unit);
+        if (j == 0) {
+          p.part_ml[slot * 2 + 0] = m_run;
+          p.part_ml[slot * 2 + 1] = l_run;
+        }
+      }
+    }
+  }
+}
+
 template <int D, bool FP8>
 int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   dim3 grid((unsigned)(p.n_part * p.hkv * p.gtiles * batch));
@@ -423,12 +599,29 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   // grid over all CUs instead of filling some to their register limit.
   const int64_t cap = pto_hip::ctx().attn_waves_per_cu;
   const size_t lds = cap > 0 ? (size_t)(163840 / cap) / 1024 * 1024 : 0;
-  if (bf16)
-    hipLaunchKernelGGL((attn_partition_kernel<D, true, FP8>), grid, dim3(64), lds, stream, p);
-  else if constexpr (!FP8)
-    hipLaunchKernelGGL((attn_partition_kernel<D, false, false>), grid, dim3(64), lds, stream, p);
-  else
+  if (!bf16 && FP8)
     return pto_hip::fail(PTO_HIP_ERR_UNSUPPORTED, "paged_attention: an FP8E4M3FN cache needs a BF16 query");
+  if (p.n_wg > 0) {
+    if constexpr (D == 128) {
+      // 12 wavefronts per CU (3 per SIMD) by default; "attn_waves_per_cu" 8 selects 2 per SIMD.
+      const bool eight = cap == 8;
+      dim3 bgrid(p.n_wg), bblock(eight ? 512 : 768);
+      if (bf16 && eight)
+        hipLaunchKernelGGL((attn_balanced_kernel<D, true, FP8, 8>), bgrid, bblock, 0, stream, p);
+      else if (bf16)
+        hipLaunchKernelGGL((attn_balanced_kernel<D, true, FP8, 12>), bgrid, bblock, 0, stream, p);
+      else if constexpr (!FP8) {
+        if (eight)
+          hipLaunchKernelGGL((attn_balanced_kernel<D, false, false, 8>), bgrid, bblock, 0, stream, p);
+        else
+          hipLaunchKernelGGL((attn_balanced_kernel<D, false, false, 12>), bgrid, bblock, 0, stream, p);
+      }
+    }
+  } else if (bf16) {
+    hipLaunchKernelGGL((attn_partition_kernel<D, true, FP8>), grid, dim3(64), lds, stream, p);
+  } else if constexpr (!FP8) {
+    hipLaunchKernelGGL((attn_partition_kernel<D, false, false>), grid, dim3(64), lds, stream, p);
+  }
   PTO_CHECK_HIP(hipGetLastError());
   // "attn_skip_merge" leaves the partials unmerged: a timing aid that isolates the streaming
   // kernel; results are not valid in that mode.

@@ -641,6 +641,8 @@ int pto_hip_set_option(const char* name, int64_t value) {
     c.attn_tokens_per_partition = value;
   } else if (!std::strcmp(name, "gemm_variant")) {
     c.gemm_variant = value;
+  } else if (!std::strcmp(name, "attn_variant")) {
+    c.attn_variant = value;
   } else if (!std::strcmp(name, "attn_skip_merge")) {
     c.attn_skip_merge = value != 0;
   } else if (!std::strcmp(name, "attn_waves_per_cu")) {
@@ -660,6 +662,7 @@ int pto_hip_get_option(const char* name, int64_t* value) {
   else if (!std::strcmp(name, "gemm_variant")) *value = c.gemm_variant;
   else if (!std::strcmp(name, "attn_waves_per_cu")) *value = c.attn_waves_per_cu;
   else if (!std::strcmp(name, "attn_skip_merge")) *value = c.attn_skip_merge;
+  else if (!std::strcmp(name, "attn_variant")) *value = c.attn_variant;
   else return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
   return PTO_HIP_OK;
 }

@@ -17,8 +17,10 @@ ATOL, RTOL = 1e-2, 2e-2
 
 
 def _run(worker, inp, tpp=0):
-    """tpp = tokens per context partition; 0 lets the library choose."""
-    worker.set_option("attn_tokens_per_partition", tpp)
+    """tpp = 0: the default streaming kernel; tpp > 0: the partition-grid kernel with that many
+    tokens per context partition; tpp < 0: the partition-grid kernel with its own choice."""
+    worker.set_option("attn_variant", 0 if tpp == 0 else 1)
+    worker.set_option("attn_tokens_per_partition", max(tpp, 0))
     dev = [t.cuda() if isinstance(t, torch.Tensor) and i != 6 else t for i, t in enumerate(inp.args())]
     dev[5].fill_(float("nan"))
     torch.cuda.synchronize()
@@ -26,6 +28,7 @@ def _run(worker, inp, tpp=0):
         h(*dev)
     worker.sync()
     worker.set_option("attn_tokens_per_partition", 0)
+    worker.set_option("attn_variant", 0)
     return dev[5].cpu()
 
 
@@ -42,7 +45,7 @@ def _check(out, ref):
     assert err <= ATOL + RTOL * ref.abs().max().item()
 
 
-@pytest.mark.parametrize("tpp", [0, 128, 512, 4096])
+@pytest.mark.parametrize("tpp", [0, -1, 128, 512, 4096])
 def test_small_config_matches_golden(worker, tpp):
     """B16 Hq32 Hkv8 D128 bs128, ctx~U[512,4096], permutation table (reduced pool)."""
     inp = workloads.attention_small(seed=0, pool_blocks=None)
@@ -67,7 +70,7 @@ def test_shapes_and_edges(worker, batch, hq, hkv, d, bs, ctxs):
                                            block_size=bs, context_lens=ctxs, ctx_range=(1, max(max(ctxs), 1)),
                                            seed=7)
     ref = _golden(inp)
-    for tpp in (0, 32, 256):
+    for tpp in (0, -1, 32, 256):
         out = _run(worker, inp, tpp)
         _check(out, ref)
     if 0 in ctxs:
@@ -80,6 +83,7 @@ def test_fp16_cache(worker):
     inp = workloads.paged_attention_inputs(batch=3, num_heads=16, kv_head_num=4, context_lens=[300, 17, 129],
                                            ctx_range=(1, 300), dtype=torch.float16, seed=3)
     _check(_run(worker, inp), _golden(inp))
+    _check(_run(worker, inp, -1), _golden(inp))
 
 
 def test_duplicate_table_entries(worker):
@@ -89,13 +93,14 @@ def test_duplicate_table_entries(worker):
     g = torch.Generator().manual_seed(11)
     inp.block_table = torch.randint(0, 16, inp.block_table.shape, generator=g, dtype=torch.int32)
     _check(_run(worker, inp), _golden(inp))
+    _check(_run(worker, inp, -1), _golden(inp))
 
 
 def test_block_permutation_invariance_is_bit_exact(worker):
     """Moving physical blocks and permuting the table consistently must not change one bit."""
     inp = workloads.paged_attention_inputs(batch=4, num_heads=32, kv_head_num=8, context_lens=[640, 129, 1024, 77],
                                            ctx_range=(1, 1024), pool_blocks=64, seed=9)
-    out_a = _run(worker, inp, 128)
+    out_a = _run(worker, inp, 0)
     g = torch.Generator().manual_seed(123)
     perm = torch.randperm(64, generator=g)          # new position of old block p is perm[p]
     rows = 8 * 128
@@ -107,7 +112,8 @@ def test_block_permutation_invariance_is_bit_exact(worker):
     inp.key_cache = kc2.reshape(-1, 128)
     inp.value_cache = vc2.reshape(-1, 128)
     inp.block_table = perm[inp.block_table.long()].to(torch.int32)
-    out_b = _run(worker, inp, 128)
+    out_b = _run(worker, inp, 0)
+    assert torch.equal(_run(worker, inp, 128), _run(worker, inp, 128))
     assert torch.equal(out_a, out_b)
 
 
@@ -152,7 +158,7 @@ def test_fp8_cache_matches_golden(worker, batch, hq, hkv, bs, ctxs):
                                            context_lens=ctxs, ctx_range=(1, max(ctxs)), fp8_kv=True, seed=11)
     assert inp.key_cache.dtype == torch.float8_e4m3fn
     ref = _golden(inp)
-    for tpp in (0, 64, 512):
+    for tpp in (0, -1, 64, 512):
         _check(_run(worker, inp, tpp), ref)
 
 
