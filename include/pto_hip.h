@@ -241,7 +241,13 @@ PTO_HIP_API int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* args,
  *  "attn_waves_per_cu"          cap on resident attention wavefronts per CU, 0 = none (default)
  *  "attn_skip_merge"            1 = launch only the streaming attention kernel and leave the
  *                               partition partials unmerged (kernel timing aid; output invalid)
- *  "gemm_variant"               FFN GEMM tiling: 0 = default choice, 1..2 = fixed alternatives
+ *  "attn_variant"               0 = one wavefront per (sequence, KV head, partition) (default),
+ *                               1 = one pinned workgroup per CU over a balanced list of those
+ *                               items (head_dim 128 only)
+ *  "gemm_variant"               FFN GEMM tiling: 0 = default choice, 1..3 = fixed alternatives
+ *  "w8a16_wgs_per_cu"           workgroups per CU the W8A16 k split aims at (default 2)
+ *  "w8a16_min_steps"            fewest 32-row steps per wavefront before k is split further
+ *                               (default 4)
  */
 PTO_HIP_API int pto_hip_set_option(const char* name, int64_t value);
 PTO_HIP_API int pto_hip_get_option(const char* name, int64_t* value);

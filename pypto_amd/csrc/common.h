@@ -52,9 +52,11 @@ struct Context {
   // options
   int64_t attn_tokens_per_partition = 0;
   int64_t attn_waves_per_cu = 0;
-  int64_t attn_variant = 0;  // 0 streaming form (head_dim 128), 1 partition grid
+  int64_t attn_variant = 0;  // 0 partition grid, 1 balanced form (head_dim 128)
   int64_t attn_skip_merge = 0;
   int64_t gemm_variant = 0;
+  int64_t w8a16_wgs_per_cu = 2;  // workgroups of the W8A16 partial kernel aimed at per compute unit
+  int64_t w8a16_min_steps = 4;   // fewest 32-row steps per wavefront before k is split further
 };
 
 Context& ctx();
@@ -63,6 +65,42 @@ Context& ctx();
 int workspace(size_t bytes, void** ptr);
 // Returns `n` zeroed int counters (grown on demand; same caveat as workspace()).
 int counters(size_t n, int** ptr);
+
+// ---- W8A16 decode projections, shared with the composed decoder layer -------------------
+constexpr int kW8Slab = 128;  // output channels per workgroup of the partial kernel
+constexpr int kW8MaxM = 32;   // rows of a partial slab (activation rows are at most this many)
+// fp32 partial sums of a projection, one [32, N] slab per k split: element (s, m, n) of
+// projection i is part[i][(s * 32 + m) * N + n].  They live in the shared workspace.
+struct W8Partials {
+  float* part[2];
+  int splits;
+};
+// Launches the partial kernel for x[M, K] @ wq0[K, N] (and wq1 when non-null).
+int w8a16_partials(const void* x, const void* wq0, const void* wq1, int64_t m, int64_t k, int64_t n,
+                   int x_dtype, hipStream_t st, W8Partials* out);
+// out = cast(sum_s(part0) * scale0 [-> SiLU(.) * (sum_s(part1) * scale1)] [+ residual]).
+int w8a16_finish(const W8Partials& parts, const float* scale0, const float* scale1, const void* residual,
+                 int res_dtype, void* out, int out_dtype, int64_t m, int64_t n, hipStream_t st);
+// sum_out = sum_s(part) * scale + residual (fp32); normed_out = cast(RMSNorm(sum_out) * gamma).
+bool w8a16_finish_norm_fits(int64_t n);
+int w8a16_finish_norm(const W8Partials& parts, const float* scale, const void* residual, int res_dtype,
+                      float* sum_out, const float* gamma, void* normed_out, int out_dtype, int64_t m,
+                      int64_t n, float eps, hipStream_t st);
+
+// RoPE + K/V append reading either final fp32 projections (qkv_scale null, splits 1) or the
+// partial sums of the q/k/v projection (summed in split order and scaled per channel).
+int rope_kv_cache_update(const float* qkv, const float* qkv_scale, int splits, int64_t split_stride,
+                         const int32_t* seq_lens, const float* rope_cos, const float* rope_sin,
+                         const int32_t* block_table, void* key_cache, void* value_cache, void* q_out,
+                         int64_t batch, int64_t num_heads, int64_t kv_head_num, int64_t head_dim,
+                         int64_t block_size, int64_t max_num_blocks_per_req, int64_t max_pos,
+                         int64_t pool_rows, int dtype, void* stream);
+int cast_from_f32(const float* in, void* out, size_t n, int out_dtype, hipStream_t st);
+// pto_hip_paged_attention with an optional second output: the result rounded to the query dtype.
+int paged_attention(const void* query, const void* key_cache, const void* value_cache,
+                    const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
+                    const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
+                    const float* v_scale, void* stream);
 
 inline int dtype_bytes(int dt) {
   switch (dt) {

@@ -6,14 +6,11 @@
 // examples/models/08_llama_mini.py:384-483; golden
 // tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:255-287), with the
 // projections taking int8 weights and per-channel scales.  The reference submits one task per
-// tile through its scheduler; here the layer is eleven kernel launches in stream order.
+// tile through its scheduler; here the layer is twelve kernel launches in stream order; each projection is a partial-sum
+// kernel whose finish is folded into the elementwise step that follows it.
 #include <hip/hip_runtime.h>
 
 #include "common.h"
-
-namespace pto_hip {
-int cast_from_f32(const float* in, void* out, size_t n, int out_dtype, hipStream_t st);
-}
 
 extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, void* stream) {
   using namespace pto_hip;
@@ -39,11 +36,11 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
 
   // Layer-private intermediates (the kernels' own scratch lives in the shared workspace).
   auto up = [](size_t n) { return (n + 255) / 256 * 256; };
-  const size_t sz_normed = up((size_t)b * h * 2), sz_qkv = up((size_t)b * qkv_n * 4),
+  const size_t sz_normed = up((size_t)b * h * 2),
                sz_q = up((size_t)b * hq * d * 2), sz_attn = up((size_t)b * hq * d * 4),
                sz_attn16 = up((size_t)b * hq * d * 2), sz_resid = up((size_t)b * h * 4),
                sz_h = up((size_t)b * inter * 2);
-  const size_t total = sz_normed + sz_qkv + sz_q + sz_attn + sz_attn16 + sz_resid + sz_normed + sz_h;
+  const size_t total = sz_normed + sz_q + sz_attn + sz_attn16 + sz_resid + sz_normed + sz_h;
   if (total > cx.layer_ws_bytes) {
     PTO_CHECK_HIP(hipDeviceSynchronize());
     if (cx.layer_ws) PTO_CHECK_HIP(hipFree(cx.layer_ws));
@@ -54,7 +51,6 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
   }
   char* w = reinterpret_cast<char*>(cx.layer_ws);
   void* normed = w;              w += sz_normed;
-  float* qkv = (float*)w;        w += sz_qkv;
   void* q16 = w;                 w += sz_q;
   float* attn = (float*)w;       w += sz_attn;
   void* attn16 = w;              w += sz_attn16;
@@ -63,31 +59,35 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
   void* hbuf = w;
 
   int rc;
+  W8Partials parts{};
   // 1. input RMSNorm -> activation dtype
   if ((rc = pto_hip_rms_norm(a->hidden_states, a->gamma_in, normed, b, h, a->eps, dt, dt, stream))) return rc;
-  // 2. QKV projection (fp32 out)
-  if ((rc = pto_hip_w8a16_matmul(normed, a->wqkv_q, a->wqkv_s, nullptr, qkv, b, h, qkv_n, dt, 0, PTO_HIP_FP32, stream)))
-    return rc;
-  // 3. RoPE at pos = seq_len - 1, append K/V, rotated Q
-  if ((rc = pto_hip_rope_kv_cache_update(qkv, a->seq_lens, a->rope_cos, a->rope_sin, a->block_table, a->key_cache,
-                                         a->value_cache, q16, b, hq, hkv, d, a->block_size,
-                                         a->max_num_blocks_per_req, a->max_pos, a->pool_rows, dt, stream)))
+  // 2. QKV projection, left as k-split partial sums
+  if ((rc = w8a16_partials(normed, a->wqkv_q, nullptr, b, h, qkv_n, dt, st, &parts))) return rc;
+  // 3. finish of the projection + RoPE at pos = seq_len - 1, append K/V, rotated Q
+  if ((rc = rope_kv_cache_update(parts.part[0], a->wqkv_s, parts.splits, (int64_t)kW8MaxM * qkv_n, a->seq_lens,
+                                 a->rope_cos, a->rope_sin, a->block_table, a->key_cache, a->value_cache, q16, b,
+                                 hq, hkv, d, a->block_size, a->max_num_blocks_per_req, a->max_pos, a->pool_rows,
+                                 dt, stream)))
     return rc;
   // 4. paged attention over seq_len tokens (including the one just written)
   float scale = 1.0f / sqrtf((float)d);
   uint32_t scale_bits;
   __builtin_memcpy(&scale_bits, &scale, 4);
   const int64_t cfg[7] = {b, hq, hkv, d, a->block_size, a->max_num_blocks_per_req, (int64_t)scale_bits};
-  if ((rc = pto_hip_paged_attention(q16, a->key_cache, a->value_cache, a->block_table, a->seq_lens, attn, cfg, dt, dt,
-                                    nullptr, nullptr, stream)))
+  if ((rc = paged_attention(q16, a->key_cache, a->value_cache, a->block_table, a->seq_lens, attn, attn16, cfg, dt, dt,
+                            nullptr, nullptr, stream)))
     return rc;
-  if ((rc = cast_from_f32(attn, attn16, (size_t)b * hq * d, dt, st))) return rc;
-  // 5. o_proj + residual -> fp32
-  if ((rc = pto_hip_w8a16_matmul(attn16, a->wo_q, a->wo_s, a->hidden_states, resid1, b, hq * d, h, dt, dt,
-                                 PTO_HIP_FP32, stream)))
-    return rc;
-  // 6. post-attention RMSNorm
-  if ((rc = pto_hip_rms_norm(resid1, a->gamma_post, normed2, b, h, a->eps, PTO_HIP_FP32, dt, stream))) return rc;
+  // 5. o_proj; 6. its finish + residual -> fp32, post-attention RMSNorm -> activation dtype
+  if ((rc = w8a16_partials(attn16, a->wo_q, nullptr, b, hq * d, h, dt, st, &parts))) return rc;
+  if (w8a16_finish_norm_fits(h)) {
+    if ((rc = w8a16_finish_norm(parts, a->wo_s, a->hidden_states, dt, resid1, a->gamma_post, normed2, dt, b, h,
+                                a->eps, st)))
+      return rc;
+  } else {
+    if ((rc = w8a16_finish(parts, a->wo_s, nullptr, a->hidden_states, dt, resid1, PTO_HIP_FP32, b, h, st))) return rc;
+    if ((rc = pto_hip_rms_norm(resid1, a->gamma_post, normed2, b, h, a->eps, PTO_HIP_FP32, dt, stream))) return rc;
+  }
   // 7. gate/up + SwiGLU -> h (activation dtype), 8. down + residual -> out
   if ((rc = pto_hip_w8a16_swiglu(normed2, a->wg_q, a->wg_s, a->wu_q, a->wu_s, hbuf, b, h, inter, dt, dt, stream)))
     return rc;

@@ -37,6 +37,8 @@ struct AttnParams {
   const int32_t* block_table;
   const int32_t* ctx_lens;
   float* out;
+  void* out16;     // optional second copy of the result in the 16-bit activation type
+  int out16_bf16;
   float* part_o;   // [B*Hq, n_part, D]
   float* part_ml;  // [B*Hq, n_part, 2]  (running max in log2 units, row sum)
   const float* k_scale;  // [pool_blocks, Hkv] for an e4m3 cache, else null
@@ -500,7 +502,15 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
   }
   const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
-  for (int k = 0; k < D / 64; ++k) p.out[(size_t)row * D + k * 64 + lane] = o[k] * inv;
+  for (int k = 0; k < D / 64; ++k) {
+    const float y = o[k] * inv;
+    const size_t idx = (size_t)row * D + k * 64 + lane;
+    p.out[idx] = y;
+    if (p.out16) {
+      if (p.out16_bf16) reinterpret_cast<__bf16*>(p.out16)[idx] = (__bf16)y;
+      else reinterpret_cast<_Float16*>(p.out16)[idx] = (_Float16)y;
+    }
+  }
 }
 
 
@@ -635,12 +645,11 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
 
 }  // namespace
 
-extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
-                                       const void* value_cache, const int32_t* block_table,
-                                       const int32_t* context_lens, float* out,
-                                       const int64_t* config, int q_dtype, int kv_dtype,
-                                       const float* k_scale, const float* v_scale, void* stream) {
-  using namespace pto_hip;
+namespace pto_hip {
+int paged_attention(const void* query, const void* key_cache, const void* value_cache,
+                    const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
+                    const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
+                    const float* v_scale, void* stream) {
   Context& cx = ctx();
   if (!cx.initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(config != nullptr, "paged_attention: config is null");
@@ -684,6 +693,8 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
   p.block_table = block_table;
   p.ctx_lens = context_lens;
   p.out = out;
+  p.out16 = nullptr;
+  p.out16_bf16 = q_dtype == PTO_HIP_BF16;
   p.k_scale = k_scale;
   p.v_scale = v_scale;
   p.batch = (int)batch;
@@ -730,10 +741,29 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
     p.part_o = reinterpret_cast<float*>(ws);
     p.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + o_bytes);
   }
-  if (fp8) {
-    if (d == 128) return launch<128, true>(p, (int)batch, bf16, (hipStream_t)stream);
-    return launch<256, true>(p, (int)batch, bf16, (hipStream_t)stream);
-  }
-  if (d == 128) return launch<128, false>(p, (int)batch, bf16, (hipStream_t)stream);
-  return launch<256, false>(p, (int)batch, bf16, (hipStream_t)stream);
+  // "attn_variant" 1 selects the balanced form (one pinned workgroup per CU) for head_dim 128;
+  // head_dim 256 needs more LDS than its wavefronts per CU allow.
+  p.n_wg = (cx.attn_variant == 1 && d == 128) ? cx.num_cu : 0;
+  // The merge kernel writes the 16-bit copy; without a merge a cast kernel follows.
+  const bool merged = p.n_part > 1 && !cx.attn_skip_merge;
+  if (merged) p.out16 = out16;
+  int rc;
+  if (fp8)
+    rc = d == 128 ? launch<128, true>(p, (int)batch, bf16, (hipStream_t)stream)
+                  : launch<256, true>(p, (int)batch, bf16, (hipStream_t)stream);
+  else
+    rc = d == 128 ? launch<128, false>(p, (int)batch, bf16, (hipStream_t)stream)
+                  : launch<256, false>(p, (int)batch, bf16, (hipStream_t)stream);
+  if (rc || !out16 || merged) return rc;
+  return cast_from_f32(out, out16, (size_t)batch * hq * d, q_dtype, (hipStream_t)stream);
+}
+}  // namespace pto_hip
+
+extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
+                                       const void* value_cache, const int32_t* block_table,
+                                       const int32_t* context_lens, float* out,
+                                       const int64_t* config, int q_dtype, int kv_dtype,
+                                       const float* k_scale, const float* v_scale, void* stream) {
+  return pto_hip::paged_attention(query, key_cache, value_cache, block_table, context_lens, out, nullptr, config,
+                                  q_dtype, kv_dtype, k_scale, v_scale, stream);
 }

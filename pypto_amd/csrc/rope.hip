@@ -13,7 +13,10 @@
 namespace {
 
 struct RopeParams {
-  const float* qkv;        // [B, (Hq + 2*Hkv) * D] fp32 projections
+  const float* qkv;        // [B, (Hq + 2*Hkv) * D] fp32 projections, or their k-split partial sums
+  const float* scale;      // per-channel scales of the partial sums; null when qkv is final
+  int splits;              // partial slabs to sum (1 when qkv is final)
+  int64_t split_stride;    // elements between consecutive partial slabs
   const int32_t* seq_lens; // [B]
   const float* cos;        // [max_pos, D/2]
   const float* sin;
@@ -31,7 +34,23 @@ __global__ __launch_bounds__(128) void rope_kv_kernel(RopeParams p) {
   const int b = blockIdx.x, head = blockIdx.y;
   const int half = p.d / 2;
   const int pos = p.seq_lens[b] - 1;
-  const float* src = p.qkv + ((size_t)b * (p.hq + 2 * p.hkv) + head) * p.d;
+  const size_t src = ((size_t)b * (p.hq + 2 * p.hkv) + head) * p.d;
+  // channel value: sum of the partial slabs in split order, times the channel scale
+  // (loads go out four at a time; the additions keep the order)
+  auto fetch = [&](int i) {
+    float v = 0.f;
+    const float* q = p.qkv + src + i;
+    int s = 0;
+    for (; s + 4 <= p.splits; s += 4) {
+      float t[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) t[u] = q[(size_t)(s + u) * p.split_stride];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v += t[u];
+    }
+    for (; s < p.splits; ++s) v += q[(size_t)s * p.split_stride];
+    return p.scale ? v * p.scale[(size_t)head * p.d + i] : v;
+  };
   const bool is_q = head < p.hq, is_k = !is_q && head < p.hq + p.hkv;
   T* dst;
   if (is_q) {
@@ -52,7 +71,7 @@ __global__ __launch_bounds__(128) void rope_kv_kernel(RopeParams p) {
   }
   const int cpos = pos < 0 ? 0 : (pos >= p.max_pos ? p.max_pos - 1 : pos);
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
-    const float lo = src[i], hi = src[i + half];
+    const float lo = fetch(i), hi = fetch(i + half);
     if (is_q || is_k) {
       const float c = p.cos[(size_t)cpos * half + i], s = p.sin[(size_t)cpos * half + i];
       dst[i] = (T)(lo * c - hi * s);
@@ -86,13 +105,13 @@ int cast_from_f32(const float* in, void* out, size_t n, int out_dtype, hipStream
 }
 }  // namespace pto_hip
 
-extern "C" int pto_hip_rope_kv_cache_update(const float* qkv, const int32_t* seq_lens, const float* rope_cos,
-                                            const float* rope_sin, const int32_t* block_table,
-                                            void* key_cache, void* value_cache, void* q_out, int64_t batch,
-                                            int64_t num_heads, int64_t kv_head_num, int64_t head_dim,
-                                            int64_t block_size, int64_t max_num_blocks_per_req,
-                                            int64_t max_pos, int64_t pool_rows, int dtype, void* stream) {
-  using namespace pto_hip;
+namespace pto_hip {
+int rope_kv_cache_update(const float* qkv, const float* qkv_scale, int splits, int64_t split_stride,
+                         const int32_t* seq_lens, const float* rope_cos, const float* rope_sin,
+                         const int32_t* block_table, void* key_cache, void* value_cache, void* q_out,
+                         int64_t batch, int64_t num_heads, int64_t kv_head_num, int64_t head_dim,
+                         int64_t block_size, int64_t max_num_blocks_per_req, int64_t max_pos,
+                         int64_t pool_rows, int dtype, void* stream) {
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(batch >= 0 && batch < 65536, "rope_kv_cache_update: batch %lld out of range", (long long)batch);
   if (batch == 0) return PTO_HIP_OK;
@@ -108,6 +127,9 @@ extern "C" int pto_hip_rope_kv_cache_update(const float* qkv, const int32_t* seq
                 "rope_kv_cache_update: null tensor pointer");
   RopeParams p{};
   p.qkv = qkv;
+  p.scale = qkv_scale;
+  p.splits = splits;
+  p.split_stride = split_stride;
   p.seq_lens = seq_lens;
   p.cos = rope_cos;
   p.sin = rope_sin;
@@ -130,4 +152,16 @@ extern "C" int pto_hip_rope_kv_cache_update(const float* qkv, const int32_t* seq
     hipLaunchKernelGGL(rope_kv_kernel<_Float16>, grid, dim3(128), 0, (hipStream_t)stream, p);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
+}
+}  // namespace pto_hip
+
+extern "C" int pto_hip_rope_kv_cache_update(const float* qkv, const int32_t* seq_lens, const float* rope_cos,
+                                            const float* rope_sin, const int32_t* block_table,
+                                            void* key_cache, void* value_cache, void* q_out, int64_t batch,
+                                            int64_t num_heads, int64_t kv_head_num, int64_t head_dim,
+                                            int64_t block_size, int64_t max_num_blocks_per_req,
+                                            int64_t max_pos, int64_t pool_rows, int dtype, void* stream) {
+  return pto_hip::rope_kv_cache_update(qkv, nullptr, 1, 0, seq_lens, rope_cos, rope_sin, block_table, key_cache,
+                                       value_cache, q_out, batch, num_heads, kv_head_num, head_dim, block_size,
+                                       max_num_blocks_per_req, max_pos, pool_rows, dtype, stream);
 }

@@ -648,7 +648,12 @@ int pto_hip_set_option(const char* name, int64_t value) {
   } else if (!std::strcmp(name, "attn_waves_per_cu")) {
     PTO_CHECK_ARG(value >= 0 && value <= 16, "attn_waves_per_cu must be in [0, 16]");
     c.attn_waves_per_cu = value;
-
+  } else if (!std::strcmp(name, "w8a16_wgs_per_cu")) {
+    PTO_CHECK_ARG(value >= 1 && value <= 16, "w8a16_wgs_per_cu must be in [1, 16]");
+    c.w8a16_wgs_per_cu = value;
+  } else if (!std::strcmp(name, "w8a16_min_steps")) {
+    PTO_CHECK_ARG(value >= 1 && value <= 1024, "w8a16_min_steps must be in [1, 1024]");
+    c.w8a16_min_steps = value;
   } else {
     return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
   }
@@ -663,6 +668,8 @@ int pto_hip_get_option(const char* name, int64_t* value) {
   else if (!std::strcmp(name, "attn_waves_per_cu")) *value = c.attn_waves_per_cu;
   else if (!std::strcmp(name, "attn_skip_merge")) *value = c.attn_skip_merge;
   else if (!std::strcmp(name, "attn_variant")) *value = c.attn_variant;
+  else if (!std::strcmp(name, "w8a16_wgs_per_cu")) *value = c.w8a16_wgs_per_cu;
+  else if (!std::strcmp(name, "w8a16_min_steps")) *value = c.w8a16_min_steps;
   else return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
   return PTO_HIP_OK;
 }

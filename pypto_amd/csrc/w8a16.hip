@@ -5,42 +5,48 @@
 // projection.py:145-177) with int8 weights and one fp32 scale per output channel.  Decode
 // batches are small (M <= 32), so the work is reading the weights once: HBM-bound.
 //
-//   * one wavefront owns a 32 x 256 output slab over a k range; per 16-k step it reads 8 bytes
-//     (8 output channels) of 8 k-rows per lane - full 256-byte rows per 32 lanes - widens the
-//     int8 codes to fp32 and packs them, transposed, straight into MFMA B operands (the high
-//     halves of the fp32 values are exact bf16), then issues 8 v_mfma_f32_32x32x16;
-//   * k is split across wavefronts to fill the machine; the fp32 partial slabs are summed, scaled
-//     per channel and finished (residual add, SwiGLU, cast) by a second small kernel, in a fixed
-//     order so results are reproducible.
+//   * a workgroup of four wavefronts owns 128 output channels over a k range; the wavefronts
+//     take the range's 32-row steps in turn.  Per step a lane reads 8 bytes (8 channels) of 8
+//     k-rows - whole 128-byte row segments per 16 lanes - keeps the next step's loads in flight,
+//     widens the int8 codes to fp32 and packs them, transposed, straight into MFMA B operands
+//     (the high halves of the fp32 values are exact bf16), then issues 16 v_mfma_f32_16x16x32;
+//   * the four accumulators are summed through LDS in a fixed order, so one workgroup writes
+//     one fp32 partial slab; k is split across workgroups only as far as filling the machine
+//     needs;
+//   * the partial slabs are summed in split order, scaled per channel and finished by a small
+//     second kernel: residual add / SwiGLU / cast, or residual add + RMSNorm of the whole row.
+//     The RoPE kernel reads the q/k/v partials directly.
 #include <hip/hip_runtime.h>
 
 #include "common.h"
 
 namespace {
 
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
 
-constexpr int kSlab = 256;   // output channels per wavefront
-constexpr int kStep = 16;    // k per MFMA step
-constexpr int kMaxM = 32;
+constexpr int kSlab = pto_hip::kW8Slab;  // output channels per workgroup
+constexpr int kStep = 32;                // k rows per step
+constexpr int kWaves = 4;
+constexpr int kMaxM = pto_hip::kW8MaxM;
+constexpr int kUnit = kStep * kWaves;    // k rows one round of the wavefronts covers
 
 struct GemvParams {
-  const uint16_t* x;   // [M, K] 16-bit activations
-  const int8_t* wq;    // [K, N]
-  float* part;         // [splits, 32, N]
-  int m, k, n, splits, k_per_split;
+  const uint16_t* x;    // [M, K] 16-bit activations
+  const int8_t* wq[2];  // [K, N] each; the second is the up projection of a gate/up pair
+  float* part[2];       // [splits, 32, N] each
+  int m, k, n, slabs, n_mats, splits, k_per_split;
 };
 
 template <bool BF16>
-__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
   if constexpr (BF16) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   } else {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
 }
@@ -57,73 +63,143 @@ __device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
   }
 }
 
+struct Stage {
+  uint2 w[8];    // 8 channels of k rows kg*8 .. kg*8+7
+  u32x4 xa[2];   // activations of rows c and c+16, k = kg*8 .. +8
+};
+
 template <bool BF16>
-__global__ __launch_bounds__(64) void w8a16_partial_kernel(GemvParams p) {
-  const int lane = threadIdx.x;
-  const int c = lane & 31, kg = lane >> 5;
-  const int slab = blockIdx.x, split = blockIdx.y;
+__global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void w8a16_partial_kernel(GemvParams p) {
+  constexpr int kHalf = kWaves / 2;
+  __shared__ float red[kHalf * kMaxM * kSlab];  // 32 KiB
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: row addresses stay scalar
+  const int c = lane & 15, kg = lane >> 4;
+
+  const int per_split = p.slabs * p.n_mats;
+  const int split = blockIdx.x / per_split, rem = blockIdx.x % per_split;
+  const int mat = rem / p.slabs, slab = rem % p.slabs;
   const int k_begin = split * p.k_per_split;
   const int k_end = min(p.k, k_begin + p.k_per_split);
-  int n0 = slab * kSlab + c * 8;
-  const bool n_ok = n0 < p.n;
-  if (!n_ok) n0 = p.n - 8;  // keep the loads inside the matrix; the lane's results are dropped
+  const int n_steps = (k_end - k_begin + kStep - 1) / kStep;
 
-  const int8_t* wp = p.wq + n0;
-  const uint16_t* xp = p.x + (size_t)min(c, p.m - 1) * p.k + kg * 8;
-  const bool m_ok = c < p.m;
+  const int n0 = slab * kSlab + c * 8;
+  const uint16_t* xp0 = p.x + (size_t)min(c, p.m - 1) * p.k + kg * 8;
+  const uint16_t* xp1 = p.x + (size_t)min(c + 16, p.m - 1) * p.k + kg * 8;
+  const bool m0_ok = c < p.m, m1_ok = c + 16 < p.m;
 
-  f32x16 acc[8];
+  f32x4 acc[8][2];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+    for (int h = 0; h < 2; ++h) acc[i][h] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  uint2 w[8];
-  u32x4 xa;
-  auto load_step = [&](int k0) {
-    // past the end: re-read the last step (cache hit) so every load is unconditional
-    k0 = min(k0, k_end - kStep);
+  // Loads never depend on a condition, so the number of requests in flight is known at compile
+  // time: steps past the end re-read the wavefront's last one (a cache hit), and a last step
+  // that would reach past row k is moved back to end at row k - the rows it then repeats are
+  // multiplied by zeroed activations.  A row address is a wavefront-uniform row base plus a
+  // per-lane offset that never changes.
+  const int last_step = wave < n_steps ? wave + (n_steps - 1 - wave) / kWaves * kWaves : n_steps - 1;
+  const int8_t* wbase = p.wq[mat];
+  const uint32_t lane_off = (uint32_t)min(n0, p.n - 8) + (uint32_t)(kg * 8) * (uint32_t)p.n;
+  auto step_row = [&](int step) { return min(k_begin + step * kStep, p.k - kStep); };
+  auto load = [&](Stage& s, int step) {
+    const int kstep = step_row(min(step, last_step));
+    s.xa[0] = *reinterpret_cast<const u32x4*>(xp0 + kstep);
+    s.xa[1] = *reinterpret_cast<const u32x4*>(xp1 + kstep);
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
-      w[e] = *reinterpret_cast<const uint2*>(wp + (size_t)(k0 + kg * 8 + e) * p.n);
-    xa = *reinterpret_cast<const u32x4*>(xp + k0);
+    for (int e = 0; e < 8; ++e) {
+      const int8_t* row = wbase + (size_t)(kstep + e) * p.n;  // uniform
+      s.w[e] = *reinterpret_cast<const uint2*>(row + lane_off);
+    }
   };
-
-  load_step(k_begin);
-  for (int k0 = k_begin; k0 < k_end; k0 += kStep) {
-    uint2 cw[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) cw[e] = w[e];
-    u32x4 cx = xa;
-    if (!m_ok) cx = u32x4{0u, 0u, 0u, 0u};
-    load_step(k0 + kStep);
+  auto compute = [&](const Stage& s, int step) {
+    const int row0 = step_row(step) + kg * 8;  // first of this lane's 8 rows
+    const bool k_ok = row0 >= k_begin + step * kStep && row0 < k_end;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    const u32x4 a0 = (k_ok && m0_ok) ? s.xa[0] : z;
+    const u32x4 a1 = (k_ok && m1_ok) ? s.xa[1] : z;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       // channel n0 + i: its 8 k-values, as packed pairs (k, k+1)
       u32x4 b;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const uint32_t w0 = i < 4 ? cw[2 * q].x : cw[2 * q].y;
-        const uint32_t w1 = i < 4 ? cw[2 * q + 1].x : cw[2 * q + 1].y;
+        const uint32_t w0 = i < 4 ? s.w[2 * q].x : s.w[2 * q].y;
+        const uint32_t w1 = i < 4 ? s.w[2 * q + 1].x : s.w[2 * q + 1].y;
         const float f0 = (float)(int8_t)(w0 >> ((i & 3) * 8));
         const float f1 = (float)(int8_t)(w1 >> ((i & 3) * 8));
         b[q] = pack_pair<BF16>(f0, f1);
       }
-      acc[i] = mfma32<BF16>(cx, b, acc[i]);
+      acc[i][0] = mfma16<BF16>(a0, b, acc[i][0]);
+      acc[i][1] = mfma16<BF16>(a1, b, acc[i][1]);
+      __builtin_amdgcn_sched_barrier(0);  // keep the conversions next to their MFMAs
     }
+  };
+
+  // Wavefront w takes steps w, w + kWaves, ...; two register stages, one in flight while the
+  // other is consumed (three or four workgroups share a compute unit, so a dozen or more steps
+  // are in flight per unit).  The trip count is rounded up to even: a surplus step multiplies
+  // by zero.
+  Stage sa, sb;
+  load(sa, wave);
+  for (int s = wave; s < n_steps; s += 2 * kWaves) {
+    load(sb, s + kWaves);
+    compute(sa, s);
+    load(sa, s + 2 * kWaves);
+    compute(sb, s + kWaves);
   }
 
-  if (!n_ok) return;
-  // acc[i][r]: row m = (r/4)*8 + kg*4 + r%4, channel n0 + i
-  float* out = p.part + (size_t)split * kMaxM * p.n + n0;
+  // ---- sum the accumulators: upper half -> LDS -> lower half -> LDS -> all threads ----------
+  // acc[i][h][r]: row m = h*16 + 4*kg + r, channel c*8 + i of the slab.
+  if (wave >= kHalf) {
+    float* dst = red + (wave - kHalf) * (kMaxM * kSlab) + lane;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int m = (r >> 2) * 8 + kg * 4 + (r & 3);
-    float4 lo = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-    float4 hi = {acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
-    float4* dst = reinterpret_cast<float4*>(out + (size_t)m * p.n);
-    dst[0] = lo;
-    dst[1] = hi;
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) dst[((i * 2 + h) * 4 + r) * 64] = acc[i][h][r];
+  }
+  __syncthreads();
+  if (wave < kHalf) {
+    const float* src = red + wave * (kMaxM * kSlab) + lane;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[i][h][r] += src[((i * 2 + h) * 4 + r) * 64];
+  }
+  __syncthreads();
+  if (wave < kHalf) {
+    float* dst = red + wave * (kMaxM * kSlab);
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = h * 16 + 4 * kg + r;
+        float4 lo = {acc[0][h][r], acc[1][h][r], acc[2][h][r], acc[3][h][r]};
+        float4 hi = {acc[4][h][r], acc[5][h][r], acc[6][h][r], acc[7][h][r]};
+        float4* d4 = reinterpret_cast<float4*>(dst + m * kSlab + c * 8);
+        d4[0] = lo;
+        d4[1] = hi;
+      }
+  }
+  __syncthreads();
+  // thread t sums float4 chunk (t % 32) of rows t/32, t/32 + 8, ... over the remaining slices
+  constexpr int kRowsPerPass = kWaves * 64 / 32;
+#pragma unroll
+  for (int m = tid >> 5; m < kMaxM; m += kRowsPerPass) {
+    const int ch = (tid & 31) * 4;
+    float4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < kHalf; ++w) {
+      const float4 v = *reinterpret_cast<const float4*>(red + w * (kMaxM * kSlab) + m * kSlab + ch);
+      a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+    }
+    const int n = slab * kSlab + ch;
+    if (n < p.n) *reinterpret_cast<float4*>(p.part[mat] + ((size_t)split * kMaxM + m) * p.n + n) = a;
   }
 }
 
@@ -137,40 +213,130 @@ struct FinishParams {
   int m, n, splits, res_dtype, out_dtype;
 };
 
-__device__ __forceinline__ float load_as_f32(const void* p, size_t i, int dt) {
-  if (dt == PTO_HIP_FP32) return reinterpret_cast<const float*>(p)[i];
-  if (dt == PTO_HIP_BF16) return (float)reinterpret_cast<const __bf16*>(p)[i];
-  return (float)reinterpret_cast<const _Float16*>(p)[i];
+__device__ __forceinline__ float4 load4_as_f32(const void* p, size_t i, int dt) {
+  if (dt == PTO_HIP_FP32) return *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + i);
+  const uint2 v = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p) + i);
+  if (dt == PTO_HIP_BF16)
+    return float4{__builtin_bit_cast(float, v.x << 16), __builtin_bit_cast(float, v.x & 0xffff0000u),
+                  __builtin_bit_cast(float, v.y << 16), __builtin_bit_cast(float, v.y & 0xffff0000u)};
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  const h2 a = __builtin_bit_cast(h2, v.x), b = __builtin_bit_cast(h2, v.y);
+  return float4{(float)a.x, (float)a.y, (float)b.x, (float)b.y};
 }
-__device__ __forceinline__ void store_from_f32(void* p, size_t i, int dt, float v) {
-  if (dt == PTO_HIP_FP32) reinterpret_cast<float*>(p)[i] = v;
-  else if (dt == PTO_HIP_BF16) reinterpret_cast<__bf16*>(p)[i] = (__bf16)v;
-  else reinterpret_cast<_Float16*>(p)[i] = (_Float16)v;
+__device__ __forceinline__ void store4_from_f32(void* p, size_t i, int dt, float4 v) {
+  if (dt == PTO_HIP_FP32) {
+    *reinterpret_cast<float4*>(reinterpret_cast<float*>(p) + i) = v;
+  } else if (dt == PTO_HIP_BF16) {
+    typedef __bf16 b4 __attribute__((ext_vector_type(4)));
+    *reinterpret_cast<b4*>(reinterpret_cast<__bf16*>(p) + i) = b4{(__bf16)v.x, (__bf16)v.y, (__bf16)v.z, (__bf16)v.w};
+  } else {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    *reinterpret_cast<h4*>(reinterpret_cast<_Float16*>(p) + i) =
+        h4{(_Float16)v.x, (_Float16)v.y, (_Float16)v.z, (_Float16)v.w};
+  }
+}
+
+// Sum of the k splits of four channels, in split order, times the channel scales.  Loads go out
+// four at a time; the additions keep the order.
+__device__ __forceinline__ float4 sum_splits(const float* part, const float* scale, int splits, int m, int n,
+                                             int nn) {
+  float4 a = {0.f, 0.f, 0.f, 0.f};
+  const size_t stride = (size_t)kMaxM * nn;
+  const float* src = part + (size_t)m * nn + n;
+  int s = 0;
+  for (; s + 4 <= splits; s += 4) {
+    float4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = *reinterpret_cast<const float4*>(src + (size_t)(s + j) * stride);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { a.x += v[j].x; a.y += v[j].y; a.z += v[j].z; a.w += v[j].w; }
+  }
+  for (; s < splits; ++s) {
+    const float4 v = *reinterpret_cast<const float4*>(src + (size_t)s * stride);
+    a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+  }
+  const float4 sc = *reinterpret_cast<const float4*>(scale + n);
+  return float4{a.x * sc.x, a.y * sc.y, a.z * sc.z, a.w * sc.w};
+}
+
+__device__ __forceinline__ float silu_mul(float g, float u) {
+  return g * __frcp_rn(1.f + __expf(-g)) * u;  // SiLU(gate) * up, device form of 01_ffn.py:70-75
 }
 
 __global__ __launch_bounds__(256) void w8a16_finish_kernel(FinishParams p) {
-  const int n = blockIdx.x * 256 + threadIdx.x;
+  const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
   const int m = blockIdx.y;
   if (n >= p.n) return;
-  float a = 0.f;
-  for (int s = 0; s < p.splits; ++s) a += p.part0[((size_t)s * kMaxM + m) * p.n + n];
-  a *= p.scale0[n];
+  float4 a = sum_splits(p.part0, p.scale0, p.splits, m, n, p.n);
   if (p.part1) {
-    float u = 0.f;
-    for (int s = 0; s < p.splits; ++s) u += p.part1[((size_t)s * kMaxM + m) * p.n + n];
-    u *= p.scale1[n];
-    a = a * __frcp_rn(1.f + __expf(-a)) * u;  // SiLU(gate) * up, device form of 01_ffn.py:70-75
+    const float4 u = sum_splits(p.part1, p.scale1, p.splits, m, n, p.n);
+    a = float4{silu_mul(a.x, u.x), silu_mul(a.y, u.y), silu_mul(a.z, u.z), silu_mul(a.w, u.w)};
   }
   const size_t idx = (size_t)m * p.n + n;
-  if (p.residual) a += load_as_f32(p.residual, idx, p.res_dtype);
-  store_from_f32(p.out, idx, p.out_dtype, a);
+  if (p.residual) {
+    const float4 r = load4_as_f32(p.residual, idx, p.res_dtype);
+    a.x += r.x; a.y += r.y; a.z += r.z; a.w += r.w;
+  }
+  store4_from_f32(p.out, idx, p.out_dtype, a);
+}
+
+// Finish of a projection followed by RMSNorm of the sum with the residual: one workgroup per
+// row, the row (n <= 4 * kNormThreads * kNormVec channels) kept in registers between the two passes.
+// Writes the fp32 sum (the next residual) and the normalised row.
+constexpr int kNormVec = 2;
+constexpr int kNormThreads = 1024;
+struct FinishNormParams {
+  const float* part;
+  const float* scale;
+  const void* residual;  // [M, N] in res_dtype
+  float* sum_out;        // [M, N] fp32
+  const float* gamma;    // [N]
+  void* normed_out;      // [M, N] in out_dtype
+  int n, splits, res_dtype, out_dtype;
+  float eps;
+};
+
+__global__ __launch_bounds__(kNormThreads) void w8a16_finish_norm_kernel(FinishNormParams p) {
+  const int m = blockIdx.x;
+  float4 v[kNormVec];
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < kNormVec; ++u) {
+    const int n = (threadIdx.x + u * kNormThreads) * 4;
+    if (n < p.n) {
+      float4 a = sum_splits(p.part, p.scale, p.splits, m, n, p.n);
+      const float4 r = load4_as_f32(p.residual, (size_t)m * p.n + n, p.res_dtype);
+      a.x += r.x; a.y += r.y; a.z += r.z; a.w += r.w;
+      v[u] = a;
+      *reinterpret_cast<float4*>(p.sum_out + (size_t)m * p.n + n) = a;
+      ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+  __shared__ float wsum[kNormThreads / 64];
+  if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int w = 0; w < kNormThreads / 64; ++w) tot += wsum[w];
+  const float inv = rsqrtf(tot / (float)p.n + p.eps);
+#pragma unroll
+  for (int u = 0; u < kNormVec; ++u) {
+    const int n = (threadIdx.x + u * kNormThreads) * 4;
+    if (n < p.n) {
+      const float4 g = *reinterpret_cast<const float4*>(p.gamma + n);
+      const float4 y = {v[u].x * inv * g.x, v[u].y * inv * g.y, v[u].z * inv * g.z, v[u].w * inv * g.w};
+      store4_from_f32(p.normed_out, (size_t)m * p.n + n, p.out_dtype, y);
+    }
+  }
 }
 
 int check_common(const char* what, int64_t m, int64_t k, int64_t n, int x_dtype, int out_dtype) {
   using namespace pto_hip;
   PTO_CHECK_ARG(m >= 0 && m <= kMaxM, "%s: M = %lld rows, this decode kernel takes at most %d", what,
                 (long long)m, kMaxM);
-  PTO_CHECK_ARG(k >= kStep && k % kStep == 0, "%s: K = %lld must be a positive multiple of %d", what,
+  PTO_CHECK_ARG(k >= kStep && k % 16 == 0, "%s: K = %lld must be a multiple of 16, at least %d", what,
                 (long long)k, kStep);
   PTO_CHECK_ARG(n >= 8 && n % 8 == 0, "%s: N = %lld must be a positive multiple of 8", what, (long long)n);
   PTO_CHECK_ARG(k < (1 << 30) && n < (1 << 30), "%s: shape too large", what);
@@ -181,38 +347,95 @@ int check_common(const char* what, int64_t m, int64_t k, int64_t n, int x_dtype,
   return PTO_HIP_OK;
 }
 
-// k splits: enough wavefronts for two per SIMD, each with at least 8 steps of work.
-int choose_splits(int64_t k, int64_t n) {
-  const int64_t slabs = (n + kSlab - 1) / kSlab;
-  const int64_t want = (int64_t)pto_hip::ctx().num_cu * 8;
-  int64_t s = (want + slabs - 1) / slabs;
-  const int64_t max_s = k / (kStep * 8) > 0 ? k / (kStep * 8) : 1;
-  if (s > max_s) s = max_s;
-  if (s < 1) s = 1;
-  return (int)s;
+// k splits: a few workgroups per compute unit, each wavefront with at least a few steps when k
+// allows, split boundaries on multiples of the rows one round of the wavefronts covers.
+void choose_splits(int64_t k, int64_t slabs_total, int* splits, int* k_per_split) {
+  const pto_hip::Context& cx = pto_hip::ctx();
+  const int64_t units = (k + kUnit - 1) / kUnit;
+  int64_t want = (cx.w8a16_wgs_per_cu * cx.num_cu) / slabs_total;
+  if (want < 1) want = 1;
+  int64_t per = (units + want - 1) / want;
+  if (per < cx.w8a16_min_steps) per = units >= cx.w8a16_min_steps ? cx.w8a16_min_steps : units;
+  *splits = (int)((units + per - 1) / per);
+  *k_per_split = (int)(per * kUnit);
 }
 
-int launch_partial(const void* x, const void* wq, float* part, int64_t m, int64_t k, int64_t n, int splits,
-                   int x_dtype, hipStream_t st) {
+}  // namespace
+
+namespace pto_hip {
+
+int w8a16_partials(const void* x, const void* wq0, const void* wq1, int64_t m, int64_t k, int64_t n,
+                   int x_dtype, hipStream_t st, W8Partials* out) {
   GemvParams p{};
   p.x = reinterpret_cast<const uint16_t*>(x);
-  p.wq = reinterpret_cast<const int8_t*>(wq);
-  p.part = part;
+  p.wq[0] = reinterpret_cast<const int8_t*>(wq0);
+  p.wq[1] = reinterpret_cast<const int8_t*>(wq1);
   p.m = (int)m;
   p.k = (int)k;
   p.n = (int)n;
-  p.splits = splits;
-  p.k_per_split = (int)(((k + splits - 1) / splits + kStep - 1) / kStep * kStep);
-  dim3 grid((unsigned)((n + kSlab - 1) / kSlab), (unsigned)splits);
+  p.slabs = (int)((n + kSlab - 1) / kSlab);
+  p.n_mats = wq1 ? 2 : 1;
+  choose_splits(k, (int64_t)p.slabs * p.n_mats, &p.splits, &p.k_per_split);
+  const size_t one = (size_t)p.splits * kMaxM * n * sizeof(float);
+  void* ws = nullptr;
+  int rc = workspace(one * p.n_mats, &ws);
+  if (rc) return rc;
+  p.part[0] = reinterpret_cast<float*>(ws);
+  p.part[1] = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + one);
+  const dim3 grid((unsigned)(p.slabs * p.n_mats * p.splits));
   if (x_dtype == PTO_HIP_BF16)
-    hipLaunchKernelGGL(w8a16_partial_kernel<true>, grid, dim3(64), 0, st, p);
+    hipLaunchKernelGGL(w8a16_partial_kernel<true>, grid, dim3(kWaves * 64), 0, st, p);
   else
-    hipLaunchKernelGGL(w8a16_partial_kernel<false>, grid, dim3(64), 0, st, p);
+    hipLaunchKernelGGL(w8a16_partial_kernel<false>, grid, dim3(kWaves * 64), 0, st, p);
+  PTO_CHECK_HIP(hipGetLastError());
+  out->part[0] = p.part[0];
+  out->part[1] = wq1 ? p.part[1] : nullptr;
+  out->splits = p.splits;
+  return PTO_HIP_OK;
+}
+
+int w8a16_finish(const W8Partials& parts, const float* scale0, const float* scale1, const void* residual,
+                 int res_dtype, void* out, int out_dtype, int64_t m, int64_t n, hipStream_t st) {
+  FinishParams f{};
+  f.part0 = parts.part[0];
+  f.part1 = parts.part[1];
+  f.scale0 = scale0;
+  f.scale1 = scale1;
+  f.residual = residual;
+  f.out = out;
+  f.m = (int)m;
+  f.n = (int)n;
+  f.splits = parts.splits;
+  f.res_dtype = res_dtype;
+  f.out_dtype = out_dtype;
+  hipLaunchKernelGGL(w8a16_finish_kernel, dim3((unsigned)((n / 4 + 255) / 256), (unsigned)m), dim3(256), 0, st, f);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
 }
 
-}  // namespace
+bool w8a16_finish_norm_fits(int64_t n) { return n % 4 == 0 && n <= 4 * kNormThreads * kNormVec; }
+
+int w8a16_finish_norm(const W8Partials& parts, const float* scale, const void* residual, int res_dtype,
+                      float* sum_out, const float* gamma, void* normed_out, int out_dtype, int64_t m,
+                      int64_t n, float eps, hipStream_t st) {
+  FinishNormParams f{};
+  f.part = parts.part[0];
+  f.scale = scale;
+  f.residual = residual;
+  f.sum_out = sum_out;
+  f.gamma = gamma;
+  f.normed_out = normed_out;
+  f.n = (int)n;
+  f.splits = parts.splits;
+  f.res_dtype = res_dtype;
+  f.out_dtype = out_dtype;
+  f.eps = eps;
+  hipLaunchKernelGGL(w8a16_finish_norm_kernel, dim3((unsigned)m), dim3(kNormThreads), 0, st, f);
+  PTO_CHECK_HIP(hipGetLastError());
+  return PTO_HIP_OK;
+}
+
+}  // namespace pto_hip
 
 extern "C" int pto_hip_w8a16_matmul(const void* x, const void* w_q, const float* w_scale,
                                     const void* residual, void* out, int64_t m, int64_t k, int64_t n,
@@ -223,28 +446,17 @@ extern "C" int pto_hip_w8a16_matmul(const void* x, const void* w_q, const float*
   if (rc) return rc;
   if (m == 0) return PTO_HIP_OK;
   PTO_CHECK_ARG(x && w_q && w_scale && out, "w8a16_matmul: null tensor pointer");
-  PTO_CHECK_ARG(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_q % 8 == 0), "w8a16_matmul: misaligned operand");
+  PTO_CHECK_ARG(((uintptr_t)x % 16 == 0) && ((uintptr_t)w_q % 8 == 0) && ((uintptr_t)w_scale % 16 == 0) &&
+                    ((uintptr_t)out % 16 == 0) && ((uintptr_t)residual % 16 == 0),
+                "w8a16_matmul: misaligned operand");
+  if (residual)
+    PTO_CHECK_ARG(res_dtype == PTO_HIP_FP32 || res_dtype == PTO_HIP_BF16 || res_dtype == PTO_HIP_FP16,
+                  "w8a16_matmul: residual dtype %s not in {FP32, BF16, FP16}", dtype_name(res_dtype));
   hipStream_t st = (hipStream_t)stream;
-  const int splits = choose_splits(k, n);
-  // split s of the last step may start before k_end - kStep only if k_per_split >= kStep: true here
-  void* ws = nullptr;
-  rc = workspace((size_t)splits * kMaxM * n * sizeof(float), &ws);
+  W8Partials parts{};
+  rc = w8a16_partials(x, w_q, nullptr, m, k, n, x_dtype, st, &parts);
   if (rc) return rc;
-  rc = launch_partial(x, w_q, reinterpret_cast<float*>(ws), m, k, n, splits, x_dtype, st);
-  if (rc) return rc;
-  FinishParams f{};
-  f.part0 = reinterpret_cast<const float*>(ws);
-  f.scale0 = w_scale;
-  f.residual = residual;
-  f.out = out;
-  f.m = (int)m;
-  f.n = (int)n;
-  f.splits = splits;
-  f.res_dtype = res_dtype;
-  f.out_dtype = out_dtype;
-  hipLaunchKernelGGL(w8a16_finish_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)m), dim3(256), 0, st, f);
-  PTO_CHECK_HIP(hipGetLastError());
-  return PTO_HIP_OK;
+  return w8a16_finish(parts, w_scale, nullptr, residual, res_dtype, out, out_dtype, m, n, st);
 }
 
 extern "C" int pto_hip_w8a16_swiglu(const void* x, const void* wg_q, const float* wg_scale,
@@ -256,31 +468,12 @@ extern "C" int pto_hip_w8a16_swiglu(const void* x, const void* wg_q, const float
   if (rc) return rc;
   if (m == 0) return PTO_HIP_OK;
   PTO_CHECK_ARG(x && wg_q && wg_scale && wu_q && wu_scale && out, "w8a16_swiglu: null tensor pointer");
-  PTO_CHECK_ARG(((uintptr_t)x % 16 == 0) && ((uintptr_t)wg_q % 8 == 0) && ((uintptr_t)wu_q % 8 == 0),
+  PTO_CHECK_ARG(((uintptr_t)x % 16 == 0) && ((uintptr_t)wg_q % 8 == 0) && ((uintptr_t)wu_q % 8 == 0) &&
+                    ((uintptr_t)wg_scale % 16 == 0) && ((uintptr_t)wu_scale % 16 == 0) && ((uintptr_t)out % 16 == 0),
                 "w8a16_swiglu: misaligned operand");
   hipStream_t st = (hipStream_t)stream;
-  const int splits = choose_splits(k, n);
-  const size_t one = (size_t)splits * kMaxM * n * sizeof(float);
-  void* ws = nullptr;
-  rc = workspace(2 * one, &ws);
+  W8Partials parts{};
+  rc = w8a16_partials(x, wg_q, wu_q, m, k, n, x_dtype, st, &parts);
   if (rc) return rc;
-  float* p0 = reinterpret_cast<float*>(ws);
-  float* p1 = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + one);
-  rc = launch_partial(x, wg_q, p0, m, k, n, splits, x_dtype, st);
-  if (rc) return rc;
-  rc = launch_partial(x, wu_q, p1, m, k, n, splits, x_dtype, st);
-  if (rc) return rc;
-  FinishParams f{};
-  f.part0 = p0;
-  f.part1 = p1;
-  f.scale0 = wg_scale;
-  f.scale1 = wu_scale;
-  f.out = out;
-  f.m = (int)m;
-  f.n = (int)n;
-  f.splits = splits;
-  f.out_dtype = out_dtype;
-  hipLaunchKernelGGL(w8a16_finish_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)m), dim3(256), 0, st, f);
-  PTO_CHECK_HIP(hipGetLastError());
-  return PTO_HIP_OK;
+  return w8a16_finish(parts, wg_scale, wu_scale, nullptr, 0, out, out_dtype, m, n, st);
 }

@@ -17,10 +17,11 @@ ATOL, RTOL = 1e-2, 2e-2
 
 
 def _run(worker, inp, tpp=0):
-    """tpp = 0: the default streaming kernel; tpp > 0: the partition-grid kernel with that many
-    tokens per context partition; tpp < 0: the partition-grid kernel with its own choice."""
-    worker.set_option("attn_variant", 0 if tpp == 0 else 1)
-    worker.set_option("attn_tokens_per_partition", max(tpp, 0))
+    """tpp = 0: the default partition-grid kernel with its own choice of partition size; tpp > 0:
+    the same with that many tokens per context partition; tpp < 0: the balanced form (one pinned
+    workgroup per CU) with -tpp - 1 tokens per partition (-1: its own choice)."""
+    worker.set_option("attn_variant", 1 if tpp < 0 else 0)
+    worker.set_option("attn_tokens_per_partition", tpp if tpp > 0 else max(-tpp - 1, 0))
     dev = [t.cuda() if isinstance(t, torch.Tensor) and i != 6 else t for i, t in enumerate(inp.args())]
     dev[5].fill_(float("nan"))
     torch.cuda.synchronize()
