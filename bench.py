@@ -8,7 +8,9 @@ A step is one paged-attention decode pass over one batch of the "small" configur
 a pool of 1024 blocks, permutation block table).  The step rotates through several identical KV
 pools so the working set stays larger than the 256 MB last-level cache.  The printed JSON line
 carries the whole-step throughput (`value`), the roofline of the dominant kernel, the FFN block
-at LLaMA-7B shape as a second measurement, and the CPU oracle timed on this machine's host cores.
+at LLaMA-7B shape as a second measurement, two more HBM-bound workloads of the same path (the
+long-context e4m3 attention configuration and one W8A16 decoder-layer decode step), and the CPU
+oracle timed on this machine's host cores.
 """
 
 from __future__ import annotations
@@ -24,6 +26,15 @@ HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 KV_POOLS = 4                   # 4 x 537 MB of K+V, cycled
 
+# HBM bytes one launch of the dominant kernel moves, from hardware counters: rocprofv3 --pmc
+# FETCH_SIZE and --pmc WRITE_SIZE (KiB per dispatch) of this script, each scaled by what the same
+# counter reads for a plain 1 GiB device copy (FETCH_SIZE reads 0.5 KiB per KiB copied, WRITE_SIZE
+# 1.0).  The counter runs and their figures are in profiles/bench_attention_small_ffn_llama7b.md.
+PMC_FETCH_KIB = 74364.9
+PMC_FETCH_SCALE = 1048576.0 / 524320.0
+PMC_WRITE_KIB = 1284.9
+PMC_WRITE_SCALE = 1.0
+
 
 def main() -> int:
     ap = argparse.ArgumentParser()
@@ -32,6 +43,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--no-ffn", action="store_true", help="skip the FFN measurement")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the long-context e4m3 attention and decoder-layer measurements")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy, a known-size reference for HBM byte counters")
     args = ap.parse_args()
@@ -42,7 +55,8 @@ def main() -> int:
     import torch
 
     from pypto_amd import workloads
-    from pypto_amd.runtime import ChipWorker, RunConfig, benchmark, ffn_block, paged_attention
+    from pypto_amd.runtime import (ChipWorker, RunConfig, benchmark, decoder_layer_decode, ffn_block,
+                                   paged_attention)
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -100,16 +114,18 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "attn_partition_kernel<128, true>",
+            "kernel": "attn_partition_kernel<128, true, false>",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "kernel_us": round(kernel_us, 2),
-            "traffic": None,
+            "traffic": round((PMC_FETCH_KIB * PMC_FETCH_SCALE + PMC_WRITE_KIB * PMC_WRITE_SCALE) * 1024),
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this script, scaled by a 1 GiB copy",
         },
     }
     handle.unregister()
+    del pools[1:], arg_sets
 
     # ---- FFN block at LLaMA-7B shape (second half of the metric) ------------------------------
     if not args.no_ffn:
@@ -131,6 +147,49 @@ def main() -> int:
             "bound": "mfma",
         }
         del f
+
+    # ---- the path's other HBM-bound workloads ---------------------------------------------------
+    if not args.no_extra:
+        lf = workloads.attention_long_fp8(seed=0, device="cuda")
+        torch.cuda.synchronize()
+        with worker.register(paged_attention) as lh:
+            largs = [lf.args()]
+            benchmark(lh, largs, rounds=3, warmup=0)
+            lstats = benchmark(lh, largs, rounds=10, warmup=0)
+        lbytes = lf.algorithmic_bytes()
+        result["attention_long_fp8"] = {
+            "workload": "paged-attention decode long: B64 Hq64 Hkv8 D128 bs128 ctx~U[8192,32768], e4m3 KV with "
+                        "one fp32 scale per (block, KV head), dequantised in-kernel",
+            "algorithmic_bytes_per_step": lbytes,
+            "us_per_step": round(lstats.device_wall_us, 1),
+            "achieved": round(lbytes / lstats.device_wall_us / 1e3, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(lbytes / lstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "bound": "hbm",
+        }
+        del lf, largs
+        torch.cuda.empty_cache()
+        dl = workloads.decoder_layer_inputs(device="cuda")
+        torch.cuda.synchronize()
+        with worker.register(decoder_layer_decode) as dh:
+            dargs = [dl.args()]
+            benchmark(dh, dargs, rounds=5, warmup=0)
+            dstats = benchmark(dh, dargs, rounds=20, warmup=0)
+        dbytes = dl.algorithmic_bytes()
+        result["decoder_layer"] = {
+            "workload": "decoder-layer decode step: H4096 Hq32 Hkv8 D128 I14336 B32 ctx4096, int8 weights with "
+                        "per-channel scales, bf16 activations and paged KV",
+            "algorithmic_bytes_per_step": dbytes,
+            "us_per_step": round(dstats.device_wall_us, 1),
+            "achieved": round(dbytes / dstats.device_wall_us / 1e3, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(dbytes / dstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "bound": "hbm",
+        }
+        del dl, dargs
+        torch.cuda.empty_cache()
 
     # ---- CPU baseline: the oracle on this machine's host cores --------------------------------
     if not args.no_cpu_baseline:
