@@ -128,6 +128,10 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *      tensors: qkv[B,(Hq+2Hkv)*D] fp32, seq_lens[B] i32, rope_cos[max_pos,D/2], rope_sin,
  *               block_table[B*max_blocks] i32, key_cache (INOUT), value_cache (INOUT), q_out[B*Hq,D]
  *      scalars: num_heads, kv_head_num, head_dim, block_size
+ *  "rope_kv_cache_update_fp8"  the same with FP8E4M3FN caches, quantised on write
+ *      tensors: qkv, seq_lens, rope_cos, rope_sin, block_table, key_cache (INOUT), value_cache (INOUT),
+ *               k_scale[pool,Hkv] fp32 (INOUT), v_scale (INOUT), q_out[B*Hq,D]
+ *      scalars: num_heads, kv_head_num, head_dim, block_size
  *  "decoder_layer_decode"  examples/models/qwen3_jit/qwen3_decode.py:47-113
  *      tensors: hidden_states[B,H], seq_lens, block_table, key_cache (INOUT), value_cache (INOUT),
  *               rope_cos, rope_sin, gamma_in[H], gamma_post[H], wqkv_q, wqkv_s, wo_q, wo_s, wg_q, wg_s,
@@ -204,6 +208,20 @@ PTO_HIP_API int pto_hip_rope_kv_cache_update(const float* qkv, const int32_t* se
                                              int64_t num_heads, int64_t kv_head_num, int64_t head_dim,
                                              int64_t block_size, int64_t max_num_blocks_per_req,
                                              int64_t max_pos, int64_t pool_rows, int dtype, void* stream);
+
+/* The same step for an FP8E4M3FN cache: the new K/V rows are quantised on write with the running
+ * per-(block, KV head) scale the e4m3 attention path reads (k_scale/v_scale FP32 [pool_blocks, Hkv],
+ * updated in place).  First token of a block: scale = amax(row)/448; later tokens: the scale only
+ * grows, and when it does the block's earlier rows are re-coded.  The reference has no quantised
+ * cache; the float step is examples/models/qwen3_jit/kernels/attention.py:39-102. */
+PTO_HIP_API int pto_hip_rope_kv_cache_update_fp8(const float* qkv, const int32_t* seq_lens,
+                                                 const float* rope_cos, const float* rope_sin,
+                                                 const int32_t* block_table, void* key_cache,
+                                                 void* value_cache, float* k_scale, float* v_scale,
+                                                 void* q_out, int64_t batch, int64_t num_heads,
+                                                 int64_t kv_head_num, int64_t head_dim, int64_t block_size,
+                                                 int64_t max_num_blocks_per_req, int64_t max_pos,
+                                                 int64_t pool_blocks, int q_dtype, void* stream);
 
 /* One decoder layer, one new token per sequence (examples/models/qwen3_jit/qwen3_decode.py:47-113):
  * RMSNorm -> QKV -> RoPE + K/V append -> paged attention -> o_proj + residual -> RMSNorm ->

@@ -40,6 +40,7 @@ from .attention import (  # noqa: F401
 from .ffn import ffn_block, ffn_swiglu, rms_norm, swiglu  # noqa: F401
 from .layer import (  # noqa: F401
     decoder_layer_decode,
+    kv_append_fp8,
     quantize_w8,
     rope_cos_sin,
     rope_rotate_half,

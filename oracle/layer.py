@@ -7,6 +7,10 @@ TEST INFRASTRUCTURE ONLY — see ``oracle/__init__.py``.
                                    position = seq_len - 1, K/V row written into the cache)
 * layer composition                test_llama_7b_mini_1h.py:119-198,
                                    tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:255-287
+* e4m3 quantise-on-write of the appended K/V rows (``kv_append_fp8``): the reference has no
+  quantised cache; closed form stated in the function.  PARITY UNPINNED against the
+  reference (nothing there to pin it); pinned against ``quantize_kv_fp8`` of a block
+  written in one go when the first row holds the block's maximum.
 * W8A16 (int8 weights, per-output-channel fp32 scale): the reference has no
   such path; closed form ``w_q = clamp(round(w / s), -127, 127)``,
   ``s = amax_col / 127``, ``y = (x @ w_q) * s``.
@@ -16,7 +20,7 @@ from __future__ import annotations
 
 import torch
 
-from .attention import encode_scale, paged_attention_golden
+from .attention import FP8_E4M3_MAX, encode_scale, paged_attention_golden
 from .ffn import rms_norm, swiglu
 
 
@@ -42,6 +46,43 @@ def rope_rotate_half(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> t
     xf = x.float()
     lo, hi = xf[..., :half], xf[..., half:]
     return torch.cat([lo * cos - hi * sin, hi * cos + lo * sin], dim=-1)
+
+
+def kv_append_fp8(codes: torch.Tensor, scale: torch.Tensor, new_rows: torch.Tensor, blocks, tokens,
+                  block_size: int):
+    """Append one fp32 row per (sequence, KV head) to an e4m3 cache with a running scale.
+
+    The reference has no quantised cache; this is the write side of the contract
+    ``quantize_kv_fp8`` states (code = e4m3(x / scale), nearest even, scale per
+    (block, KV head)).  ``codes`` [pool_blocks*Hkv*bs, D] float8_e4m3fn and ``scale``
+    [pool_blocks, Hkv] fp32 are updated copies; ``new_rows`` is [B, Hkv, D] fp32,
+    ``blocks[b]`` / ``tokens[b]`` the physical block and the slot inside it.
+
+    slot 0: scale = amax(row)/448 (1 if the row is all zero) - the block's old content
+    is stale.  slot t > 0: scale' = max(scale, amax(row)/448); if it grew, rows 0..t-1
+    are re-coded as e4m3(code * scale / scale').  The row is stored as
+    e4m3(clamp(row / scale', +-448)).
+    """
+    codes = codes.clone()
+    scale = scale.clone()
+    b, kv, d = new_rows.shape
+    view = codes.view(-1, kv, block_size, d)  # [pool_blocks, Hkv, bs, D]
+    for bi in range(b):
+        blk, t = int(blocks[bi]), int(tokens[bi])
+        for h in range(kv):
+            row = new_rows[bi, h].float()
+            cand = row.abs().max() / FP8_E4M3_MAX
+            if t == 0:
+                new = cand if cand > 0 else torch.tensor(1.0)
+            else:
+                old = scale[blk, h]
+                new = torch.maximum(old, cand)
+                if new > old:
+                    prev = view[blk, h, :t].float() * old / new
+                    view[blk, h, :t] = prev.clamp(-FP8_E4M3_MAX, FP8_E4M3_MAX).to(torch.float8_e4m3fn)
+            view[blk, h, t] = (row / new).clamp(-FP8_E4M3_MAX, FP8_E4M3_MAX).to(torch.float8_e4m3fn)
+            scale[blk, h] = new
+    return codes, scale
 
 
 def quantize_w8(w: torch.Tensor):

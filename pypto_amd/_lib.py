@@ -23,6 +23,7 @@ EXPORTS = (
     "pto_hip_benchmark", "pto_hip_paged_attention", "pto_hip_paged_gather", "pto_hip_rms_norm",
     "pto_hip_ffn_swiglu", "pto_hip_set_option", "pto_hip_get_option",
     "pto_hip_w8a16_matmul", "pto_hip_w8a16_swiglu", "pto_hip_rope_kv_cache_update",
+    "pto_hip_rope_kv_cache_update_fp8",
     "pto_hip_decoder_layer_decode",
 )
 
@@ -93,6 +94,7 @@ def load() -> C.CDLL:
         "pto_hip_w8a16_swiglu": [vp, vp, vp, vp, vp, vp, i64, i64, i64, C.c_int, C.c_int, vp],
         "pto_hip_rope_kv_cache_update": [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64,
                                          C.c_int, vp],
+        "pto_hip_rope_kv_cache_update_fp8": [vp] * 10 + [i64] * 8 + [C.c_int, vp],
         "pto_hip_decoder_layer_decode": [vp, vp],
         "pto_hip_set_option": [C.c_char_p, i64],
         "pto_hip_get_option": [C.c_char_p, C.POINTER(i64)],

@@ -80,13 +80,15 @@ enum ProgramKind {
   kW8a16Matmul,
   kW8a16Swiglu,
   kRopeKvCacheUpdate,
+  kRopeKvCacheUpdateFp8,
   kDecoderLayerDecode,
   kNumPrograms
 };
 
 const char* const kProgramNames[kNumPrograms] = {
     "paged_attention", "paged_gather",  "rms_norm",           "ffn_swiglu",          "ffn_block",
-    "w8a16_matmul",    "w8a16_swiglu",  "rope_kv_cache_update", "decoder_layer_decode"};
+    "w8a16_matmul",    "w8a16_swiglu",  "rope_kv_cache_update", "rope_kv_cache_update_fp8",
+    "decoder_layer_decode"};
 
 std::mutex g_mu;
 std::vector<int> g_callables;  // callable id -> ProgramKind, -1 once unregistered
@@ -313,6 +315,44 @@ int run_w8a16_swiglu(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns,
                               (int)t[5].dtype, stream);
 }
 
+int run_rope_kv_fp8(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream) {
+  PTO_CHECK_ARG(nt == 10 && ns == 4,
+                "rope_kv_cache_update_fp8: expected qkv, seq_lens, rope_cos, rope_sin, block_table, key_cache, "
+                "value_cache, k_scale, v_scale, q_out + scalars num_heads, kv_head_num, head_dim, block_size; "
+                "got %d + %d", nt, ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor("rope_kv_cache_update_fp8", "operand", t[i], 1, 2);
+    if (rc) return rc;
+  }
+  const int64_t hq = (int64_t)s[0], hkv = (int64_t)s[1], d = (int64_t)s[2], bs = (int64_t)s[3];
+  PTO_CHECK_ARG(hq > 0 && hkv > 0 && d > 0 && bs > 0, "rope_kv_cache_update_fp8: non-positive scalar");
+  const int64_t batch = numel(t[1]);
+  PTO_CHECK_ARG(t[0].dtype == PTO_HIP_FP32 && numel(t[0]) == batch * (hq + 2 * hkv) * d,
+                "rope_kv_cache_update_fp8: qkv must be FP32 [B, (Hq+2Hkv)*D]");
+  PTO_CHECK_ARG(t[1].dtype == PTO_HIP_INT32 && t[4].dtype == PTO_HIP_INT32,
+                "rope_kv_cache_update_fp8: seq_lens and block_table must be INT32");
+  PTO_CHECK_ARG(t[2].dtype == PTO_HIP_FP32 && t[3].dtype == PTO_HIP_FP32 && numel(t[2]) == numel(t[3]) &&
+                    d % 2 == 0 && numel(t[2]) % (d / 2) == 0,
+                "rope_kv_cache_update_fp8: rope_cos/rope_sin must be FP32 [max_pos, D/2]");
+  PTO_CHECK_ARG(batch > 0 ? numel(t[4]) % batch == 0 : true,
+                "rope_kv_cache_update_fp8: block_table must be [B, max_blocks]");
+  PTO_CHECK_ARG(t[5].dtype == PTO_HIP_FP8E4M3FN && t[6].dtype == PTO_HIP_FP8E4M3FN && numel(t[5]) == numel(t[6]) &&
+                    numel(t[5]) % (hkv * bs * d) == 0,
+                "rope_kv_cache_update_fp8: caches must be FP8E4M3FN [pool_blocks*Hkv*bs, D]");
+  const int64_t pool_blocks = numel(t[5]) / (hkv * bs * d);
+  PTO_CHECK_ARG(t[7].dtype == PTO_HIP_FP32 && t[8].dtype == PTO_HIP_FP32 && numel(t[7]) == pool_blocks * hkv &&
+                    numel(t[8]) == pool_blocks * hkv,
+                "rope_kv_cache_update_fp8: k_scale/v_scale must be FP32 [pool_blocks, Hkv]");
+  PTO_CHECK_ARG((t[9].dtype == PTO_HIP_BF16 || t[9].dtype == PTO_HIP_FP16) && numel(t[9]) == batch * hq * d,
+                "rope_kv_cache_update_fp8: q_out must be BF16 or FP16 [B*Hq, D]");
+  return pto_hip_rope_kv_cache_update_fp8(
+      reinterpret_cast<const float*>(tptr(t[0])), reinterpret_cast<const int32_t*>(tptr(t[1])),
+      reinterpret_cast<const float*>(tptr(t[2])), reinterpret_cast<const float*>(tptr(t[3])),
+      reinterpret_cast<const int32_t*>(tptr(t[4])), tptr_mut(t[5]), tptr_mut(t[6]),
+      reinterpret_cast<float*>(tptr_mut(t[7])), reinterpret_cast<float*>(tptr_mut(t[8])), tptr_mut(t[9]), batch, hq,
+      hkv, d, bs, batch ? numel(t[4]) / batch : 1, numel(t[2]) / (d / 2), pool_blocks, (int)t[9].dtype, stream);
+}
+
 int run_rope_kv(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream) {
   PTO_CHECK_ARG(nt == 8 && ns == 4,
                 "rope_kv_cache_update: expected qkv, seq_lens, rope_cos, rope_sin, block_table, key_cache, "
@@ -415,6 +455,7 @@ int dispatch(int kind, const PtoHipChipTensor* t, int nt, const uint64_t* s, int
     case kW8a16Matmul: return run_w8a16_matmul(t, nt, s, ns, stream);
     case kW8a16Swiglu: return run_w8a16_swiglu(t, nt, s, ns, stream);
     case kRopeKvCacheUpdate: return run_rope_kv(t, nt, s, ns, stream);
+    case kRopeKvCacheUpdateFp8: return run_rope_kv_fp8(t, nt, s, ns, stream);
     case kDecoderLayerDecode: return run_decoder_layer(t, nt, s, ns, stream);
     default: return fail(PTO_HIP_ERR_NOT_FOUND, "unknown program kind %d", kind);
   }

@@ -75,12 +75,16 @@ w8a16_swiglu = HipProgram("w8a16_swiglu", (IN, IN, IN, IN, IN, OUT))
 rope_kv_cache_update = HipProgram(
     "rope_kv_cache_update", (IN, IN, IN, IN, IN, INOUT, INOUT, OUT),
     scalars=("num_heads", "kv_head_num", "head_dim", "block_size"))
+rope_kv_cache_update_fp8 = HipProgram(
+    "rope_kv_cache_update_fp8", (IN, IN, IN, IN, IN, INOUT, INOUT, INOUT, INOUT, OUT),
+    scalars=("num_heads", "kv_head_num", "head_dim", "block_size"))
 decoder_layer_decode = HipProgram(
     "decoder_layer_decode", (IN, IN, IN, INOUT, INOUT) + (IN,) * 14 + (OUT,),
     scalars=("num_heads", "kv_head_num", "head_dim", "block_size", "eps"))
 
 PROGRAMS = {p.name: p for p in (paged_attention, paged_gather, rms_norm, ffn_swiglu, ffn_block, w8a16_matmul,
-                                w8a16_swiglu, rope_kv_cache_update, decoder_layer_decode)}
+                                w8a16_swiglu, rope_kv_cache_update, rope_kv_cache_update_fp8,
+                                decoder_layer_decode)}
 
 
 @dataclass

@@ -5,7 +5,8 @@ import torch
 
 import oracle
 from pypto_amd import workloads
-from pypto_amd.runtime import (decoder_layer_decode, rope_kv_cache_update, validate_golden, w8a16_matmul,
+from pypto_amd.runtime import (decoder_layer_decode, rope_kv_cache_update, rope_kv_cache_update_fp8,
+                               validate_golden, w8a16_matmul,
                                w8a16_matmul_residual, w8a16_swiglu)
 
 pytestmark = pytest.mark.gpu
@@ -100,6 +101,73 @@ def test_rope_position_out_of_range_is_reported(worker):
         with worker.register(rope_kv_cache_update) as h:
             h(qkv, bad, inp.rope_cos, inp.rope_sin, inp.block_table, inp.key_cache.clone(), inp.value_cache.clone(),
               q_out, 2, 1, 128, 16)
+
+
+def _fp8_append_case(seq, bs, seed, grow=1.0):
+    b, hq, hkv, d = len(seq), 4, 2, 128
+    inp = workloads.decoder_layer_inputs(batch=b, hidden=256, num_heads=hq, kv_head_num=hkv, head_dim=d,
+                                         intermediate=512, block_size=bs, context_lens=seq, seed=seed)
+    pool_blocks = inp.key_cache.shape[0] // (hkv * bs)
+    kc, ks = oracle.quantize_kv_fp8(inp.key_cache, pool_blocks, hkv, bs)
+    vc, vs = oracle.quantize_kv_fp8(inp.value_cache, pool_blocks, hkv, bs)
+    g = torch.Generator().manual_seed(seed + 1)
+    qkv = torch.randn(b, (hq + 2 * hkv) * d, generator=g) * grow
+    return inp, qkv, kc, ks, vc, vs, (b, hq, hkv, d)
+
+
+@pytest.mark.parametrize("seq,bs,grow", [([17, 1, 40, 16], 16, 1.0), ([33, 64, 65], 32, 8.0), ([5, 128], 128, 0.01)])
+def test_rope_kv_cache_update_fp8(worker, seq, bs, grow):
+    """Quantise-on-write: V rows (no rotation) bit-exact against the oracle, scales exact, K rows
+    within one e4m3 step (the rotation's fp32 products may fuse differently), rest untouched."""
+    inp, qkv, kc, ks, vc, vs, (b, hq, hkv, d) = _fp8_append_case(seq, bs, seed=21, grow=grow)
+    kc_d, ks_d, vc_d, vs_d = kc.clone(), ks.clone(), vc.clone(), vs.clone()
+    q_out = torch.zeros(b * hq, d, dtype=torch.bfloat16)
+    with worker.register(rope_kv_cache_update_fp8) as h:
+        h(qkv, inp.seq_lens, inp.rope_cos, inp.rope_sin, inp.block_table, kc_d, vc_d, ks_d, vs_d, q_out, hq, hkv, d, bs)
+    pos = torch.tensor(seq) - 1
+    cos, sin = inp.rope_cos[pos].unsqueeze(1), inp.rope_sin[pos].unsqueeze(1)
+    q = oracle.rope_rotate_half(qkv[:, :hq * d].reshape(b, hq, d), cos, sin).to(torch.bfloat16)
+    k = oracle.rope_rotate_half(qkv[:, hq * d:(hq + hkv) * d].reshape(b, hkv, d), cos, sin)
+    v = qkv[:, (hq + hkv) * d:].reshape(b, hkv, d)
+    table = inp.block_table.reshape(b, -1)
+    blocks = [int(table[i, int(pos[i]) // bs]) for i in range(b)]
+    tokens = [int(pos[i]) % bs for i in range(b)]
+    ref_vc, ref_vs = oracle.kv_append_fp8(vc, vs, v, blocks, tokens, bs)
+    ref_kc, ref_ks = oracle.kv_append_fp8(kc, ks, k, blocks, tokens, bs)
+    assert torch.allclose(q_out.float(), q.reshape(-1, d).float(), atol=2e-2, rtol=1e-2)
+    assert torch.equal(vs_d, ref_vs)
+    assert torch.equal(vc_d.view(torch.uint8), ref_vc.view(torch.uint8))
+    assert torch.allclose(ks_d, ref_ks, rtol=1e-6)
+    got_k = oracle.dequant_kv_fp8(kc_d, ks_d, bs)
+    want_k = oracle.dequant_kv_fp8(ref_kc, ref_ks, bs)
+    step = ref_ks.max() * 32.0  # largest e4m3 step (between 416 and 448) in value units
+    assert ((got_k - want_k).abs() <= step).all()
+    assert (kc_d.view(torch.uint8) != ref_kc.view(torch.uint8)).float().mean() < 1e-3
+    # blocks that received no token keep codes and scales
+    untouched = torch.ones(ks.shape[0], dtype=torch.bool)
+    untouched[blocks] = False
+    assert torch.equal(ks_d[untouched], ks[untouched]) and torch.equal(vs_d[untouched], vs[untouched])
+    rows = untouched.repeat_interleave(hkv * bs)
+    assert torch.equal(vc_d.view(torch.uint8)[rows], vc.view(torch.uint8)[rows])
+
+
+def test_fp8_append_then_attention_matches_bf16_path(worker):
+    """The appended token is visible to the e4m3 attention path: decode over the updated cache
+    agrees with the oracle's attention on the oracle-updated cache."""
+    from pypto_amd.runtime import paged_attention
+    seq, bs = [70, 33, 128], 32
+    inp, qkv, kc, ks, vc, vs, (b, hq, hkv, d) = _fp8_append_case(seq, bs, seed=31)
+    q_out = torch.zeros(b * hq, d, dtype=torch.bfloat16)
+    with worker.register(rope_kv_cache_update_fp8) as h:
+        h(qkv, inp.seq_lens, inp.rope_cos, inp.rope_sin, inp.block_table, kc, vc, ks, vs, q_out, hq, hkv, d, bs)
+    max_blocks = inp.block_table.numel() // b
+    config = torch.tensor([b, hq, hkv, d, bs, max_blocks, oracle.attention.encode_scale(1.0 / d ** 0.5)],
+                          dtype=torch.int64)
+    out = torch.zeros(b * hq, d)
+    with worker.register(paged_attention) as h:
+        h(q_out, kc, vc, inp.block_table, inp.seq_lens, out, config, ks, vs)
+    ref = oracle.paged_attention_golden(q_out, kc, vc, inp.block_table, inp.seq_lens, config, ks, vs)
+    validate_golden({"out": out}, {"out": ref}, rtol=2e-2, atol=1e-2)
 
 
 def _oracle_layer(inp):

@@ -91,3 +91,41 @@ def test_w8a16_closed_form():
     ref = (x.double() @ wq.double()) * s.double()
     assert torch.allclose(y.double(), ref, atol=1e-5, rtol=1e-5)
     assert torch.allclose(y, x.float() @ w, atol=2e-2)
+
+
+def test_kv_append_fp8_properties():
+    """Pins of the quantise-on-write oracle that do not restate its formula."""
+    torch.manual_seed(0)
+    bs, d, kv = 8, 16, 2
+    rows = torch.randn(bs, 1, kv, d)
+    # (1) If the first row holds the block's maximum, the scale never changes and appending the
+    # rows one by one gives exactly the codes of quantising the finished block in one go.
+    rows[0, 0, :, 0] = 10.0
+    codes = torch.zeros(4 * kv * bs, d).to(torch.float8_e4m3fn)
+    codes[:] = torch.tensor(3.0).to(torch.float8_e4m3fn)  # stale content must not matter
+    scale = torch.full((4, kv), 123.0)
+    for t in range(bs):
+        codes, scale = oracle.kv_append_fp8(codes, scale, rows[t], [2], [t], bs)
+    block = rows[:, 0].permute(1, 0, 2).reshape(kv * bs, d)  # [Hkv*bs, D] of block 2
+    full = torch.zeros(4 * kv * bs, d)
+    full[2 * kv * bs:3 * kv * bs] = block
+    ref_codes, ref_scale = oracle.quantize_kv_fp8(full, 4, kv, bs)
+    got = codes.view(torch.uint8).reshape(4, kv * bs, d)[2]
+    want = ref_codes.view(torch.uint8).reshape(4, kv * bs, d)[2]
+    assert torch.equal(got, want)
+    assert torch.equal(scale[2], ref_scale[2])
+    # other blocks untouched
+    assert (codes.view(torch.uint8).reshape(4, -1)[[0, 1, 3]] == torch.tensor(3.0).to(torch.float8_e4m3fn).view(torch.uint8)).all()
+    # (2) Growing rows: the scale is the running amax/448 and every stored value stays within half
+    # an e4m3 step (2^-4 relative) per re-coding of the true value.
+    codes = torch.zeros(kv * bs, d).to(torch.float8_e4m3fn)
+    scale = torch.ones(1, kv)
+    grow = torch.randn(bs, 1, kv, d) * torch.arange(1, bs + 1).reshape(bs, 1, 1, 1)
+    for t in range(bs):
+        codes, scale = oracle.kv_append_fp8(codes, scale, grow[t], [0], [t], bs)
+        amax = grow[:t + 1, 0].abs().amax(dim=(0, 2))
+        assert torch.allclose(scale[0], amax / 448.0, rtol=1e-6)
+    deq = oracle.dequant_kv_fp8(codes, scale, bs).reshape(kv, bs, d)
+    true = grow[:, 0].permute(1, 0, 2)
+    bound = (bs * 2.0 ** -4) * true.abs() + (scale[0].reshape(kv, 1, 1) * 2.0 ** -9) * bs
+    assert ((deq - true).abs() <= bound).all()
