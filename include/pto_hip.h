@@ -136,6 +136,7 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *      tensors: hidden_states[B,H], seq_lens, block_table, key_cache (INOUT), value_cache (INOUT),
  *               rope_cos, rope_sin, gamma_in[H], gamma_post[H], wqkv_q, wqkv_s, wo_q, wo_s, wg_q, wg_s,
  *               wu_q, wu_s, wd_q, wd_s, out[B,H]
+ *               (FP8E4M3FN caches: k_scale, v_scale [pool,Hkv] fp32 (INOUT) follow value_cache)
  *      scalars: num_heads, kv_head_num, head_dim, block_size, eps (f32 bits)
  */
 PTO_HIP_API int pto_hip_register(const char* program_name, int* callable_id);
@@ -225,7 +226,8 @@ PTO_HIP_API int pto_hip_rope_kv_cache_update_fp8(const float* qkv, const int32_t
 
 /* One decoder layer, one new token per sequence (examples/models/qwen3_jit/qwen3_decode.py:47-113):
  * RMSNorm -> QKV -> RoPE + K/V append -> paged attention -> o_proj + residual -> RMSNorm ->
- * SwiGLU FFN + residual.  Projection weights are INT8 [in, out] with FP32 per-output scales. */
+ * SwiGLU FFN + residual.  Projection weights are INT8 [in, out] with FP32 per-output scales.
+ * With e4m3 caches pool_rows is still the row count of each cache (pool_blocks * Hkv * block_size). */
 typedef struct PtoHipDecoderLayerArgs {
   const void* hidden_states;  /* [B, H] dtype */
   const int32_t* seq_lens;    /* [B] context length including the new token */
@@ -251,6 +253,10 @@ typedef struct PtoHipDecoderLayerArgs {
   int64_t block_size, max_num_blocks_per_req, max_pos, pool_rows;
   float eps;
   int32_t dtype;              /* PTO_HIP_BF16 or PTO_HIP_FP16 */
+  int32_t kv_dtype;           /* 0 = caches hold `dtype`; PTO_HIP_FP8E4M3FN = e4m3 caches, quantised on write */
+  int32_t reserved;
+  float* k_scale;             /* [pool_blocks, Hkv] FP32, updated in place (e4m3 caches only) */
+  float* v_scale;
 } PtoHipDecoderLayerArgs;
 PTO_HIP_API int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* args, void* stream);
 

@@ -104,7 +104,7 @@ def decoder_layer_decode(
     rope_cos, rope_sin, gamma_in, gamma_post,
     wqkv_q, wqkv_s, wo_q, wo_s, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s,
     *, num_heads: int, kv_head_num: int, head_dim: int, block_size: int,
-    max_num_blocks_per_req: int, eps: float = 1e-6,
+    max_num_blocks_per_req: int, eps: float = 1e-6, k_scale=None, v_scale=None,
 ):
     """One LLaMA-style decoder layer, one new token per sequence.
 
@@ -114,7 +114,11 @@ def decoder_layer_decode(
     + residual (test_qwen3_decode_scope3_mixed.py:255-287).  Activations are
     rounded to the activation dtype wherever the model path casts.
 
-    Returns (out [B, H] act dtype, key_cache, value_cache) — caches are updated copies.
+    With float8_e4m3fn caches (``k_scale``/``v_scale`` [pool_blocks, Hkv] given) the new rows
+    are quantised on write (``kv_append_fp8``) from their fp32 values.
+
+    Returns (out [B, H] act dtype, key_cache, value_cache) — caches are updated copies — and,
+    for e4m3 caches, the updated (k_scale, v_scale) as two more elements.
     """
     act = hidden.dtype
     b, h = hidden.shape
@@ -132,23 +136,30 @@ def decoder_layer_decode(
     cos = rope_cos[pos].unsqueeze(1)  # [B, 1, D/2]
     sin = rope_sin[pos].unsqueeze(1)
     q = rope_rotate_half(q, cos, sin).to(act)
-    k = rope_rotate_half(k, cos, sin).to(act)
-    v = v.to(act)
-
     table = block_table.reshape(b, max_num_blocks_per_req).long()
-    for bi in range(b):
-        p = int(pos[bi])
-        blk = int(table[bi, p // bs])
-        for hh in range(kv):
-            row = (blk * kv + hh) * bs + p % bs
-            key_cache[row] = k[bi, hh]
-            value_cache[row] = v[bi, hh]
+    fp8 = key_cache.dtype == torch.float8_e4m3fn
+    if fp8:
+        blocks = [int(table[bi, int(pos[bi]) // bs]) for bi in range(b)]
+        tokens = [int(pos[bi]) % bs for bi in range(b)]
+        key_cache, k_scale = kv_append_fp8(key_cache, k_scale, rope_rotate_half(k, cos, sin), blocks, tokens, bs)
+        value_cache, v_scale = kv_append_fp8(value_cache, v_scale, v.float(), blocks, tokens, bs)
+    else:
+        k = rope_rotate_half(k, cos, sin).to(act)
+        v = v.to(act)
+        for bi in range(b):
+            p = int(pos[bi])
+            blk = int(table[bi, p // bs])
+            for hh in range(kv):
+                row = (blk * kv + hh) * bs + p % bs
+                key_cache[row] = k[bi, hh]
+                value_cache[row] = v[bi, hh]
 
     config = torch.tensor(
         [b, hq, kv, d, bs, max_num_blocks_per_req, encode_scale(1.0 / (d ** 0.5))], dtype=torch.int64
     )
     attn = paged_attention_golden(
-        q.reshape(b * hq, d), key_cache, value_cache, block_table, seq_lens, config
+        q.reshape(b * hq, d), key_cache, value_cache, block_table, seq_lens, config,
+        k_scale if fp8 else None, v_scale if fp8 else None,
     ).reshape(b, hq * d).to(act)
 
     resid1 = w8a16_matmul(attn, wo_q, wo_s) + hidden.float()
@@ -158,4 +169,6 @@ def decoder_layer_decode(
     mlp = swiglu(gate, up).to(act)
     down = w8a16_matmul(mlp, wd_q, wd_s)
     out = (down + resid1).to(act)
+    if fp8:
+        return out, key_cache, value_cache, k_scale, v_scale
     return out, key_cache, value_cache

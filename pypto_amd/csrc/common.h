@@ -95,6 +95,12 @@ int rope_kv_cache_update(const float* qkv, const float* qkv_scale, int splits, i
                          int64_t batch, int64_t num_heads, int64_t kv_head_num, int64_t head_dim,
                          int64_t block_size, int64_t max_num_blocks_per_req, int64_t max_pos,
                          int64_t pool_rows, int dtype, void* stream);
+int rope_kv_cache_update_fp8(const float* qkv, const float* qkv_scale, int splits, int64_t split_stride,
+                             const int32_t* seq_lens, const float* rope_cos, const float* rope_sin,
+                             const int32_t* block_table, void* key_cache, void* value_cache, float* k_scale,
+                             float* v_scale, void* q_out, int64_t batch, int64_t num_heads, int64_t kv_head_num,
+                             int64_t head_dim, int64_t block_size, int64_t max_num_blocks_per_req,
+                             int64_t max_pos, int64_t pool_blocks, int q_dtype, void* stream);
 int cast_from_f32(const float* in, void* out, size_t n, int out_dtype, hipStream_t st);
 // pto_hip_paged_attention with an optional second output: the result rounded to the query dtype.
 int paged_attention(const void* query, const void* key_cache, const void* value_cache,

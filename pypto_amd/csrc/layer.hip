@@ -26,6 +26,11 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
                 "decoder_layer_decode: bad model dimensions");
   PTO_CHECK_ARG(a->dtype == PTO_HIP_BF16 || a->dtype == PTO_HIP_FP16,
                 "decoder_layer_decode: activation dtype %s not in {BF16, FP16}", dtype_name(a->dtype));
+  const bool fp8kv = a->kv_dtype == PTO_HIP_FP8E4M3FN;
+  PTO_CHECK_ARG(a->kv_dtype == 0 || a->kv_dtype == a->dtype || fp8kv,
+                "decoder_layer_decode: cache dtype %s must be the activation dtype or FP8E4M3FN",
+                dtype_name(a->kv_dtype));
+  PTO_CHECK_ARG(!fp8kv || (a->k_scale && a->v_scale), "decoder_layer_decode: e4m3 caches need k_scale and v_scale");
   PTO_CHECK_ARG(a->hidden_states && a->out && a->seq_lens && a->block_table && a->key_cache && a->value_cache &&
                     a->rope_cos && a->rope_sin && a->gamma_in && a->gamma_post && a->wqkv_q && a->wqkv_s &&
                     a->wo_q && a->wo_s && a->wg_q && a->wg_s && a->wu_q && a->wu_s && a->wd_q && a->wd_s,
@@ -65,18 +70,26 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
   // 2. QKV projection, left as k-split partial sums
   if ((rc = w8a16_partials(normed, a->wqkv_q, nullptr, b, h, qkv_n, dt, st, &parts))) return rc;
   // 3. finish of the projection + RoPE at pos = seq_len - 1, append K/V, rotated Q
-  if ((rc = rope_kv_cache_update(parts.part[0], a->wqkv_s, parts.splits, (int64_t)kW8MaxM * qkv_n, a->seq_lens,
-                                 a->rope_cos, a->rope_sin, a->block_table, a->key_cache, a->value_cache, q16, b,
-                                 hq, hkv, d, a->block_size, a->max_num_blocks_per_req, a->max_pos, a->pool_rows,
-                                 dt, stream)))
-    return rc;
+  if (fp8kv) {
+    const int64_t pool_blocks = a->pool_rows / (hkv * a->block_size);
+    rc = rope_kv_cache_update_fp8(parts.part[0], a->wqkv_s, parts.splits, (int64_t)kW8MaxM * qkv_n, a->seq_lens,
+                                  a->rope_cos, a->rope_sin, a->block_table, a->key_cache, a->value_cache, a->k_scale,
+                                  a->v_scale, q16, b, hq, hkv, d, a->block_size, a->max_num_blocks_per_req,
+                                  a->max_pos, pool_blocks, dt, stream);
+  } else {
+    rc = rope_kv_cache_update(parts.part[0], a->wqkv_s, parts.splits, (int64_t)kW8MaxM * qkv_n, a->seq_lens,
+                              a->rope_cos, a->rope_sin, a->block_table, a->key_cache, a->value_cache, q16, b, hq,
+                              hkv, d, a->block_size, a->max_num_blocks_per_req, a->max_pos, a->pool_rows, dt, stream);
+  }
+  if (rc) return rc;
   // 4. paged attention over seq_len tokens (including the one just written)
   float scale = 1.0f / sqrtf((float)d);
   uint32_t scale_bits;
   __builtin_memcpy(&scale_bits, &scale, 4);
   const int64_t cfg[7] = {b, hq, hkv, d, a->block_size, a->max_num_blocks_per_req, (int64_t)scale_bits};
-  if ((rc = paged_attention(q16, a->key_cache, a->value_cache, a->block_table, a->seq_lens, attn, attn16, cfg, dt, dt,
-                            nullptr, nullptr, stream)))
+  if ((rc = paged_attention(q16, a->key_cache, a->value_cache, a->block_table, a->seq_lens, attn, attn16, cfg, dt,
+                            fp8kv ? PTO_HIP_FP8E4M3FN : dt, fp8kv ? a->k_scale : nullptr,
+                            fp8kv ? a->v_scale : nullptr, stream)))
     return rc;
   // 5. o_proj; 6. its finish + residual -> fp32, post-attention RMSNorm -> activation dtype
   if ((rc = w8a16_partials(attn16, a->wo_q, nullptr, b, hq * d, h, dt, st, &parts))) return rc;

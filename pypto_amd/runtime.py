@@ -82,6 +82,11 @@ decoder_layer_decode = HipProgram(
     "decoder_layer_decode", (IN, IN, IN, INOUT, INOUT) + (IN,) * 14 + (OUT,),
     scalars=("num_heads", "kv_head_num", "head_dim", "block_size", "eps"))
 
+# the same layer over FP8E4M3FN caches: k_scale, v_scale follow value_cache
+decoder_layer_decode_fp8kv = HipProgram(
+    "decoder_layer_decode", (IN, IN, IN, INOUT, INOUT, INOUT, INOUT) + (IN,) * 14 + (OUT,),
+    scalars=("num_heads", "kv_head_num", "head_dim", "block_size", "eps"))
+
 PROGRAMS = {p.name: p for p in (paged_attention, paged_gather, rms_norm, ffn_swiglu, ffn_block, w8a16_matmul,
                                 w8a16_swiglu, rope_kv_cache_update, rope_kv_cache_update_fp8,
                                 decoder_layer_decode)}

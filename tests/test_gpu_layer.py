@@ -5,7 +5,7 @@ import torch
 
 import oracle
 from pypto_amd import workloads
-from pypto_amd.runtime import (decoder_layer_decode, rope_kv_cache_update, rope_kv_cache_update_fp8,
+from pypto_amd.runtime import (decoder_layer_decode, decoder_layer_decode_fp8kv, rope_kv_cache_update, rope_kv_cache_update_fp8,
                                validate_golden, w8a16_matmul,
                                w8a16_matmul_residual, w8a16_swiglu)
 
@@ -199,3 +199,30 @@ def test_decoder_layer_decode(worker, batch, ctxs):
     assert torch.allclose(inp.value_cache.float(), ref_v.float(), atol=2e-2, rtol=1e-2)
     changed = (inp.key_cache != kc0).any(dim=1).sum().item()
     assert changed <= batch * 2
+
+
+def test_decoder_layer_decode_fp8_kv(worker):
+    """The same reduced layer over e4m3 caches: rows quantised on write, attention dequantises."""
+    batch = 6
+    ctxs = [100, 1, 257, 33, 128, 129]
+    inp = workloads.decoder_layer_inputs(batch=batch, hidden=1024, num_heads=8, kv_head_num=2, head_dim=128,
+                                         intermediate=2816, block_size=128, context_lens=ctxs, seed=8)
+    pool_blocks = inp.key_cache.shape[0] // (2 * 128)
+    kc, ks = oracle.quantize_kv_fp8(inp.key_cache, pool_blocks, 2, 128)
+    vc, vs = oracle.quantize_kv_fp8(inp.value_cache, pool_blocks, 2, 128)
+    w = inp.weights
+    ref_out, ref_k, ref_v, ref_ks, ref_vs = oracle.decoder_layer_decode(
+        inp.hidden, inp.seq_lens, inp.block_table, kc, vc, inp.rope_cos, inp.rope_sin,
+        inp.gamma_in, inp.gamma_post, *w["qkv"], *w["o"], *w["gate"], *w["up"], *w["down"],
+        num_heads=inp.num_heads, kv_head_num=inp.kv_head_num, head_dim=inp.head_dim, block_size=inp.block_size,
+        max_num_blocks_per_req=inp.max_num_blocks_per_req, eps=inp.eps, k_scale=ks, v_scale=vs)
+    kc_d, vc_d, ks_d, vs_d = kc.clone(), vc.clone(), ks.clone(), vs.clone()
+    args = list(inp.args())
+    args[3:5] = [kc_d, vc_d, ks_d, vs_d]
+    with worker.register(decoder_layer_decode_fp8kv) as h:
+        h(*args)
+    validate_golden({"out": inp.out.float()}, {"out": ref_out.float()}, rtol=2e-2, atol=2e-2)
+    assert torch.allclose(ks_d, ref_ks, rtol=1e-2) and torch.allclose(vs_d, ref_vs, rtol=1e-2)
+    got = oracle.dequant_kv_fp8(vc_d, vs_d, 128)
+    want = oracle.dequant_kv_fp8(ref_v, ref_vs, 128)
+    assert ((got - want).abs() <= ref_vs.max() * 32.0 + 1e-6).all()
