@@ -260,6 +260,27 @@ typedef struct PtoHipDecoderLayerArgs {
 } PtoHipDecoderLayerArgs;
 PTO_HIP_API int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* args, void* stream);
 
+/* ---- manifest -> program ------------------------------------------------------------------
+ * The reference describes a compiled program by a kernel_config.py manifest (ORCHESTRATION +
+ * KERNELS[{func_id, name, core_type, signature}], python/pypto/backend/pto_backend.py:933-1045)
+ * and runs it by compiling every kernel (python/pypto/runtime/device_runner.py:505-664).  Here a
+ * recognised manifest maps to one fused program name for pto_hip_register: the 4-kernel
+ * paged-attention set (qk_matmul/pv_matmul on aic, softmax_prepare/online_update and the optional
+ * init_inplace on aiv), the
+ * matmul + swiglu FFN chain, a single rms_norm kernel, paged_gather.  orch_dirs may be null when
+ * the manifest carries no signature.  PTO_HIP_ERR_NOT_FOUND when nothing matches.  Needs no
+ * device: callable before pto_hip_init.  *program_name points at a static string. */
+enum { PTO_HIP_CORE_AIC = 0, PTO_HIP_CORE_AIV = 1 };
+enum { PTO_HIP_DIR_IN = 0, PTO_HIP_DIR_OUT = 1, PTO_HIP_DIR_INOUT = 2 };
+typedef struct PtoHipManifestKernel {
+  int32_t func_id;
+  int32_t core_type;  /* PTO_HIP_CORE_AIC / PTO_HIP_CORE_AIV */
+  const char* name;
+} PtoHipManifestKernel;
+PTO_HIP_API int pto_hip_select_program(const char* orchestration_name, const PtoHipManifestKernel* kernels,
+                                       int32_t n_kernels, const int32_t* orch_dirs, int32_t n_orch_tensors,
+                                       const char** program_name);
+
 /* ---- tuning knobs (integers by name; unknown names are PTO_HIP_ERR_NOT_FOUND) ------------
  *  "attn_tokens_per_partition"  0 = choose from the device's CU count (default)
  *  "attn_waves_per_cu"          cap on resident attention wavefronts per CU, 0 = none (default)

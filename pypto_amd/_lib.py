@@ -24,7 +24,7 @@ EXPORTS = (
     "pto_hip_ffn_swiglu", "pto_hip_set_option", "pto_hip_get_option",
     "pto_hip_w8a16_matmul", "pto_hip_w8a16_swiglu", "pto_hip_rope_kv_cache_update",
     "pto_hip_rope_kv_cache_update_fp8",
-    "pto_hip_decoder_layer_decode",
+    "pto_hip_decoder_layer_decode", "pto_hip_select_program",
 )
 
 
@@ -41,6 +41,10 @@ class ChipTensor(C.Structure):
         ("dtype", C.c_uint32),
         ("reserved", C.c_uint32),
     ]
+
+
+class ManifestKernel(C.Structure):
+    _fields_ = [("func_id", C.c_int32), ("core_type", C.c_int32), ("name", C.c_char_p)]
 
 
 class DeviceInfo(C.Structure):
@@ -96,6 +100,8 @@ def load() -> C.CDLL:
                                          C.c_int, vp],
         "pto_hip_rope_kv_cache_update_fp8": [vp] * 10 + [i64] * 8 + [C.c_int, vp],
         "pto_hip_decoder_layer_decode": [vp, vp],
+        "pto_hip_select_program": [C.c_char_p, C.POINTER(ManifestKernel), C.c_int32, C.POINTER(C.c_int32),
+                                   C.c_int32, C.POINTER(C.c_char_p)],
         "pto_hip_set_option": [C.c_char_p, i64],
         "pto_hip_get_option": [C.c_char_p, C.POINTER(i64)],
     }
