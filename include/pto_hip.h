@@ -283,12 +283,13 @@ PTO_HIP_API int pto_hip_select_program(const char* orchestration_name, const Pto
 
 /* ---- tuning knobs (integers by name; unknown names are PTO_HIP_ERR_NOT_FOUND) ------------
  *  "attn_tokens_per_partition"  0 = choose from the device's CU count (default)
- *  "attn_waves_per_cu"          cap on resident attention wavefronts per CU, 0 = none (default)
+ *  "attn_waves_per_cu"          cap on resident attention wavefronts per CU, 0 = none (default); for
+ *                               the evenly split form the wavefronts per CU (0 = 4, at most 8)
  *  "attn_skip_merge"            1 = launch only the streaming attention kernel and leave the
  *                               partition partials unmerged (kernel timing aid; output invalid)
- *  "attn_variant"               0 = one wavefront per (sequence, KV head, partition) (default),
- *                               1 = one pinned workgroup per CU over a balanced list of those
- *                               items (head_dim 128 only)
+ *  "attn_variant"               0 = one wavefront per (sequence, KV head, partition), 1 = one pinned
+ *                               workgroup per CU and the chunk list cut evenly over their wavefronts,
+ *                               -1 = by launch size (default)
  *  "gemm_variant"               FFN GEMM tiling: 0 = default choice, 1..3 = fixed alternatives
  *  "w8a16_wgs_per_cu"           workgroups per CU the W8A16 k split aims at (default 2)
  *  "w8a16_min_steps"            fewest 32-row steps per wavefront before k is split further

@@ -52,7 +52,7 @@ struct Context {
   // options
   int64_t attn_tokens_per_partition = 0;
   int64_t attn_waves_per_cu = 0;
-  int64_t attn_variant = 0;  // 0 partition grid, 1 balanced form (head_dim 128)
+  int64_t attn_variant = -1;  // -1 by launch size, 0 partition grid, 1 evenly split form
   int64_t attn_skip_merge = 0;
   int64_t gemm_variant = 0;
   int64_t w8a16_wgs_per_cu = 2;  // workgroups of the W8A16 partial kernel aimed at per compute unit

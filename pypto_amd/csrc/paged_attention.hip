@@ -15,6 +15,8 @@
 //   * the query group of a KV head (padded to 16 rows) stays in registers as B operand.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include <type_traits>
 
 #include "common.h"
@@ -44,7 +46,8 @@ struct AttnParams {
   const float* k_scale;  // [pool_blocks, Hkv] for an e4m3 cache, else null
   const float* v_scale;
   int batch, hq, hkv, group, gtiles, bs, max_blocks, tpp, n_part;
-  int n_wg;  // streaming form: resident workgroups (one per CU)
+  int n_wg;        // evenly split form: resident workgroups (one per CU); 0 = partition grid
+  int lean_waves;  // ... and wavefronts in each
   float scale_log2e;
 };
 
@@ -185,6 +188,117 @@ __device__ __forceinline__ u32x4 fp8x8_to_bf16x8(uint32_t w0, uint32_t w1) {
                fp8x2_to_bf16x2(w1, true)};
 }
 
+// S^T = K Q^T for one chunk: two 16x16 tiles, rows = tokens, columns = query heads.
+template <int D, bool BF16, bool FP8>
+__device__ __forceinline__ void qk_scores(const KFrag<D, FP8>& kf, const u32x4 (&qf)[D / 32], f32x4& s0, f32x4& s1) {
+  s0 = f32x4{0.f, 0.f, 0.f, 0.f};
+  s1 = f32x4{0.f, 0.f, 0.f, 0.f};
+  if constexpr (FP8) {
+#pragma unroll
+    for (int s2 = 0; s2 < D / 64; ++s2) {
+      s0 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[0][s2][0], kf.t[0][s2][1]), qf[2 * s2], s0);
+      s1 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[1][s2][0], kf.t[1][s2][1]), qf[2 * s2], s1);
+      s0 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[0][s2][2], kf.t[0][s2][3]), qf[2 * s2 + 1], s0);
+      s1 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[1][s2][2], kf.t[1][s2][3]), qf[2 * s2 + 1], s1);
+    }
+  } else {
+#pragma unroll
+    for (int s = 0; s < D / 32; ++s) {
+      s0 = mfma16<BF16>(kf.t[0][s], qf[s], s0);
+      s1 = mfma16<BF16>(kf.t[1][s], qf[s], s1);
+    }
+  }
+}
+
+// Online softmax of one chunk's scores and O^T += V^T P^T.  vf holds the chunk's V rows (rows
+// past tok_end are zeroed here).
+template <int D, bool BF16, bool FP8>
+__device__ __forceinline__ void softmax_pv(f32x4 s0, f32x4 s1, VFrag<D, FP8>& vf, int tok, int tok_end, int j,
+                                           float k_mul, f32x4 (&acc)[D / 128][8], float& m_run, float& l_run) {
+  float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sv[e] *= k_mul;
+  const bool partial = tok + kChunk > tok_end;
+  if (partial) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int t = tok + (e >> 2) * 16 + j * 4 + (e & 3);
+      if (t >= tok_end) sv[e] = -INFINITY;
+    }
+  }
+
+  // ---- online softmax (column-wise: every lane of a column agrees on the maximum) ----
+  float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
+                   fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+  mx = fmaxf(mx, __shfl_xor(mx, 16));
+  mx = fmaxf(mx, __shfl_xor(mx, 32));
+  if (__builtin_amdgcn_ballot_w64(mx > m_run) != 0) {
+    // Some column's maximum grew: rescale the running sum and the accumulators.
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    m_run = m_new;
+    l_run *= alpha;
+#pragma unroll
+    for (int set = 0; set < D / 128; ++set)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[set][i] *= alpha;
+  }
+  u32x4 pf;
+  float psum = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e += 2) {
+    float ra, rb;
+    pf[e >> 1] = round_pack<BF16>(__builtin_amdgcn_exp2f(sv[e] - m_run),
+                                  __builtin_amdgcn_exp2f(sv[e + 1] - m_run), ra, rb);
+    psum += ra + rb;
+  }
+  l_run += psum;
+
+  if (partial) {
+    // Rows past the end may hold anything; keep them out of the PV product.
+#pragma unroll
+    for (int set = 0; set < D / 128; ++set)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int t = tok + (e >> 2) * 16 + j * 4 + (e & 3);
+        if (t >= tok_end) vf.t[set][e] = typename std::conditional<FP8, uint2, u32x4>::type{};
+      }
+  }
+
+  // ---- O^T += V^T P^T : transpose each lane's 8 tokens x 8 elements, then 8 MFMAs ----
+#pragma unroll
+  for (int set = 0; set < D / 128; ++set) {
+    u32x4 vw[8];  // the lane's 8 tokens x 8 elements as 16-bit values
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      if constexpr (FP8) vw[e] = fp8x8_to_bf16x8(vf.t[set][e].x, vf.t[set][e].y);
+      else vw[e] = vf.t[set][e];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
+      u32x4 vt;
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk)
+        vt[kk] = __builtin_amdgcn_perm(vw[2 * kk + 1][i >> 1], vw[2 * kk][i >> 1], sel);
+      acc[set][i] = mfma16<BF16>(vt, pf, acc[set][i]);
+    }
+  }
+}
+
+// Re-expresses the accumulators in another V scale (e4m3 cache, block change).
+template <int D>
+__device__ __forceinline__ void change_unit(f32x4 (&acc)[D / 128][8], float& v_unit, float v_next) {
+  if (v_next != v_unit) {
+    const float r = v_unit / v_next;
+#pragma unroll
+    for (int set = 0; set < D / 128; ++set)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[set][i] *= r;
+    v_unit = v_next;
+  }
+}
+
 // Attention of one query group (16 padded columns) over the chunks tok_first, tok_first +
 // tok_step, ... < tok_end of one (sequence, KV head): on return acc holds O^T in units of v_unit,
 // m_run the running maximum (log2 units) and l_run the row sum, both per column and already
@@ -229,6 +343,13 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
       win_ks = ok ? p.k_scale[(size_t)win_blk * p.hkv + h] : 1.f;
       win_vs = ok ? p.v_scale[(size_t)win_blk * p.hkv + h] : 1.f;
     }
+    if (!preloaded) {
+      // A refill inside the chunk loop sits on a rarely taken branch.  Consuming the loaded
+      // registers here keeps the wait for them on that branch; left to the first use after the
+      // branch rejoins, it would become a wait for every load in flight on every iteration.
+      asm volatile("" : "+v"(win_blk));
+      if constexpr (FP8) asm volatile("" : "+v"(win_ks), "+v"(win_vs));
+    }
   };
   load_window(tok_first / p.bs, true);
 
@@ -254,139 +375,49 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
   m_run = kMinMax;
   l_run = 0.f;
 
-  // Software pipeline: K of chunk n+1 is requested as soon as QK^T of chunk n has consumed
-  // the K registers, V of chunk n at the top of iteration n.  All loads are unconditional (the
-  // look-ahead past the last chunk re-reads the first tile, a cache hit) so that the number of
-  // requests in flight at each wait is known at compile time.
-  KFrag<D, FP8> kf;
-  VFrag<D, FP8> vf;
-  size_t o0 = tile_offset(tok_first + 16), o1 = o0;
-  o1 = o0;
-  o0 = tile_offset(tok_first);
-  // e4m3 cache: a chunk lies inside one block (block_size is a multiple of 32), whose two scales
-  // apply to the whole chunk.  The accumulators are kept in units of the current block's V
-  // scale, v_unit; they are converted when the block changes and once more at the end.
-  float k_mul = p.scale_log2e, v_next = 1.f, k_next = p.scale_log2e;
+  float k_mul = p.scale_log2e;
   v_unit = 1.f;
-  if constexpr (FP8) {
-    k_mul = p.scale_log2e * scale_k();
-    v_unit = scale_v();
-  }
-  load_k<D, FP8>(kf, kc + o0, kc + o1, lane);
-  load_v<D, FP8>(vf, vc + o0, vc + o1, voff);
-  stage_k<D, FP8>(kf, kbuf, lane);
-
-  for (int tok = tok_first; tok < tok_end; tok += tok_step) {
-    o1 = tile_offset(tok + tok_step + 16);
-    o0 = tile_offset(tok + tok_step);
+  {
+    // Software pipeline: K of chunk n+1 is requested as soon as QK^T of chunk n has consumed
+    // the K registers, V of chunk n+1 after PV of chunk n.  All loads are unconditional (the
+    // look-ahead past the last chunk re-reads the first tile, a cache hit) so that the number of
+    // requests in flight at each wait is known at compile time.
+    KFrag<D, FP8> kf;
+    VFrag<D, FP8> vf;
+    size_t o1 = tile_offset(tok_first + 16);
+    size_t o0 = tile_offset(tok_first);
+    // e4m3 cache: a chunk lies inside one block (block_size is a multiple of 32), whose two scales
+    // apply to the whole chunk.  The accumulators are kept in units of the current block's V
+    // scale, v_unit; they are converted when the block changes and once more at the end.
+    float v_next = 1.f, k_next = p.scale_log2e;
     if constexpr (FP8) {
-      k_next = p.scale_log2e * scale_k();
-      v_next = scale_v();
+      k_mul = p.scale_log2e * scale_k();
+      v_unit = scale_v();
     }
-
-    // ---- S^T = K Q^T : two 16x16 tiles, rows = tokens, columns = query heads ----
-    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-    fetch_k<D, FP8>(kf, kbuf, c, j);
-    if constexpr (FP8) {
-#pragma unroll
-      for (int s2 = 0; s2 < D / 64; ++s2) {
-        s0 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[0][s2][0], kf.t[0][s2][1]), qf[2 * s2], s0);
-        s1 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[1][s2][0], kf.t[1][s2][1]), qf[2 * s2], s1);
-        s0 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[0][s2][2], kf.t[0][s2][3]), qf[2 * s2 + 1], s0);
-        s1 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[1][s2][2], kf.t[1][s2][3]), qf[2 * s2 + 1], s1);
-      }
-    } else {
-#pragma unroll
-      for (int s = 0; s < D / 32; ++s) {
-        s0 = mfma16<BF16>(kf.t[0][s], qf[s], s0);
-        s1 = mfma16<BF16>(kf.t[1][s], qf[s], s1);
-      }
-    }
-    load_k<D, FP8>(kf, kc + o0, kc + o1, lane);  // next chunk, into the registers QK^T just released
-
-    float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
-#pragma unroll
-    for (int e = 0; e < 8; ++e) sv[e] *= k_mul;
-    const bool partial = tok + kChunk > tok_end;
-    if (partial) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int t = tok + (e >> 2) * 16 + j * 4 + (e & 3);
-        if (t >= tok_end) sv[e] = -INFINITY;
-      }
-    }
-
-    // ---- online softmax (column-wise: every lane of a column agrees on the maximum) ----
-    float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
-                     fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    if (__builtin_amdgcn_ballot_w64(mx > m_run) != 0) {
-      // Some column's maximum grew: rescale the running sum and the accumulators.
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-      m_run = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int set = 0; set < D / 128; ++set)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[set][i] *= alpha;
-    }
-    u32x4 pf;
-    float psum = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; e += 2) {
-      float ra, rb;
-      pf[e >> 1] = round_pack<BF16>(__builtin_amdgcn_exp2f(sv[e] - m_run),
-                                    __builtin_amdgcn_exp2f(sv[e + 1] - m_run), ra, rb);
-      psum += ra + rb;
-    }
-    l_run += psum;
-
-    if (partial) {
-      // Rows past the end may hold anything; keep them out of the PV product.
-#pragma unroll
-      for (int set = 0; set < D / 128; ++set)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int t = tok + (e >> 2) * 16 + j * 4 + (e & 3);
-          if (t >= tok_end) vf.t[set][e] = typename std::conditional<FP8, uint2, u32x4>::type{};
-        }
-    }
-
-    // ---- O^T += V^T P^T : transpose each lane's 8 tokens x 8 elements, then 8 MFMAs ----
-#pragma unroll
-    for (int set = 0; set < D / 128; ++set) {
-      u32x4 vw[8];  // the lane's 8 tokens x 8 elements as 16-bit values
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        if constexpr (FP8) vw[e] = fp8x8_to_bf16x8(vf.t[set][e].x, vf.t[set][e].y);
-        else vw[e] = vf.t[set][e];
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
-        u32x4 vt;
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk)
-          vt[kk] = __builtin_amdgcn_perm(vw[2 * kk + 1][i >> 1], vw[2 * kk][i >> 1], sel);
-        acc[set][i] = mfma16<BF16>(vt, pf, acc[set][i]);
-      }
-    }
-    if constexpr (FP8) {
-      // Next chunk may belong to another block: re-express the accumulators in its V scale.
-      if (v_next != v_unit) {
-        const float r = v_unit / v_next;
-#pragma unroll
-        for (int set = 0; set < D / 128; ++set)
-#pragma unroll
-          for (int i = 0; i < 8; ++i) acc[set][i] *= r;
-        v_unit = v_next;
-      }
-      k_mul = k_next;
-    }
-    load_v<D, FP8>(vf, vc + o0, vc + o1, voff);  // next chunk, into the registers PV just released
+    load_k<D, FP8>(kf, kc + o0, kc + o1, lane);
+    load_v<D, FP8>(vf, vc + o0, vc + o1, voff);
     stage_k<D, FP8>(kf, kbuf, lane);
+
+    for (int tok = tok_first; tok < tok_end; tok += tok_step) {
+      o1 = tile_offset(tok + tok_step + 16);
+      o0 = tile_offset(tok + tok_step);
+      if constexpr (FP8) {
+        k_next = p.scale_log2e * scale_k();
+        v_next = scale_v();
+      }
+      f32x4 s0, s1;
+      fetch_k<D, FP8>(kf, kbuf, c, j);
+      qk_scores<D, BF16, FP8>(kf, qf, s0, s1);
+      load_k<D, FP8>(kf, kc + o0, kc + o1, lane);  // next chunk, into the registers QK^T just released
+      softmax_pv<D, BF16, FP8>(s0, s1, vf, tok, tok_end, j, k_mul, acc, m_run, l_run);
+      if constexpr (FP8) {
+        // Next chunk may belong to another block: re-express the accumulators in its V scale.
+        change_unit<D>(acc, v_unit, v_next);
+        k_mul = k_next;
+      }
+      load_v<D, FP8>(vf, vc + o0, vc + o1, voff);  // next chunk, into the registers PV just released
+      stage_k<D, FP8>(kf, kbuf, lane);
+    }
   }
 
   // Row sum over the four k-groups of a column.
@@ -515,68 +546,105 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
 
 
 // ---------------------------------------------------------------------------------------------
-// Balanced form of the partition kernel.  Under HBM saturation every CU gets about the same
-// share of the bandwidth, so the launch lasts as long as the CU with the most bytes to fetch;
-// the hardware dispatcher, left alone, parks between 2 and 12 single-wavefront workgroups on a
-// CU.  Here one workgroup of kBalWaves wavefronts is pinned to each CU (its LDS use allows only
-// one) and the non-empty (sequence, KV head, query tile, partition) items, enumerated densely,
-// are dealt round-robin: item i goes to workgroup i mod n_wg.  Every CU then fetches the same
-// number of partitions, give or take one.  Partials and their merge are those of the
-// partition-grid kernel.
+// Evenly split form.  A launch of the partition grid lasts as long as its slowest wavefront: one
+// wavefront streams its partition with one or two chunks in flight, i.e. at a rate set by the
+// memory latency, partitions differ in length, and the hardware dispatcher parks between 2 and
+// 12 single-wavefront workgroups on a CU.  Here the work is cut by bytes instead: all
+// (sequence, KV head, query tile, 32-token chunk) items, in that order, form one list of N items,
+// one workgroup is pinned to every CU (its LDS request allows only one) and wavefront w of the
+// W_tot = min(resident wavefronts, N) participating ones takes the items c with
+// floor(c * W_tot / N) = w - a contiguous, non-empty run, equal to within one chunk for every wavefront.  A run that crosses into another (sequence, head)
+// ends one partial result and starts the next; the partial of wavefront w for pair q (q counting
+// (sequence, head, tile) triples) goes to slot q + w, which is unique, and the slots of one pair
+// are consecutive, so the merge kernel finds them from the same arithmetic.
 // ---------------------------------------------------------------------------------------------
-template <int D, bool BF16, bool FP8, int kBalWaves>
-__global__ __launch_bounds__(kBalWaves * 64) void attn_balanced_kernel(AttnParams p) {
-  __shared__ __attribute__((aligned(16))) char k_lds[kBalWaves][KStage<D, FP8>::kBytes];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+constexpr int kLeanMaxWaves = 8;
+
+__device__ __forceinline__ int seq_chunks(const AttnParams& p, int ctx) {
+  const int max_ctx = p.max_blocks * p.bs;
+  ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
+  return (ctx + kChunk - 1) / kChunk;
+}
+
+// Number of items of all sequences (wave-uniform).  lane i of pass b0 looks at sequence b0 + i.
+__device__ __forceinline__ long long lean_total(const AttnParams& p, int lane, int hg_count) {
+  long long total = 0;
+  for (int b0 = 0; b0 < p.batch; b0 += 64) {
+    long long n = (b0 + lane < p.batch) ? (long long)seq_chunks(p, p.ctx_lens[b0 + lane]) * hg_count : 0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) n += __shfl_xor(n, off);
+    total += n;
+  }
+  return total;
+}
+
+// Sequence holding item s (0 <= s < total): its index, the number of items before it and its
+// chunk count, all wave-uniform.
+__device__ __forceinline__ void lean_locate(const AttnParams& p, int lane, int hg_count, long long s, int& b,
+                                            long long& first_item, int& chunks) {
+  long long base = 0;
+  b = -1;
+  first_item = 0;
+  chunks = 0;
+  for (int b0 = 0; b0 < p.batch; b0 += 64) {
+    const int ch = (b0 + lane < p.batch) ? seq_chunks(p, p.ctx_lens[b0 + lane]) : 0;
+    const long long n = (long long)ch * hg_count;
+    long long incl = n;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const long long up = __shfl_up(incl, off);
+      if (lane >= off) incl += up;
+    }
+    const long long lo = base + incl - n;
+    const unsigned long long hit = __ballot(n > 0 && lo <= s && s < lo + n);
+    if (hit) {
+      const int src = __ffsll((long long)hit) - 1;
+      b = b0 + src;
+      first_item = __shfl(lo, src);
+      chunks = __shfl(ch, src);
+      return;
+    }
+    base += __shfl(incl, 63);
+  }
+}
+
+template <int D, bool BF16, bool FP8>
+__global__ __launch_bounds__(kLeanMaxWaves * 64) void attn_lean_kernel(AttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) char lean_lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, j = lane >> 4;
   const int hg_count = p.hkv * p.gtiles;
   const int max_ctx = p.max_blocks * p.bs;
-  const int n_workers = p.n_wg * kBalWaves;
+  char* kbuf = lean_lds + wave * KStage<D, FP8>::kBytes;
 
-  if (p.n_part == 1) {
-    // No merge kernel runs: rows of empty sequences are zeroed here
-    // (09_paged_attention_spmd.py:647-651).
-    for (int row = blockIdx.x * kBalWaves + wave; row < p.batch * p.hq; row += n_workers) {
-      if (p.ctx_lens[row / p.hq] <= 0)
-        for (int d = lane; d < D; d += 64) p.out[(size_t)row * D + d] = 0.f;
-    }
-  }
+  // Wavefronts are numbered CU-fastest, so that a short item list still spreads over the CUs;
+  // with fewer items than wavefronts only the first `total` wavefronts take part, which keeps
+  // every participant's run non-empty (the merge relies on that).
+  const long long total = lean_total(p, lane, hg_count);
+  const long long wres = (long long)gridDim.x * (blockDim.x >> 6);
+  const long long wtot = wres < total ? wres : total;
+  const long long w = (long long)wave * gridDim.x + blockIdx.x;
+  if (w >= wtot) return;
+  long long s = (w * total + wtot - 1) / wtot;
+  const long long s_end = ((w + 1) * total + wtot - 1) / wtot;
 
-  // Items of this wavefront: blockIdx.x + n_wg * (wave + kBalWaves * k), k = 0, 1, ...
-  for (int item = blockIdx.x + p.n_wg * wave;; item += p.n_wg * kBalWaves) {
-    // Locate the item: sequence b holds items [A_b, A_b + np_b * hg_count), np_b = ceil(ctx_b / tpp).
-    int base = 0, fb = -1, foff = 0, fnp = 1;
-    for (int b0 = 0; b0 < p.batch; b0 += 64) {
-      int ctx = (b0 + lane < p.batch) ? p.ctx_lens[b0 + lane] : 0;
-      ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
-      const int n = (ctx + p.tpp - 1) / p.tpp * hg_count;
-      int incl = n;
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const int up = __shfl_up(incl, off);
-        if (lane >= off) incl += up;
-      }
-      const int lo = base + incl - n;
-      const unsigned long long hit = __ballot(n > 0 && lo <= item && item < lo + n);
-      if (hit) {
-        const int src = __ffsll((long long)hit) - 1;
-        fb = b0 + src;
-        foff = item - __shfl(lo, src);
-        fnp = __shfl(n, src) / hg_count;
-        break;
-      }
-      base += __shfl(incl, 63);
-    }
-    if (fb < 0) break;  // past the last item (uniform over the wavefront)
-    const int b = __builtin_amdgcn_readfirstlane(fb);
-    const int np = __builtin_amdgcn_readfirstlane(fnp);
-    const int off = __builtin_amdgcn_readfirstlane(foff);
-    const int hg = off / np, part = off % np;
+  while (s < s_end) {  // one iteration per (sequence, head, tile) the run touches
+    int b, chunks;
+    long long first_item;
+    lean_locate(p, lane, hg_count, s, b, first_item, chunks);
+    if (b < 0) break;  // cannot happen for s < total; keeps the loop finite whatever the data
+    b = __builtin_amdgcn_readfirstlane(b);
+    chunks = __builtin_amdgcn_readfirstlane(chunks);
+    const long long local = s - first_item;
+    const int hg = (int)(local / chunks), chunk = (int)(local % chunks);
+    const long long left = s_end - s;
+    const int run = (int)(left < (long long)(chunks - chunk) ? left : (long long)(chunks - chunk));
     const int h = hg / p.gtiles, gt = hg % p.gtiles;
     int ctx = p.ctx_lens[b];
     ctx = ctx > max_ctx ? max_ctx : ctx;
-    const int tok_begin = part * p.tpp;
-    const int tok_end = min(ctx, tok_begin + p.tpp);
+    const int tok_first = chunk * kChunk;
+    const int tok_end = min(ctx, (chunk + run) * kChunk);
     const int g = gt * 16 + c;
     const bool g_valid = g < p.group;
     const int hq_row = b * p.hq + h * p.group + g;
@@ -584,20 +652,100 @@ __global__ __launch_bounds__(kBalWaves * 64) void attn_balanced_kernel(AttnParam
     f32x4 acc[D / 128][8];
     float m_run, l_run, v_unit;
     const int first_window =
-        p.block_table[(size_t)b * p.max_blocks + min(tok_begin / p.bs + lane, p.max_blocks - 1)];
-    attend_range<D, BF16, FP8>(p, b, h, hq_row, g_valid, tok_begin, tok_end, kChunk, c, j, k_lds[wave],
-                               first_window, acc, m_run, l_run, v_unit);
+        p.block_table[(size_t)b * p.max_blocks + min(tok_first / p.bs + lane, p.max_blocks - 1)];
+    attend_range<D, BF16, FP8>(p, b, h, hq_row, g_valid, tok_first, tok_end, kChunk, c, j, kbuf, first_window,
+                                     acc, m_run, l_run, v_unit);
     if (g_valid) {
-      if (p.n_part == 1) {
-        store_rows<D>(p.out + (size_t)hq_row * D, acc, j, l_run > 0.f ? v_unit / l_run : 0.f);
-      } else {
-        const size_t slot = (size_t)hq_row * p.n_part + part;
-        store_rows<D>(p.part_o + slot * D, acc, j, v_unit);
-        if (j == 0) {
-          p.part_ml[slot * 2 + 0] = m_run;
-          p.part_ml[slot * 2 + 1] = l_run;
-        }
+      const size_t slot = ((size_t)((long long)b * hg_count + hg + w)) * 16 + c;
+      store_rows<D>(p.part_o + slot * D, acc, j, v_unit);
+      if (j == 0) {
+        p.part_ml[slot * 2 + 0] = m_run;
+        p.part_ml[slot * 2 + 1] = l_run;
       }
+    }
+    s += run;
+  }
+}
+
+// Merge for the evenly split form: one wavefront per output row; the row's partials are the slots
+// q + w_first .. q + w_last of its (sequence, head, tile).  Online-update algebra of
+// 04_paged_attention.py:186-215; an empty sequence gives zeros (09_paged_attention_spmd.py:647-651).
+template <int D>
+__global__ __launch_bounds__(256) void attn_lean_reduce_kernel(AttnParams p, long long wtot) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // b*Hq + query head
+  if (row >= p.batch * p.hq) return;
+  const int b = row / p.hq, hqi = row % p.hq;
+  const int h = hqi / p.group, g = hqi % p.group;
+  const int hg_count = p.hkv * p.gtiles, hg = h * p.gtiles + g / 16, gi = g % 16;
+
+  // items before sequence b, items in total, chunks of b
+  long long total = 0, before = 0;
+  int chunks = 0;
+  for (int b0 = 0; b0 < p.batch; b0 += 64) {
+    const int ch = (b0 + lane < p.batch) ? seq_chunks(p, p.ctx_lens[b0 + lane]) : 0;
+    long long n = (long long)ch * hg_count;
+    long long mine = (b0 + lane < b) ? n : 0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      n += __shfl_xor(n, off);
+      mine += __shfl_xor(mine, off);
+    }
+    total += n;
+    before += mine;
+    if (b >= b0 && b < b0 + 64) chunks = __shfl(ch, b - b0);
+  }
+
+  float o[D / 64];
+#pragma unroll
+  for (int k = 0; k < D / 64; ++k) o[k] = 0.f;
+  float l = 0.f;
+  if (chunks > 0) {
+    if (wtot > total) wtot = total;  // as in the streaming kernel
+    const long long c0 = before + (long long)hg * chunks, c1 = c0 + chunks;
+    const long long w_first = c0 * wtot / total, w_last = (c1 - 1) * wtot / total;
+    const int np = (int)(w_last - w_first + 1);
+    const size_t slot0 = ((size_t)((long long)b * hg_count + hg + w_first)) * 16 + gi;
+    const float* ml = p.part_ml + slot0 * 2;   // partial i at ml[i * 32], po[i * 16 * D]
+    const float* po = p.part_o + slot0 * D;
+    float m = kMinMax;
+    for (int i = lane; i < np; i += 64) m = fmaxf(m, ml[(size_t)i * 32]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    for (int i = lane; i < np; i += 64) l += __builtin_amdgcn_exp2f(ml[(size_t)i * 32] - m) * ml[(size_t)i * 32 + 1];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off);
+    int i = 0;
+    for (; i + 4 <= np; i += 4) {
+      float wv[4], v[4][D / 64];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        wv[u] = ml[(size_t)(i + u) * 32];
+#pragma unroll
+        for (int k = 0; k < D / 64; ++k) v[u][k] = po[(size_t)(i + u) * 16 * D + k * 64 + lane];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float wgt = __builtin_amdgcn_exp2f(wv[u] - m);
+#pragma unroll
+        for (int k = 0; k < D / 64; ++k) o[k] += wgt * v[u][k];
+      }
+    }
+    for (; i < np; ++i) {
+      const float wgt = __builtin_amdgcn_exp2f(ml[(size_t)i * 32] - m);
+#pragma unroll
+      for (int k = 0; k < D / 64; ++k) o[k] += wgt * po[(size_t)i * 16 * D + k * 64 + lane];
+    }
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+  for (int k = 0; k < D / 64; ++k) {
+    const float y = o[k] * inv;
+    const size_t idx = (size_t)row * D + k * 64 + lane;
+    p.out[idx] = y;
+    if (p.out16) {
+      if (p.out16_bf16) reinterpret_cast<__bf16*>(p.out16)[idx] = (__bf16)y;
+      else reinterpret_cast<_Float16*>(p.out16)[idx] = (_Float16)y;
     }
   }
 }
@@ -612,21 +760,31 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   if (!bf16 && FP8)
     return pto_hip::fail(PTO_HIP_ERR_UNSUPPORTED, "paged_attention: an FP8E4M3FN cache needs a BF16 query");
   if (p.n_wg > 0) {
-    if constexpr (D == 128) {
-      // 12 wavefronts per CU (3 per SIMD) by default; "attn_waves_per_cu" 8 selects 2 per SIMD.
-      const bool eight = cap == 8;
-      dim3 bgrid(p.n_wg), bblock(eight ? 512 : 768);
-      if (bf16 && eight)
-        hipLaunchKernelGGL((attn_balanced_kernel<D, true, FP8, 8>), bgrid, bblock, 0, stream, p);
-      else if (bf16)
-        hipLaunchKernelGGL((attn_balanced_kernel<D, true, FP8, 12>), bgrid, bblock, 0, stream, p);
-      else if constexpr (!FP8) {
-        if (eight)
-          hipLaunchKernelGGL((attn_balanced_kernel<D, false, false, 8>), bgrid, bblock, 0, stream, p);
-        else
-          hipLaunchKernelGGL((attn_balanced_kernel<D, false, false, 12>), bgrid, bblock, 0, stream, p);
+    // Evenly split form: one workgroup of lean_waves wavefronts per CU.  The LDS request (K stages
+    // of the wavefronts, padded past half of the CU's LDS) keeps a second workgroup off the CU.
+    const size_t lean_lds = std::max<size_t>((size_t)p.lean_waves * KStage<D, FP8>::kBytes, 84 * 1024);
+    dim3 lgrid(p.n_wg), lblock(p.lean_waves * 64);
+    auto go = [&](auto kern) -> int {
+      static bool attr_set = false;  // per instantiation
+      if (!attr_set) {
+        PTO_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_set = true;
       }
+      hipLaunchKernelGGL(kern, lgrid, lblock, lean_lds, stream, p);
+      return PTO_HIP_OK;
+    };
+    int rc = PTO_HIP_OK;
+    if (bf16) rc = go(attn_lean_kernel<D, true, FP8>);
+    else if constexpr (!FP8) rc = go(attn_lean_kernel<D, false, false>);
+    if (rc) return rc;
+    PTO_CHECK_HIP(hipGetLastError());
+    if (!pto_hip::ctx().attn_skip_merge) {
+      hipLaunchKernelGGL((attn_lean_reduce_kernel<D>), dim3((unsigned)((batch * p.hq + 3) / 4)), dim3(256), 0, stream,
+                         p, (long long)p.n_wg * p.lean_waves);
+      PTO_CHECK_HIP(hipGetLastError());
     }
+    return PTO_HIP_OK;
   } else if (bf16) {
     hipLaunchKernelGGL((attn_partition_kernel<D, true, FP8>), grid, dim3(64), lds, stream, p);
   } else if constexpr (!FP8) {
@@ -731,7 +889,12 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   PTO_CHECK_ARG((int64_t)p.n_part * batch * hkv * p.gtiles < (1ll << 31),
                 "paged_attention: batch x heads x partitions exceeds the grid limit");
 
-  if (p.n_part > 1) {
+  // Launches that may stream a gigabyte or more of cache take the evenly split form: there the
+  // spread of partition lengths costs more than that form's longer start-up (measured: +11 % on
+  // 2.8 GB with contexts of 8K-32K, nothing on 150 MB).  "attn_variant" 0/1 forces the choice.
+  const int64_t kv_bound = batch * hkv * p.gtiles * max_ctx * 2 * d * (fp8 ? 1 : 2);
+  const bool lean = cx.attn_variant >= 0 ? cx.attn_variant == 1 : kv_bound >= (1ll << 30);
+  if (p.n_part > 1 && !lean) {
     const size_t rows = (size_t)batch * hq;
     const size_t o_bytes = rows * p.n_part * d * sizeof(float);
     const size_t ml_bytes = rows * p.n_part * 2 * sizeof(float);
@@ -741,11 +904,26 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     p.part_o = reinterpret_cast<float*>(ws);
     p.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + o_bytes);
   }
-  // "attn_variant" 1 selects the balanced form (one pinned workgroup per CU) for head_dim 128;
-  // head_dim 256 needs more LDS than its wavefronts per CU allow.
-  p.n_wg = (cx.attn_variant == 1 && d == 128) ? cx.num_cu : 0;
+  // "attn_variant" 1 selects the evenly split form (one pinned workgroup per CU).
+  p.n_wg = 0;
+  if (lean) {
+    const int64_t kbytes = (fp8 ? d : 2 * d) + 16;  // K stage row pitch
+    int64_t waves = cx.attn_waves_per_cu > 0 ? cx.attn_waves_per_cu : 4;
+    if (waves > kLeanMaxWaves) waves = kLeanMaxWaves;
+    while (waves > 1 && waves * 32 * kbytes > 160 * 1024) --waves;
+    p.n_wg = cx.num_cu;
+    p.lean_waves = (int)waves;
+    // partial slots: one per (sequence, head, tile) plus one per resident wavefront
+    const size_t slots = (size_t)batch * hkv * p.gtiles + (size_t)p.n_wg * waves;
+    const size_t o_bytes = slots * 16 * d * sizeof(float), ml_bytes = slots * 16 * 2 * sizeof(float);
+    void* ws = nullptr;
+    int rc = workspace(o_bytes + ml_bytes, &ws);
+    if (rc != PTO_HIP_OK) return rc;
+    p.part_o = reinterpret_cast<float*>(ws);
+    p.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + o_bytes);
+  }
   // The merge kernel writes the 16-bit copy; without a merge a cast kernel follows.
-  const bool merged = p.n_part > 1 && !cx.attn_skip_merge;
+  const bool merged = (p.n_part > 1 || p.n_wg > 0) && !cx.attn_skip_merge;
   if (merged) p.out16 = out16;
   int rc;
   if (fp8)

@@ -702,6 +702,7 @@ int pto_hip_set_option(const char* name, int64_t value) {
   } else if (!std::strcmp(name, "gemm_variant")) {
     c.gemm_variant = value;
   } else if (!std::strcmp(name, "attn_variant")) {
+    PTO_CHECK_ARG(value >= -1 && value <= 1, "attn_variant must be -1, 0 or 1");
     c.attn_variant = value;
   } else if (!std::strcmp(name, "attn_skip_merge")) {
     c.attn_skip_merge = value != 0;

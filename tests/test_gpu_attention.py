@@ -17,11 +17,12 @@ ATOL, RTOL = 1e-2, 2e-2
 
 
 def _run(worker, inp, tpp=0):
-    """tpp = 0: the default partition-grid kernel with its own choice of partition size; tpp > 0:
-    the same with that many tokens per context partition; tpp < 0: the balanced form (one pinned
-    workgroup per CU) with -tpp - 1 tokens per partition (-1: its own choice)."""
-    worker.set_option("attn_variant", 1 if tpp < 0 else 0)
-    worker.set_option("attn_tokens_per_partition", tpp if tpp > 0 else max(-tpp - 1, 0))
+    """tpp = 0: the library's own choice of form and partition size; tpp > 0: the partition-grid
+    kernel with that many tokens per context partition; tpp < 0: the evenly split form (one pinned
+    workgroup per CU) with -tpp wavefronts per CU."""
+    worker.set_option("attn_variant", -1 if tpp == 0 else (0 if tpp > 0 else 1))
+    worker.set_option("attn_tokens_per_partition", max(tpp, 0))
+    worker.set_option("attn_waves_per_cu", max(-tpp, 0))
     dev = [t.cuda() if isinstance(t, torch.Tensor) and i != 6 else t for i, t in enumerate(inp.args())]
     dev[5].fill_(float("nan"))
     torch.cuda.synchronize()
@@ -29,7 +30,8 @@ def _run(worker, inp, tpp=0):
         h(*dev)
     worker.sync()
     worker.set_option("attn_tokens_per_partition", 0)
-    worker.set_option("attn_variant", 0)
+    worker.set_option("attn_waves_per_cu", 0)
+    worker.set_option("attn_variant", -1)
     return dev[5].cpu()
 
 
@@ -46,7 +48,7 @@ def _check(out, ref):
     assert err <= ATOL + RTOL * ref.abs().max().item()
 
 
-@pytest.mark.parametrize("tpp", [0, -1, 128, 512, 4096])
+@pytest.mark.parametrize("tpp", [0, -1, -4, -8, 128, 512, 4096])
 def test_small_config_matches_golden(worker, tpp):
     """B16 Hq32 Hkv8 D128 bs128, ctx~U[512,4096], permutation table (reduced pool)."""
     inp = workloads.attention_small(seed=0, pool_blocks=None)
@@ -71,7 +73,7 @@ def test_shapes_and_edges(worker, batch, hq, hkv, d, bs, ctxs):
                                            block_size=bs, context_lens=ctxs, ctx_range=(1, max(max(ctxs), 1)),
                                            seed=7)
     ref = _golden(inp)
-    for tpp in (0, -1, 32, 256):
+    for tpp in (0, -1, -8, 32, 256):
         out = _run(worker, inp, tpp)
         _check(out, ref)
     if 0 in ctxs:
