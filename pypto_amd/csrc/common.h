@@ -75,17 +75,19 @@ struct W8Partials {
   float* part[2];
   int splits;
 };
-// Launches the partial kernel for x[M, K] @ wq0[K, N] (and wq1 when non-null).
-int w8a16_partials(const void* x, const void* wq0, const void* wq1, int64_t m, int64_t k, int64_t n,
-                   int x_dtype, hipStream_t st, W8Partials* out);
+// Launches the partial kernel for x[M, K] @ wq0[K, N] (and wq1 when non-null).  x_blocked: x is
+// stored [K/8][32][8] - element (m, k) at ((k/8)*32 + m)*8 + k%8 - the layout the layer's own
+// producers write so that a wavefront's activation reads are whole consecutive cache lines.
+int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* wq1, int64_t m, int64_t k,
+                   int64_t n, int x_dtype, hipStream_t st, W8Partials* out);
 // out = cast(sum_s(part0) * scale0 [-> SiLU(.) * (sum_s(part1) * scale1)] [+ residual]).
 int w8a16_finish(const W8Partials& parts, const float* scale0, const float* scale1, const void* residual,
-                 int res_dtype, void* out, int out_dtype, int64_t m, int64_t n, hipStream_t st);
+                 int res_dtype, void* out, int out_dtype, bool out_blocked, int64_t m, int64_t n, hipStream_t st);
 // sum_out = sum_s(part) * scale + residual (fp32); normed_out = cast(RMSNorm(sum_out) * gamma).
 bool w8a16_finish_norm_fits(int64_t n);
 int w8a16_finish_norm(const W8Partials& parts, const float* scale, const void* residual, int res_dtype,
-                      float* sum_out, const float* gamma, void* normed_out, int out_dtype, int64_t m,
-                      int64_t n, float eps, hipStream_t st);
+                      float* sum_out, const float* gamma, void* normed_out, int out_dtype, bool out_blocked,
+                      int64_t m, int64_t n, float eps, hipStream_t st);
 
 // RoPE + K/V append reading either final fp32 projections (qkv_scale null, splits 1) or the
 // partial sums of the q/k/v projection (summed in split order and scaled per channel).
@@ -101,10 +103,17 @@ int rope_kv_cache_update_fp8(const float* qkv, const float* qkv_scale, int split
                              float* v_scale, void* q_out, int64_t batch, int64_t num_heads, int64_t kv_head_num,
                              int64_t head_dim, int64_t block_size, int64_t max_num_blocks_per_req,
                              int64_t max_pos, int64_t pool_blocks, int q_dtype, void* stream);
+// RMSNorm of at most 32 rows written in the blocked activation layout [H/8][32][8].
+bool rms_norm_blocked_fits(int64_t rows, int64_t hidden);
+int rms_norm_blocked(const void* x, const float* gamma, void* out, int64_t rows, int64_t hidden, float eps,
+                     int dtype, hipStream_t st);
 int cast_from_f32(const float* in, void* out, size_t n, int out_dtype, hipStream_t st);
 // pto_hip_paged_attention with an optional second output: the result rounded to the query dtype.
+// want_blocked asks for the copy as [Hq*D/8][32][8] over the batch rows (batch <= 32);
+// *wrote_blocked says whether that is how it was written (only a launch with a merge kernel can).
 int paged_attention(const void* query, const void* key_cache, const void* value_cache,
                     const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
+                    bool want_blocked, bool* wrote_blocked,
                     const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
                     const float* v_scale, void* stream);
 

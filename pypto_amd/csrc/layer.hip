@@ -65,10 +65,16 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
 
   int rc;
   W8Partials parts{};
+  // Activations between the layer's own kernels are kept in the blocked layout [K/8][32][8] when
+  // every producer can write it (16-byte groups of 8 channels; vectorised RMSNorm shape limits).
+  const bool blk = rms_norm_blocked_fits(b, h) && w8a16_finish_norm_fits(h) && (hq * d) % 8 == 0 && inter % 8 == 0 &&
+                   ((uintptr_t)a->hidden_states | (uintptr_t)a->gamma_in) % 16 == 0;
   // 1. input RMSNorm -> activation dtype
-  if ((rc = pto_hip_rms_norm(a->hidden_states, a->gamma_in, normed, b, h, a->eps, dt, dt, stream))) return rc;
+  if (blk) rc = rms_norm_blocked(a->hidden_states, a->gamma_in, normed, b, h, a->eps, dt, st);
+  else rc = pto_hip_rms_norm(a->hidden_states, a->gamma_in, normed, b, h, a->eps, dt, dt, stream);
+  if (rc) return rc;
   // 2. QKV projection, left as k-split partial sums
-  if ((rc = w8a16_partials(normed, a->wqkv_q, nullptr, b, h, qkv_n, dt, st, &parts))) return rc;
+  if ((rc = w8a16_partials(normed, blk, a->wqkv_q, nullptr, b, h, qkv_n, dt, st, &parts))) return rc;
   // 3. finish of the projection + RoPE at pos = seq_len - 1, append K/V, rotated Q
   if (fp8kv) {
     const int64_t pool_blocks = a->pool_rows / (hkv * a->block_size);
@@ -87,22 +93,25 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
   uint32_t scale_bits;
   __builtin_memcpy(&scale_bits, &scale, 4);
   const int64_t cfg[7] = {b, hq, hkv, d, a->block_size, a->max_num_blocks_per_req, (int64_t)scale_bits};
-  if ((rc = paged_attention(q16, a->key_cache, a->value_cache, a->block_table, a->seq_lens, attn, attn16, cfg, dt,
-                            fp8kv ? PTO_HIP_FP8E4M3FN : dt, fp8kv ? a->k_scale : nullptr,
+  bool blk_attn = false;  // the 16-bit copy is blocked only when the merge kernel wrote it
+  if ((rc = paged_attention(q16, a->key_cache, a->value_cache, a->block_table, a->seq_lens, attn, attn16, blk,
+                            &blk_attn, cfg, dt, fp8kv ? PTO_HIP_FP8E4M3FN : dt, fp8kv ? a->k_scale : nullptr,
                             fp8kv ? a->v_scale : nullptr, stream)))
     return rc;
   // 5. o_proj; 6. its finish + residual -> fp32, post-attention RMSNorm -> activation dtype
-  if ((rc = w8a16_partials(attn16, a->wo_q, nullptr, b, hq * d, h, dt, st, &parts))) return rc;
+  if ((rc = w8a16_partials(attn16, blk_attn, a->wo_q, nullptr, b, hq * d, h, dt, st, &parts))) return rc;
   if (w8a16_finish_norm_fits(h)) {
-    if ((rc = w8a16_finish_norm(parts, a->wo_s, a->hidden_states, dt, resid1, a->gamma_post, normed2, dt, b, h,
+    if ((rc = w8a16_finish_norm(parts, a->wo_s, a->hidden_states, dt, resid1, a->gamma_post, normed2, dt, blk, b, h,
                                 a->eps, st)))
       return rc;
   } else {
-    if ((rc = w8a16_finish(parts, a->wo_s, nullptr, a->hidden_states, dt, resid1, PTO_HIP_FP32, b, h, st))) return rc;
+    if ((rc = w8a16_finish(parts, a->wo_s, nullptr, a->hidden_states, dt, resid1, PTO_HIP_FP32, false, b, h, st)))
+      return rc;
     if ((rc = pto_hip_rms_norm(resid1, a->gamma_post, normed2, b, h, a->eps, PTO_HIP_FP32, dt, stream))) return rc;
   }
   // 7. gate/up + SwiGLU -> h (activation dtype), 8. down + residual -> out
-  if ((rc = pto_hip_w8a16_swiglu(normed2, a->wg_q, a->wg_s, a->wu_q, a->wu_s, hbuf, b, h, inter, dt, dt, stream)))
-    return rc;
-  return pto_hip_w8a16_matmul(hbuf, a->wd_q, a->wd_s, resid1, a->out, b, inter, h, dt, PTO_HIP_FP32, dt, stream);
+  if ((rc = w8a16_partials(normed2, blk, a->wg_q, a->wu_q, b, h, inter, dt, st, &parts))) return rc;
+  if ((rc = w8a16_finish(parts, a->wg_s, a->wu_s, nullptr, 0, hbuf, dt, blk, b, inter, st))) return rc;
+  if ((rc = w8a16_partials(hbuf, blk, a->wd_q, nullptr, b, inter, h, dt, st, &parts))) return rc;
+  return w8a16_finish(parts, a->wd_s, nullptr, resid1, PTO_HIP_FP32, a->out, dt, false, b, h, st);
 }

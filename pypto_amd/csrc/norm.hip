@@ -54,7 +54,9 @@ __global__ __launch_bounds__(kThreads) void rms_norm_kernel(const TI* __restrict
 // 16-bit rows whose length is a multiple of 8 and at most 8 * kThreads * kVecPerThread: each
 // thread keeps its 16-byte chunks in registers, so the row is read from memory once.
 constexpr int kVecPerThread = 4;
-template <typename T>
+// BLOCKED writes the output as [hidden/8][32][8] (at most 32 rows): the activation layout the
+// W8A16 projections of the decoder layer read.
+template <typename T, bool BLOCKED>
 __global__ __launch_bounds__(kThreads) void rms_norm_vec_kernel(const T* __restrict__ x,
                                                                 const float* __restrict__ gamma,
                                                                 T* __restrict__ out, int64_t hidden,
@@ -62,7 +64,8 @@ __global__ __launch_bounds__(kThreads) void rms_norm_vec_kernel(const T* __restr
   typedef __attribute__((__vector_size__(8 * sizeof(T)))) T vec8;
   const int64_t row = blockIdx.x;
   const vec8* xr = reinterpret_cast<const vec8*>(x + row * hidden);
-  vec8* orow = reinterpret_cast<vec8*>(out + row * hidden);
+  vec8* orow = BLOCKED ? reinterpret_cast<vec8*>(out) + row : reinterpret_cast<vec8*>(out + row * hidden);
+  constexpr int kOutStride = BLOCKED ? 32 : 1;  // vec8 units between consecutive 8-element groups
   const int nvec = (int)(hidden / 8);
   vec8 v[kVecPerThread];
   float ss = 0.f;
@@ -97,7 +100,7 @@ __global__ __launch_bounds__(kThreads) void rms_norm_vec_kernel(const T* __restr
       const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
 #pragma unroll
       for (int e = 0; e < 8; ++e) o[e] = (T)((float)v[u][e] * inv * g[e]);
-      orow[i] = o;
+      orow[(size_t)i * kOutStride] = o;
     }
   }
 }
@@ -129,6 +132,28 @@ int launch_out(const void* x, const float* gamma, void* out, int64_t rows, int64
 
 }  // namespace
 
+namespace pto_hip {
+bool rms_norm_blocked_fits(int64_t rows, int64_t hidden) {
+  return rows <= 32 && hidden % 8 == 0 && hidden <= 8 * kThreads * kVecPerThread;
+}
+int rms_norm_blocked(const void* x, const float* gamma, void* out, int64_t rows, int64_t hidden, float eps,
+                     int dtype, hipStream_t st) {
+  PTO_CHECK_ARG(rms_norm_blocked_fits(rows, hidden) && (dtype == PTO_HIP_BF16 || dtype == PTO_HIP_FP16) &&
+                    ((uintptr_t)x | (uintptr_t)out | (uintptr_t)gamma) % 16 == 0 && gamma != nullptr,
+                "rms_norm (blocked): unsupported shape [%lld, %lld] or operands", (long long)rows, (long long)hidden);
+  if (rows == 0) return PTO_HIP_OK;
+  dim3 grid((unsigned)rows), block(kThreads);
+  if (dtype == PTO_HIP_BF16)
+    hipLaunchKernelGGL((rms_norm_vec_kernel<__bf16, true>), grid, block, 0, st, (const __bf16*)x, gamma, (__bf16*)out,
+                       hidden, eps);
+  else
+    hipLaunchKernelGGL((rms_norm_vec_kernel<_Float16, true>), grid, block, 0, st, (const _Float16*)x, gamma,
+                       (_Float16*)out, hidden, eps);
+  PTO_CHECK_HIP(hipGetLastError());
+  return PTO_HIP_OK;
+}
+}  // namespace pto_hip
+
 extern "C" int pto_hip_rms_norm(const void* x, const float* gamma, void* out, int64_t rows,
                                 int64_t hidden, float eps, int x_dtype, int out_dtype, void* stream) {
   using namespace pto_hip;
@@ -144,10 +169,10 @@ extern "C" int pto_hip_rms_norm(const void* x, const float* gamma, void* out, in
   if (vec_ok) {
     dim3 grid((unsigned)rows), block(kThreads);
     if (x_dtype == PTO_HIP_BF16)
-      hipLaunchKernelGGL(rms_norm_vec_kernel<__bf16>, grid, block, 0, st, (const __bf16*)x, gamma,
+      hipLaunchKernelGGL((rms_norm_vec_kernel<__bf16, false>), grid, block, 0, st, (const __bf16*)x, gamma,
                          (__bf16*)out, hidden, eps);
     else
-      hipLaunchKernelGGL(rms_norm_vec_kernel<_Float16>, grid, block, 0, st, (const _Float16*)x, gamma,
+      hipLaunchKernelGGL((rms_norm_vec_kernel<_Float16, false>), grid, block, 0, st, (const _Float16*)x, gamma,
                          (_Float16*)out, hidden, eps);
     PTO_CHECK_HIP(hipGetLastError());
     return PTO_HIP_OK;

@@ -41,6 +41,7 @@ struct AttnParams {
   float* out;
   void* out16;     // optional second copy of the result in the 16-bit activation type
   int out16_bf16;
+  int out16_blocked;  // copy stored [Hq*D/8][32][8] over the batch rows instead of [B, Hq*D]
   float* part_o;   // [B*Hq, n_part, D]
   float* part_ml;  // [B*Hq, n_part, 2]  (running max in log2 units, row sum)
   const float* k_scale;  // [pool_blocks, Hkv] for an e4m3 cache, else null
@@ -538,8 +539,13 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
     const size_t idx = (size_t)row * D + k * 64 + lane;
     p.out[idx] = y;
     if (p.out16) {
-      if (p.out16_bf16) reinterpret_cast<__bf16*>(p.out16)[idx] = (__bf16)y;
-      else reinterpret_cast<_Float16*>(p.out16)[idx] = (_Float16)y;
+      size_t i16 = idx;
+      if (p.out16_blocked) {
+        const int bb = row / p.hq, kk = (row % p.hq) * D + k * 64 + lane;  // element kk of batch row bb
+        i16 = ((size_t)(kk >> 3) * 32 + bb) * 8 + (kk & 7);
+      }
+      if (p.out16_bf16) reinterpret_cast<__bf16*>(p.out16)[i16] = (__bf16)y;
+      else reinterpret_cast<_Float16*>(p.out16)[i16] = (_Float16)y;
     }
   }
 }
@@ -744,8 +750,13 @@ __global__ __launch_bounds__(256) void attn_lean_reduce_kernel(AttnParams p, lon
     const size_t idx = (size_t)row * D + k * 64 + lane;
     p.out[idx] = y;
     if (p.out16) {
-      if (p.out16_bf16) reinterpret_cast<__bf16*>(p.out16)[idx] = (__bf16)y;
-      else reinterpret_cast<_Float16*>(p.out16)[idx] = (_Float16)y;
+      size_t i16 = idx;
+      if (p.out16_blocked) {
+        const int bb = row / p.hq, kk = (row % p.hq) * D + k * 64 + lane;  // element kk of batch row bb
+        i16 = ((size_t)(kk >> 3) * 32 + bb) * 8 + (kk & 7);
+      }
+      if (p.out16_bf16) reinterpret_cast<__bf16*>(p.out16)[i16] = (__bf16)y;
+      else reinterpret_cast<_Float16*>(p.out16)[i16] = (_Float16)y;
     }
   }
 }
@@ -806,7 +817,7 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
 namespace pto_hip {
 int paged_attention(const void* query, const void* key_cache, const void* value_cache,
                     const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
-                    const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
+                    bool want_blocked, bool* wrote_blocked, const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
                     const float* v_scale, void* stream) {
   Context& cx = ctx();
   if (!cx.initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
@@ -853,6 +864,8 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   p.out = out;
   p.out16 = nullptr;
   p.out16_bf16 = q_dtype == PTO_HIP_BF16;
+  p.out16_blocked = 0;
+  if (wrote_blocked) *wrote_blocked = false;
   p.k_scale = k_scale;
   p.v_scale = v_scale;
   p.batch = (int)batch;
@@ -924,7 +937,12 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   }
   // The merge kernel writes the 16-bit copy; without a merge a cast kernel follows.
   const bool merged = (p.n_part > 1 || p.n_wg > 0) && !cx.attn_skip_merge;
-  if (merged) p.out16 = out16;
+  if (merged) {
+    // the merge kernel writes the copy, blocked on request; without a merge a cast kernel writes it row-major
+    p.out16 = out16;
+    p.out16_blocked = (out16 && want_blocked) ? 1 : 0;
+    if (wrote_blocked) *wrote_blocked = p.out16_blocked != 0;
+  }
   int rc;
   if (fp8)
     rc = d == 128 ? launch<128, true>(p, (int)batch, bf16, (hipStream_t)stream)
@@ -942,6 +960,6 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
                                        const int32_t* context_lens, float* out,
                                        const int64_t* config, int q_dtype, int kv_dtype,
                                        const float* k_scale, const float* v_scale, void* stream) {
-  return pto_hip::paged_attention(query, key_cache, value_cache, block_table, context_lens, out, nullptr, config,
+  return pto_hip::paged_attention(query, key_cache, value_cache, block_table, context_lens, out, nullptr, false, nullptr, config,
                                   q_dtype, kv_dtype, k_scale, v_scale, stream);
 }

@@ -38,6 +38,7 @@ struct GemvParams {
   const int8_t* wq[2];  // [K, N] each; the second is the up projection of a gate/up pair
   float* part[2];       // [splits, 32, N] each
   int m, k, n, slabs, n_mats, splits, k_per_split;
+  int x_blocked;  // activations stored [K/8][32][8] (see w8a16_partials) instead of row-major
 };
 
 template <bool BF16>
@@ -84,8 +85,14 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
   const int n_steps = (k_end - k_begin + kStep - 1) / kStep;
 
   const int n0 = slab * kSlab + c * 8;
-  const uint16_t* xp0 = p.x + (size_t)min(c, p.m - 1) * p.k + kg * 8;
-  const uint16_t* xp1 = p.x + (size_t)min(c + 16, p.m - 1) * p.k + kg * 8;
+  // Row-major x: lane (c, kg) reads 16 bytes of rows c and c+16 at k = kstep + 8*kg.  Blocked x
+  // keeps the 32 rows of each 8-k group together, so the same two reads of a wavefront cover 2 KB
+  // of consecutive bytes instead of 32 half cache lines.
+  const int x_step = p.x_blocked ? kMaxM : 1;  // elements per unit of k
+  const uint16_t* xp0 = p.x_blocked ? p.x + (size_t)(kg * kMaxM + min(c, p.m - 1)) * 8
+                                    : p.x + (size_t)min(c, p.m - 1) * p.k + kg * 8;
+  const uint16_t* xp1 = p.x_blocked ? p.x + (size_t)(kg * kMaxM + min(c + 16, p.m - 1)) * 8
+                                    : p.x + (size_t)min(c + 16, p.m - 1) * p.k + kg * 8;
   const bool m0_ok = c < p.m, m1_ok = c + 16 < p.m;
 
   f32x4 acc[8][2];
@@ -105,8 +112,8 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
   auto step_row = [&](int step) { return min(k_begin + step * kStep, p.k - kStep); };
   auto load = [&](Stage& s, int step) {
     const int kstep = step_row(min(step, last_step));
-    s.xa[0] = *reinterpret_cast<const u32x4*>(xp0 + kstep);
-    s.xa[1] = *reinterpret_cast<const u32x4*>(xp1 + kstep);
+    s.xa[0] = *reinterpret_cast<const u32x4*>(xp0 + (size_t)kstep * x_step);
+    s.xa[1] = *reinterpret_cast<const u32x4*>(xp1 + (size_t)kstep * x_step);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int8_t* row = wbase + (size_t)(kstep + e) * p.n;  // uniform
@@ -211,7 +218,11 @@ struct FinishParams {
   const void* residual; // [M, N] in res_dtype, or null
   void* out;            // [M, N]
   int m, n, splits, res_dtype, out_dtype;
+  int out_blocked;  // write out as [N/8][32][8] for the next projection
 };
+
+// Element index of (row m, channel n) in the blocked activation layout [N/8][32][8].
+__device__ __forceinline__ size_t blocked_index(int m, int n) { return ((size_t)(n >> 3) * kMaxM + m) * 8 + (n & 7); }
 
 __device__ __forceinline__ float4 load4_as_f32(const void* p, size_t i, int dt) {
   if (dt == PTO_HIP_FP32) return *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + i);
@@ -277,7 +288,7 @@ __global__ __launch_bounds__(256) void w8a16_finish_kernel(FinishParams p) {
     const float4 r = load4_as_f32(p.residual, idx, p.res_dtype);
     a.x += r.x; a.y += r.y; a.z += r.z; a.w += r.w;
   }
-  store4_from_f32(p.out, idx, p.out_dtype, a);
+  store4_from_f32(p.out, p.out_blocked ? blocked_index(m, n) : idx, p.out_dtype, a);
 }
 
 // Finish of a projection followed by RMSNorm of the sum with the residual: one workgroup per
@@ -293,6 +304,7 @@ struct FinishNormParams {
   const float* gamma;    // [N]
   void* normed_out;      // [M, N] in out_dtype
   int n, splits, res_dtype, out_dtype;
+  int out_blocked;
   float eps;
 };
 
@@ -327,7 +339,7 @@ __global__ __launch_bounds__(kNormThreads) void w8a16_finish_norm_kernel(FinishN
     if (n < p.n) {
       const float4 g = *reinterpret_cast<const float4*>(p.gamma + n);
       const float4 y = {v[u].x * inv * g.x, v[u].y * inv * g.y, v[u].z * inv * g.z, v[u].w * inv * g.w};
-      store4_from_f32(p.normed_out, (size_t)m * p.n + n, p.out_dtype, y);
+      store4_from_f32(p.normed_out, p.out_blocked ? blocked_index(m, n) : (size_t)m * p.n + n, p.out_dtype, y);
     }
   }
 }
@@ -364,7 +376,7 @@ void choose_splits(int64_t k, int64_t slabs_total, int* splits, int* k_per_split
 
 namespace pto_hip {
 
-int w8a16_partials(const void* x, const void* wq0, const void* wq1, int64_t m, int64_t k, int64_t n,
+int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* wq1, int64_t m, int64_t k, int64_t n,
                    int x_dtype, hipStream_t st, W8Partials* out) {
   GemvParams p{};
   p.x = reinterpret_cast<const uint16_t*>(x);
@@ -375,6 +387,7 @@ int w8a16_partials(const void* x, const void* wq0, const void* wq1, int64_t m, i
   p.n = (int)n;
   p.slabs = (int)((n + kSlab - 1) / kSlab);
   p.n_mats = wq1 ? 2 : 1;
+  p.x_blocked = x_blocked ? 1 : 0;
   choose_splits(k, (int64_t)p.slabs * p.n_mats, &p.splits, &p.k_per_split);
   const size_t one = (size_t)p.splits * kMaxM * n * sizeof(float);
   void* ws = nullptr;
@@ -395,7 +408,7 @@ int w8a16_partials(const void* x, const void* wq0, const void* wq1, int64_t m, i
 }
 
 int w8a16_finish(const W8Partials& parts, const float* scale0, const float* scale1, const void* residual,
-                 int res_dtype, void* out, int out_dtype, int64_t m, int64_t n, hipStream_t st) {
+                 int res_dtype, void* out, int out_dtype, bool out_blocked, int64_t m, int64_t n, hipStream_t st) {
   FinishParams f{};
   f.part0 = parts.part[0];
   f.part1 = parts.part[1];
@@ -408,6 +421,7 @@ int w8a16_finish(const W8Partials& parts, const float* scale0, const float* scal
   f.splits = parts.splits;
   f.res_dtype = res_dtype;
   f.out_dtype = out_dtype;
+  f.out_blocked = out_blocked ? 1 : 0;
   hipLaunchKernelGGL(w8a16_finish_kernel, dim3((unsigned)((n / 4 + 255) / 256), (unsigned)m), dim3(256), 0, st, f);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
@@ -416,8 +430,8 @@ int w8a16_finish(const W8Partials& parts, const float* scale0, const float* scal
 bool w8a16_finish_norm_fits(int64_t n) { return n % 4 == 0 && n <= 4 * kNormThreads * kNormVec; }
 
 int w8a16_finish_norm(const W8Partials& parts, const float* scale, const void* residual, int res_dtype,
-                      float* sum_out, const float* gamma, void* normed_out, int out_dtype, int64_t m,
-                      int64_t n, float eps, hipStream_t st) {
+                      float* sum_out, const float* gamma, void* normed_out, int out_dtype, bool out_blocked,
+                      int64_t m, int64_t n, float eps, hipStream_t st) {
   FinishNormParams f{};
   f.part = parts.part[0];
   f.scale = scale;
@@ -429,6 +443,7 @@ int w8a16_finish_norm(const W8Partials& parts, const float* scale, const void* r
   f.splits = parts.splits;
   f.res_dtype = res_dtype;
   f.out_dtype = out_dtype;
+  f.out_blocked = out_blocked ? 1 : 0;
   f.eps = eps;
   hipLaunchKernelGGL(w8a16_finish_norm_kernel, dim3((unsigned)m), dim3(kNormThreads), 0, st, f);
   PTO_CHECK_HIP(hipGetLastError());
@@ -454,9 +469,9 @@ extern "C" int pto_hip_w8a16_matmul(const void* x, const void* w_q, const float*
                   "w8a16_matmul: residual dtype %s not in {FP32, BF16, FP16}", dtype_name(res_dtype));
   hipStream_t st = (hipStream_t)stream;
   W8Partials parts{};
-  rc = w8a16_partials(x, w_q, nullptr, m, k, n, x_dtype, st, &parts);
+  rc = w8a16_partials(x, false, w_q, nullptr, m, k, n, x_dtype, st, &parts);
   if (rc) return rc;
-  return w8a16_finish(parts, w_scale, nullptr, residual, res_dtype, out, out_dtype, m, n, st);
+  return w8a16_finish(parts, w_scale, nullptr, residual, res_dtype, out, out_dtype, false, m, n, st);
 }
 
 extern "C" int pto_hip_w8a16_swiglu(const void* x, const void* wg_q, const float* wg_scale,
@@ -473,7 +488,7 @@ extern "C" int pto_hip_w8a16_swiglu(const void* x, const void* wg_q, const float
                 "w8a16_swiglu: misaligned operand");
   hipStream_t st = (hipStream_t)stream;
   W8Partials parts{};
-  rc = w8a16_partials(x, wg_q, wu_q, m, k, n, x_dtype, st, &parts);
+  rc = w8a16_partials(x, false, wg_q, wu_q, m, k, n, x_dtype, st, &parts);
   if (rc) return rc;
-  return w8a16_finish(parts, wg_scale, wu_scale, nullptr, 0, out, out_dtype, m, n, st);
+  return w8a16_finish(parts, wg_scale, wu_scale, nullptr, 0, out, out_dtype, false, m, n, st);
 }
