@@ -291,9 +291,9 @@ PTO_HIP_API int pto_hip_select_program(const char* orchestration_name, const Pto
  *                               workgroup per CU and the chunk list cut evenly over their wavefronts,
  *                               -1 = by launch size (default)
  *  "gemm_variant"               FFN GEMM tiling: 0 = default choice, 1..3 = fixed alternatives
- *  "w8a16_wgs_per_cu"           workgroups per CU the W8A16 k split aims at (default 2)
+ *  "w8a16_wgs_per_cu"           workgroups per CU the W8A16 k split aims at (default 1)
  *  "w8a16_min_steps"            fewest 32-row steps per wavefront before k is split further
- *                               (default 4)
+ *                               (default 8)
  */
 PTO_HIP_API int pto_hip_set_option(const char* name, int64_t value);
 PTO_HIP_API int pto_hip_get_option(const char* name, int64_t* value);

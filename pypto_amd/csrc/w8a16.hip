@@ -29,9 +29,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
 
 constexpr int kSlab = pto_hip::kW8Slab;  // output channels per workgroup
 constexpr int kStep = 32;                // k rows per step
-constexpr int kWaves = 4;
 constexpr int kMaxM = pto_hip::kW8MaxM;
-constexpr int kUnit = kStep * kWaves;    // k rows one round of the wavefronts covers
+constexpr int kWavesPerWg = 4;           // wavefronts per workgroup of the partial kernel
 
 struct GemvParams {
   const uint16_t* x;    // [M, K] 16-bit activations
@@ -69,10 +68,13 @@ struct Stage {
   u32x4 xa[2];   // activations of rows c and c+16, k = kg*8 .. +8
 };
 
-template <bool BF16>
-__global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void w8a16_partial_kernel(GemvParams p) {
+// kWaves wavefronts per workgroup, kStages register stages per wavefront (kStages - 1 in flight),
+// kOcc wavefronts per SIMD the register budget is cut for.
+template <bool BF16, int kWaves, int kStages, int kOcc>
+__global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOcc, kOcc))) void w8a16_partial_kernel(
+    GemvParams p) {
   constexpr int kHalf = kWaves / 2;
-  __shared__ float red[kHalf * kMaxM * kSlab];  // 32 KiB
+  __shared__ float red[kHalf * kMaxM * kSlab];  // 16 KiB per wavefront of the lower half
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: row addresses stay scalar
   const int c = lane & 15, kg = lane >> 4;
@@ -144,17 +146,18 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
     }
   };
 
-  // Wavefront w takes steps w, w + kWaves, ...; two register stages, one in flight while the
-  // other is consumed (three or four workgroups share a compute unit, so a dozen or more steps
-  // are in flight per unit).  The trip count is rounded up to even: a surplus step multiplies
-  // by zero.
-  Stage sa, sb;
-  load(sa, wave);
-  for (int s = wave; s < n_steps; s += 2 * kWaves) {
-    load(sb, s + kWaves);
-    compute(sa, s);
-    load(sa, s + 2 * kWaves);
-    compute(sb, s + kWaves);
+  // Wavefront w takes steps w, w + kWaves, ...; kStages register stages, all but the one being
+  // consumed in flight.  The trip count is rounded up to whole rounds of kStages: surplus steps
+  // multiply by zero.
+  Stage st[kStages];
+#pragma unroll
+  for (int u = 0; u < kStages - 1; ++u) load(st[u], wave + u * kWaves);
+  for (int s = wave; s < n_steps; s += kStages * kWaves) {
+#pragma unroll
+    for (int u = 0; u < kStages; ++u) {
+      load(st[(u + kStages - 1) % kStages], s + (u + kStages - 1) * kWaves);
+      compute(st[u], s + u * kWaves);
+    }
   }
 
   // ---- sum the accumulators: upper half -> LDS -> lower half -> LDS -> all threads ----------
@@ -361,7 +364,8 @@ int check_common(const char* what, int64_t m, int64_t k, int64_t n, int x_dtype,
 
 // k splits: a few workgroups per compute unit, each wavefront with at least a few steps when k
 // allows, split boundaries on multiples of the rows one round of the wavefronts covers.
-void choose_splits(int64_t k, int64_t slabs_total, int* splits, int* k_per_split) {
+void choose_splits(int64_t k, int64_t slabs_total, int waves, int* splits, int* k_per_split) {
+  const int kUnit = kStep * waves;  // k rows one round of the wavefronts covers
   const pto_hip::Context& cx = pto_hip::ctx();
   const int64_t units = (k + kUnit - 1) / kUnit;
   int64_t want = (cx.w8a16_wgs_per_cu * cx.num_cu) / slabs_total;
@@ -388,7 +392,7 @@ int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* w
   p.slabs = (int)((n + kSlab - 1) / kSlab);
   p.n_mats = wq1 ? 2 : 1;
   p.x_blocked = x_blocked ? 1 : 0;
-  choose_splits(k, (int64_t)p.slabs * p.n_mats, &p.splits, &p.k_per_split);
+  choose_splits(k, (int64_t)p.slabs * p.n_mats, kWavesPerWg, &p.splits, &p.k_per_split);
   const size_t one = (size_t)p.splits * kMaxM * n * sizeof(float);
   void* ws = nullptr;
   int rc = workspace(one * p.n_mats, &ws);
@@ -396,10 +400,13 @@ int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* w
   p.part[0] = reinterpret_cast<float*>(ws);
   p.part[1] = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + one);
   const dim3 grid((unsigned)(p.slabs * p.n_mats * p.splits));
+  // Four wavefronts x two stages: measured best in the decoder layer against 2, 4 and 8 wavefronts
+  // with 2-4 stages (more requests in flight per CU only lengthened the memory queueing delay).
+  const dim3 block((unsigned)kWavesPerWg * 64);
   if (x_dtype == PTO_HIP_BF16)
-    hipLaunchKernelGGL(w8a16_partial_kernel<true>, grid, dim3(kWaves * 64), 0, st, p);
+    hipLaunchKernelGGL((w8a16_partial_kernel<true, kWavesPerWg, 2, 4>), grid, block, 0, st, p);
   else
-    hipLaunchKernelGGL(w8a16_partial_kernel<false>, grid, dim3(kWaves * 64), 0, st, p);
+    hipLaunchKernelGGL((w8a16_partial_kernel<false, kWavesPerWg, 2, 4>), grid, block, 0, st, p);
   PTO_CHECK_HIP(hipGetLastError());
   out->part[0] = p.part[0];
   out->part[1] = wq1 ? p.part[1] : nullptr;
