@@ -7,8 +7,10 @@
 // projection (mlp.py:60).
 //
 // One MFMA GEMM kernel serves both matmuls:
-//   * block tile (64*MT) x 256 x 64, four wavefronts, each owning (32*MT) x 128 of the tile as
-//     MT x 4 accumulators of v_mfma_f32_32x32x16;
+//   * block tile 256 x 256 x 64, eight wavefronts (two per SIMD, so the MFMA pipe has a second
+//     instruction stream while one waits on memory or the barrier), each owning 128 x 64 of the
+//     tile as 4 x 2 accumulators of v_mfma_f32_32x32x16; a four-wavefront form (128 x 128 each)
+//     and a 128-row tile for small shapes are kept as variants;
 //   * both operands go HBM -> VGPR -> LDS as coalesced 16-byte chunks in their memory layout:
 //     A rows ([M, K], k contiguous) are read back with ds_read_b128; B rows ([K, N], n
 //     contiguous) are read back with the transposing ds_read_b64_tr_b16, which hands every
@@ -74,9 +76,19 @@ __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
 
 // EDGE = false assumes m, n, k are multiples of the tile; EDGE = true clamps every address into
 // the operands (so all loads stay unconditional) and zeroes the A chunks that lie past k.
-template <int MT, int NBUF, bool DUAL, bool BF16, bool EDGE, typename OutT>
-__global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
-  constexpr int BM = 64 * MT;
+// Wavefront grid WM x WN over the (32*MT*WM) x 256 tile: each wavefront owns (32*MT) x (32*NT)
+// as MT x NT accumulators, NT = 8 / WN.  2 x 2 wavefronts with 4 x 4 accumulators run one
+// wavefront per SIMD; 2 x 4 wavefronts with 4 x 2 accumulators run two per SIMD, so the MFMA pipe
+// has a second instruction stream to draw from while one waits on memory or a barrier.
+template <int MT, int WM, int WN, bool DUAL, bool BF16, bool EDGE, typename OutT>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
+  constexpr int NBUF = 2;
+  constexpr int NT = (BN / 32) / WN;        // B fragments (32 columns each) per wavefront
+  constexpr int T = 64 * WM * WN;           // threads
+  constexpr int BM = 32 * MT * WM;
+  constexpr int NA = BM * 8 / T;            // 16-byte A chunks per thread and tile
+  constexpr int NB = BK * 32 / T;           // 16-byte B chunks per thread and tile
+  static_assert(NT >= 1 && (!DUAL || NT % 2 == 0), "gate/up pass needs gate and up columns in every wavefront");
   constexpr int A_ELEMS = BM * LDK;
   constexpr int B_ELEMS = BK * LDN;
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
@@ -85,7 +97,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int wm = wave & 1, wn = wave >> 1;
+  const int wm = wave % WM, wn = wave / WM;
 
   const int ntiles = p.tiles_m * p.tiles_n;
   const int logical = xcd_remap(blockIdx.x, ntiles * p.splits);
@@ -97,9 +109,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   const int n0 = tn * (DUAL ? BN / 2 : BN);
 
   // ---- global -> register staging ---------------------------------------------------
-  // A: thread owns 16-byte chunk (tid % 8) of rows tid/8 + 32*i.
+  // A: thread owns 16-byte chunk (tid % 8) of rows tid/8 + (T/8)*i.
   const int a_chunk = tid & 7, a_row = tid >> 3;
-  // B: thread owns 16-byte chunk (tid % 32) of k rows tid/32 + 8*i; in the gate/up pass chunks
+  // B: thread owns 16-byte chunk (tid % 32) of k rows tid/32 + (T/32)*i; in the gate/up pass chunks
   // 0..15 come from the gate weights and 16..31 from the up weights (same output columns).
   const int b_chunk = tid & 31, b_row = tid >> 5;
   const uint16_t* bsrc;
@@ -112,17 +124,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     b_col = n0 + b_chunk * 8;
   }
   if (EDGE) b_col = min(b_col, p.n - 8);
-  const uint16_t* a_ptr[2 * MT];
+  const uint16_t* a_ptr[NA];
 #pragma unroll
-  for (int i = 0; i < 2 * MT; ++i) {
-    int r = m0 + a_row + 32 * i;
+  for (int i = 0; i < NA; ++i) {
+    int r = m0 + a_row + (T / 8) * i;
     if (EDGE) r = min(r, p.m - 1);
     a_ptr[i] = p.a + (int64_t)r * p.lda + k_begin + a_chunk * 8;
   }
   const uint16_t* b_ptr = bsrc + (int64_t)(k_begin + b_row) * p.ldb + b_col;
 
-  u32x4 ra[2 * MT];
-  u32x4 rb[8];
+  u32x4 ra[NA];
+  u32x4 rb[NB];
   auto load_a = [&](int k0, int i) {
     if constexpr (EDGE) {
       const int ka = min(k0 + a_chunk * 8, klen - 8) - a_chunk * 8;  // clamped tile origin for A
@@ -136,34 +148,34 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   };
   auto load_b = [&](int k0, int i) {
     if constexpr (EDGE) {
-      const int kk = min(k0 + b_row + 8 * i, klen - 1) - b_row;
+      const int kk = min(k0 + b_row + (T / 32) * i, klen - 1) - b_row;
       rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)kk * p.ldb);
     } else {
-      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)(k0 + 8 * i) * p.ldb);
+      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)(k0 + (T / 32) * i) * p.ldb);
     }
   };
   auto load_tile = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 2 * MT; ++i) load_a(k0, i);
+    for (int i = 0; i < NA; ++i) load_a(k0, i);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) load_b(k0, i);
+    for (int i = 0; i < NB; ++i) load_b(k0, i);
   };
   auto store_tile = [&](int buf) {
     uint16_t* da = sa + buf * A_ELEMS;
 #pragma unroll
-    for (int i = 0; i < 2 * MT; ++i)
-      *reinterpret_cast<u32x4*>(da + (a_row + 32 * i) * LDK + a_chunk * 8) = ra[i];
+    for (int i = 0; i < NA; ++i)
+      *reinterpret_cast<u32x4*>(da + (a_row + (T / 8) * i) * LDK + a_chunk * 8) = ra[i];
     uint16_t* db = sb + buf * B_ELEMS;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      *reinterpret_cast<u32x4*>(db + (b_row + 8 * i) * LDN + b_chunk * 8) = rb[i];
+    for (int i = 0; i < NB; ++i)
+      *reinterpret_cast<u32x4*>(db + (b_row + (T / 32) * i) * LDN + b_chunk * 8) = rb[i];
   };
 
-  f32x16 acc[MT][4];
+  f32x16 acc[MT][NT];
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int jn = 0; jn < 4; ++jn)
+    for (int jn = 0; jn < NT; ++jn)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][jn][r] = 0.f;
 
@@ -175,16 +187,18 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   //     next 8 k-rows.
   const int a_frag = (wm * MT * 32 + (lane & 31)) * LDK + (lane >> 5) * 8;
   const int grp = lane >> 4, sub = lane & 15;
-  int b_frag[4];
+  int b_frag[NT];
 #pragma unroll
-  for (int jn = 0; jn < 4; ++jn) {
-    const int col = DUAL ? ((jn >> 1) * (BN / 2) + wn * 64 + (jn & 1) * 32) : (wn * 128 + jn * 32);
+  for (int jn = 0; jn < NT; ++jn) {
+    // gate/up pass: the first NT/2 fragments are gate columns, the rest the up columns of the same outputs
+    const int col = DUAL ? ((jn / (NT / 2)) * (BN / 2) + wn * (16 * NT) + (jn % (NT / 2)) * 32)
+                         : (wn * (32 * NT) + jn * 32);
     b_frag[jn] = ((grp >> 1) * 8 + (sub >> 2)) * LDN + col + (grp & 1) * 16 + (sub & 3) * 4;
   }
 
   // One LDS read of the fragment set for k-step `ks` of buffer `buf`: r < MT reads A fragment r,
   // the rest read half (4 k-rows) of a B fragment.
-  u32x4 fa[2][MT], fb[2][4];
+  u32x4 fa[2][MT], fb[2][NT];
   auto read_one = [&](int buf, int ks, int set, int r) {
     if (r < MT) {
       fa[set][r] = *reinterpret_cast<const u32x4*>(sa + buf * A_ELEMS + a_frag + ks * 16 + r * 32 * LDK);
@@ -196,8 +210,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
       fb[set][jn][half * 2 + 1] = v.y;
     }
   };
-  constexpr int kReads = MT + 8;                              // LDS reads per k-step
-  constexpr int kSlots = MT * 4;                              // MFMAs per k-step
+  constexpr int kReads = MT + 2 * NT;                         // LDS reads per k-step
+  constexpr int kSlots = MT * NT;                             // MFMAs per k-step
+  static_assert(kSlots >= NA && kSlots >= NB, "one LDS write / global load per MFMA slot");
   constexpr int kReadsPerSlot = (kReads + kSlots - 1) / kSlots;
   constexpr int kSteps = BK / 16;
 
@@ -224,18 +239,19 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     for (int ks = 0; ks < kSteps; ++ks) {
 #pragma unroll
       for (int q = 0; q < kSlots; ++q) {
-        const int i = q / 4, jn = q % 4;
+        const int i = q / NT, jn = q % NT;
         acc[i][jn] = mfma32<BF16>(fa[ks & 1][i], fb[ks & 1][jn], acc[i][jn]);
         if (ks + 1 < kSteps) {
 #pragma unroll
           for (int r = q * kReadsPerSlot; r < (q + 1) * kReadsPerSlot; ++r)
             if (r < kReads) read_one(buf, ks + 1, (ks + 1) & 1, r);
         }
-        if (ks == 0 && q < 2 * MT)
-          *reinterpret_cast<u32x4*>(da + (a_row + 32 * q) * LDK + a_chunk * 8) = ra[q];
-        if (ks == 1 && q < 8) *reinterpret_cast<u32x4*>(db + (b_row + 8 * q) * LDN + b_chunk * 8) = rb[q];
-        if (ks == 2 && q < 2 * MT) load_a(k_next, q);
-        if (ks == 3 && q < 8) load_b(k_next, q);
+        if (ks == 0 && q < NA)
+          *reinterpret_cast<u32x4*>(da + (a_row + (T / 8) * q) * LDK + a_chunk * 8) = ra[q];
+        if (ks == 1 && q < NB)
+          *reinterpret_cast<u32x4*>(db + (b_row + (T / 32) * q) * LDN + b_chunk * 8) = rb[q];
+        if (ks == 2 && q < NA) load_a(k_next, q);
+        if (ks == 3 && q < NB) load_b(k_next, q);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -256,15 +272,15 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
       if (row >= p.m) continue;
       if constexpr (DUAL) {
 #pragma unroll
-        for (int jn = 0; jn < 2; ++jn) {
-          const int col = n0 + wn * 64 + jn * 32 + (lane & 31);
+        for (int jn = 0; jn < NT / 2; ++jn) {
+          const int col = n0 + wn * (16 * NT) + jn * 32 + (lane & 31);
           if (col < p.n)
-            store_out<OutT>(c + (int64_t)row * p.ldc + col, silu(acc[i][jn][r]) * acc[i][jn + 2][r]);
+            store_out<OutT>(c + (int64_t)row * p.ldc + col, silu(acc[i][jn][r]) * acc[i][jn + NT / 2][r]);
         }
       } else {
 #pragma unroll
-        for (int jn = 0; jn < 4; ++jn) {
-          const int col = n0 + wn * 128 + jn * 32 + (lane & 31);
+        for (int jn = 0; jn < NT; ++jn) {
+          const int col = n0 + wn * (32 * NT) + jn * 32 + (lane & 31);
           if (col < p.n) {
             if (p.splits > 1)
               unsafeAtomicAdd(reinterpret_cast<float*>(p.c) + (int64_t)row * p.ldc + col, acc[i][jn][r]);
@@ -278,32 +294,33 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 }
 
 
-template <int MT, int NBUF, bool DUAL, bool BF16, bool EDGE, typename OutT>
+template <int MT, int WM, int WN, bool DUAL, bool BF16, bool EDGE, typename OutT>
 int launch_gemm_e(GemmParams p, hipStream_t st) {
-  constexpr int BM = 64 * MT;
+  constexpr int BM = 32 * MT * WM;
+  constexpr int NBUF = 2;
   p.tiles_m = (p.m + BM - 1) / BM;
   const int bn_out = DUAL ? BN / 2 : BN;
   p.tiles_n = (p.n + bn_out - 1) / bn_out;
   const size_t smem = (size_t)NBUF * (BM * LDK + BK * LDN) * sizeof(uint16_t);
-  auto kern = gemm_kernel<MT, NBUF, DUAL, BF16, EDGE, OutT>;
+  auto kern = gemm_kernel<MT, WM, WN, DUAL, BF16, EDGE, OutT>;
   static bool attr_set = false;  // per instantiation
   if (!attr_set) {
     PTO_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(256), smem, st, p);
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(64 * WM * WN), smem, st, p);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
 }
 
-template <int MT, int NBUF, bool DUAL, bool BF16, typename OutT>
+template <int MT, int WM, int WN, bool DUAL, bool BF16, typename OutT>
 int launch_gemm(GemmParams p, hipStream_t st) {
-  constexpr int BM_ = 64 * MT;
+  constexpr int BM_ = 32 * MT * WM;
   const bool edge = p.m % BM_ != 0 || p.n % (DUAL ? BN / 2 : BN) != 0 || p.k % BK != 0 ||
                     (p.splits > 1 && p.k_per_split % BK != 0);
-  return edge ? launch_gemm_e<MT, NBUF, DUAL, BF16, true, OutT>(p, st)
-              : launch_gemm_e<MT, NBUF, DUAL, BF16, false, OutT>(p, st);
+  return edge ? launch_gemm_e<MT, WM, WN, DUAL, BF16, true, OutT>(p, st)
+              : launch_gemm_e<MT, WM, WN, DUAL, BF16, false, OutT>(p, st);
 }
 
 __global__ __launch_bounds__(256) void zero_kernel(float4* p, size_t n4) {
@@ -316,20 +333,22 @@ int launch_variant(GemmParams p, hipStream_t st) {
   const int64_t variant = pto_hip::ctx().gemm_variant;
   p.splits = 1;
   p.k_per_split = p.k;
-  // variant 1: 256x256 tile; variant 2: 128x256 tile; variant 3: 256x256 tile, k split in two.
-  // variant 0 prefers the large tile; when that leaves CUs without a workgroup it splits k in
-  // two for a contiguous fp32 output (sum of two terms: the result does not depend on which
-  // half arrives first) and otherwise falls back to the smaller tile.
+  // variant 0 (default) and 4: 256x256 tile, eight wavefronts (two per SIMD); variants 1-3 keep four
+  // wavefronts (one per SIMD): 1 = 256x256 tile, 2 = 128x256 tile, 3 = 256x256 tile with k split in two.
+  // When the large tile leaves CUs without a workgroup, variants 0 and 4 split k in two for a
+  // contiguous fp32 output (sum of two terms: the result does not depend on which half arrives
+  // first); variant 0 otherwise falls back to the smaller tile.
   const int64_t big_tiles = (int64_t)((p.m + 255) / 256) * ((p.n + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256));
   const bool can_split = !DUAL && sizeof(OutT) == 4 && p.ldc == p.n && ((int64_t)p.m * p.n) % 4 == 0 &&
                          p.k >= 4 * BK;
+  const bool eight = variant == 0 || variant == 4;
   bool split = variant == 3 && can_split;
   bool small = variant == 2;
-  if (variant == 0 && big_tiles < pto_hip::ctx().num_cu) {
+  if (eight && big_tiles < pto_hip::ctx().num_cu) {
     if (can_split && big_tiles * 2 >= pto_hip::ctx().num_cu / 2) split = true;
-    else small = true;
+    else if (variant == 0) small = true;
   }
-  if (small) return launch_gemm<2, 2, DUAL, BF16, OutT>(p, st);
+  if (small) return launch_gemm<2, 2, 2, DUAL, BF16, OutT>(p, st);
   if (split) {
     p.splits = 2;
     p.k_per_split = ((p.k + 2 * BK - 1) / (2 * BK)) * BK;
@@ -337,7 +356,8 @@ int launch_variant(GemmParams p, hipStream_t st) {
     hipLaunchKernelGGL(zero_kernel, dim3(1024), dim3(256), 0, st, reinterpret_cast<float4*>(p.c), n4);
     PTO_CHECK_HIP(hipGetLastError());
   }
-  return launch_gemm<4, 2, DUAL, BF16, OutT>(p, st);
+  if (eight) return launch_gemm<4, 2, 4, DUAL, BF16, OutT>(p, st);
+  return launch_gemm<4, 2, 2, DUAL, BF16, OutT>(p, st);
 }
 
 template <bool DUAL>
