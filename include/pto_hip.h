@@ -290,10 +290,11 @@ PTO_HIP_API int pto_hip_select_program(const char* orchestration_name, const Pto
  *  "attn_variant"               0 = one wavefront per (sequence, KV head, partition), 1 = one pinned
  *                               workgroup per CU and the chunk list cut evenly over their wavefronts,
  *                               -1 = by launch size (default)
- *  "gemm_variant"               FFN GEMM tiling: 0 = default choice (256x256 tile, 8 wavefronts),
- *                               1..3 = 4-wavefront alternatives (256-row tile, 128-row tile, 256-row
- *                               tile with k split in two), 4 = 8 wavefronts without the small-tile
- *                               fallback
+ *  "gemm_variant"               FFN GEMM tiling: 0 = default choice (8 wavefronts; 256x256 tile, or
+ *                               128x256 when that leaves CUs idle), 1..3 = 4-wavefront alternatives
+ *                               (256-row tile, 128-row tile, 256-row tile with k split in two),
+ *                               4 = 8 wavefronts, 256-row tile, k split when CUs would idle,
+ *                               5 = 8 wavefronts, 128-row tile
  *  "w8a16_wgs_per_cu"           workgroups per CU the W8A16 k split aims at (default 1)
  *  "w8a16_min_steps"            fewest 32-row steps per wavefront before k is split further
  *                               (default 8)

@@ -333,30 +333,27 @@ int launch_variant(GemmParams p, hipStream_t st) {
   const int64_t variant = pto_hip::ctx().gemm_variant;
   p.splits = 1;
   p.k_per_split = p.k;
-  // variant 0 (default) and 4: 256x256 tile, eight wavefronts (two per SIMD); variants 1-3 keep four
-  // wavefronts (one per SIMD): 1 = 256x256 tile, 2 = 128x256 tile, 3 = 256x256 tile with k split in two.
-  // When the large tile leaves CUs without a workgroup, variants 0 and 4 split k in two for a
-  // contiguous fp32 output (sum of two terms: the result does not depend on which half arrives
-  // first); variant 0 otherwise falls back to the smaller tile.
+  // variant 0 (default): eight wavefronts (two per SIMD) on a 256x256 tile, or on a 128x256 tile
+  // when the large one would leave CUs without a workgroup (measured on the LLaMA-7B down pass:
+  // 183 us against 223 us for the large tile with k split in two and fp32 atomics).
+  // variants 1-3 keep four wavefronts (one per SIMD): 1 = 256x256 tile, 2 = 128x256 tile,
+  // 3 = 256x256 tile with k split in two (contiguous fp32 output; a two-term sum does not depend
+  // on which half arrives first).  4 = eight wavefronts, 256x256 tile, k split in two when CUs
+  // would idle.  5 = eight wavefronts, 128x256 tile.
   const int64_t big_tiles = (int64_t)((p.m + 255) / 256) * ((p.n + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256));
   const bool can_split = !DUAL && sizeof(OutT) == 4 && p.ldc == p.n && ((int64_t)p.m * p.n) % 4 == 0 &&
                          p.k >= 4 * BK;
-  const bool eight = variant == 0 || variant == 4;
-  bool split = variant == 3 && can_split;
-  bool small = variant == 2;
-  if (eight && big_tiles < pto_hip::ctx().num_cu) {
-    if (can_split && big_tiles * 2 >= pto_hip::ctx().num_cu / 2) split = true;
-    else if (variant == 0) small = true;
-  }
-  if (small) return launch_gemm<2, 2, 2, DUAL, BF16, OutT>(p, st);
-  if (split) {
+  const bool few = big_tiles < pto_hip::ctx().num_cu;
+  if (variant == 5 || (variant == 0 && few)) return launch_gemm<2, 2, 4, DUAL, BF16, OutT>(p, st);
+  if (variant == 2) return launch_gemm<2, 2, 2, DUAL, BF16, OutT>(p, st);
+  if (can_split && (variant == 3 || (variant == 4 && few))) {
     p.splits = 2;
     p.k_per_split = ((p.k + 2 * BK - 1) / (2 * BK)) * BK;
     const size_t n4 = (size_t)p.m * p.n / 4;
     hipLaunchKernelGGL(zero_kernel, dim3(1024), dim3(256), 0, st, reinterpret_cast<float4*>(p.c), n4);
     PTO_CHECK_HIP(hipGetLastError());
   }
-  if (eight) return launch_gemm<4, 2, 4, DUAL, BF16, OutT>(p, st);
+  if (variant == 0 || variant == 4) return launch_gemm<4, 2, 4, DUAL, BF16, OutT>(p, st);
   return launch_gemm<4, 2, 2, DUAL, BF16, OutT>(p, st);
 }
 

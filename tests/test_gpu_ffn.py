@@ -41,7 +41,7 @@ def test_ffn_reference_example_fp32(worker):
     assert torch.allclose(out, oracle.ffn_swiglu(x, wg, wu, wd), rtol=3e-3, atol=3e-3)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
 def test_ffn_tiny_fp16(worker, variant):
     """x[128,512] fp16, I=1024, weights N(0,0.02), seed 0; max-abs 1e-2 / rel 2e-2."""
     inp = workloads.ffn_tiny(seed=0)
@@ -56,7 +56,7 @@ def test_ffn_tiny_fp16(worker, variant):
     validate_golden({"out": inp.out}, {"out": ref32}, rtol=2e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("t,h,i", [(256, 512, 1024), (100, 264, 520), (512, 1024, 2816)])
 def test_ffn_block_bf16(worker, variant, t, h, i):
     """RMSNorm prologue + SwiGLU FFN, bf16, incl. shapes that are not tile multiples."""
