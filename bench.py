@@ -133,8 +133,10 @@ def main() -> int:
         torch.cuda.synchronize()
         with worker.register(ffn_block) as fh:
             fargs = [(f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.out, f.eps)]
-            benchmark(fh, fargs, rounds=10, warmup=0)
-            fstats = benchmark(fh, fargs, rounds=20, warmup=0)
+            # the clocks need some tens of milliseconds of MFMA load to settle: the first rounds of a
+            # process run ~10 % slower than the steady state
+            benchmark(fh, fargs, rounds=40, warmup=0)
+            fstats = benchmark(fh, fargs, rounds=40, warmup=0)
         tflops = f.flops() / fstats.device_wall_us / 1e6
         result["ffn"] = {
             "workload": "FFN LLaMA-7B: T2048 H4096 I11008 bf16, RMSNorm prologue, SwiGLU, fp32 accumulate",
