@@ -30,9 +30,9 @@ KV_POOLS = 4                   # 4 x 537 MB of K+V, cycled
 # FETCH_SIZE and --pmc WRITE_SIZE (KiB per dispatch) of this script, each scaled by what the same
 # counter reads for a plain 1 GiB device copy (FETCH_SIZE reads 0.5 KiB per KiB copied, WRITE_SIZE
 # 1.0).  The counter runs and their figures are in profiles/bench_attention_small_ffn_llama7b.md.
-PMC_FETCH_KIB = 74364.9
-PMC_FETCH_SCALE = 1048576.0 / 524320.0
-PMC_WRITE_KIB = 1284.9
+PMC_FETCH_KIB = 74372.5
+PMC_FETCH_SCALE = 1048576.0 / 524321.0
+PMC_WRITE_KIB = 1284.8
 PMC_WRITE_SCALE = 1.0
 
 
