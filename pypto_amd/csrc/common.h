@@ -40,10 +40,6 @@ struct Context {
   // Grow-only device scratch for partial results (attention partitions, FFN intermediates).
   void* workspace = nullptr;
   size_t workspace_bytes = 0;
-  // Zero-initialised arrival counters for kernels whose last workgroup merges partial results;
-  // every such kernel leaves them zero again.
-  int* counters = nullptr;
-  size_t counters_len = 0;
   // Intermediates of the composed decoder layer (grow-only).
   void* layer_ws = nullptr;
   size_t layer_ws_bytes = 0;
@@ -63,8 +59,6 @@ Context& ctx();
 // Returns a workspace of at least `bytes` (reallocates if too small; stream-ordered callers
 // must not hold an older pointer across a growing call).
 int workspace(size_t bytes, void** ptr);
-// Returns `n` zeroed int counters (grown on demand; same caveat as workspace()).
-int counters(size_t n, int** ptr);
 
 // ---- W8A16 decode projections, shared with the composed decoder layer -------------------
 constexpr int kW8Slab = 128;  // output channels per workgroup of the partial kernel

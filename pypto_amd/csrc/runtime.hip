@@ -50,25 +50,6 @@ int workspace(size_t bytes, void** ptr) {
   return PTO_HIP_OK;
 }
 
-int counters(size_t n, int** ptr) {
-  Context& c = ctx();
-  if (n > c.counters_len) {
-    PTO_CHECK_HIP(hipDeviceSynchronize());
-    if (c.layer_ws) PTO_CHECK_HIP(hipFree(c.layer_ws));
-  c.layer_ws = nullptr;
-  c.layer_ws_bytes = 0;
-  if (c.counters) PTO_CHECK_HIP(hipFree(c.counters));
-    c.counters = nullptr;
-    c.counters_len = 0;
-    size_t want = n + n / 2 + 1024;
-    PTO_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&c.counters), want * sizeof(int)));
-    PTO_CHECK_HIP(hipMemset(c.counters, 0, want * sizeof(int)));
-    c.counters_len = want;
-  }
-  *ptr = c.counters;
-  return PTO_HIP_OK;
-}
-
 namespace {
 
 enum ProgramKind {
@@ -538,9 +519,6 @@ int pto_hip_close(void) {
   if (c.layer_ws) PTO_CHECK_HIP(hipFree(c.layer_ws));
   c.layer_ws = nullptr;
   c.layer_ws_bytes = 0;
-  if (c.counters) PTO_CHECK_HIP(hipFree(c.counters));
-  c.counters = nullptr;
-  c.counters_len = 0;
   c.initialized = false;
   {
     std::lock_guard<std::mutex> lk(g_mu);
