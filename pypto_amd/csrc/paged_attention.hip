@@ -487,6 +487,7 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
 // Merge of the per-partition (m, l, o): the online-update algebra of
 // examples/models/04_paged_attention.py:186-215 applied across partitions, then o / l.
 // One wavefront per output row; partitions are read four at a time so that their loads overlap.
+constexpr int kReduceFast = 8;  // partition counts up to this take the single-round-trip path
 template <int D>
 __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
   const int lane = threadIdx.x & 63;
@@ -499,6 +500,52 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
   const int np = (ctx + p.tpp - 1) / p.tpp;
   const float* ml = p.part_ml + (size_t)row * p.n_part * 2;
   const float* po = p.part_o + (size_t)row * p.n_part * D;
+  if (p.n_part <= kReduceFast) {
+    // Few partitions: every slot the row could use is fetched at once, before the context length
+    // is known, so the launch is one memory round trip instead of three; slots past np (never
+    // written, or stale) are dropped by select, not by a zero weight.
+    float pm[kReduceFast], pl[kReduceFast], pv[kReduceFast][D / 64];
+#pragma unroll
+    for (int u = 0; u < kReduceFast; ++u) {
+      const int i = min(u, p.n_part - 1);
+      pm[u] = ml[2 * i];
+      pl[u] = ml[2 * i + 1];
+#pragma unroll
+      for (int k = 0; k < D / 64; ++k) pv[u][k] = po[(size_t)i * D + k * 64 + lane];
+    }
+    float m = kMinMax;
+#pragma unroll
+    for (int u = 0; u < kReduceFast; ++u) m = u < np ? fmaxf(m, pm[u]) : m;
+    float l = 0.f, o[D / 64];
+#pragma unroll
+    for (int k = 0; k < D / 64; ++k) o[k] = 0.f;
+#pragma unroll
+    for (int u = 0; u < kReduceFast; ++u) {
+      const float wgt = __builtin_amdgcn_exp2f(pm[u] - m);
+      if (u < np) {
+        l += wgt * pl[u];
+#pragma unroll
+        for (int k = 0; k < D / 64; ++k) o[k] += wgt * pv[u][k];
+      }
+    }
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+    for (int k = 0; k < D / 64; ++k) {
+      const float y = o[k] * inv;
+      const size_t idx = (size_t)row * D + k * 64 + lane;
+      p.out[idx] = y;
+      if (p.out16) {
+        size_t i16 = idx;
+        if (p.out16_blocked) {
+          const int bb = row / p.hq, kk = (row % p.hq) * D + k * 64 + lane;
+          i16 = ((size_t)(kk >> 3) * 32 + bb) * 8 + (kk & 7);
+        }
+        if (p.out16_bf16) reinterpret_cast<__bf16*>(p.out16)[i16] = (__bf16)y;
+        else reinterpret_cast<_Float16*>(p.out16)[i16] = (_Float16)y;
+      }
+    }
+    return;
+  }
   // lane i holds (m, l) of partitions i, i+64, ...
   float m = kMinMax;
   for (int i = lane; i < np; i += 64) m = fmaxf(m, ml[2 * i]);
