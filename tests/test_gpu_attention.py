@@ -82,6 +82,35 @@ def test_shapes_and_edges(worker, batch, hq, hkv, d, bs, ctxs):
         assert (out[i * rows:(i + 1) * rows] == 0).all()
 
 
+@pytest.mark.parametrize(
+    "batch,num_heads,head_dim,block_size,context_len,max_model_len",
+    [
+        # the reference's own configuration list (one KV head, uniform context length):
+        # tests/st/runtime/framework_and_models/test_paged_attention_multi_config.py:689-720
+        (4, 16, 128, 64, 1024, 2048),
+        (4, 16, 128, 128, 1024, 2048),
+        (4, 64, 128, 64, 1024, 2048),
+        (4, 64, 256, 64, 1024, 2048),
+        (4, 16, 128, 64, 1000, 2048),
+        (4, 16, 128, 64, 700, 2048),
+        (4, 16, 128, 128, 500, 2048),
+        (1, 16, 128, 64, 64, 2048),
+        (1, 16, 128, 64, 50, 2048),
+        (2, 16, 128, 64, 100, 2048),
+        (1, 16, 128, 64, 1000, 2048),
+        (4, 64, 128, 64, 700, 2048),
+    ],
+)
+def test_reference_multi_config_list(worker, batch, num_heads, head_dim, block_size, context_len, max_model_len):
+    inp = workloads.paged_attention_inputs(batch=batch, num_heads=num_heads, kv_head_num=1, head_dim=head_dim,
+                                           block_size=block_size, context_lens=[context_len] * batch,
+                                           ctx_range=(1, context_len),
+                                           max_num_blocks_per_req=max_model_len // block_size, seed=13)
+    ref = _golden(inp)
+    for tpp in (0, -4):
+        _check(_run(worker, inp, tpp), ref)
+
+
 def test_fp16_cache(worker):
     inp = workloads.paged_attention_inputs(batch=3, num_heads=16, kv_head_num=4, context_lens=[300, 17, 129],
                                            ctx_range=(1, 300), dtype=torch.float16, seed=3)
