@@ -201,7 +201,8 @@ def main() -> int:
         host = [t.cpu() for t in (p.query, p.key_cache, p.value_cache, p.block_table, p.context_lens, p.config)]
         times = []
         oracle.paged_attention_golden(*host)  # warm-up
-        for _ in range(3):
+        t_begin = time.perf_counter()
+        while len(times) < 5 or (time.perf_counter() - t_begin < 10.0 and len(times) < 400):
             t0 = time.perf_counter()
             oracle.paged_attention_golden(*host)
             times.append(time.perf_counter() - t0)
@@ -211,8 +212,8 @@ def main() -> int:
             "unit": "GB/s",
             "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": "one full step of the same workload (torch block-loop golden), median of 3 after 1 warm-up; "
-                      f"{med * 1e3:.1f} ms per step, os.cpu_count()={os.cpu_count()}",
+            "sample": f"full steps of the same workload (torch block-loop golden) for ~10 s after 1 warm-up: median of "
+                      f"{len(times)} steps, {med * 1e3:.1f} ms per step, os.cpu_count()={os.cpu_count()}",
         }
 
     if args.calibrate_copy:
