@@ -48,3 +48,30 @@ def test_calls_before_init_fail_loudly():
     assert lib.pto_hip_set_option(b"no_such_option", 1) == _lib.ERR_NOT_FOUND
     with pytest.raises(ValueError, match="unknown option"):
         _lib.check(lib.pto_hip_set_option(b"no_such_option", 1))
+
+
+def test_options_round_trip_and_ranges():
+    """Every documented knob can be set and read back; out-of-range values are ValueError."""
+    lib = _lib.load()
+    knobs = {"attn_tokens_per_partition": 256, "attn_waves_per_cu": 4, "attn_skip_merge": 1, "attn_variant": 1,
+             "gemm_variant": 2, "w8a16_wgs_per_cu": 3, "w8a16_min_steps": 16}
+    for name, value in knobs.items():
+        old = ctypes.c_int64(-99)
+        _lib.check(lib.pto_hip_get_option(name.encode(), ctypes.byref(old)))
+        _lib.check(lib.pto_hip_set_option(name.encode(), value))
+        got = ctypes.c_int64(-99)
+        _lib.check(lib.pto_hip_get_option(name.encode(), ctypes.byref(got)))
+        assert got.value == value, name
+        _lib.check(lib.pto_hip_set_option(name.encode(), old.value))
+    for name, bad in (("attn_variant", 2), ("attn_waves_per_cu", 17), ("attn_tokens_per_partition", -1),
+                      ("w8a16_wgs_per_cu", 0), ("w8a16_min_steps", 0)):
+        with pytest.raises(ValueError, match=name):
+            _lib.check(lib.pto_hip_set_option(name.encode(), bad))
+    with pytest.raises(ValueError, match="unknown option"):
+        _lib.check(lib.pto_hip_get_option(b"nope", ctypes.byref(ctypes.c_int64())))
+
+
+def test_manifest_kernel_layout_matches_header():
+    # PtoHipManifestKernel: i32 func_id, i32 core_type, const char* name
+    assert ctypes.sizeof(_lib.ManifestKernel) == 16
+    assert _lib.ManifestKernel.name.offset == 8
