@@ -168,6 +168,10 @@ PTO_HIP_API int pto_hip_paged_attention(const void* query, const void* key_cache
                                         const int64_t* config, int q_dtype, int kv_dtype,
                                         const float* k_scale, const float* v_scale, void* stream);
 
+/* out[i, :] = src[block_table[idx / bs] * bs + idx % bs, col_offset : col_offset + size]
+ * (src/ir/op/tensor_ops/paged_gather.cpp:74-199), bit-exact, asynchronous on the stream.  An index
+ * that addresses a block outside block_table or a row outside src is skipped and reported by
+ * the next pto_hip_sync. */
 PTO_HIP_API int pto_hip_paged_gather(const void* src, const int32_t* indices,
                                      const int32_t* block_table, void* out, int64_t n_indices,
                                      int64_t src_rows, int64_t src_hidden, int64_t table_len,

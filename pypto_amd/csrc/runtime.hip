@@ -582,8 +582,11 @@ int pto_hip_sync(void* stream) {
   // Device-side argument errors of launches that do not block are reported here.
   int flags[2] = {0, 0};
   PTO_CHECK_HIP(hipMemcpy(flags, ctx().flags, sizeof(flags), hipMemcpyDeviceToHost));
-  if (flags[1]) {
-    PTO_CHECK_HIP(hipMemset(ctx().flags + 1, 0, sizeof(int)));
+  if (flags[0] || flags[1]) {
+    PTO_CHECK_HIP(hipMemset(ctx().flags, 0, sizeof(flags)));
+    if (flags[0])
+      return fail(PTO_HIP_ERR_INVALID_VALUE,
+                  "paged_gather: an index addresses a block outside block_table or a row outside src");
     return fail(PTO_HIP_ERR_INVALID_VALUE,
                 "rope_kv_cache_update: a decode position lies outside the rope table, the block table or the cache");
   }
