@@ -3,8 +3,8 @@
 // Semantics of tensor.paged_gather (src/ir/op/tensor_ops/paged_gather.cpp:74-199; golden in
 // tests/st/runtime/ops/test_paged_gather.py:68-78).  Pure index arithmetic and byte copies, so
 // results are bit-exact for every element type.  The reference lowers this to a scalar per-row
-// DMA loop on one core; here one 64-lane wavefront copies one row with 16-byte accesses when
-// the row segment is 16-byte aligned, bytes otherwise.
+// DMA loop on one core; here a group of lanes copies one row with 16-byte accesses when the row
+// segment is 16-byte aligned, bytes otherwise, and a wavefront has several rows in flight.
 #include <hip/hip_runtime.h>
 
 #include "common.h"
@@ -21,30 +21,53 @@ struct GatherParams {
   int* error_flag;  // set to 1 when an index falls outside the table or the pool
 };
 
-__global__ __launch_bounds__(256) void paged_gather_kernel(GatherParams p) {
+// One lane group of `lanes_per_row` lanes (a power of two, 1..64) copies one row; a wavefront
+// takes kUnroll sets of 64 / lanes_per_row rows (4 sets for rows up to 1 KB, 1 for longer rows,
+// which already keep a wavefront's lanes busy), and issues the index loads of all sets, then
+// the table loads, then the copies, so that the three dependent accesses of a row overlap with
+// those of the others.
+template <int kUnroll>
+__global__ __launch_bounds__(256) void paged_gather_kernel(GatherParams p, int lanes_per_row) {
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= p.n) return;
-  const int64_t li = p.indices[row];
-  const int64_t lb = li / p.bs;
-  if (li < 0 || lb >= p.table_len) {
-    if (lane == 0) *p.error_flag = 1;
-    return;
+  const int rows_per_set = 64 / lanes_per_row;
+  const int group = lane / lanes_per_row, sub = lane % lanes_per_row;
+  const int64_t wave_id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t row0 = wave_id * (rows_per_set * kUnroll) + group;
+
+  int64_t li[kUnroll], phys[kUnroll];
+  bool ok[kUnroll];
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const int64_t row = row0 + (int64_t)u * rows_per_set;
+    ok[u] = row < p.n;
+    li[u] = ok[u] ? p.indices[row] : 0;
   }
-  const int64_t phys = (int64_t)p.table[lb] * p.bs + li % p.bs;
-  if (phys < 0 || phys >= p.src_rows) {
-    if (lane == 0) *p.error_flag = 1;
-    return;
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const int64_t lb = li[u] / p.bs;
+    const bool in_table = li[u] >= 0 && lb < p.table_len;
+    if (ok[u] && !in_table && sub == 0) *p.error_flag = 1;
+    ok[u] = ok[u] && in_table;
+    phys[u] = ok[u] ? (int64_t)p.table[lb] * p.bs + li[u] % p.bs : 0;
   }
-  const uint8_t* s = p.src + phys * p.src_row_bytes + p.col_off_bytes;
-  uint8_t* d = p.out + row * p.out_row_bytes;
-  const int64_t nb = p.out_row_bytes;
-  if ((((uintptr_t)s | (uintptr_t)d | (uintptr_t)nb) & 15) == 0) {
-    const uint4* s4 = reinterpret_cast<const uint4*>(s);
-    uint4* d4 = reinterpret_cast<uint4*>(d);
-    for (int64_t i = lane; i < nb / 16; i += 64) d4[i] = s4[i];
-  } else {
-    for (int64_t i = lane; i < nb; i += 64) d[i] = s[i];
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    if (!ok[u]) continue;
+    if (phys[u] < 0 || phys[u] >= p.src_rows) {
+      if (sub == 0) *p.error_flag = 1;
+      continue;
+    }
+    const int64_t row = row0 + (int64_t)u * rows_per_set;
+    const uint8_t* s = p.src + phys[u] * p.src_row_bytes + p.col_off_bytes;
+    uint8_t* d = p.out + row * p.out_row_bytes;
+    const int64_t nb = p.out_row_bytes;
+    if ((((uintptr_t)s | (uintptr_t)d | (uintptr_t)nb) & 15) == 0) {
+      const uint4* s4 = reinterpret_cast<const uint4*>(s);
+      uint4* d4 = reinterpret_cast<uint4*>(d);
+      for (int64_t i = sub; i < nb / 16; i += lanes_per_row) d4[i] = s4[i];
+    } else {
+      for (int64_t i = sub; i < nb; i += lanes_per_row) d[i] = s[i];
+    }
   }
 }
 
@@ -86,9 +109,16 @@ extern "C" int pto_hip_paged_gather(const void* src, const int32_t* indices,
   p.out_row_bytes = size * elem_bytes;
   p.col_off_bytes = col_offset * elem_bytes;
   p.error_flag = flag;
-  const int64_t blocks = (n_indices + 3) / 4;
+  // lanes per row: enough 16-byte lanes to cover a row segment in one pass, as a power of two
+  int lanes_per_row = 64;
+  while (lanes_per_row > 1 && (int64_t)(lanes_per_row / 2) * 16 >= p.out_row_bytes) lanes_per_row /= 2;
+  const int unroll = p.out_row_bytes <= 1024 ? 4 : 1;
+  const int64_t rows_per_wave = (int64_t)(64 / lanes_per_row) * unroll;
+  const int64_t waves = (n_indices + rows_per_wave - 1) / rows_per_wave;
+  const int64_t blocks = (waves + 3) / 4;
   PTO_CHECK_ARG(blocks < (1ll << 31), "paged_gather: too many indices (%lld)", (long long)n_indices);
-  hipLaunchKernelGGL(paged_gather_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p);
+  if (unroll == 1) hipLaunchKernelGGL(paged_gather_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, st, p, lanes_per_row);
+  else hipLaunchKernelGGL(paged_gather_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, st, p, lanes_per_row);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
 }
