@@ -225,3 +225,36 @@ def test_fp8_rejects_small_blocks(worker):
                                            context_lens=[40], ctx_range=(1, 40), fp8_kv=True, seed=13)
     with pytest.raises(ValueError, match="block_size % 32"):
         _run(worker, inp)
+
+
+def test_full_size_long_fp8_config_properties(worker):
+    """B64 Hq64 Hkv8 ctx~U[8192,32768] e4m3 (2.8 GB of cache, built on the GPU): the two launch
+    forms cut the work differently (fixed partitions vs even chunk runs) and must agree; three
+    whole sequences are checked against the oracle on the CPU."""
+    inp = workloads.attention_long_fp8(seed=0, device="cuda")
+    outs = {}
+    for name, variant in (("grid", 0), ("split", 1), ("auto", -1)):
+        worker.set_option("attn_variant", variant)
+        inp.out.fill_(float("nan"))
+        with worker.register(paged_attention) as h:
+            h(*inp.args())
+        worker.sync()
+        outs[name] = inp.out.clone()
+    worker.set_option("attn_variant", -1)
+    assert torch.isfinite(outs["grid"]).all()
+    assert (outs["grid"] - outs["split"]).abs().max().item() < 2e-3
+    assert torch.equal(outs["auto"], outs["split"])  # a launch of this size takes the evenly split form
+    cfg = inp.config.tolist()
+    b, hq, hkv, d, bs, mb = cfg[:6]
+    table = inp.block_table.reshape(b, mb)
+    for seq in (0, 17, 63):
+        nblk = (int(inp.context_lens[seq]) + bs - 1) // bs
+        blocks = table[seq, :nblk].long()
+        rows = (blocks[:, None, None] * hkv * bs + torch.arange(hkv, device="cuda")[None, :, None] * bs
+                + torch.arange(bs, device="cuda")[None, None, :]).reshape(-1)
+        sub_cfg = torch.tensor([1, hq, hkv, d, bs, nblk, cfg[6]], dtype=torch.int64)
+        ref = oracle.paged_attention_golden(
+            inp.query[seq * hq:(seq + 1) * hq].cpu(), inp.key_cache[rows].cpu(), inp.value_cache[rows].cpu(),
+            torch.arange(nblk, dtype=torch.int32), inp.context_lens[seq:seq + 1].cpu(), sub_cfg,
+            inp.k_scale[blocks].cpu(), inp.v_scale[blocks].cpu())
+        _check(outs["split"][seq * hq:(seq + 1) * hq].cpu(), ref)
