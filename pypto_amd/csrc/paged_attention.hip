@@ -951,9 +951,10 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
 
   // Launches that may stream a gigabyte or more of cache take the evenly split form: there the
   // spread of partition lengths costs more than that form's longer start-up (measured: +11 % on
-  // 2.8 GB with contexts of 8K-32K, nothing on 150 MB).  "attn_variant" 0/1 forces the choice.
+  // 2.8 GB with contexts of 8K-32K, nothing on 150 MB).  head_dim 256 stays on the partition grid:
+  // the pinned workgroup's register budget makes that kernel spill.  "attn_variant" 0/1 forces the choice.
   const int64_t kv_bound = batch * hkv * p.gtiles * max_ctx * 2 * d * (fp8 ? 1 : 2);
-  const bool lean = cx.attn_variant >= 0 ? cx.attn_variant == 1 : kv_bound >= (1ll << 30);
+  const bool lean = cx.attn_variant >= 0 ? cx.attn_variant == 1 : (d == 128 && kv_bound >= (1ll << 30));
   if (p.n_part > 1 && !lean) {
     const size_t rows = (size_t)batch * hq;
     const size_t o_bytes = rows * p.n_part * d * sizeof(float);
