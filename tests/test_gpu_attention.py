@@ -258,3 +258,20 @@ def test_full_size_long_fp8_config_properties(worker):
             torch.arange(nblk, dtype=torch.int32), inp.context_lens[seq:seq + 1].cpu(), sub_cfg,
             inp.k_scale[blocks].cpu(), inp.v_scale[blocks].cpu())
         _check(outs["split"][seq * hq:(seq + 1) * hq].cpu(), ref)
+
+
+def test_many_sequences_with_gaps(worker):
+    """130 sequences (three 64-wide passes of the in-kernel prefix scans), a third of them empty."""
+    g = torch.Generator().manual_seed(23)
+    ctxs = torch.randint(0, 300, (130,), generator=g)
+    ctxs[torch.rand(130, generator=g) < 0.33] = 0
+    ctxs[64] = 0
+    ctxs[129] = 299
+    inp = workloads.paged_attention_inputs(batch=130, num_heads=8, kv_head_num=2, head_dim=128, block_size=32,
+                                           context_lens=ctxs.tolist(), ctx_range=(1, 300), seed=29)
+    ref = _golden(inp)
+    for tpp in (0, -1, -8, 64):
+        out = _run(worker, inp, tpp)
+        _check(out, ref)
+        empty = (ctxs == 0).repeat_interleave(8)
+        assert (out[empty] == 0).all()
