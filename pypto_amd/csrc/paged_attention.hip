@@ -661,8 +661,9 @@ __device__ __forceinline__ void lean_locate(const AttnParams& p, int lane, int h
   }
 }
 
+// head_dim 256 needs more than 256 registers per wavefront: four wavefronts (one per SIMD) there.
 template <int D, bool BF16, bool FP8>
-__global__ __launch_bounds__(kLeanMaxWaves * 64) void attn_lean_kernel(AttnParams p) {
+__global__ __launch_bounds__((D == 128 ? kLeanMaxWaves : 4) * 64) void attn_lean_kernel(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char lean_lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -951,10 +952,10 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
 
   // Launches that may stream a gigabyte or more of cache take the evenly split form: there the
   // spread of partition lengths costs more than that form's longer start-up (measured: +11 % on
-  // 2.8 GB with contexts of 8K-32K, nothing on 150 MB).  head_dim 256 stays on the partition grid:
-  // the pinned workgroup's register budget makes that kernel spill.  "attn_variant" 0/1 forces the choice.
+  // 2.8 GB of e4m3 cache with contexts of 8K-32K, +13 % on 2.7 GB at head_dim 256, within 3 % either
+  // way when all contexts are equal, nothing on 150 MB).  "attn_variant" 0/1 forces the choice.
   const int64_t kv_bound = batch * hkv * p.gtiles * max_ctx * 2 * d * (fp8 ? 1 : 2);
-  const bool lean = cx.attn_variant >= 0 ? cx.attn_variant == 1 : (d == 128 && kv_bound >= (1ll << 30));
+  const bool lean = cx.attn_variant >= 0 ? cx.attn_variant == 1 : kv_bound >= (1ll << 30);
   if (p.n_part > 1 && !lean) {
     const size_t rows = (size_t)batch * hq;
     const size_t o_bytes = rows * p.n_part * d * sizeof(float);
@@ -970,7 +971,7 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   if (lean) {
     const int64_t kbytes = (fp8 ? d : 2 * d) + 16;  // K stage row pitch
     int64_t waves = cx.attn_waves_per_cu > 0 ? cx.attn_waves_per_cu : 4;
-    if (waves > kLeanMaxWaves) waves = kLeanMaxWaves;
+    if (waves > (d == 128 ? kLeanMaxWaves : 4)) waves = d == 128 ? kLeanMaxWaves : 4;
     while (waves > 1 && waves * 32 * kbytes > 160 * 1024) --waves;
     p.n_wg = cx.num_cu;
     p.lean_waves = (int)waves;
