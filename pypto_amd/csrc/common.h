@@ -72,8 +72,12 @@ struct W8Partials {
 // Launches the partial kernel for x[M, K] @ wq0[K, N] (and wq1 when non-null).  x_blocked: x is
 // stored [K/8][32][8] - element (m, k) at ((k/8)*32 + m)*8 + k%8 - the layout the layer's own
 // producers write so that a wavefront's activation reads are whole consecutive cache lines.
+// w16: the weights are 16-bit values of the activation type instead of int8 codes (the finish
+// kernels then take null scales).
 int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* wq1, int64_t m, int64_t k,
-                   int64_t n, int x_dtype, hipStream_t st, W8Partials* out);
+                   int64_t n, int x_dtype, hipStream_t st, W8Partials* out, bool w16 = false);
+// Grow-only device scratch for intermediates that must survive calls which use workspace().
+int layer_workspace(size_t bytes, void** ptr);
 // out = cast(sum_s(part0) * scale0 [-> SiLU(.) * (sum_s(part1) * scale1)] [+ residual]).
 int w8a16_finish(const W8Partials& parts, const float* scale0, const float* scale1, const void* residual,
                  int res_dtype, void* out, int out_dtype, bool out_blocked, int64_t m, int64_t n, hipStream_t st);

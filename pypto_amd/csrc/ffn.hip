@@ -18,7 +18,9 @@
 //   * in the gate/up pass the 256 LDS columns are 128 gate + 128 up columns of the same output
 //     range, so SiLU(gate) * up is applied on the accumulators and only h is written;
 //   * workgroup ids are remapped so that the ids sharing an XCD (id mod 8) work on neighbouring
-//     tiles and share operands in that XCD's L2.
+//     tiles and share operands in that XCD's L2;
+//   * at decode-size token counts (at most 64 rows) the block is bound by reading the weights
+//     once and runs as skinny projections instead (ffn_skinny below).
 #include <hip/hip_runtime.h>
 
 #include "common.h"
@@ -391,6 +393,43 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* a, const flo
   if (row < m && col < n) c[(int64_t)row * n + col] = b1 ? silu(g) * u : g;
 }
 
+constexpr int64_t kSkinnyMaxTokens = 64;
+
+int ffn_skinny(const void* x, const float* gamma, const void* w_gate, const void* w_up, const void* w_down,
+               void* out, int64_t tokens, int64_t hidden, int64_t intermediate, float eps, int dtype,
+               int out_dtype, hipStream_t st) {
+  using namespace pto_hip;
+  const int eb = dtype_bytes(dtype), ob = dtype_bytes(out_dtype);
+  auto up = [](size_t n) { return (n + 255) / 256 * 256; };
+  // intermediates of one 32-row pass, in the blocked activation layout [K/8][32][8]
+  const size_t sz_xn = up((size_t)kW8MaxM * hidden * eb), sz_h = up((size_t)kW8MaxM * intermediate * eb);
+  void* lws = nullptr;
+  int rc = layer_workspace(sz_xn + sz_h, &lws);
+  if (rc) return rc;
+  void* xn = lws;
+  void* hbuf = reinterpret_cast<char*>(lws) + sz_xn;
+  const bool blk_x = gamma != nullptr && rms_norm_blocked_fits(kW8MaxM, hidden);
+  for (int64_t r0 = 0; r0 < tokens; r0 += kW8MaxM) {
+    const int64_t m = tokens - r0 < kW8MaxM ? tokens - r0 : kW8MaxM;
+    const void* xr = reinterpret_cast<const char*>(x) + (size_t)r0 * hidden * eb;
+    const void* a1 = xr;
+    if (gamma) {
+      if (blk_x) rc = rms_norm_blocked(xr, gamma, xn, m, hidden, eps, dtype, st);
+      else rc = pto_hip_rms_norm(xr, gamma, xn, m, hidden, eps, dtype, dtype, st);
+      if (rc) return rc;
+      a1 = xn;
+    }
+    W8Partials parts{};
+    if ((rc = w8a16_partials(a1, gamma && blk_x, w_gate, w_up, m, hidden, intermediate, dtype, st, &parts, true)))
+      return rc;
+    if ((rc = w8a16_finish(parts, nullptr, nullptr, nullptr, 0, hbuf, dtype, true, m, intermediate, st))) return rc;
+    if ((rc = w8a16_partials(hbuf, true, w_down, nullptr, m, intermediate, hidden, dtype, st, &parts, true))) return rc;
+    void* outr = reinterpret_cast<char*>(out) + (size_t)r0 * hidden * ob;
+    if ((rc = w8a16_finish(parts, nullptr, nullptr, nullptr, 0, outr, out_dtype, false, m, hidden, st))) return rc;
+  }
+  return PTO_HIP_OK;
+}
+
 }  // namespace
 
 extern "C" int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void* w_gate,
@@ -408,6 +447,16 @@ extern "C" int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void*
   const int eb = dtype_bytes(dtype);
   PTO_CHECK_ARG(dtype == PTO_HIP_BF16 || dtype == PTO_HIP_FP16 || dtype == PTO_HIP_FP32,
                 "ffn: dtype %s not in {BF16, FP16, FP32}", dtype_name(dtype));
+
+  // Decode-size token counts: the weights dominate the traffic (HBM-bound), so the block runs as
+  // skinny projections - the kernels of the W8A16 path with 16-bit weights - 32 rows at a time.
+  const bool sixteen = dtype == PTO_HIP_BF16 || dtype == PTO_HIP_FP16;
+  if (sixteen && tokens <= kSkinnyMaxTokens && ctx().gemm_variant == 0 && hidden % 16 == 0 && hidden >= 32 &&
+      intermediate % 16 == 0 && intermediate >= 32 &&
+      ((uintptr_t)x | (uintptr_t)w_gate | (uintptr_t)w_up | (uintptr_t)w_down | (uintptr_t)out |
+       (uintptr_t)gamma) % 16 == 0 &&
+      (out_dtype == PTO_HIP_FP32 || out_dtype == dtype))
+    return ffn_skinny(x, gamma, w_gate, w_up, w_down, out, tokens, hidden, intermediate, eps, dtype, out_dtype, st);
 
   const size_t xn_bytes = gamma ? ((size_t)tokens * hidden * eb + 255) / 256 * 256 : 0;
   const size_t h_bytes = (size_t)tokens * intermediate * eb;

@@ -46,15 +46,12 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
                sz_attn16 = up((size_t)b * hq * d * 2), sz_resid = up((size_t)b * h * 4),
                sz_h = up((size_t)b * inter * 2);
   const size_t total = sz_normed + sz_q + sz_attn + sz_attn16 + sz_resid + sz_normed + sz_h;
-  if (total > cx.layer_ws_bytes) {
-    PTO_CHECK_HIP(hipDeviceSynchronize());
-    if (cx.layer_ws) PTO_CHECK_HIP(hipFree(cx.layer_ws));
-    cx.layer_ws = nullptr;
-    cx.layer_ws_bytes = 0;
-    PTO_CHECK_HIP(hipMalloc(&cx.layer_ws, total));
-    cx.layer_ws_bytes = total;
+  void* lws = nullptr;
+  {
+    int rc0 = layer_workspace(total, &lws);
+    if (rc0) return rc0;
   }
-  char* w = reinterpret_cast<char*>(cx.layer_ws);
+  char* w = reinterpret_cast<char*>(lws);
   void* normed = w;              w += sz_normed;
   void* q16 = w;                 w += sz_q;
   float* attn = (float*)w;       w += sz_attn;

@@ -50,6 +50,20 @@ int workspace(size_t bytes, void** ptr) {
   return PTO_HIP_OK;
 }
 
+int layer_workspace(size_t bytes, void** ptr) {
+  Context& c = ctx();
+  if (bytes > c.layer_ws_bytes) {
+    PTO_CHECK_HIP(hipDeviceSynchronize());
+    if (c.layer_ws) PTO_CHECK_HIP(hipFree(c.layer_ws));
+    c.layer_ws = nullptr;
+    c.layer_ws_bytes = 0;
+    PTO_CHECK_HIP(hipMalloc(&c.layer_ws, bytes));
+    c.layer_ws_bytes = bytes;
+  }
+  *ptr = c.layer_ws;
+  return PTO_HIP_OK;
+}
+
 namespace {
 
 enum ProgramKind {

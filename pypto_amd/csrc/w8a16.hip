@@ -18,6 +18,8 @@
 //     The RoPE kernel reads the q/k/v partials directly.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -34,7 +36,7 @@ constexpr int kWavesPerWg = 4;           // wavefronts per workgroup of the part
 
 struct GemvParams {
   const uint16_t* x;    // [M, K] 16-bit activations
-  const int8_t* wq[2];  // [K, N] each; the second is the up projection of a gate/up pair
+  const void* wq[2];    // [K, N] each (int8 codes or 16-bit weights); the second is the up projection of a pair
   float* part[2];       // [splits, 32, N] each
   int m, k, n, slabs, n_mats, splits, k_per_split;
   int x_blocked;  // activations stored [K/8][32][8] (see w8a16_partials) instead of row-major
@@ -63,14 +65,17 @@ __device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
   }
 }
 
+// W8: int8 weight codes (8 bytes = 8 channels per row and lane); otherwise 16-bit weights of the
+// activation type (16 bytes = 8 channels).
+template <bool W8>
 struct Stage {
-  uint2 w[8];    // 8 channels of k rows kg*8 .. kg*8+7
-  u32x4 xa[2];   // activations of rows c and c+16, k = kg*8 .. +8
+  typename std::conditional<W8, uint2, u32x4>::type w[8];  // 8 channels of k rows kg*8 .. kg*8+7
+  u32x4 xa[2];                                             // activations of rows c and c+16, k = kg*8 .. +8
 };
 
 // kWaves wavefronts per workgroup, kStages register stages per wavefront (kStages - 1 in flight),
 // kOcc wavefronts per SIMD the register budget is cut for.
-template <bool BF16, int kWaves, int kStages, int kOcc>
+template <bool BF16, bool W8, int kWaves, int kStages, int kOcc>
 __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOcc, kOcc))) void w8a16_partial_kernel(
     GemvParams p) {
   constexpr int kHalf = kWaves / 2;
@@ -109,20 +114,22 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
   // multiplied by zeroed activations.  A row address is a wavefront-uniform row base plus a
   // per-lane offset that never changes.
   const int last_step = wave < n_steps ? wave + (n_steps - 1 - wave) / kWaves * kWaves : n_steps - 1;
-  const int8_t* wbase = p.wq[mat];
+  constexpr int kWBytes = W8 ? 1 : 2;  // bytes per weight
+  typedef typename std::conditional<W8, uint2, u32x4>::type wvec_t;
+  const char* wbase = reinterpret_cast<const char*>(p.wq[mat]);
   const uint32_t lane_off = (uint32_t)min(n0, p.n - 8) + (uint32_t)(kg * 8) * (uint32_t)p.n;
   auto step_row = [&](int step) { return min(k_begin + step * kStep, p.k - kStep); };
-  auto load = [&](Stage& s, int step) {
+  auto load = [&](Stage<W8>& s, int step) {
     const int kstep = step_row(min(step, last_step));
     s.xa[0] = *reinterpret_cast<const u32x4*>(xp0 + (size_t)kstep * x_step);
     s.xa[1] = *reinterpret_cast<const u32x4*>(xp1 + (size_t)kstep * x_step);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int8_t* row = wbase + (size_t)(kstep + e) * p.n;  // uniform
-      s.w[e] = *reinterpret_cast<const uint2*>(row + lane_off);
+      const char* row = wbase + (size_t)(kstep + e) * p.n * kWBytes;  // uniform
+      s.w[e] = *reinterpret_cast<const wvec_t*>(row + (size_t)lane_off * kWBytes);
     }
   };
-  auto compute = [&](const Stage& s, int step) {
+  auto compute = [&](const Stage<W8>& s, int step) {
     const int row0 = step_row(step) + kg * 8;  // first of this lane's 8 rows
     const bool k_ok = row0 >= k_begin + step * kStep && row0 < k_end;
     const u32x4 z = {0u, 0u, 0u, 0u};
@@ -132,13 +139,20 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
     for (int i = 0; i < 8; ++i) {
       // channel n0 + i: its 8 k-values, as packed pairs (k, k+1)
       u32x4 b;
+      if constexpr (W8) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint32_t w0 = i < 4 ? s.w[2 * q].x : s.w[2 * q].y;
-        const uint32_t w1 = i < 4 ? s.w[2 * q + 1].x : s.w[2 * q + 1].y;
-        const float f0 = (float)(int8_t)(w0 >> ((i & 3) * 8));
-        const float f1 = (float)(int8_t)(w1 >> ((i & 3) * 8));
-        b[q] = pack_pair<BF16>(f0, f1);
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t w0 = i < 4 ? s.w[2 * q].x : s.w[2 * q].y;
+          const uint32_t w1 = i < 4 ? s.w[2 * q + 1].x : s.w[2 * q + 1].y;
+          const float f0 = (float)(int8_t)(w0 >> ((i & 3) * 8));
+          const float f1 = (float)(int8_t)(w1 >> ((i & 3) * 8));
+          b[q] = pack_pair<BF16>(f0, f1);
+        }
+      } else {
+        // 16-bit weights: element i of rows 2q and 2q+1 (an 8x8 transpose in registers)
+        const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) b[q] = __builtin_amdgcn_perm(s.w[2 * q + 1][i >> 1], s.w[2 * q][i >> 1], sel);
       }
       acc[i][0] = mfma16<BF16>(a0, b, acc[i][0]);
       acc[i][1] = mfma16<BF16>(a1, b, acc[i][1]);
@@ -149,7 +163,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
   // Wavefront w takes steps w, w + kWaves, ...; kStages register stages, all but the one being
   // consumed in flight.  The trip count is rounded up to whole rounds of kStages: surplus steps
   // multiply by zero.
-  Stage st[kStages];
+  Stage<W8> st[kStages];
 #pragma unroll
   for (int u = 0; u < kStages - 1; ++u) load(st[u], wave + u * kWaves);
   for (int s = wave; s < n_steps; s += kStages * kWaves) {
@@ -269,6 +283,7 @@ __device__ __forceinline__ float4 sum_splits(const float* part, const float* sca
     const float4 v = *reinterpret_cast<const float4*>(src + (size_t)s * stride);
     a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
   }
+  if (!scale) return a;  // unquantised weights
   const float4 sc = *reinterpret_cast<const float4*>(scale + n);
   return float4{a.x * sc.x, a.y * sc.y, a.z * sc.z, a.w * sc.w};
 }
@@ -381,11 +396,11 @@ void choose_splits(int64_t k, int64_t slabs_total, int waves, int* splits, int* 
 namespace pto_hip {
 
 int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* wq1, int64_t m, int64_t k, int64_t n,
-                   int x_dtype, hipStream_t st, W8Partials* out) {
+                   int x_dtype, hipStream_t st, W8Partials* out, bool w16) {
   GemvParams p{};
   p.x = reinterpret_cast<const uint16_t*>(x);
-  p.wq[0] = reinterpret_cast<const int8_t*>(wq0);
-  p.wq[1] = reinterpret_cast<const int8_t*>(wq1);
+  p.wq[0] = wq0;
+  p.wq[1] = wq1;
   p.m = (int)m;
   p.k = (int)k;
   p.n = (int)n;
@@ -403,10 +418,14 @@ int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* w
   // Four wavefronts x two stages: measured best in the decoder layer against 2, 4 and 8 wavefronts
   // with 2-4 stages (more requests in flight per CU only lengthened the memory queueing delay).
   const dim3 block((unsigned)kWavesPerWg * 64);
-  if (x_dtype == PTO_HIP_BF16)
-    hipLaunchKernelGGL((w8a16_partial_kernel<true, kWavesPerWg, 2, 4>), grid, block, 0, st, p);
-  else
-    hipLaunchKernelGGL((w8a16_partial_kernel<false, kWavesPerWg, 2, 4>), grid, block, 0, st, p);
+  const bool bf = x_dtype == PTO_HIP_BF16;
+  if (w16) {  // twice the bytes per stage: three wavefronts per SIMD
+    if (bf) hipLaunchKernelGGL((w8a16_partial_kernel<true, false, kWavesPerWg, 2, 3>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((w8a16_partial_kernel<false, false, kWavesPerWg, 2, 3>), grid, block, 0, st, p);
+  } else {
+    if (bf) hipLaunchKernelGGL((w8a16_partial_kernel<true, true, kWavesPerWg, 2, 4>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((w8a16_partial_kernel<false, true, kWavesPerWg, 2, 4>), grid, block, 0, st, p);
+  }
   PTO_CHECK_HIP(hipGetLastError());
   out->part[0] = p.part[0];
   out->part[1] = wq1 ? p.part[1] : nullptr;
