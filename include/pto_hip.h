@@ -182,7 +182,9 @@ PTO_HIP_API int pto_hip_rms_norm(const void* x, const float* gamma, void* out, i
                                  int64_t hidden, float eps, int x_dtype, int out_dtype,
                                  void* stream);
 
-/* out = (silu(x Wg) * (x Wu)) Wd ; gamma != NULL adds the RMSNorm prologue (ffn_block). */
+/* out = (silu(x Wg) * (x Wu)) Wd ; gamma != NULL adds the RMSNorm prologue (ffn_block).
+ * Up to 64 tokens run as weight-streaming skinny projections (HBM-bound), more as MFMA-tiled
+ * GEMMs; both forms accumulate in fp32 and round the SwiGLU product to `dtype` once. */
 PTO_HIP_API int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void* w_gate,
                                    const void* w_up, const void* w_down, void* out,
                                    int64_t tokens, int64_t hidden, int64_t intermediate,
@@ -190,8 +192,9 @@ PTO_HIP_API int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void
 
 /* W8A16 decode projection (no counterpart in the reference, which has no quantised weights; the
  * contract is its projection kernel's, examples/models/qwen3_jit/kernels/projection.py:145-177,
- * x @ W with W [in, out]):  out[M<=32, N] = (x[M,K] @ w_q[K,N]) * w_scale[N] (+ residual[M,N]).
- * x is BF16/FP16, w_q INT8, accumulation fp32; residual may be NULL. */
+ * x @ W with W [in, out]):  out[M, N] = (x[M,K] @ w_q[K,N]) * w_scale[N] (+ residual[M,N]).
+ * x is BF16/FP16, w_q INT8, accumulation fp32; residual may be NULL.  Built for decode: the
+ * weights stream from HBM once per 32 rows of x, so M beyond a few dozen rows belongs to a GEMM. */
 PTO_HIP_API int pto_hip_w8a16_matmul(const void* x, const void* w_q, const float* w_scale,
                                      const void* residual, void* out, int64_t m, int64_t k, int64_t n,
                                      int x_dtype, int res_dtype, int out_dtype, void* stream);

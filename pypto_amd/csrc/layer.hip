@@ -6,9 +6,11 @@
 // examples/models/08_llama_mini.py:384-483; golden
 // tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:255-287), with the
 // projections taking int8 weights and per-channel scales.  The reference submits one task per
-// tile through its scheduler; here the layer is twelve kernel launches in stream order; each projection is a partial-sum
+// tile through its scheduler; here the layer is eleven kernel launches in stream order; each projection is a partial-sum
 // kernel whose finish is folded into the elementwise step that follows it.
 #include <hip/hip_runtime.h>
+
+#include <algorithm>
 
 #include "common.h"
 
@@ -19,9 +21,28 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
   PTO_CHECK_ARG(a != nullptr, "decoder_layer_decode: null argument block");
   const int64_t b = a->batch, h = a->hidden, hq = a->num_heads, hkv = a->kv_head_num, d = a->head_dim,
                 inter = a->intermediate;
-  PTO_CHECK_ARG(b >= 0 && b <= 32, "decoder_layer_decode: batch %lld, this decode path takes at most 32",
-                (long long)b);
+  PTO_CHECK_ARG(b >= 0 && b < (1 << 20), "decoder_layer_decode: batch %lld out of range", (long long)b);
   if (b == 0) return PTO_HIP_OK;
+  if (b > kW8MaxM) {
+    // The projections hold 32 rows per pass: larger batches run as consecutive groups of 32
+    // sequences in stream order (each group's rows of the block table, lengths and activations;
+    // the caches and weights are shared).
+    PTO_CHECK_ARG(a->hidden_states && a->out && a->seq_lens && a->block_table,
+                  "decoder_layer_decode: null tensor pointer");
+    PTO_CHECK_ARG(a->dtype == PTO_HIP_BF16 || a->dtype == PTO_HIP_FP16,
+                  "decoder_layer_decode: activation dtype %s not in {BF16, FP16}", dtype_name(a->dtype));
+    for (int64_t b0 = 0; b0 < b; b0 += kW8MaxM) {
+      PtoHipDecoderLayerArgs part = *a;
+      part.batch = std::min<int64_t>(kW8MaxM, b - b0);
+      part.hidden_states = reinterpret_cast<const char*>(a->hidden_states) + (size_t)b0 * h * 2;
+      part.out = reinterpret_cast<char*>(a->out) + (size_t)b0 * h * 2;
+      part.seq_lens = a->seq_lens + b0;
+      part.block_table = a->block_table + b0 * a->max_num_blocks_per_req;
+      const int rc = pto_hip_decoder_layer_decode(&part, stream);
+      if (rc) return rc;
+    }
+    return PTO_HIP_OK;
+  }
   PTO_CHECK_ARG(h > 0 && hq > 0 && hkv > 0 && d > 0 && inter > 0 && hq % hkv == 0,
                 "decoder_layer_decode: bad model dimensions");
   PTO_CHECK_ARG(a->dtype == PTO_HIP_BF16 || a->dtype == PTO_HIP_FP16,

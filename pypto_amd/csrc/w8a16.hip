@@ -18,6 +18,7 @@
 //     The RoPE kernel reads the q/k/v partials directly.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <type_traits>
 
 #include "common.h"
@@ -362,10 +363,14 @@ __global__ __launch_bounds__(kNormThreads) void w8a16_finish_norm_kernel(FinishN
   }
 }
 
+template <typename P>
+P* byte_offset(P* base, int64_t bytes) {
+  return reinterpret_cast<P*>(reinterpret_cast<uintptr_t>(base) + (uintptr_t)bytes);
+}
+
 int check_common(const char* what, int64_t m, int64_t k, int64_t n, int x_dtype, int out_dtype) {
   using namespace pto_hip;
-  PTO_CHECK_ARG(m >= 0 && m <= kMaxM, "%s: M = %lld rows, this decode kernel takes at most %d", what,
-                (long long)m, kMaxM);
+  PTO_CHECK_ARG(m >= 0 && m < (1 << 20), "%s: M = %lld rows out of range", what, (long long)m);
   PTO_CHECK_ARG(k >= kStep && k % 16 == 0, "%s: K = %lld must be a multiple of 16, at least %d", what,
                 (long long)k, kStep);
   PTO_CHECK_ARG(n >= 8 && n % 8 == 0, "%s: N = %lld must be a positive multiple of 8", what, (long long)n);
@@ -494,10 +499,19 @@ extern "C" int pto_hip_w8a16_matmul(const void* x, const void* w_q, const float*
     PTO_CHECK_ARG(res_dtype == PTO_HIP_FP32 || res_dtype == PTO_HIP_BF16 || res_dtype == PTO_HIP_FP16,
                   "w8a16_matmul: residual dtype %s not in {FP32, BF16, FP16}", dtype_name(res_dtype));
   hipStream_t st = (hipStream_t)stream;
-  W8Partials parts{};
-  rc = w8a16_partials(x, false, w_q, nullptr, m, k, n, x_dtype, st, &parts);
-  if (rc) return rc;
-  return w8a16_finish(parts, w_scale, nullptr, residual, res_dtype, out, out_dtype, false, m, n, st);
+  // The kernel holds 32 rows of x per pass; more rows stream the weights once per pass, in order
+  // on the stream (the partial buffer is reused).
+  for (int64_t r0 = 0; r0 < m; r0 += kMaxM) {
+    const int64_t rows = std::min<int64_t>(kMaxM, m - r0);
+    W8Partials parts{};
+    rc = w8a16_partials(byte_offset(x, r0 * k * 2), false, w_q, nullptr, rows, k, n, x_dtype, st, &parts);
+    if (rc) return rc;
+    rc = w8a16_finish(parts, w_scale, nullptr,
+                      residual ? byte_offset(residual, r0 * n * dtype_bytes(res_dtype)) : nullptr, res_dtype,
+                      byte_offset(out, r0 * n * dtype_bytes(out_dtype)), out_dtype, false, rows, n, st);
+    if (rc) return rc;
+  }
+  return PTO_HIP_OK;
 }
 
 extern "C" int pto_hip_w8a16_swiglu(const void* x, const void* wg_q, const float* wg_scale,
@@ -513,8 +527,14 @@ extern "C" int pto_hip_w8a16_swiglu(const void* x, const void* wg_q, const float
                     ((uintptr_t)wg_scale % 16 == 0) && ((uintptr_t)wu_scale % 16 == 0) && ((uintptr_t)out % 16 == 0),
                 "w8a16_swiglu: misaligned operand");
   hipStream_t st = (hipStream_t)stream;
-  W8Partials parts{};
-  rc = w8a16_partials(x, false, wg_q, wu_q, m, k, n, x_dtype, st, &parts);
-  if (rc) return rc;
-  return w8a16_finish(parts, wg_scale, wu_scale, nullptr, 0, out, out_dtype, false, m, n, st);
+  for (int64_t r0 = 0; r0 < m; r0 += kMaxM) {  // 32 rows per pass, as in w8a16_matmul
+    const int64_t rows = std::min<int64_t>(kMaxM, m - r0);
+    W8Partials parts{};
+    rc = w8a16_partials(byte_offset(x, r0 * k * 2), false, wg_q, wu_q, rows, k, n, x_dtype, st, &parts);
+    if (rc) return rc;
+    rc = w8a16_finish(parts, wg_scale, wu_scale, nullptr, 0, byte_offset(out, r0 * n * dtype_bytes(out_dtype)),
+                      out_dtype, false, rows, n, st);
+    if (rc) return rc;
+  }
+  return PTO_HIP_OK;
 }

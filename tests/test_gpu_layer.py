@@ -52,12 +52,34 @@ def test_w8a16_swiglu(worker):
 
 
 def test_w8a16_argument_rules(worker):
-    x = torch.zeros(33, 64, dtype=torch.bfloat16)
-    wq = torch.zeros(64, 64, dtype=torch.int8)
+    wq = torch.zeros(40, 64, dtype=torch.int8)
     s = torch.ones(64)
-    with pytest.raises(ValueError, match="at most 32"):
+    with pytest.raises(ValueError, match="multiple of 16"):
         with worker.register(w8a16_matmul) as h:
-            h(x, wq, s, torch.zeros(33, 64))
+            h(torch.zeros(4, 40, dtype=torch.bfloat16), wq, s, torch.zeros(4, 64))
+
+
+@pytest.mark.parametrize("m", [33, 64, 75])
+def test_w8a16_more_than_one_row_pass(worker, m):
+    """Row counts beyond one 32-row pass: every pass reuses the partial buffer in stream order."""
+    torch.manual_seed(m)
+    k, n = 512, 384
+    x = (torch.randn(m, k) * 0.5).to(torch.bfloat16)
+    wq = torch.randint(-127, 128, (k, n), dtype=torch.int8)
+    wu = torch.randint(-127, 128, (k, n), dtype=torch.int8)
+    s = torch.rand(n) * 0.01 + 0.001
+    su = torch.rand(n) * 0.01 + 0.001
+    res = torch.randn(m, n)
+    out = torch.zeros(m, n)
+    with worker.register(w8a16_matmul_residual) as h:
+        h(x, wq, s, res, out)
+    ref = oracle.w8a16_matmul(x, wq, s) + res
+    validate_golden({"out": out}, {"out": ref}, rtol=1e-3, atol=1e-3)
+    out2 = torch.zeros(m, n, dtype=torch.bfloat16)
+    with worker.register(w8a16_swiglu) as h:
+        h(x, wq, s, wu, su, out2)
+    ref2 = oracle.swiglu(oracle.w8a16_matmul(x, wq, s), oracle.w8a16_matmul(x, wu, su)).to(torch.bfloat16)
+    validate_golden({"out": out2.float()}, {"out": ref2.float()}, rtol=1e-2, atol=1e-3)
 
 
 def test_rope_kv_cache_update(worker):
@@ -179,7 +201,7 @@ def _oracle_layer(inp):
         max_num_blocks_per_req=inp.max_num_blocks_per_req, eps=inp.eps)
 
 
-@pytest.mark.parametrize("batch,ctxs", [(4, [100, 1, 257, 33]), (32, None)])
+@pytest.mark.parametrize("batch,ctxs", [(4, [100, 1, 257, 33]), (32, None), (45, None)])
 def test_decoder_layer_decode(worker, batch, ctxs):
     """Reduced model (H1024, Hq8, Hkv2, D128, I2816), same pipeline as the full configuration."""
     if ctxs is None:
