@@ -114,7 +114,7 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "attn_partition_kernel<128, true, false>",
+            "kernel": "attn_partition_kernel<128, true, false, 1>",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",

@@ -297,6 +297,9 @@ PTO_HIP_API int pto_hip_select_program(const char* orchestration_name, const Pto
  *  "attn_variant"               0 = one wavefront per (sequence, KV head, partition), 1 = one pinned
  *                               workgroup per CU and the chunk list cut evenly over their wavefronts,
  *                               -1 = by launch size (default)
+ *  "attn_group_tiles"           cap on the 16-head query tiles one wavefront carries: 0 = the whole KV
+ *                               group up to 64 heads (32 at head_dim 256), the cache read once per
+ *                               group (default); 1, 2, 4 = at most that many, read once per wavefront
  *  "gemm_variant"               FFN GEMM tiling: 0 = default choice (8 wavefronts; 256x256 tile, or
  *                               128x256 when that leaves CUs idle), 1..3 = 4-wavefront alternatives
  *                               (256-row tile, 128-row tile, 256-row tile with k split in two),

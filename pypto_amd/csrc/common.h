@@ -50,6 +50,7 @@ struct Context {
   int64_t attn_waves_per_cu = 0;
   int64_t attn_variant = -1;  // -1 by launch size, 0 partition grid, 1 evenly split form
   int64_t attn_skip_merge = 0;
+  int64_t attn_group_tiles = 0;  // cap on the query tiles one wavefront carries (0 = by group size)
   int64_t gemm_variant = 0;
   int64_t w8a16_wgs_per_cu = 1;  // workgroups of the W8A16 partial kernel aimed at per compute unit
   int64_t w8a16_min_steps = 8;   // fewest 32-row steps per wavefront before k is split further

@@ -47,6 +47,7 @@ struct AttnParams {
   const float* k_scale;  // [pool_blocks, Hkv] for an e4m3 cache, else null
   const float* v_scale;
   int batch, hq, hkv, group, gtiles, bs, max_blocks, tpp, n_part;
+  int gt_rows;     // query rows one wavefront covers: 16 x its tile count; gtiles = ceil(group / gt_rows)
   int n_wg;        // evenly split form: resident workgroups (one per CU); 0 = partition grid
   int lean_waves;  // ... and wavefronts in each
   float scale_log2e;
@@ -211,11 +212,12 @@ __device__ __forceinline__ void qk_scores(const KFrag<D, FP8>& kf, const u32x4 (
   }
 }
 
-// Online softmax of one chunk's scores and O^T += V^T P^T.  vf holds the chunk's V rows (rows
-// past tok_end are zeroed here).
-template <int D, bool BF16, bool FP8>
-__device__ __forceinline__ void softmax_pv(f32x4 s0, f32x4 s1, VFrag<D, FP8>& vf, int tok, int tok_end, int j,
-                                           float k_mul, f32x4 (&acc)[D / 128][8], float& m_run, float& l_run) {
+// Online softmax of one chunk's scores for one 16-column query tile: returns the chunk's
+// probabilities rounded to the activation type, packed as the B operand of O^T += V^T P^T, and
+// updates the tile's running maximum, row sum and (on a new maximum) its accumulators.
+template <int D, bool BF16>
+__device__ __forceinline__ u32x4 softmax_chunk(f32x4 s0, f32x4 s1, int tok, int tok_end, int j, float k_mul,
+                                               f32x4 (&acc)[D / 128][8], float& m_run, float& l_run) {
   float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
 #pragma unroll
   for (int e = 0; e < 8; ++e) sv[e] *= k_mul;
@@ -254,8 +256,16 @@ __device__ __forceinline__ void softmax_pv(f32x4 s0, f32x4 s1, VFrag<D, FP8>& vf
     psum += ra + rb;
   }
   l_run += psum;
+  return pf;
+}
 
-  if (partial) {
+// O^T += V^T P^T for the GT query tiles of a wavefront.  vf holds the chunk's V rows (rows past
+// tok_end are zeroed here); each lane's 8 tokens x 8 elements are transposed once and feed the
+// MFMAs of every tile.
+template <int D, bool BF16, bool FP8, int GT>
+__device__ __forceinline__ void pv_chunk(VFrag<D, FP8>& vf, const u32x4 (&pf)[GT], int tok, int tok_end, int j,
+                                         f32x4 (&acc)[GT][D / 128][8]) {
+  if (tok + kChunk > tok_end) {
     // Rows past the end may hold anything; keep them out of the PV product.
 #pragma unroll
     for (int set = 0; set < D / 128; ++set)
@@ -265,8 +275,6 @@ __device__ __forceinline__ void softmax_pv(f32x4 s0, f32x4 s1, VFrag<D, FP8>& vf
         if (t >= tok_end) vf.t[set][e] = typename std::conditional<FP8, uint2, u32x4>::type{};
       }
   }
-
-  // ---- O^T += V^T P^T : transpose each lane's 8 tokens x 8 elements, then 8 MFMAs ----
 #pragma unroll
   for (int set = 0; set < D / 128; ++set) {
     u32x4 vw[8];  // the lane's 8 tokens x 8 elements as 16-bit values
@@ -282,44 +290,51 @@ __device__ __forceinline__ void softmax_pv(f32x4 s0, f32x4 s1, VFrag<D, FP8>& vf
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk)
         vt[kk] = __builtin_amdgcn_perm(vw[2 * kk + 1][i >> 1], vw[2 * kk][i >> 1], sel);
-      acc[set][i] = mfma16<BF16>(vt, pf, acc[set][i]);
+#pragma unroll
+      for (int t = 0; t < GT; ++t) acc[t][set][i] = mfma16<BF16>(vt, pf[t], acc[t][set][i]);
     }
   }
 }
 
 // Re-expresses the accumulators in another V scale (e4m3 cache, block change).
-template <int D>
-__device__ __forceinline__ void change_unit(f32x4 (&acc)[D / 128][8], float& v_unit, float v_next) {
+template <int D, int GT>
+__device__ __forceinline__ void change_unit(f32x4 (&acc)[GT][D / 128][8], float& v_unit, float v_next) {
   if (v_next != v_unit) {
     const float r = v_unit / v_next;
 #pragma unroll
-    for (int set = 0; set < D / 128; ++set)
+    for (int t = 0; t < GT; ++t)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[set][i] *= r;
+      for (int set = 0; set < D / 128; ++set)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[t][set][i] *= r;
     v_unit = v_next;
   }
 }
 
-// Attention of one query group (16 padded columns) over the chunks tok_first, tok_first +
-// tok_step, ... < tok_end of one (sequence, KV head): on return acc holds O^T in units of v_unit,
-// m_run the running maximum (log2 units) and l_run the row sum, both per column and already
-// summed over the wavefront.  tok_first must be a multiple of 32 below tok_end.
-template <int D, bool BF16, bool FP8>
-__device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, int hq_row, bool g_valid,
+// Attention of GT query tiles (16 padded columns each; tile t covers the query heads g0 + 16 t ..
+// of the KV group, hq_row0 being the output row of head g0) over the chunks tok_first, tok_first +
+// tok_step, ... < tok_end of one (sequence, KV head): on return acc[t] holds O^T in units of
+// v_unit, m_run[t] the running maximum (log2 units) and l_run[t] the row sum, both per column and
+// already summed over the wavefront.  tok_first must be a multiple of 32 below tok_end.  Every K
+// and V byte is loaded once and used by all GT tiles.
+template <int D, bool BF16, bool FP8, int GT>
+__device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, int hq_row0, int g0,
                                              int tok_first, int tok_end, int tok_step, int c, int j,
-                                             char* kbuf, int first_window, f32x4 (&acc)[D / 128][8],
-                                             float& m_run, float& l_run, float& v_unit) {
+                                             char* kbuf, int first_window, f32x4 (&acc)[GT][D / 128][8],
+                                             float (&m_run)[GT], float (&l_run)[GT], float& v_unit) {
   const int lane = j * 16 + c;
   // Query fragments (B operand): column = query head; k-group j of step s holds the elements
   // its K fragment holds: (s*4+j)*8..+8, or for an e4m3 cache ((s/2)*4+j)*16 + (s%2)*8..+8.
-  u32x4 qf[D / 32];
-  {
-    const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + (size_t)hq_row * D;
+  u32x4 qf[GT][D / 32];
+#pragma unroll
+  for (int t = 0; t < GT; ++t) {
+    const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + (size_t)(hq_row0 + t * 16 + c) * D;
+    const bool g_valid = g0 + t * 16 + c < p.group;
 #pragma unroll
     for (int s = 0; s < D / 32; ++s) {
       u32x4 z = {0u, 0u, 0u, 0u};
       const int el = FP8 ? ((s >> 1) * 4 + j) * 16 + (s & 1) * 8 : (s * 4 + j) * 8;
-      qf[s] = g_valid ? *reinterpret_cast<const u32x4*>(qrow + el) : z;
+      qf[t][s] = g_valid ? *reinterpret_cast<const u32x4*>(qrow + el) : z;
     }
   }
 
@@ -370,11 +385,14 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
   auto scale_v = [&]() { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, win_vs), slot_of_tile)); };
 
 #pragma unroll
-  for (int set = 0; set < D / 128; ++set)
+  for (int t = 0; t < GT; ++t) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[set][i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  m_run = kMinMax;
-  l_run = 0.f;
+    for (int set = 0; set < D / 128; ++set)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[t][set][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m_run[t] = kMinMax;
+    l_run[t] = 0.f;
+  }
 
   float k_mul = p.scale_log2e;
   v_unit = 1.f;
@@ -406,14 +424,19 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
         k_next = p.scale_log2e * scale_k();
         v_next = scale_v();
       }
-      f32x4 s0, s1;
+      f32x4 s0[GT], s1[GT];
       fetch_k<D, FP8>(kf, kbuf, c, j);
-      qk_scores<D, BF16, FP8>(kf, qf, s0, s1);
+#pragma unroll
+      for (int t = 0; t < GT; ++t) qk_scores<D, BF16, FP8>(kf, qf[t], s0[t], s1[t]);
       load_k<D, FP8>(kf, kc + o0, kc + o1, lane);  // next chunk, into the registers QK^T just released
-      softmax_pv<D, BF16, FP8>(s0, s1, vf, tok, tok_end, j, k_mul, acc, m_run, l_run);
+      u32x4 pf[GT];
+#pragma unroll
+      for (int t = 0; t < GT; ++t)
+        pf[t] = softmax_chunk<D, BF16>(s0[t], s1[t], tok, tok_end, j, k_mul, acc[t], m_run[t], l_run[t]);
+      pv_chunk<D, BF16, FP8, GT>(vf, pf, tok, tok_end, j, acc);
       if constexpr (FP8) {
         // Next chunk may belong to another block: re-express the accumulators in its V scale.
-        change_unit<D>(acc, v_unit, v_next);
+        change_unit<D, GT>(acc, v_unit, v_next);
         k_mul = k_next;
       }
       load_v<D, FP8>(vf, vc + o0, vc + o1, voff);  // next chunk, into the registers PV just released
@@ -422,11 +445,14 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
   }
 
   // Row sum over the four k-groups of a column.
-  l_run += __shfl_xor(l_run, 16);
-  l_run += __shfl_xor(l_run, 32);
+#pragma unroll
+  for (int t = 0; t < GT; ++t) {
+    l_run[t] += __shfl_xor(l_run[t], 16);
+    l_run[t] += __shfl_xor(l_run[t], 32);
+  }
 }
 
-template <int D, bool BF16, bool FP8>
+template <int D, bool BF16, bool FP8, int GT>
 __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   const int lane = threadIdx.x;
   const int c = lane & 15;   // MFMA row / column index of this lane
@@ -451,35 +477,42 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
   const int tok_begin = part * p.tpp;
   const int tok_end = min(ctx, tok_begin + p.tpp);
-  const int g = gt * 16 + c;               // query head within the KV group
-  const bool g_valid = g < p.group;
-  const int hq_row = b * p.hq + h * p.group + g;
+  const int g0 = gt * (16 * GT);            // first query head of this wavefront within the KV group
+  const int hq_row0 = b * p.hq + h * p.group + g0;
 
   if (tok_begin >= tok_end) {
     // Nothing to read.  An empty sequence yields zeros (09_paged_attention_spmd.py:647-651).
-    if (p.n_part == 1 && g_valid) {
-      float* o = p.out + (size_t)hq_row * D;
+    if (p.n_part == 1) {
 #pragma unroll
-      for (int i = 0; i < D / 4; ++i) o[j * (D / 4) + i] = 0.f;
+      for (int t = 0; t < GT; ++t) {
+        if (g0 + t * 16 + c >= p.group) continue;
+        float* o = p.out + (size_t)(hq_row0 + t * 16 + c) * D;
+#pragma unroll
+        for (int i = 0; i < D / 4; ++i) o[j * (D / 4) + i] = 0.f;
+      }
     }
     return;
   }
 
   __shared__ __attribute__((aligned(16))) char k_lds[KStage<D, FP8>::kBytes];
-  f32x4 acc[D / 128][8];
-  float m_run, l_run, v_unit;
-  attend_range<D, BF16, FP8>(p, b, h, hq_row, g_valid, tok_begin, tok_end, kChunk, c, j, k_lds, first_window, acc,
-                             m_run, l_run, v_unit);
+  f32x4 acc[GT][D / 128][8];
+  float m_run[GT], l_run[GT], v_unit;
+  attend_range<D, BF16, FP8, GT>(p, b, h, hq_row0, g0, tok_begin, tok_end, kChunk, c, j, k_lds, first_window, acc,
+                                 m_run, l_run, v_unit);
 
-  if (!g_valid) return;
-  if (p.n_part == 1) {
-    store_rows<D>(p.out + (size_t)hq_row * D, acc, j, l_run > 0.f ? v_unit / l_run : 0.f);
-  } else {
-    const size_t slot = (size_t)hq_row * p.n_part + part;
-    store_rows<D>(p.part_o + slot * D, acc, j, v_unit);
-    if (j == 0) {
-      p.part_ml[slot * 2 + 0] = m_run;
-      p.part_ml[slot * 2 + 1] = l_run;
+#pragma unroll
+  for (int t = 0; t < GT; ++t) {
+    if (g0 + t * 16 + c >= p.group) continue;
+    const int hq_row = hq_row0 + t * 16 + c;
+    if (p.n_part == 1) {
+      store_rows<D>(p.out + (size_t)hq_row * D, acc[t], j, l_run[t] > 0.f ? v_unit / l_run[t] : 0.f);
+    } else {
+      const size_t slot = (size_t)hq_row * p.n_part + part;
+      store_rows<D>(p.part_o + slot * D, acc[t], j, v_unit);
+      if (j == 0) {
+        p.part_ml[slot * 2 + 0] = m_run[t];
+        p.part_ml[slot * 2 + 1] = l_run[t];
+      }
     }
   }
 }
@@ -661,9 +694,12 @@ __device__ __forceinline__ void lean_locate(const AttnParams& p, int lane, int h
   }
 }
 
-// head_dim 256 needs more than 256 registers per wavefront: four wavefronts (one per SIMD) there.
-template <int D, bool BF16, bool FP8>
-__global__ __launch_bounds__((D == 128 ? kLeanMaxWaves : 4) * 64) void attn_lean_kernel(AttnParams p) {
+// head_dim 256 and more than one query tile per wavefront need more than 256 registers per
+// wavefront: four wavefronts (one per SIMD) there.
+constexpr int lean_max_waves(int d, int gt) { return d == 128 && gt == 1 ? kLeanMaxWaves : 4; }
+
+template <int D, bool BF16, bool FP8, int GT>
+__global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char lean_lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -699,22 +735,23 @@ __global__ __launch_bounds__((D == 128 ? kLeanMaxWaves : 4) * 64) void attn_lean
     ctx = ctx > max_ctx ? max_ctx : ctx;
     const int tok_first = chunk * kChunk;
     const int tok_end = min(ctx, (chunk + run) * kChunk);
-    const int g = gt * 16 + c;
-    const bool g_valid = g < p.group;
-    const int hq_row = b * p.hq + h * p.group + g;
+    const int g0 = gt * (16 * GT);
+    const int hq_row0 = b * p.hq + h * p.group + g0;
 
-    f32x4 acc[D / 128][8];
-    float m_run, l_run, v_unit;
+    f32x4 acc[GT][D / 128][8];
+    float m_run[GT], l_run[GT], v_unit;
     const int first_window =
         p.block_table[(size_t)b * p.max_blocks + min(tok_first / p.bs + lane, p.max_blocks - 1)];
-    attend_range<D, BF16, FP8>(p, b, h, hq_row, g_valid, tok_first, tok_end, kChunk, c, j, kbuf, first_window,
-                                     acc, m_run, l_run, v_unit);
-    if (g_valid) {
-      const size_t slot = ((size_t)((long long)b * hg_count + hg + w)) * 16 + c;
-      store_rows<D>(p.part_o + slot * D, acc, j, v_unit);
+    attend_range<D, BF16, FP8, GT>(p, b, h, hq_row0, g0, tok_first, tok_end, kChunk, c, j, kbuf, first_window,
+                                   acc, m_run, l_run, v_unit);
+#pragma unroll
+    for (int t = 0; t < GT; ++t) {
+      if (g0 + t * 16 + c >= p.group) continue;
+      const size_t slot = ((size_t)((long long)b * hg_count + hg + w)) * (16 * GT) + t * 16 + c;
+      store_rows<D>(p.part_o + slot * D, acc[t], j, v_unit);
       if (j == 0) {
-        p.part_ml[slot * 2 + 0] = m_run;
-        p.part_ml[slot * 2 + 1] = l_run;
+        p.part_ml[slot * 2 + 0] = m_run[t];
+        p.part_ml[slot * 2 + 1] = l_run[t];
       }
     }
     s += run;
@@ -731,7 +768,8 @@ __global__ __launch_bounds__(256) void attn_lean_reduce_kernel(AttnParams p, lon
   if (row >= p.batch * p.hq) return;
   const int b = row / p.hq, hqi = row % p.hq;
   const int h = hqi / p.group, g = hqi % p.group;
-  const int hg_count = p.hkv * p.gtiles, hg = h * p.gtiles + g / 16, gi = g % 16;
+  const int rows = p.gt_rows;  // rows per partial slot
+  const int hg_count = p.hkv * p.gtiles, hg = h * p.gtiles + g / rows, gi = g % rows;
 
   // items before sequence b, items in total, chunks of b
   long long total = 0, before = 0;
@@ -759,14 +797,15 @@ __global__ __launch_bounds__(256) void attn_lean_reduce_kernel(AttnParams p, lon
     const long long c0 = before + (long long)hg * chunks, c1 = c0 + chunks;
     const long long w_first = c0 * wtot / total, w_last = (c1 - 1) * wtot / total;
     const int np = (int)(w_last - w_first + 1);
-    const size_t slot0 = ((size_t)((long long)b * hg_count + hg + w_first)) * 16 + gi;
-    const float* ml = p.part_ml + slot0 * 2;   // partial i at ml[i * 32], po[i * 16 * D]
+    const size_t slot0 = ((size_t)((long long)b * hg_count + hg + w_first)) * rows + gi;
+    const float* ml = p.part_ml + slot0 * 2;   // partial i at ml[i * ml_step], po[i * po_step]
     const float* po = p.part_o + slot0 * D;
+    const size_t ml_step = (size_t)rows * 2, po_step = (size_t)rows * D;
     float m = kMinMax;
-    for (int i = lane; i < np; i += 64) m = fmaxf(m, ml[(size_t)i * 32]);
+    for (int i = lane; i < np; i += 64) m = fmaxf(m, ml[(size_t)i * ml_step]);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
-    for (int i = lane; i < np; i += 64) l += __builtin_amdgcn_exp2f(ml[(size_t)i * 32] - m) * ml[(size_t)i * 32 + 1];
+    for (int i = lane; i < np; i += 64) l += __builtin_amdgcn_exp2f(ml[(size_t)i * ml_step] - m) * ml[(size_t)i * ml_step + 1];
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off);
     int i = 0;
@@ -774,9 +813,9 @@ __global__ __launch_bounds__(256) void attn_lean_reduce_kernel(AttnParams p, lon
       float wv[4], v[4][D / 64];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        wv[u] = ml[(size_t)(i + u) * 32];
+        wv[u] = ml[(size_t)(i + u) * ml_step];
 #pragma unroll
-        for (int k = 0; k < D / 64; ++k) v[u][k] = po[(size_t)(i + u) * 16 * D + k * 64 + lane];
+        for (int k = 0; k < D / 64; ++k) v[u][k] = po[(size_t)(i + u) * po_step + k * 64 + lane];
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
@@ -786,9 +825,9 @@ __global__ __launch_bounds__(256) void attn_lean_reduce_kernel(AttnParams p, lon
       }
     }
     for (; i < np; ++i) {
-      const float wgt = __builtin_amdgcn_exp2f(ml[(size_t)i * 32] - m);
+      const float wgt = __builtin_amdgcn_exp2f(ml[(size_t)i * ml_step] - m);
 #pragma unroll
-      for (int k = 0; k < D / 64; ++k) o[k] += wgt * po[(size_t)i * 16 * D + k * 64 + lane];
+      for (int k = 0; k < D / 64; ++k) o[k] += wgt * po[(size_t)i * po_step + k * 64 + lane];
     }
   }
   const float inv = l > 0.f ? 1.f / l : 0.f;
@@ -809,7 +848,7 @@ __global__ __launch_bounds__(256) void attn_lean_reduce_kernel(AttnParams p, lon
   }
 }
 
-template <int D, bool FP8>
+template <int D, bool FP8, int GT>
 int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   dim3 grid((unsigned)(p.n_part * p.hkv * p.gtiles * batch));
   // Unused dynamic LDS caps the wavefronts resident per CU so that the dispatcher spreads the
@@ -834,8 +873,8 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
       return PTO_HIP_OK;
     };
     int rc = PTO_HIP_OK;
-    if (bf16) rc = go(attn_lean_kernel<D, true, FP8>);
-    else if constexpr (!FP8) rc = go(attn_lean_kernel<D, false, false>);
+    if (bf16) rc = go(attn_lean_kernel<D, true, FP8, GT>);
+    else if constexpr (!FP8) rc = go(attn_lean_kernel<D, false, false, GT>);
     if (rc) return rc;
     PTO_CHECK_HIP(hipGetLastError());
     if (!pto_hip::ctx().attn_skip_merge) {
@@ -845,9 +884,9 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
     }
     return PTO_HIP_OK;
   } else if (bf16) {
-    hipLaunchKernelGGL((attn_partition_kernel<D, true, FP8>), grid, dim3(64), lds, stream, p);
+    hipLaunchKernelGGL((attn_partition_kernel<D, true, FP8, GT>), grid, dim3(64), lds, stream, p);
   } else if constexpr (!FP8) {
-    hipLaunchKernelGGL((attn_partition_kernel<D, false, false>), grid, dim3(64), lds, stream, p);
+    hipLaunchKernelGGL((attn_partition_kernel<D, false, false, GT>), grid, dim3(64), lds, stream, p);
   }
   PTO_CHECK_HIP(hipGetLastError());
   // "attn_skip_merge" leaves the partials unmerged: a timing aid that isolates the streaming
@@ -920,7 +959,13 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   p.hq = (int)hq;
   p.hkv = (int)hkv;
   p.group = (int)(hq / hkv);
-  p.gtiles = (p.group + 15) / 16;
+  // Query tiles (16 heads each) one wavefront carries: the whole KV group when it fits, so that
+  // K and V are read once per group, not once per tile.
+  // "attn_group_tiles" caps the count (1 = one tile per wavefront, the KV read once per tile).
+  int gt = p.group <= 16 ? 1 : (p.group <= 32 || d == 256) ? 2 : 4;
+  if (cx.attn_group_tiles > 0 && gt > cx.attn_group_tiles) gt = (int)cx.attn_group_tiles;
+  p.gt_rows = 16 * gt;
+  p.gtiles = (p.group + p.gt_rows - 1) / p.gt_rows;
   p.bs = (int)bs;
   p.max_blocks = (int)max_blocks;
   p.scale_log2e = scale * kLog2e;
@@ -971,13 +1016,13 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   if (lean) {
     const int64_t kbytes = (fp8 ? d : 2 * d) + 16;  // K stage row pitch
     int64_t waves = cx.attn_waves_per_cu > 0 ? cx.attn_waves_per_cu : 4;
-    if (waves > (d == 128 ? kLeanMaxWaves : 4)) waves = d == 128 ? kLeanMaxWaves : 4;
+    if (waves > lean_max_waves((int)d, gt)) waves = lean_max_waves((int)d, gt);
     while (waves > 1 && waves * 32 * kbytes > 160 * 1024) --waves;
     p.n_wg = cx.num_cu;
     p.lean_waves = (int)waves;
     // partial slots: one per (sequence, head, tile) plus one per resident wavefront
     const size_t slots = (size_t)batch * hkv * p.gtiles + (size_t)p.n_wg * waves;
-    const size_t o_bytes = slots * 16 * d * sizeof(float), ml_bytes = slots * 16 * 2 * sizeof(float);
+    const size_t o_bytes = slots * p.gt_rows * d * sizeof(float), ml_bytes = slots * p.gt_rows * 2 * sizeof(float);
     void* ws = nullptr;
     int rc = workspace(o_bytes + ml_bytes, &ws);
     if (rc != PTO_HIP_OK) return rc;
@@ -993,12 +1038,17 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     if (wrote_blocked) *wrote_blocked = p.out16_blocked != 0;
   }
   int rc;
-  if (fp8)
-    rc = d == 128 ? launch<128, true>(p, (int)batch, bf16, (hipStream_t)stream)
-                  : launch<256, true>(p, (int)batch, bf16, (hipStream_t)stream);
-  else
-    rc = d == 128 ? launch<128, false>(p, (int)batch, bf16, (hipStream_t)stream)
-                  : launch<256, false>(p, (int)batch, bf16, (hipStream_t)stream);
+  hipStream_t hs = (hipStream_t)stream;
+  const int nb = (int)batch;
+  if (d == 128) {
+    if (fp8) rc = gt == 1 ? launch<128, true, 1>(p, nb, bf16, hs) : gt == 2 ? launch<128, true, 2>(p, nb, bf16, hs)
+                                                                           : launch<128, true, 4>(p, nb, bf16, hs);
+    else rc = gt == 1 ? launch<128, false, 1>(p, nb, bf16, hs) : gt == 2 ? launch<128, false, 2>(p, nb, bf16, hs)
+                                                                         : launch<128, false, 4>(p, nb, bf16, hs);
+  } else {
+    if (fp8) rc = gt == 1 ? launch<256, true, 1>(p, nb, bf16, hs) : launch<256, true, 2>(p, nb, bf16, hs);
+    else rc = gt == 1 ? launch<256, false, 1>(p, nb, bf16, hs) : launch<256, false, 2>(p, nb, bf16, hs);
+  }
   if (rc || !out16 || merged) return rc;
   return cast_from_f32(out, out16, (size_t)batch * hq * d, q_dtype, (hipStream_t)stream);
 }

@@ -696,6 +696,9 @@ int pto_hip_set_option(const char* name, int64_t value) {
     c.attn_tokens_per_partition = value;
   } else if (!std::strcmp(name, "gemm_variant")) {
     c.gemm_variant = value;
+  } else if (!std::strcmp(name, "attn_group_tiles")) {
+    PTO_CHECK_ARG(value == 0 || value == 1 || value == 2 || value == 4, "attn_group_tiles must be 0, 1, 2 or 4");
+    c.attn_group_tiles = value;
   } else if (!std::strcmp(name, "attn_variant")) {
     PTO_CHECK_ARG(value >= -1 && value <= 1, "attn_variant must be -1, 0 or 1");
     c.attn_variant = value;
@@ -724,6 +727,7 @@ int pto_hip_get_option(const char* name, int64_t* value) {
   else if (!std::strcmp(name, "attn_waves_per_cu")) *value = c.attn_waves_per_cu;
   else if (!std::strcmp(name, "attn_skip_merge")) *value = c.attn_skip_merge;
   else if (!std::strcmp(name, "attn_variant")) *value = c.attn_variant;
+  else if (!std::strcmp(name, "attn_group_tiles")) *value = c.attn_group_tiles;
   else if (!std::strcmp(name, "w8a16_wgs_per_cu")) *value = c.w8a16_wgs_per_cu;
   else if (!std::strcmp(name, "w8a16_min_steps")) *value = c.w8a16_min_steps;
   else return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);

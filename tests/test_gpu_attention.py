@@ -111,6 +111,40 @@ def test_reference_multi_config_list(worker, batch, num_heads, head_dim, block_s
         _check(_run(worker, inp, tpp), ref)
 
 
+@pytest.mark.parametrize(
+    "hq,hkv,d,fp8,dtype",
+    [
+        (24, 1, 128, False, torch.bfloat16),    # 24 heads on one KV head: two tiles, the second half padding
+        (64, 2, 128, False, torch.bfloat16),    # groups of 32: two full tiles
+        (40, 1, 128, False, torch.float16),     # 40: four tiles, the last all padding
+        (64, 1, 128, True, torch.bfloat16),     # 64 on an e4m3 cache
+        (80, 1, 128, False, torch.bfloat16),    # 80: two wavefront tiles of four
+        (48, 1, 256, False, torch.bfloat16),    # head_dim 256: two tiles per wavefront, two wavefront tiles
+        (32, 1, 256, True, torch.bfloat16),
+    ],
+)
+def test_wide_query_groups(worker, hq, hkv, d, fp8, dtype):
+    """KV groups wider than one 16-head MFMA tile: one wavefront carries up to four tiles and reads
+    the cache once for all of them; capping the tile count (one tile per wavefront, the cache read
+    once per tile) must give the same result."""
+    ctxs = [700, 0, 33, 1300, 128]
+    inp = workloads.paged_attention_inputs(batch=len(ctxs), num_heads=hq, kv_head_num=hkv, head_dim=d, block_size=64,
+                                           context_lens=ctxs, ctx_range=(1, 1300), dtype=dtype, fp8_kv=fp8, seed=21)
+    ref = _golden(inp)
+    for tpp in (0, 256, -4):
+        out = _run(worker, inp, tpp)
+        _check(out, ref)
+        assert (out[hq:2 * hq] == 0).all()      # the empty sequence
+    worker.set_option("attn_group_tiles", 1)
+    try:
+        one = _run(worker, inp, 256)
+    finally:
+        worker.set_option("attn_group_tiles", 0)
+    _check(one, ref)
+    # same partitions, same per-row arithmetic: the tile count changes nothing in a row's result
+    assert torch.equal(one, _run(worker, inp, 256))
+
+
 def test_fp16_cache(worker):
     inp = workloads.paged_attention_inputs(batch=3, num_heads=16, kv_head_num=4, context_lens=[300, 17, 129],
                                            ctx_range=(1, 300), dtype=torch.float16, seed=3)
