@@ -183,8 +183,9 @@ PTO_HIP_API int pto_hip_rms_norm(const void* x, const float* gamma, void* out, i
                                  void* stream);
 
 /* out = (silu(x Wg) * (x Wu)) Wd ; gamma != NULL adds the RMSNorm prologue (ffn_block).
- * Up to 64 tokens run as weight-streaming skinny projections (HBM-bound), more as MFMA-tiled
- * GEMMs; both forms accumulate in fp32 and round the SwiGLU product to `dtype` once. */
+ * Up to 32 tokens run as weight-streaming skinny projections (HBM-bound), more as MFMA-tiled
+ * GEMMs (with k split over several workgroups per tile while the tiles alone would leave CUs
+ * idle); every form accumulates in fp32 and rounds the SwiGLU product to `dtype` once. */
 PTO_HIP_API int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void* w_gate,
                                    const void* w_up, const void* w_down, void* out,
                                    int64_t tokens, int64_t hidden, int64_t intermediate,
@@ -301,7 +302,8 @@ PTO_HIP_API int pto_hip_select_program(const char* orchestration_name, const Pto
  *                               group up to 64 heads (32 at head_dim 256), the cache read once per
  *                               group (default); 1, 2, 4 = at most that many, read once per wavefront
  *  "gemm_variant"               FFN GEMM tiling: 0 = default choice (8 wavefronts; 256x256 tile, or
- *                               128x256 when that leaves CUs idle), 1..3 = 4-wavefront alternatives
+ *                               128x256 when that leaves CUs idle, with k split while that still does;
+ *                               skinny projections up to 32 tokens), 1..3 = 4-wavefront alternatives
  *                               (256-row tile, 128-row tile, 256-row tile with k split in two),
  *                               4 = 8 wavefronts, 256-row tile, k split when CUs would idle,
  *                               5 = 8 wavefronts, 128-row tile

@@ -19,9 +19,13 @@
 //     range, so SiLU(gate) * up is applied on the accumulators and only h is written;
 //   * workgroup ids are remapped so that the ids sharing an XCD (id mod 8) work on neighbouring
 //     tiles and share operands in that XCD's L2;
-//   * at decode-size token counts (at most 64 rows) the block is bound by reading the weights
+//   * with a few hundred rows the tiles alone leave most CUs idle: k is then split over several
+//     workgroups per tile, each writing an fp32 slab, and a finish kernel sums the slabs in
+//     split order (plus SwiGLU for the gate/up pass);
+//   * at decode-size token counts (at most 32 rows) the block is bound by reading the weights
 //     once and runs as skinny projections instead (ffn_skinny below).
 #include <hip/hip_runtime.h>
+#include <algorithm>
 
 #include "common.h"
 
@@ -48,7 +52,8 @@ struct GemmParams {
   int64_t lda, ldb, ldc;
   int m, n, k;
   int tiles_m, tiles_n;
-  int splits, k_per_split;  // split-K: fp32 output accumulated with atomics into zeroed memory
+  int splits, k_per_split;  // split-K: each split writes its own fp32 slab, a second kernel sums them
+  float* slabs;             // [splits][DUAL ? 2 : 1][m][n] when splits > 1
 };
 
 template <bool BF16>
@@ -76,13 +81,14 @@ __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
   return base + local;
 }
 
-// EDGE = false assumes m, n, k are multiples of the tile; EDGE = true clamps every address into
-// the operands (so all loads stay unconditional) and zeroes the A chunks that lie past k.
+// EDGE = 0 assumes m, n, k are multiples of the tile.  EDGE = 1: only m is ragged - the A row
+// pointers are clamped once, the loop is the same.  EDGE = 2 clamps every address into the
+// operands (so all loads stay unconditional) and zeroes the A chunks that lie past k.
 // Wavefront grid WM x WN over the (32*MT*WM) x 256 tile: each wavefront owns (32*MT) x (32*NT)
 // as MT x NT accumulators, NT = 8 / WN.  2 x 2 wavefronts with 4 x 4 accumulators run one
 // wavefront per SIMD; 2 x 4 wavefronts with 4 x 2 accumulators run two per SIMD, so the MFMA pipe
 // has a second instruction stream to draw from while one waits on memory or a barrier.
-template <int MT, int WM, int WN, bool DUAL, bool BF16, bool EDGE, typename OutT>
+template <int MT, int WM, int WN, bool DUAL, bool BF16, int EDGE, typename OutT>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   constexpr int NBUF = 2;
   constexpr int NT = (BN / 32) / WN;        // B fragments (32 columns each) per wavefront
@@ -125,12 +131,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
     bsrc = p.b0;
     b_col = n0 + b_chunk * 8;
   }
-  if (EDGE) b_col = min(b_col, p.n - 8);
+  if (EDGE == 2) b_col = min(b_col, p.n - 8);
   const uint16_t* a_ptr[NA];
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
     int r = m0 + a_row + (T / 8) * i;
-    if (EDGE) r = min(r, p.m - 1);
+    if (EDGE != 0) r = min(r, p.m - 1);
     a_ptr[i] = p.a + (int64_t)r * p.lda + k_begin + a_chunk * 8;
   }
   const uint16_t* b_ptr = bsrc + (int64_t)(k_begin + b_row) * p.ldb + b_col;
@@ -138,7 +144,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   u32x4 ra[NA];
   u32x4 rb[NB];
   auto load_a = [&](int k0, int i) {
-    if constexpr (EDGE) {
+    if constexpr (EDGE == 2) {
       const int ka = min(k0 + a_chunk * 8, klen - 8) - a_chunk * 8;  // clamped tile origin for A
       const bool a_ok = k0 + a_chunk * 8 < klen;
       u32x4 v = *reinterpret_cast<const u32x4*>(a_ptr[i] + ka);
@@ -149,7 +155,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
     }
   };
   auto load_b = [&](int k0, int i) {
-    if constexpr (EDGE) {
+    if constexpr (EDGE == 2) {
       const int kk = min(k0 + b_row + (T / 32) * i, klen - 1) - b_row;
       rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)kk * p.ldb);
     } else {
@@ -272,22 +278,28 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
     for (int r = 0; r < 16; ++r) {
       const int row = row_base + i * 32 + (r >> 2) * 8 + (r & 3);
       if (row >= p.m) continue;
+      const int64_t mn = (int64_t)p.m * p.n;
       if constexpr (DUAL) {
 #pragma unroll
         for (int jn = 0; jn < NT / 2; ++jn) {
           const int col = n0 + wn * (16 * NT) + jn * 32 + (lane & 31);
-          if (col < p.n)
-            store_out<OutT>(c + (int64_t)row * p.ldc + col, silu(acc[i][jn][r]) * acc[i][jn + NT / 2][r]);
+          if (col < p.n) {
+            if (p.splits > 1) {
+              float* s = p.slabs + (int64_t)split * 2 * mn + (int64_t)row * p.n + col;
+              s[0] = acc[i][jn][r];
+              s[mn] = acc[i][jn + NT / 2][r];
+            } else {
+              store_out<OutT>(c + (int64_t)row * p.ldc + col, silu(acc[i][jn][r]) * acc[i][jn + NT / 2][r]);
+            }
+          }
         }
       } else {
 #pragma unroll
         for (int jn = 0; jn < NT; ++jn) {
           const int col = n0 + wn * (32 * NT) + jn * 32 + (lane & 31);
           if (col < p.n) {
-            if (p.splits > 1)
-              unsafeAtomicAdd(reinterpret_cast<float*>(p.c) + (int64_t)row * p.ldc + col, acc[i][jn][r]);
-            else
-              store_out<OutT>(c + (int64_t)row * p.ldc + col, acc[i][jn][r]);
+            if (p.splits > 1) p.slabs[(int64_t)split * mn + (int64_t)row * p.n + col] = acc[i][jn][r];
+            else store_out<OutT>(c + (int64_t)row * p.ldc + col, acc[i][jn][r]);
           }
         }
       }
@@ -296,7 +308,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
 }
 
 
-template <int MT, int WM, int WN, bool DUAL, bool BF16, bool EDGE, typename OutT>
+template <int MT, int WM, int WN, bool DUAL, bool BF16, int EDGE, typename OutT>
 int launch_gemm_e(GemmParams p, hipStream_t st) {
   constexpr int BM = 32 * MT * WM;
   constexpr int NBUF = 2;
@@ -319,44 +331,106 @@ int launch_gemm_e(GemmParams p, hipStream_t st) {
 template <int MT, int WM, int WN, bool DUAL, bool BF16, typename OutT>
 int launch_gemm(GemmParams p, hipStream_t st) {
   constexpr int BM_ = 32 * MT * WM;
-  const bool edge = p.m % BM_ != 0 || p.n % (DUAL ? BN / 2 : BN) != 0 || p.k % BK != 0 ||
-                    (p.splits > 1 && p.k_per_split % BK != 0);
-  return edge ? launch_gemm_e<MT, WM, WN, DUAL, BF16, true, OutT>(p, st)
-              : launch_gemm_e<MT, WM, WN, DUAL, BF16, false, OutT>(p, st);
+  const bool edge = p.n % (DUAL ? BN / 2 : BN) != 0 || p.k % BK != 0 || (p.splits > 1 && p.k_per_split % BK != 0);
+  if (edge) return launch_gemm_e<MT, WM, WN, DUAL, BF16, 2, OutT>(p, st);
+  if (p.m % BM_ != 0) return launch_gemm_e<MT, WM, WN, DUAL, BF16, 1, OutT>(p, st);
+  return launch_gemm_e<MT, WM, WN, DUAL, BF16, 0, OutT>(p, st);
 }
 
-__global__ __launch_bounds__(256) void zero_kernel(float4* p, size_t n4) {
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256)
-    p[i] = float4{0.f, 0.f, 0.f, 0.f};
+// Sum of the split-K slabs in split order (so the result does not depend on which workgroup
+// finished first), then SwiGLU for the gate/up pass, cast and store.  n is a multiple of 4.
+constexpr int kMaxSplits = 16;
+constexpr int kSplitBatch = 8;  // slabs loaded before the first add
+template <bool DUAL, typename OutT>
+__global__ __launch_bounds__(256) void gemm_finish_kernel(const float* slabs, OutT* c, int64_t ldc, int m, int n,
+                                                          int splits) {
+  const int nq = n / 4;
+  const int64_t quads = (int64_t)m * nq, mn = (int64_t)m * n;
+  constexpr int kMats = DUAL ? 2 : 1;
+  for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < quads; q += (int64_t)gridDim.x * 256) {
+    const int64_t row = q / nq;
+    const int col = (int)(q % nq) * 4;
+    const float* src = slabs + row * n + col;
+    float4 t[kMats];
+#pragma unroll
+    for (int mat = 0; mat < kMats; ++mat) t[mat] = float4{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < splits; s0 += kSplitBatch) {
+      float4 v[kSplitBatch][kMats];
+#pragma unroll
+      for (int sp = 0; sp < kSplitBatch; ++sp)
+#pragma unroll
+        for (int mat = 0; mat < kMats; ++mat)
+          v[sp][mat] = *reinterpret_cast<const float4*>(src + ((int64_t)min(s0 + sp, splits - 1) * kMats + mat) * mn);
+#pragma unroll
+      for (int mat = 0; mat < kMats; ++mat)
+#pragma unroll
+        for (int sp = 0; sp < kSplitBatch; ++sp)
+          if (s0 + sp < splits) {
+            t[mat].x += v[sp][mat].x;
+            t[mat].y += v[sp][mat].y;
+            t[mat].z += v[sp][mat].z;
+            t[mat].w += v[sp][mat].w;
+          }
+    }
+    float4 y = t[0];
+    if constexpr (DUAL) y = float4{silu(t[0].x) * t[1].x, silu(t[0].y) * t[1].y, silu(t[0].z) * t[1].z, silu(t[0].w) * t[1].w};
+    OutT* dst = c + row * ldc + col;
+    store_out<OutT>(dst + 0, y.x);
+    store_out<OutT>(dst + 1, y.y);
+    store_out<OutT>(dst + 2, y.z);
+    store_out<OutT>(dst + 3, y.w);
+  }
+}
+
+template <bool DUAL, typename OutT>
+int launch_finish(const GemmParams& p, hipStream_t st) {
+  const int64_t quads = (int64_t)p.m * (p.n / 4);
+  const unsigned blocks = (unsigned)std::min<int64_t>((quads + 255) / 256, 4096);
+  hipLaunchKernelGGL((gemm_finish_kernel<DUAL, OutT>), dim3(blocks), dim3(256), 0, st, p.slabs,
+                     reinterpret_cast<OutT*>(p.c), p.ldc, p.m, p.n, p.splits);
+  PTO_CHECK_HIP(hipGetLastError());
+  return PTO_HIP_OK;
 }
 
 template <bool DUAL, bool BF16, typename OutT>
 int launch_variant(GemmParams p, hipStream_t st) {
   const int64_t variant = pto_hip::ctx().gemm_variant;
+  const int64_t num_cu = pto_hip::ctx().num_cu;
   p.splits = 1;
   p.k_per_split = p.k;
+  p.slabs = nullptr;
   // variant 0 (default): eight wavefronts (two per SIMD) on a 256x256 tile, or on a 128x256 tile
   // when the large one would leave CUs without a workgroup (measured on the LLaMA-7B down pass:
-  // 183 us against 223 us for the large tile with k split in two and fp32 atomics).
+  // 183 us against 223 us for the large tile with k split in two); when even the small tile
+  // covers at most half of the CUs (a few hundred tokens), k is split over up to eight
+  // workgroups per tile, each writing an fp32 slab that a second kernel sums in split order.
   // variants 1-3 keep four wavefronts (one per SIMD): 1 = 256x256 tile, 2 = 128x256 tile,
-  // 3 = 256x256 tile with k split in two (contiguous fp32 output; a two-term sum does not depend
-  // on which half arrives first).  4 = eight wavefronts, 256x256 tile, k split in two when CUs
-  // would idle.  5 = eight wavefronts, 128x256 tile.
-  const int64_t big_tiles = (int64_t)((p.m + 255) / 256) * ((p.n + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256));
-  const bool can_split = !DUAL && sizeof(OutT) == 4 && p.ldc == p.n && ((int64_t)p.m * p.n) % 4 == 0 &&
-                         p.k >= 4 * BK;
-  const bool few = big_tiles < pto_hip::ctx().num_cu;
-  if (variant == 5 || (variant == 0 && few)) return launch_gemm<2, 2, 4, DUAL, BF16, OutT>(p, st);
-  if (variant == 2) return launch_gemm<2, 2, 2, DUAL, BF16, OutT>(p, st);
-  if (can_split && (variant == 3 || (variant == 4 && few))) {
-    p.splits = 2;
-    p.k_per_split = ((p.k + 2 * BK - 1) / (2 * BK)) * BK;
-    const size_t n4 = (size_t)p.m * p.n / 4;
-    hipLaunchKernelGGL(zero_kernel, dim3(1024), dim3(256), 0, st, reinterpret_cast<float4*>(p.c), n4);
-    PTO_CHECK_HIP(hipGetLastError());
+  // 3 = 256x256 tile with k split in two.  4 = eight wavefronts, 256x256 tile, k split in two
+  // when CUs would idle.  5 = eight wavefronts, 128x256 tile.
+  const int64_t tiles_n = (p.n + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256);
+  const int64_t big_tiles = (int64_t)((p.m + 255) / 256) * tiles_n;
+  const int64_t small_tiles = (int64_t)((p.m + 127) / 128) * tiles_n;
+  const bool few = big_tiles < num_cu;
+  int want = 1;
+  if (variant == 3 || (variant == 4 && few)) want = 2;
+  if (variant == 0 && few && small_tiles * 2 <= num_cu) want = (int)std::min<int64_t>(kMaxSplits, num_cu / small_tiles);
+  if (want > 1 && p.k >= 4 * BK * want && p.n % 4 == 0) {
+    p.k_per_split = ((p.k + want * BK - 1) / (want * BK)) * BK;
+    p.splits = (p.k + p.k_per_split - 1) / p.k_per_split;
+    if (p.splits > 1) {
+      void* ws = nullptr;
+      const int rc = pto_hip::layer_workspace((size_t)p.splits * (DUAL ? 2 : 1) * p.m * p.n * sizeof(float), &ws);
+      if (rc) return rc;
+      p.slabs = reinterpret_cast<float*>(ws);
+    }
   }
-  if (variant == 0 || variant == 4) return launch_gemm<4, 2, 4, DUAL, BF16, OutT>(p, st);
-  return launch_gemm<4, 2, 2, DUAL, BF16, OutT>(p, st);
+  int rc;
+  if (variant == 5 || (variant == 0 && few)) rc = launch_gemm<2, 2, 4, DUAL, BF16, OutT>(p, st);
+  else if (variant == 2) rc = launch_gemm<2, 2, 2, DUAL, BF16, OutT>(p, st);
+  else if (variant == 0 || variant == 4) rc = launch_gemm<4, 2, 4, DUAL, BF16, OutT>(p, st);
+  else rc = launch_gemm<4, 2, 2, DUAL, BF16, OutT>(p, st);
+  if (rc || p.splits == 1) return rc;
+  return launch_finish<DUAL, OutT>(p, st);
 }
 
 template <bool DUAL>
@@ -393,7 +467,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* a, const flo
   if (row < m && col < n) c[(int64_t)row * n + col] = b1 ? silu(g) * u : g;
 }
 
-constexpr int64_t kSkinnyMaxTokens = 64;
+constexpr int64_t kSkinnyMaxTokens = 32;
 
 int ffn_skinny(const void* x, const float* gamma, const void* w_gate, const void* w_up, const void* w_down,
                void* out, int64_t tokens, int64_t hidden, int64_t intermediate, float eps, int dtype,

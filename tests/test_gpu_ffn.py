@@ -91,7 +91,8 @@ def test_ffn_llama7b_linearity_and_sample(worker):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("t,h,i", [(1, 512, 1024), (16, 512, 1024), (32, 1024, 2816), (33, 512, 1024), (64, 1024, 2816)])
 def test_ffn_block_decode_sizes(worker, dtype, t, h, i):
-    """Decode-size token counts take the skinny-projection path (weights read once per 32 rows)."""
+    """Decode-size token counts: the skinny-projection path up to 32 tokens (weights read once),
+    the k-split tiled path above."""
     inp = workloads.ffn_inputs(tokens=t, hidden=h, intermediate=i, seed=3, dtype=dtype)
     with worker.register(ffn_block) as hd:
         hd(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, inp.out, inp.eps)
@@ -105,6 +106,29 @@ def test_ffn_block_decode_sizes(worker, dtype, t, h, i):
         hd(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, inp.out, inp.eps)
     worker.set_option("gemm_variant", 0)
     assert torch.allclose(out_skinny.float(), inp.out.float(), rtol=2e-2, atol=2e-3)
+
+
+@pytest.mark.parametrize("dtype,out_fp32", [(torch.bfloat16, False), (torch.float16, False), (torch.bfloat16, True)])
+@pytest.mark.parametrize("t,h,i", [(65, 1024, 2816), (100, 2048, 1000), (130, 1024, 2816), (256, 4096, 1024), (384, 512, 4096)])
+def test_ffn_block_few_hundred_tokens(worker, dtype, out_fp32, t, h, i):
+    """A few hundred tokens leave most CUs without an output tile: k is split over several
+    workgroups per tile (fp32 slabs summed in split order), for the gate/up pass too."""
+    inp = workloads.ffn_inputs(tokens=t, hidden=h, intermediate=i, seed=5, dtype=dtype)
+    out = torch.zeros(t, h, dtype=torch.float32) if out_fp32 else inp.out
+    with worker.register(ffn_block) as hd:
+        hd(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, out, inp.eps)
+    ref = oracle.ffn_block(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, inp.eps)
+    validate_golden({"out": out.float()}, {"out": ref.float()}, rtol=2e-2, atol=1e-2)
+    first = out.clone()
+    # unsplit tiles compute the same block; a second split run is bit-identical (no atomics)
+    worker.set_option("gemm_variant", 5)
+    with worker.register(ffn_block) as hd:
+        hd(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, out, inp.eps)
+    worker.set_option("gemm_variant", 0)
+    assert torch.allclose(first.float(), out.float(), rtol=2e-2, atol=2e-3)
+    with worker.register(ffn_block) as hd:
+        hd(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, out, inp.eps)
+    assert torch.equal(first, out)
 
 
 def test_ffn_swiglu_decode_size_without_norm(worker):
