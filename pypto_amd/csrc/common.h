@@ -8,6 +8,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <string>
+#include <vector>
 
 #include "pto_hip.h"
 
@@ -43,6 +44,9 @@ struct Context {
   // Intermediates of the composed decoder layer (grow-only).
   void* layer_ws = nullptr;
   size_t layer_ws_bytes = 0;
+  // Buffers the two scratch areas outgrew.  They stay allocated until pto_hip_close: launches
+  // recorded into a HIP graph keep the address they were recorded with.
+  std::vector<void*> retired;
   // 256 bytes of device flags written by kernels that report bad indices to the host.
   int* flags = nullptr;
   // options
@@ -57,8 +61,10 @@ struct Context {
 };
 
 Context& ctx();
-// Returns a workspace of at least `bytes` (reallocates if too small; stream-ordered callers
-// must not hold an older pointer across a growing call).
+// Returns a workspace of at least `bytes`.  A request beyond the current size allocates a new
+// buffer of at least twice the old size and retires the old one without freeing it, so that
+// queued work and launches recorded into a HIP graph stay valid; it fails while a stream is
+// being captured (allocation is not allowed then): make each call once before capturing it.
 int workspace(size_t bytes, void** ptr);
 
 // ---- W8A16 decode projections, shared with the composed decoder layer -------------------

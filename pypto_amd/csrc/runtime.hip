@@ -6,6 +6,7 @@
 // order; there is no task graph and no scheduler thread.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -34,34 +35,35 @@ Context& ctx() {
   return c;
 }
 
+namespace {
+// Grows *buf to at least `bytes`.  The outgrown buffer is retired, not freed: work already
+// queued and launches recorded into a HIP graph go on using it.  Doubling bounds the retired
+// memory by the size of the live buffer.
+int grow_scratch(void** buf, size_t* have, size_t bytes) {
+  if (bytes <= *have) return PTO_HIP_OK;
+  Context& c = ctx();
+  const size_t want = std::max(bytes + bytes / 4, 2 * *have);
+  void* fresh = nullptr;
+  PTO_CHECK_HIP(hipMalloc(&fresh, want));
+  if (*buf) c.retired.push_back(*buf);
+  *buf = fresh;
+  *have = want;
+  return PTO_HIP_OK;
+}
+}  // namespace
+
 int workspace(size_t bytes, void** ptr) {
   Context& c = ctx();
-  if (bytes > c.workspace_bytes) {
-    // Work queued on any stream may still read the old buffer.
-    PTO_CHECK_HIP(hipDeviceSynchronize());
-    if (c.workspace) PTO_CHECK_HIP(hipFree(c.workspace));
-    c.workspace = nullptr;
-    c.workspace_bytes = 0;
-    size_t want = bytes + bytes / 4;
-    PTO_CHECK_HIP(hipMalloc(&c.workspace, want));
-    c.workspace_bytes = want;
-  }
+  const int rc = grow_scratch(&c.workspace, &c.workspace_bytes, bytes);
   *ptr = c.workspace;
-  return PTO_HIP_OK;
+  return rc;
 }
 
 int layer_workspace(size_t bytes, void** ptr) {
   Context& c = ctx();
-  if (bytes > c.layer_ws_bytes) {
-    PTO_CHECK_HIP(hipDeviceSynchronize());
-    if (c.layer_ws) PTO_CHECK_HIP(hipFree(c.layer_ws));
-    c.layer_ws = nullptr;
-    c.layer_ws_bytes = 0;
-    PTO_CHECK_HIP(hipMalloc(&c.layer_ws, bytes));
-    c.layer_ws_bytes = bytes;
-  }
+  const int rc = grow_scratch(&c.layer_ws, &c.layer_ws_bytes, bytes);
   *ptr = c.layer_ws;
-  return PTO_HIP_OK;
+  return rc;
 }
 
 namespace {
@@ -533,6 +535,8 @@ int pto_hip_close(void) {
   if (c.layer_ws) PTO_CHECK_HIP(hipFree(c.layer_ws));
   c.layer_ws = nullptr;
   c.layer_ws_bytes = 0;
+  for (void* old : c.retired) PTO_CHECK_HIP(hipFree(old));
+  c.retired.clear();
   c.initialized = false;
   {
     std::lock_guard<std::mutex> lk(g_mu);
