@@ -107,7 +107,7 @@ __device__ __forceinline__ void store_rows(float* o, const f32x4 (&acc)[D / 128]
 // With an e4m3 cache a 16-byte K load holds 16 elements, i.e. the operands of two MFMA k-steps:
 //   K fragment [tile][s2]: token tile*16 + c, elements (s2*4 + j)*16 .. +16  (steps 2*s2, 2*s2+1)
 //   V fragment [set][e]  : 8 bytes, token as above, elements (set*16 + c)*8 .. +8
-// Codes are widened to bf16 exactly (scale 1); the per-(block, head) scales are applied to the
+// Codes are widened to the activation type exactly (scale 1); the per-(block, head) scales are applied to the
 // scores and to the accumulators in fp32.
 template <int D, bool FP8>
 struct KFrag {
@@ -178,16 +178,26 @@ __device__ __forceinline__ void load_v(VFrag<D, FP8>& v, const char* base0, cons
       v.t[set][e] = *reinterpret_cast<const vec_t*>((e < 4 ? base0 : base1) + voff + set * kSet + (e & 3) * kRow);
 }
 
-// Two e4m3 codes (low or high half of a dword) -> two packed bf16, exact.
-__device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w, bool hi) {
-  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-  const bf16x2 r = hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true)
-                      : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
-  return __builtin_bit_cast(uint32_t, r);
+// Two e4m3 codes (low or high half of a dword) -> two packed bf16 or fp16 values; both types
+// hold every e4m3 value exactly.
+template <bool BF16>
+__device__ __forceinline__ uint32_t fp8x2_widen(uint32_t w, bool hi) {
+  if constexpr (BF16) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const bf16x2 r = hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true)
+                        : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
+    return __builtin_bit_cast(uint32_t, r);
+  } else {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    const f16x2 r = hi ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true)
+                       : __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false);
+    return __builtin_bit_cast(uint32_t, r);
+  }
 }
-__device__ __forceinline__ u32x4 fp8x8_to_bf16x8(uint32_t w0, uint32_t w1) {
-  return u32x4{fp8x2_to_bf16x2(w0, false), fp8x2_to_bf16x2(w0, true), fp8x2_to_bf16x2(w1, false),
-               fp8x2_to_bf16x2(w1, true)};
+template <bool BF16>
+__device__ __forceinline__ u32x4 fp8x8_widen(uint32_t w0, uint32_t w1) {
+  return u32x4{fp8x2_widen<BF16>(w0, false), fp8x2_widen<BF16>(w0, true), fp8x2_widen<BF16>(w1, false),
+               fp8x2_widen<BF16>(w1, true)};
 }
 
 // S^T = K Q^T for one chunk: two 16x16 tiles, rows = tokens, columns = query heads.
@@ -198,10 +208,10 @@ __device__ __forceinline__ void qk_scores(const KFrag<D, FP8>& kf, const u32x4 (
   if constexpr (FP8) {
 #pragma unroll
     for (int s2 = 0; s2 < D / 64; ++s2) {
-      s0 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[0][s2][0], kf.t[0][s2][1]), qf[2 * s2], s0);
-      s1 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[1][s2][0], kf.t[1][s2][1]), qf[2 * s2], s1);
-      s0 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[0][s2][2], kf.t[0][s2][3]), qf[2 * s2 + 1], s0);
-      s1 = mfma16<BF16>(fp8x8_to_bf16x8(kf.t[1][s2][2], kf.t[1][s2][3]), qf[2 * s2 + 1], s1);
+      s0 = mfma16<BF16>(fp8x8_widen<BF16>(kf.t[0][s2][0], kf.t[0][s2][1]), qf[2 * s2], s0);
+      s1 = mfma16<BF16>(fp8x8_widen<BF16>(kf.t[1][s2][0], kf.t[1][s2][1]), qf[2 * s2], s1);
+      s0 = mfma16<BF16>(fp8x8_widen<BF16>(kf.t[0][s2][2], kf.t[0][s2][3]), qf[2 * s2 + 1], s0);
+      s1 = mfma16<BF16>(fp8x8_widen<BF16>(kf.t[1][s2][2], kf.t[1][s2][3]), qf[2 * s2 + 1], s1);
     }
   } else {
 #pragma unroll
@@ -280,7 +290,7 @@ __device__ __forceinline__ void pv_chunk(VFrag<D, FP8>& vf, const u32x4 (&pf)[GT
     u32x4 vw[8];  // the lane's 8 tokens x 8 elements as 16-bit values
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      if constexpr (FP8) vw[e] = fp8x8_to_bf16x8(vf.t[set][e].x, vf.t[set][e].y);
+      if constexpr (FP8) vw[e] = fp8x8_widen<BF16>(vf.t[set][e].x, vf.t[set][e].y);
       else vw[e] = vf.t[set][e];
     }
 #pragma unroll
@@ -855,8 +865,6 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   // grid over all CUs instead of filling some to their register limit.
   const int64_t cap = pto_hip::ctx().attn_waves_per_cu;
   const size_t lds = cap > 0 ? (size_t)(163840 / cap) / 1024 * 1024 : 0;
-  if (!bf16 && FP8)
-    return pto_hip::fail(PTO_HIP_ERR_UNSUPPORTED, "paged_attention: an FP8E4M3FN cache needs a BF16 query");
   if (p.n_wg > 0) {
     // Evenly split form: one workgroup of lean_waves wavefronts per CU.  The LDS request (K stages
     // of the wavefronts, padded past half of the CU's LDS) keeps a second workgroup off the CU.
@@ -874,7 +882,7 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
     };
     int rc = PTO_HIP_OK;
     if (bf16) rc = go(attn_lean_kernel<D, true, FP8, GT>);
-    else if constexpr (!FP8) rc = go(attn_lean_kernel<D, false, false, GT>);
+    else rc = go(attn_lean_kernel<D, false, FP8, GT>);
     if (rc) return rc;
     PTO_CHECK_HIP(hipGetLastError());
     if (!pto_hip::ctx().attn_skip_merge) {
@@ -885,8 +893,8 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
     return PTO_HIP_OK;
   } else if (bf16) {
     hipLaunchKernelGGL((attn_partition_kernel<D, true, FP8, GT>), grid, dim3(64), lds, stream, p);
-  } else if constexpr (!FP8) {
-    hipLaunchKernelGGL((attn_partition_kernel<D, false, false, GT>), grid, dim3(64), lds, stream, p);
+  } else {
+    hipLaunchKernelGGL((attn_partition_kernel<D, false, FP8, GT>), grid, dim3(64), lds, stream, p);
   }
   PTO_CHECK_HIP(hipGetLastError());
   // "attn_skip_merge" leaves the partials unmerged: a timing aid that isolates the streaming

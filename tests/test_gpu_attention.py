@@ -228,6 +228,17 @@ def test_fp8_cache_matches_golden(worker, batch, hq, hkv, bs, ctxs):
         _check(_run(worker, inp, tpp), ref)
 
 
+def test_fp8_cache_with_fp16_query(worker):
+    """e4m3 codes widen exactly to fp16 as well: an fp16 query runs on the quantised cache."""
+    inp = workloads.paged_attention_inputs(batch=3, num_heads=32, kv_head_num=4, block_size=64,
+                                           context_lens=[300, 17, 1029], ctx_range=(1, 1029), fp8_kv=True,
+                                           dtype=torch.float16, seed=17)
+    assert inp.query.dtype == torch.float16 and inp.key_cache.dtype == torch.float8_e4m3fn
+    ref = _golden(inp)
+    for tpp in (0, -2, 128):
+        _check(_run(worker, inp, tpp), ref)
+
+
 def test_fp8_quantiser_agrees_with_oracle():
     """The input builder's quantiser and the oracle's are the same function of the data."""
     g = torch.Generator().manual_seed(0)

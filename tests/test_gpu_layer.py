@@ -223,12 +223,13 @@ def test_decoder_layer_decode(worker, batch, ctxs):
     assert changed <= batch * 2
 
 
-def test_decoder_layer_decode_fp8_kv(worker):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_decoder_layer_decode_fp8_kv(worker, dtype):
     """The same reduced layer over e4m3 caches: rows quantised on write, attention dequantises."""
     batch = 6
     ctxs = [100, 1, 257, 33, 128, 129]
     inp = workloads.decoder_layer_inputs(batch=batch, hidden=1024, num_heads=8, kv_head_num=2, head_dim=128,
-                                         intermediate=2816, block_size=128, context_lens=ctxs, seed=8)
+                                         intermediate=2816, block_size=128, context_lens=ctxs, seed=8, dtype=dtype)
     pool_blocks = inp.key_cache.shape[0] // (2 * 128)
     kc, ks = oracle.quantize_kv_fp8(inp.key_cache, pool_blocks, 2, 128)
     vc, vs = oracle.quantize_kv_fp8(inp.value_cache, pool_blocks, 2, 128)
