@@ -44,7 +44,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--no-ffn", action="store_true", help="skip the FFN measurement")
     ap.add_argument("--no-extra", action="store_true",
-                    help="skip the long-context e4m3 attention and decoder-layer measurements")
+                    help="skip the other workloads of the path: long-context e4m3 attention, decoder layer, "
+                         "FFN at 16 tokens, 64-head MQA attention")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy, a known-size reference for HBM byte counters")
     args = ap.parse_args()
@@ -191,6 +192,48 @@ def main() -> int:
             "bound": "hbm",
         }
         del dl, dargs
+        torch.cuda.empty_cache()
+        # FFN block at a decode-size token count: bound by reading the 16-bit weights once
+        fd = [workloads.ffn_inputs(tokens=16, hidden=4096, intermediate=11008, seed=s, device="cuda") for s in (0, 1)]
+        torch.cuda.synchronize()
+        with worker.register(ffn_block) as fh:
+            fdargs = [(f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.out, f.eps) for f in fd]
+            benchmark(fh, fdargs, rounds=10, warmup=0)
+            fdstats = benchmark(fh, fdargs, rounds=40, warmup=0)
+        wbytes = 3 * 4096 * 11008 * 2 + 2 * 16 * 4096 * 2
+        result["ffn_decode"] = {
+            "workload": "FFN LLaMA-7B at 16 tokens: H4096 I11008 bf16 weights streamed once, RMSNorm prologue, SwiGLU",
+            "algorithmic_bytes_per_step": wbytes,
+            "us_per_step": round(fdstats.device_wall_us, 1),
+            "achieved": round(wbytes / fdstats.device_wall_us / 1e3, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(wbytes / fdstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "bound": "hbm",
+        }
+        del fd, fdargs
+        torch.cuda.empty_cache()
+        # 64 query heads on one KV head (the reference's q_tile 64 shape at a serving size)
+        mq = workloads.paged_attention_inputs(batch=256, num_heads=64, kv_head_num=1, head_dim=128, block_size=128,
+                                              ctx_range=(2048, 4096), seed=0, device="cuda")
+        torch.cuda.synchronize()
+        with worker.register(paged_attention) as mh:
+            margs = [mq.args()]
+            benchmark(mh, margs, rounds=5, warmup=0)
+            mstats = benchmark(mh, margs, rounds=20, warmup=0)
+        mbytes = mq.algorithmic_bytes()
+        result["attention_mqa64"] = {
+            "workload": "paged-attention decode, 64 query heads per KV head: B256 Hq64 Hkv1 D128 bs128 "
+                        "ctx~U[2048,4096] bf16 KV; the cache is counted once",
+            "algorithmic_bytes_per_step": mbytes,
+            "us_per_step": round(mstats.device_wall_us, 1),
+            "achieved": round(mbytes / mstats.device_wall_us / 1e3, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(mbytes / mstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "bound": "hbm",
+        }
+        del mq, margs
         torch.cuda.empty_cache()
 
     # ---- CPU baseline: the oracle on this machine's host cores --------------------------------
