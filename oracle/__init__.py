@@ -17,6 +17,13 @@ Pinning status (what fixes each function independently of its own formula):
                                  on gathered dense K/V, softmax invariants
                                  (uniform scores -> mean of V, dominant score ->
                                  that V row), partition independence.
+* ``stages.*``                — pinned: the reference's kernel-level known answers
+                                 (all-ones scores -> m = scale, P = 1, l = block
+                                 size; the four is_first / is_last cases on its
+                                 constant state), and the block-by-block task
+                                 loop built from them reproduces
+                                 ``paged_attention_golden`` to 1e-4
+                                 (tests/test_oracle_stages.py).
 * ``ffn_swiglu`` / ``ffn_block`` — pinned: ``torch.nn.functional.silu`` form in
                                  fp64, committed seeded fixture.
 * ``rms_norm``                — pinned: ``torch.nn.functional.rms_norm``.
@@ -37,6 +44,7 @@ from .attention import (  # noqa: F401
     paged_gather,
     quantize_kv_fp8,
 )
+from . import stages  # noqa: F401
 from .ffn import ffn_block, ffn_swiglu, rms_norm, swiglu  # noqa: F401
 from .layer import (  # noqa: F401
     decoder_layer_decode,
