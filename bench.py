@@ -45,7 +45,7 @@ def main() -> int:
     ap.add_argument("--no-ffn", action="store_true", help="skip the FFN measurement")
     ap.add_argument("--no-extra", action="store_true",
                     help="skip the other workloads of the path: long-context e4m3 attention, decoder layer, "
-                         "FFN at 16 tokens, 64-head MQA attention")
+                         "the layer with bf16 weights, FFN at 16 tokens, 64-head MQA attention")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy, a known-size reference for HBM byte counters")
     args = ap.parse_args()
@@ -56,8 +56,8 @@ def main() -> int:
     import torch
 
     from pypto_amd import workloads
-    from pypto_amd.runtime import (ChipWorker, RunConfig, benchmark, decoder_layer_decode, ffn_block,
-                                   paged_attention)
+    from pypto_amd.runtime import (ChipWorker, RunConfig, benchmark, decoder_layer_decode, decoder_layer_decode_w16,
+                                   ffn_block, paged_attention)
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -192,6 +192,27 @@ def main() -> int:
             "bound": "hbm",
         }
         del dl, dargs
+        torch.cuda.empty_cache()
+        # the same layer with the reference's 16-bit weights
+        dw = workloads.decoder_layer_inputs(device="cuda", int8_weights=False)
+        torch.cuda.synchronize()
+        with worker.register(decoder_layer_decode_w16) as dh:
+            dwargs = [dw.args()]
+            benchmark(dh, dwargs, rounds=5, warmup=0)
+            dwstats = benchmark(dh, dwargs, rounds=20, warmup=0)
+        dwbytes = dw.algorithmic_bytes()
+        result["decoder_layer_w16"] = {
+            "workload": "decoder-layer decode step with bf16 weights (the reference's layer): H4096 Hq32 Hkv8 D128 "
+                        "I14336 B32 ctx4096, bf16 activations and paged KV",
+            "algorithmic_bytes_per_step": dwbytes,
+            "us_per_step": round(dwstats.device_wall_us, 1),
+            "achieved": round(dwbytes / dwstats.device_wall_us / 1e3, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(dwbytes / dwstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "bound": "hbm",
+        }
+        del dw, dwargs
         torch.cuda.empty_cache()
         # FFN block at a decode-size token count: bound by reading the 16-bit weights once
         fd = [workloads.ffn_inputs(tokens=16, hidden=4096, intermediate=11008, seed=s, device="cuda") for s in (0, 1)]

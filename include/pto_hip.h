@@ -136,7 +136,8 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *      tensors: hidden_states[B,H], seq_lens, block_table, key_cache (INOUT), value_cache (INOUT),
  *               rope_cos, rope_sin, gamma_in[H], gamma_post[H], wqkv_q, wqkv_s, wo_q, wo_s, wg_q, wg_s,
  *               wu_q, wu_s, wd_q, wd_s, out[B,H]
- *               (FP8E4M3FN caches: k_scale, v_scale [pool,Hkv] fp32 (INOUT) follow value_cache)
+ *               (16-bit weights, as in the reference: wqkv, wo, wg, wu, wd without the *_s tensors;
+ *                FP8E4M3FN caches: k_scale, v_scale [pool,Hkv] fp32 (INOUT) follow value_cache)
  *      scalars: num_heads, kv_head_num, head_dim, block_size, eps (f32 bits)
  */
 PTO_HIP_API int pto_hip_register(const char* program_name, int* callable_id);
@@ -234,7 +235,9 @@ PTO_HIP_API int pto_hip_rope_kv_cache_update_fp8(const float* qkv, const int32_t
 
 /* One decoder layer, one new token per sequence (examples/models/qwen3_jit/qwen3_decode.py:47-113):
  * RMSNorm -> QKV -> RoPE + K/V append -> paged attention -> o_proj + residual -> RMSNorm ->
- * SwiGLU FFN + residual.  Projection weights are INT8 [in, out] with FP32 per-output scales.
+ * SwiGLU FFN + residual.  Projection weights are [in, out]: either the reference's 16-bit weights
+ * (all *_s pointers NULL; golden tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:255-287)
+ * or INT8 codes with FP32 per-output scales.
  * With e4m3 caches pool_rows is still the row count of each cache (pool_blocks * Hkv * block_size). */
 typedef struct PtoHipDecoderLayerArgs {
   const void* hidden_states;  /* [B, H] dtype */
@@ -246,8 +249,8 @@ typedef struct PtoHipDecoderLayerArgs {
   const float* rope_sin;
   const float* gamma_in;      /* [H] */
   const float* gamma_post;    /* [H] */
-  const void* wqkv_q;         /* [H, (Hq+2Hkv)*D] int8 */
-  const float* wqkv_s;
+  const void* wqkv_q;         /* [H, (Hq+2Hkv)*D] int8, or `dtype` when the scales are NULL */
+  const float* wqkv_s;        /* [out channels] FP32; all five scales NULL = 16-bit weights */
   const void* wo_q;           /* [Hq*D, H] */
   const float* wo_s;
   const void* wg_q;           /* [H, I] */

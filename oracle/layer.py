@@ -94,9 +94,11 @@ def quantize_w8(w: torch.Tensor):
     return w_q, scale.contiguous()
 
 
-def w8a16_matmul(x: torch.Tensor, w_q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
-    """``(x @ w_q) * scale`` with fp32 accumulation -> fp32."""
-    return torch.matmul(x.float(), w_q.float()) * scale.float().reshape(1, -1)
+def w8a16_matmul(x: torch.Tensor, w_q: torch.Tensor, scale: torch.Tensor | None) -> torch.Tensor:
+    """``(x @ w_q) * scale`` with fp32 accumulation -> fp32.  ``scale=None``: unquantised weights, the
+    plain fp32 product of the reference's projections (test_qwen3_decode_scope3_mixed.py:271,280-284)."""
+    y = torch.matmul(x.float(), w_q.float())
+    return y if scale is None else y * scale.float().reshape(1, -1)
 
 
 def decoder_layer_decode(
@@ -113,6 +115,9 @@ def decoder_layer_decode(
     attention over ``seq_len`` tokens -> o_proj + residual -> RMSNorm -> SwiGLU FFN
     + residual (test_qwen3_decode_scope3_mixed.py:255-287).  Activations are
     rounded to the activation dtype wherever the model path casts.
+
+    Each weight comes with its per-channel scale (int8 codes) or with ``None`` (16-bit weights,
+    the reference's own layer).
 
     With float8_e4m3fn caches (``k_scale``/``v_scale`` [pool_blocks, Hkv] given) the new rows
     are quantised on write (``kv_append_fp8``) from their fp32 values.

@@ -5,7 +5,7 @@
 // Composition of the reference's decode layer (examples/models/qwen3_jit/qwen3_decode.py:47-113,
 // examples/models/08_llama_mini.py:384-483; golden
 // tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:255-287), with the
-// projections taking int8 weights and per-channel scales.  The reference submits one task per
+// projections taking either the reference's 16-bit weights or int8 weights and per-channel scales.  The reference submits one task per
 // tile through its scheduler; here the layer is eleven kernel launches in stream order; each projection is a partial-sum
 // kernel whose finish is folded into the elementwise step that follows it.
 #include <hip/hip_runtime.h>
@@ -47,15 +47,30 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
                 "decoder_layer_decode: bad model dimensions");
   PTO_CHECK_ARG(a->dtype == PTO_HIP_BF16 || a->dtype == PTO_HIP_FP16,
                 "decoder_layer_decode: activation dtype %s not in {BF16, FP16}", dtype_name(a->dtype));
+  // What the projection and attention kernels assume of the shapes (16-byte operand rows, whole
+  // 16-row k steps, at least one 32-row step).
+  PTO_CHECK_ARG(d == 128 || d == 256, "decoder_layer_decode: head_dim %lld not built (128, 256)", (long long)d);
+  PTO_CHECK_ARG(h % 16 == 0 && h >= 32 && inter % 16 == 0 && inter >= 32,
+                "decoder_layer_decode: hidden %lld and intermediate %lld must be multiples of 16, at least 32",
+                (long long)h, (long long)inter);
+  PTO_CHECK_ARG(a->block_size > 0 && a->block_size % 16 == 0 && a->max_num_blocks_per_req > 0 && a->max_pos > 0,
+                "decoder_layer_decode: block_size must be a positive multiple of 16, the table and RoPE tables non-empty");
   const bool fp8kv = a->kv_dtype == PTO_HIP_FP8E4M3FN;
   PTO_CHECK_ARG(a->kv_dtype == 0 || a->kv_dtype == a->dtype || fp8kv,
                 "decoder_layer_decode: cache dtype %s must be the activation dtype or FP8E4M3FN",
                 dtype_name(a->kv_dtype));
   PTO_CHECK_ARG(!fp8kv || (a->k_scale && a->v_scale), "decoder_layer_decode: e4m3 caches need k_scale and v_scale");
   PTO_CHECK_ARG(a->hidden_states && a->out && a->seq_lens && a->block_table && a->key_cache && a->value_cache &&
-                    a->rope_cos && a->rope_sin && a->gamma_in && a->gamma_post && a->wqkv_q && a->wqkv_s &&
-                    a->wo_q && a->wo_s && a->wg_q && a->wg_s && a->wu_q && a->wu_s && a->wd_q && a->wd_s,
+                    a->rope_cos && a->rope_sin && a->gamma_in && a->gamma_post && a->wqkv_q && a->wo_q && a->wg_q &&
+                    a->wu_q && a->wd_q,
                 "decoder_layer_decode: null tensor pointer");
+  // All five scales null: the weights are 16-bit values of the activation type (the reference's
+  // own layer); all five set: INT8 codes with one scale per output channel.
+  const int n_scales = (a->wqkv_s != nullptr) + (a->wo_s != nullptr) + (a->wg_s != nullptr) + (a->wu_s != nullptr) +
+                       (a->wd_s != nullptr);
+  PTO_CHECK_ARG(n_scales == 0 || n_scales == 5,
+                "decoder_layer_decode: weight scales must be given for all five projections or for none");
+  const bool w16 = n_scales == 0;
   hipStream_t st = (hipStream_t)stream;
   const int dt = a->dtype;
   const int64_t qkv_n = (hq + 2 * hkv) * d;
@@ -92,7 +107,7 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
   else rc = pto_hip_rms_norm(a->hidden_states, a->gamma_in, normed, b, h, a->eps, dt, dt, stream);
   if (rc) return rc;
   // 2. QKV projection, left as k-split partial sums
-  if ((rc = w8a16_partials(normed, blk, a->wqkv_q, nullptr, b, h, qkv_n, dt, st, &parts))) return rc;
+  if ((rc = w8a16_partials(normed, blk, a->wqkv_q, nullptr, b, h, qkv_n, dt, st, &parts, w16))) return rc;
   // 3. finish of the projection + RoPE at pos = seq_len - 1, append K/V, rotated Q
   if (fp8kv) {
     const int64_t pool_blocks = a->pool_rows / (hkv * a->block_size);
@@ -117,7 +132,7 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
                             fp8kv ? a->v_scale : nullptr, stream)))
     return rc;
   // 5. o_proj; 6. its finish + residual -> fp32, post-attention RMSNorm -> activation dtype
-  if ((rc = w8a16_partials(attn16, blk_attn, a->wo_q, nullptr, b, hq * d, h, dt, st, &parts))) return rc;
+  if ((rc = w8a16_partials(attn16, blk_attn, a->wo_q, nullptr, b, hq * d, h, dt, st, &parts, w16))) return rc;
   if (w8a16_finish_norm_fits(h)) {
     if ((rc = w8a16_finish_norm(parts, a->wo_s, a->hidden_states, dt, resid1, a->gamma_post, normed2, dt, blk, b, h,
                                 a->eps, st)))
@@ -128,8 +143,8 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
     if ((rc = pto_hip_rms_norm(resid1, a->gamma_post, normed2, b, h, a->eps, PTO_HIP_FP32, dt, stream))) return rc;
   }
   // 7. gate/up + SwiGLU -> h (activation dtype), 8. down + residual -> out
-  if ((rc = w8a16_partials(normed2, blk, a->wg_q, a->wu_q, b, h, inter, dt, st, &parts))) return rc;
+  if ((rc = w8a16_partials(normed2, blk, a->wg_q, a->wu_q, b, h, inter, dt, st, &parts, w16))) return rc;
   if ((rc = w8a16_finish(parts, a->wg_s, a->wu_s, nullptr, 0, hbuf, dt, blk, b, inter, st))) return rc;
-  if ((rc = w8a16_partials(hbuf, blk, a->wd_q, nullptr, b, inter, h, dt, st, &parts))) return rc;
+  if ((rc = w8a16_partials(hbuf, blk, a->wd_q, nullptr, b, inter, h, dt, st, &parts, w16))) return rc;
   return w8a16_finish(parts, a->wd_s, nullptr, resid1, PTO_HIP_FP32, a->out, dt, false, b, h, st);
 }

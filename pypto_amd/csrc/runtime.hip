@@ -382,16 +382,27 @@ int run_rope_kv(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hi
 }
 
 int run_decoder_layer(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream) {
-  PTO_CHECK_ARG((nt == 20 || nt == 22) && ns == 5,
-                "decoder_layer_decode: expected 20 tensors (22 with k_scale, v_scale after the FP8E4M3FN "
-                "caches) + scalars num_heads, kv_head_num, head_dim, block_size, eps; got %d + %d", nt, ns);
+  PTO_CHECK_ARG((nt == 20 || nt == 22 || nt == 15 || nt == 17) && ns == 5,
+                "decoder_layer_decode: expected 20 tensors with INT8 weights and their scales or 15 with 16-bit "
+                "weights (2 more with k_scale, v_scale after FP8E4M3FN caches) + scalars num_heads, kv_head_num, "
+                "head_dim, block_size, eps; got %d + %d", nt, ns);
   // With an e4m3 cache the two scale tensors follow value_cache; o shifts the later operands.
-  const bool fp8 = nt == 22;
+  // INT8 weights come as (codes, scales) pairs, 16-bit weights alone.
+  const bool fp8 = nt == 22 || nt == 17;
+  const bool w16 = nt == 15 || nt == 17;
   const int o = fp8 ? 2 : 0;
+  const int wstep = w16 ? 1 : 2;
   for (int i = 0; i < nt; ++i) {
     int rc = check_tensor("decoder_layer_decode", "operand", t[i], 1, 2);
     if (rc) return rc;
   }
+  const PtoHipChipTensor* w[5];   // qkv, o, gate, up, down
+  const PtoHipChipTensor* ws[5];  // their scales (INT8 weights)
+  for (int i = 0; i < 5; ++i) {
+    w[i] = &t[9 + o + i * wstep];
+    ws[i] = w16 ? nullptr : &t[10 + o + i * wstep];
+  }
+  const PtoHipChipTensor& out = t[nt - 1];
   PtoHipDecoderLayerArgs a{};
   a.hidden_states = tptr(t[0]);
   a.seq_lens = reinterpret_cast<const int32_t*>(tptr(t[1]));
@@ -407,17 +418,18 @@ int run_decoder_layer(const PtoHipChipTensor* t, int nt, const uint64_t* s, int 
   a.rope_sin = reinterpret_cast<const float*>(tptr(t[6 + o]));
   a.gamma_in = reinterpret_cast<const float*>(tptr(t[7 + o]));
   a.gamma_post = reinterpret_cast<const float*>(tptr(t[8 + o]));
-  a.wqkv_q = tptr(t[9 + o]);
-  a.wqkv_s = reinterpret_cast<const float*>(tptr(t[10 + o]));
-  a.wo_q = tptr(t[11 + o]);
-  a.wo_s = reinterpret_cast<const float*>(tptr(t[12 + o]));
-  a.wg_q = tptr(t[13 + o]);
-  a.wg_s = reinterpret_cast<const float*>(tptr(t[14 + o]));
-  a.wu_q = tptr(t[15 + o]);
-  a.wu_s = reinterpret_cast<const float*>(tptr(t[16 + o]));
-  a.wd_q = tptr(t[17 + o]);
-  a.wd_s = reinterpret_cast<const float*>(tptr(t[18 + o]));
-  a.out = tptr_mut(t[19 + o]);
+  auto scale_of = [&](int i) { return w16 ? nullptr : reinterpret_cast<const float*>(tptr(*ws[i])); };
+  a.wqkv_q = tptr(*w[0]);
+  a.wqkv_s = scale_of(0);
+  a.wo_q = tptr(*w[1]);
+  a.wo_s = scale_of(1);
+  a.wg_q = tptr(*w[2]);
+  a.wg_s = scale_of(2);
+  a.wu_q = tptr(*w[3]);
+  a.wu_s = scale_of(3);
+  a.wd_q = tptr(*w[4]);
+  a.wd_s = scale_of(4);
+  a.out = tptr_mut(out);
   PTO_CHECK_ARG(t[0].ndims == 2, "decoder_layer_decode: hidden_states must be [B, H]");
   a.batch = t[0].shapes[0];
   a.hidden = t[0].shapes[1];
@@ -428,18 +440,18 @@ int run_decoder_layer(const PtoHipChipTensor* t, int nt, const uint64_t* s, int 
   a.eps = scalar_f32(s[4]);
   PTO_CHECK_ARG(a.num_heads > 0 && a.kv_head_num > 0 && a.head_dim > 1 && a.block_size > 0,
                 "decoder_layer_decode: non-positive scalar");
-  PTO_CHECK_ARG(t[13 + o].ndims == 2, "decoder_layer_decode: w_gate must be [H, I]");
-  a.intermediate = t[13 + o].shapes[1];
+  PTO_CHECK_ARG(w[2]->ndims == 2, "decoder_layer_decode: w_gate must be [H, I]");
+  a.intermediate = w[2]->shapes[1];
   a.max_num_blocks_per_req = a.batch ? numel(t[2]) / a.batch : 1;
   a.max_pos = numel(t[5 + o]) / (a.head_dim / 2);
   a.pool_rows = numel(t[3]) / a.head_dim;
   a.dtype = (int)t[0].dtype;
   const int64_t qkv_n = (a.num_heads + 2 * a.kv_head_num) * a.head_dim;
-  PTO_CHECK_ARG(t[19 + o].dtype == t[0].dtype, "decoder_layer_decode: out must have the activation dtype");
+  PTO_CHECK_ARG(out.dtype == t[0].dtype, "decoder_layer_decode: out must have the activation dtype");
   if (fp8) {
     PTO_CHECK_ARG(t[3].dtype == PTO_HIP_FP8E4M3FN && t[4].dtype == PTO_HIP_FP8E4M3FN && t[5].dtype == PTO_HIP_FP32 &&
                       t[6].dtype == PTO_HIP_FP32,
-                  "decoder_layer_decode: with 22 tensors the caches must be FP8E4M3FN and the scales FP32");
+                  "decoder_layer_decode: with k_scale and v_scale the caches must be FP8E4M3FN and the scales FP32");
     const int64_t per_block = a.kv_head_num * a.block_size * a.head_dim;
     PTO_CHECK_ARG(numel(t[3]) % per_block == 0 && numel(t[5]) == numel(t[3]) / per_block * a.kv_head_num &&
                       numel(t[6]) == numel(t[5]) && numel(t[4]) == numel(t[3]),
@@ -448,14 +460,19 @@ int run_decoder_layer(const PtoHipChipTensor* t, int nt, const uint64_t* s, int 
     PTO_CHECK_ARG(t[3].dtype == t[0].dtype && t[4].dtype == t[0].dtype,
                   "decoder_layer_decode: caches must have the activation dtype");
   }
-  PTO_CHECK_ARG(t[9 + o].dtype == PTO_HIP_INT8 && numel(t[9 + o]) == a.hidden * qkv_n && numel(t[10 + o]) == qkv_n &&
-                    numel(t[11 + o]) == a.num_heads * a.head_dim * a.hidden && numel(t[12 + o]) == a.hidden &&
-                    numel(t[13 + o]) == a.hidden * a.intermediate && numel(t[15 + o]) == numel(t[13 + o]) &&
-                    numel(t[17 + o]) == numel(t[13 + o]) && numel(t[14 + o]) == a.intermediate &&
-                    numel(t[16 + o]) == a.intermediate && numel(t[18 + o]) == a.hidden,
-                "decoder_layer_decode: weight or scale shapes do not match the model dimensions");
+  const int64_t w_numel[5] = {a.hidden * qkv_n, a.num_heads * a.head_dim * a.hidden, a.hidden * a.intermediate,
+                              a.hidden * a.intermediate, a.intermediate * a.hidden};
+  const int64_t s_numel[5] = {qkv_n, a.hidden, a.intermediate, a.intermediate, a.hidden};
+  for (int i = 0; i < 5; ++i) {
+    PTO_CHECK_ARG(numel(*w[i]) == w_numel[i] && (w16 ? w[i]->dtype == t[0].dtype : w[i]->dtype == PTO_HIP_INT8),
+                  "decoder_layer_decode: weight %d must be %s with %lld elements", i,
+                  w16 ? "of the activation dtype" : "INT8", (long long)w_numel[i]);
+    if (!w16)
+      PTO_CHECK_ARG(ws[i]->dtype == PTO_HIP_FP32 && numel(*ws[i]) == s_numel[i],
+                    "decoder_layer_decode: scale %d must be FP32 with %lld elements", i, (long long)s_numel[i]);
+  }
   PTO_CHECK_ARG(numel(t[7 + o]) == a.hidden && numel(t[8 + o]) == a.hidden && numel(t[1]) == a.batch &&
-                    numel(t[19 + o]) == a.batch * a.hidden,
+                    numel(out) == a.batch * a.hidden,
                 "decoder_layer_decode: gamma, seq_lens or out shape mismatch");
   return pto_hip_decoder_layer_decode(&a, stream);
 }

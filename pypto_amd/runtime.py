@@ -87,6 +87,14 @@ decoder_layer_decode_fp8kv = HipProgram(
     "decoder_layer_decode", (IN, IN, IN, INOUT, INOUT, INOUT, INOUT) + (IN,) * 14 + (OUT,),
     scalars=("num_heads", "kv_head_num", "head_dim", "block_size", "eps"))
 
+# the reference's own layer: 16-bit weights, no scale tensors
+decoder_layer_decode_w16 = HipProgram(
+    "decoder_layer_decode", (IN, IN, IN, INOUT, INOUT) + (IN,) * 9 + (OUT,),
+    scalars=("num_heads", "kv_head_num", "head_dim", "block_size", "eps"))
+decoder_layer_decode_w16_fp8kv = HipProgram(
+    "decoder_layer_decode", (IN, IN, IN, INOUT, INOUT, INOUT, INOUT) + (IN,) * 9 + (OUT,),
+    scalars=("num_heads", "kv_head_num", "head_dim", "block_size", "eps"))
+
 PROGRAMS = {p.name: p for p in (paged_attention, paged_gather, rms_norm, ffn_swiglu, ffn_block, w8a16_matmul,
                                 w8a16_swiglu, rope_kv_cache_update, rope_kv_cache_update_fp8,
                                 decoder_layer_decode)}

@@ -241,7 +241,9 @@ class DecoderLayerInputs:
     rope_sin: torch.Tensor
     gamma_in: torch.Tensor
     gamma_post: torch.Tensor
-    weights: dict  # name -> (codes int8 [in,out], scale fp32 [out]) for qkv, o, gate, up, down
+    # name -> (codes int8 [in,out], scale fp32 [out]) for qkv, o, gate, up, down; with 16-bit
+    # weights (weights [in,out] of the activation dtype, None)
+    weights: dict
     out: torch.Tensor
     num_heads: int
     kv_head_num: int
@@ -251,22 +253,24 @@ class DecoderLayerInputs:
     eps: float = 1e-6
 
     def args(self) -> tuple:
-        w = self.weights
+        flat = [t for name in ("qkv", "o", "gate", "up", "down") for t in self.weights[name] if t is not None]
         return (self.hidden, self.seq_lens, self.block_table, self.key_cache, self.value_cache, self.rope_cos,
-                self.rope_sin, self.gamma_in, self.gamma_post, *w["qkv"], *w["o"], *w["gate"], *w["up"], *w["down"],
+                self.rope_sin, self.gamma_in, self.gamma_post, *flat,
                 self.out, self.num_heads, self.kv_head_num, self.head_dim, self.block_size, self.eps)
 
     def algorithmic_bytes(self) -> int:
-        """int8 weights + the K/V rows attention reads (the HBM-bound part of the step)."""
-        wbytes = sum(c.numel() for c, _ in self.weights.values())
+        """Weights + the K/V rows attention reads (the HBM-bound part of the step)."""
+        wbytes = sum(c.numel() * c.element_size() for c, _ in self.weights.values())
         kv = int(self.seq_lens.sum().item()) * self.kv_head_num * self.head_dim * 2 * self.key_cache.element_size()
         return wbytes + kv
 
 
 def decoder_layer_inputs(*, batch=32, hidden=4096, num_heads=32, kv_head_num=8, head_dim=128,
                          intermediate=14336, context=4096, block_size=128, theta=5e5,
-                         dtype=torch.bfloat16, seed=0, device="cpu", context_lens=None) -> DecoderLayerInputs:
-    """One decode step of a LLaMA-style layer: int8 weights from N(0,0.02), bf16 activations and KV."""
+                         dtype=torch.bfloat16, seed=0, device="cpu", context_lens=None,
+                         int8_weights=True) -> DecoderLayerInputs:
+    """One decode step of a LLaMA-style layer: weights from N(0,0.02) as int8 codes + scales or, with
+    ``int8_weights=False``, in the activation dtype; 16-bit activations and KV."""
     dev = torch.device(device)
     g = torch.Generator(device=dev).manual_seed(seed)
 
@@ -289,12 +293,13 @@ def decoder_layer_inputs(*, batch=32, hidden=4096, num_heads=32, kv_head_num=8, 
         off += n
     rows = total * kv_head_num * block_size
     qkv_n = (num_heads + 2 * kv_head_num) * head_dim
+    pack = quantize_w8 if int8_weights else (lambda w: (w.to(dtype), None))
     weights = {
-        "qkv": quantize_w8(rn((hidden, qkv_n), 0.02)),
-        "o": quantize_w8(rn((num_heads * head_dim, hidden), 0.02)),
-        "gate": quantize_w8(rn((hidden, intermediate), 0.02)),
-        "up": quantize_w8(rn((hidden, intermediate), 0.02)),
-        "down": quantize_w8(rn((intermediate, hidden), 0.02)),
+        "qkv": pack(rn((hidden, qkv_n), 0.02)),
+        "o": pack(rn((num_heads * head_dim, hidden), 0.02)),
+        "gate": pack(rn((hidden, intermediate), 0.02)),
+        "up": pack(rn((hidden, intermediate), 0.02)),
+        "down": pack(rn((intermediate, hidden), 0.02)),
     }
     cos, sin = rope_tables(max_blocks * block_size, head_dim, theta, device=dev)
     return DecoderLayerInputs(

@@ -129,3 +129,38 @@ def test_kv_append_fp8_properties():
     true = grow[:, 0].permute(1, 0, 2)
     bound = (bs * 2.0 ** -4) * true.abs() + (scale[0].reshape(kv, 1, 1) * 2.0 ** -9) * bs
     assert ((deq - true).abs() <= bound).all()
+
+
+def test_layer_with_16bit_weights_follows_reference_scope3_golden():
+    """One-token sequences make attention return the token's own V row, so the layer's second half
+    can be checked against the reference's golden for it (o_proj + residual, RMSNorm, SwiGLU MLP,
+    residual; tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:255-287),
+    written out here step by step."""
+    import torch
+    from pypto_amd import workloads
+    batch, hidden, hq, hkv, d, inter = 4, 256, 4, 2, 128, 512
+    inp = workloads.decoder_layer_inputs(batch=batch, hidden=hidden, num_heads=hq, kv_head_num=hkv, head_dim=d,
+                                         intermediate=inter, block_size=16, context_lens=[1] * batch, seed=3,
+                                         int8_weights=False)
+    w = inp.weights
+    out, kc, vc = oracle.decoder_layer_decode(
+        inp.hidden, inp.seq_lens, inp.block_table, inp.key_cache, inp.value_cache, inp.rope_cos, inp.rope_sin,
+        inp.gamma_in, inp.gamma_post, *w["qkv"], *w["o"], *w["gate"], *w["up"], *w["down"],
+        num_heads=hq, kv_head_num=hkv, head_dim=d, block_size=16, max_num_blocks_per_req=inp.max_num_blocks_per_req)
+    normed = oracle.rms_norm(inp.hidden, inp.gamma_in, 1e-6, out_dtype=torch.bfloat16)
+    v = (normed.float() @ w["qkv"][0].float())[:, (hq + hkv) * d:].reshape(batch, hkv, d).to(torch.bfloat16)
+    attn_out = v.repeat_interleave(hq // hkv, dim=1).reshape(batch, hq * d)
+    resid1 = attn_out.float() @ w["o"][0].float() + inp.hidden.float()
+    inv_rms = torch.rsqrt(resid1.pow(2).mean(dim=-1, keepdim=True) + 1e-6)
+    normed2 = (resid1 * inv_rms * inp.gamma_post).bfloat16()
+    gate, up = normed2.float() @ w["gate"][0].float(), normed2.float() @ w["up"][0].float()
+    mlp = (gate * torch.sigmoid(gate) * up).bfloat16()
+    want = (mlp.float() @ w["down"][0].float() + resid1).bfloat16()
+    assert torch.allclose(out.float(), want.float(), rtol=1e-2, atol=1e-3)
+    # position 0: RoPE is the identity, the appended K row is the projection itself
+    k = (normed.float() @ w["qkv"][0].float())[:, hq * d:(hq + hkv) * d].reshape(batch, hkv, d).to(torch.bfloat16)
+    table = inp.block_table.reshape(batch, -1)
+    for b in range(batch):
+        for h in range(hkv):
+            row = (int(table[b, 0]) * hkv + h) * 16
+            assert torch.equal(kc[row], k[b, h]) and torch.equal(vc[row], v[b, h])
