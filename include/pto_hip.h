@@ -132,6 +132,8 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *      tensors: qkv, seq_lens, rope_cos, rope_sin, block_table, key_cache (INOUT), value_cache (INOUT),
  *               k_scale[pool,Hkv] fp32 (INOUT), v_scale (INOUT), q_out[B*Hq,D]
  *      scalars: num_heads, kv_head_num, head_dim, block_size
+ *  "projection"            examples/models/qwen3_jit/kernels/projection.py:35-57,118-177
+ *      tensors: x[M,K], w[K,N] (dtype of x), [residual[M,N],] out[M,N] (fp32 or dtype of x)
  *  "decoder_layer_decode"  examples/models/qwen3_jit/qwen3_decode.py:47-113
  *      tensors: hidden_states[B,H], seq_lens, block_table, key_cache (INOUT), value_cache (INOUT),
  *               rope_cos, rope_sin, gamma_in[H], gamma_post[H], wqkv_q, wqkv_s, wo_q, wo_s, wg_q, wg_s,
@@ -191,6 +193,14 @@ PTO_HIP_API int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void
                                    const void* w_up, const void* w_down, void* out,
                                    int64_t tokens, int64_t hidden, int64_t intermediate,
                                    float eps, int dtype, int out_dtype, void* stream);
+
+/* out[M, N] = x[M, K] @ w[K, N] (+ residual[M, N]), 16-bit x and w of the same type, fp32
+ * accumulation, out FP32 or that type: the reference's projection kernels
+ * (examples/models/qwen3_jit/kernels/projection.py:35-57; with the residual add :118-143, with the
+ * cast of the sum :146-177).  residual may be NULL; K and N multiples of 8.  Up to 32 rows stream the
+ * weights once (HBM-bound), more rows run as an MFMA-tiled GEMM. */
+PTO_HIP_API int pto_hip_projection(const void* x, const void* w, const void* residual, void* out, int64_t m,
+                                   int64_t k, int64_t n, int dtype, int res_dtype, int out_dtype, void* stream);
 
 /* W8A16 decode projection (no counterpart in the reference, which has no quantised weights; the
  * contract is its projection kernel's, examples/models/qwen3_jit/kernels/projection.py:145-177,

@@ -38,6 +38,15 @@ def rms_norm(x: torch.Tensor, gamma: torch.Tensor | None, eps: float = 1e-6,
     return y if out_dtype is None else y.to(out_dtype)
 
 
+def projection(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor | None = None) -> torch.Tensor:
+    """``x @ w`` (+ residual) with fp32 accumulation -> fp32: the K-chunked matmul / matmul_acc of the
+    reference's projections (examples/models/qwen3_jit/kernels/projection.py:35-57) and their
+    residual forms (:118-143, :146-177; golden test_qwen3_decode_scope3_mixed.py:271-272,285-287).
+    The caller casts the sum where the model does."""
+    y = torch.matmul(x.float(), w.float())
+    return y if residual is None else y + residual.float()
+
+
 def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """``gate * sigmoid(gate) * up`` (01_ffn.py:176; device form :70-75 is the same algebra)."""
     return gate * torch.sigmoid(gate) * up

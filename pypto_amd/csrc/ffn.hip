@@ -54,7 +54,15 @@ struct GemmParams {
   int tiles_m, tiles_n;
   int splits, k_per_split;  // split-K: each split writes its own fp32 slab, a second kernel sums them
   float* slabs;             // [splits][DUAL ? 2 : 1][m][n] when splits > 1
+  const void* residual;     // optional [m, n] added to the product (single-operand pass only)
+  int res_dtype;
 };
+
+__device__ __forceinline__ float load_residual(const void* r, int dt, int64_t i) {
+  if (dt == PTO_HIP_FP32) return reinterpret_cast<const float*>(r)[i];
+  if (dt == PTO_HIP_BF16) return (float)reinterpret_cast<const __bf16*>(r)[i];
+  return (float)reinterpret_cast<const _Float16*>(r)[i];
+}
 
 template <bool BF16>
 __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
@@ -298,8 +306,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
         for (int jn = 0; jn < NT; ++jn) {
           const int col = n0 + wn * (32 * NT) + jn * 32 + (lane & 31);
           if (col < p.n) {
-            if (p.splits > 1) p.slabs[(int64_t)split * mn + (int64_t)row * p.n + col] = acc[i][jn][r];
-            else store_out<OutT>(c + (int64_t)row * p.ldc + col, acc[i][jn][r]);
+            if (p.splits > 1) {
+              p.slabs[(int64_t)split * mn + (int64_t)row * p.n + col] = acc[i][jn][r];
+            } else {
+              float v = acc[i][jn][r];
+              if (p.residual) v += load_residual(p.residual, p.res_dtype, (int64_t)row * p.n + col);
+              store_out<OutT>(c + (int64_t)row * p.ldc + col, v);
+            }
           }
         }
       }
@@ -343,7 +356,7 @@ constexpr int kMaxSplits = 16;
 constexpr int kSplitBatch = 8;  // slabs loaded before the first add
 template <bool DUAL, typename OutT>
 __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* slabs, OutT* c, int64_t ldc, int m, int n,
-                                                          int splits) {
+                                                          int splits, const void* residual, int res_dtype) {
   const int nq = n / 4;
   const int64_t quads = (int64_t)m * nq, mn = (int64_t)m * n;
   constexpr int kMats = DUAL ? 2 : 1;
@@ -374,6 +387,13 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* slabs, Ou
     }
     float4 y = t[0];
     if constexpr (DUAL) y = float4{silu(t[0].x) * t[1].x, silu(t[0].y) * t[1].y, silu(t[0].z) * t[1].z, silu(t[0].w) * t[1].w};
+    if (!DUAL && residual) {
+      const int64_t r0 = row * n + col;
+      y.x += load_residual(residual, res_dtype, r0);
+      y.y += load_residual(residual, res_dtype, r0 + 1);
+      y.z += load_residual(residual, res_dtype, r0 + 2);
+      y.w += load_residual(residual, res_dtype, r0 + 3);
+    }
     OutT* dst = c + row * ldc + col;
     store_out<OutT>(dst + 0, y.x);
     store_out<OutT>(dst + 1, y.y);
@@ -387,7 +407,7 @@ int launch_finish(const GemmParams& p, hipStream_t st) {
   const int64_t quads = (int64_t)p.m * (p.n / 4);
   const unsigned blocks = (unsigned)std::min<int64_t>((quads + 255) / 256, 4096);
   hipLaunchKernelGGL((gemm_finish_kernel<DUAL, OutT>), dim3(blocks), dim3(256), 0, st, p.slabs,
-                     reinterpret_cast<OutT*>(p.c), p.ldc, p.m, p.n, p.splits);
+                     reinterpret_cast<OutT*>(p.c), p.ldc, p.m, p.n, p.splits, p.residual, p.res_dtype);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
 }
@@ -591,4 +611,51 @@ extern "C" int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void*
   p2.n = (int)hidden;
   p2.k = (int)intermediate;
   return launch_typed<false>(p2, dtype, out_dtype, st);
+}
+
+// out[M, N] = x[M, K] @ w[K, N] (+ residual[M, N]): the reference's projection kernels
+// (examples/models/qwen3_jit/kernels/projection.py:35-57 plain, :118-143 and :146-177 with the
+// residual add and the cast of the result).  Up to 32 rows stream the weights once through the
+// skinny projection kernels; more rows go through the tiled GEMM.
+extern "C" int pto_hip_projection(const void* x, const void* w, const void* residual, void* out, int64_t m,
+                                  int64_t k, int64_t n, int dtype, int res_dtype, int out_dtype, void* stream) {
+  using namespace pto_hip;
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(m >= 0 && k > 0 && n > 0 && m < (1 << 30) && k < (1 << 30) && n < (1 << 30),
+                "projection: bad shape M=%lld K=%lld N=%lld", (long long)m, (long long)k, (long long)n);
+  if (m == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(dtype == PTO_HIP_BF16 || dtype == PTO_HIP_FP16, "projection: dtype %s not in {BF16, FP16}",
+                dtype_name(dtype));
+  PTO_CHECK_ARG(out_dtype == PTO_HIP_FP32 || out_dtype == dtype,
+                "projection: output dtype %s must be FP32 or the input dtype %s", dtype_name(out_dtype),
+                dtype_name(dtype));
+  PTO_CHECK_ARG(x && w && out, "projection: null tensor pointer");
+  if (residual)
+    PTO_CHECK_ARG(res_dtype == PTO_HIP_FP32 || res_dtype == PTO_HIP_BF16 || res_dtype == PTO_HIP_FP16,
+                  "projection: residual dtype %s not in {FP32, BF16, FP16}", dtype_name(res_dtype));
+  PTO_CHECK_ARG(k % 8 == 0 && n % 8 == 0, "projection: K = %lld and N = %lld must be multiples of 8", (long long)k,
+                (long long)n);
+  PTO_CHECK_ARG(((uintptr_t)x | (uintptr_t)w | (uintptr_t)out | (uintptr_t)residual) % 16 == 0,
+                "projection: operand pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  if (m <= kSkinnyMaxTokens && ctx().gemm_variant == 0 && k % 16 == 0 && k >= 32) {
+    W8Partials parts{};
+    int rc = w8a16_partials(x, false, w, nullptr, m, k, n, dtype, st, &parts, true);
+    if (rc) return rc;
+    return w8a16_finish(parts, nullptr, nullptr, residual, res_dtype, out, out_dtype, false, m, n, st);
+  }
+  GemmParams p{};
+  p.a = reinterpret_cast<const uint16_t*>(x);
+  p.b0 = reinterpret_cast<const uint16_t*>(w);
+  p.b1 = nullptr;
+  p.c = out;
+  p.lda = k;
+  p.ldb = n;
+  p.ldc = n;
+  p.m = (int)m;
+  p.n = (int)n;
+  p.k = (int)k;
+  p.residual = residual;
+  p.res_dtype = res_dtype;
+  return launch_typed<false>(p, dtype, out_dtype, st);
 }

@@ -79,13 +79,14 @@ enum ProgramKind {
   kRopeKvCacheUpdate,
   kRopeKvCacheUpdateFp8,
   kDecoderLayerDecode,
+  kProjection,
   kNumPrograms
 };
 
 const char* const kProgramNames[kNumPrograms] = {
     "paged_attention", "paged_gather",  "rms_norm",           "ffn_swiglu",          "ffn_block",
     "w8a16_matmul",    "w8a16_swiglu",  "rope_kv_cache_update", "rope_kv_cache_update_fp8",
-    "decoder_layer_decode"};
+    "decoder_layer_decode", "projection"};
 
 std::mutex g_mu;
 std::vector<int> g_callables;  // callable id -> ProgramKind, -1 once unregistered
@@ -292,6 +293,30 @@ int run_w8a16_matmul(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns,
                               n, (int)x.dtype, res_dt, (int)out.dtype, stream);
 }
 
+int run_projection(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
+  PTO_CHECK_ARG((nt == 3 || nt == 4) && ns == 0,
+                "projection: expected x, w, [residual,] out and no scalars, got %d + %d", nt, ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor("projection", "operand", t[i], 1, 2);
+    if (rc) return rc;
+  }
+  const PtoHipChipTensor &x = t[0], &w = t[1], &out = t[nt - 1];
+  PTO_CHECK_ARG(x.ndims == 2 && w.ndims == 2 && out.ndims == 2, "projection: x, w and out must be 2-D");
+  const int64_t m = x.shapes[0], k = x.shapes[1], n = w.shapes[1];
+  PTO_CHECK_ARG(w.dtype == x.dtype && w.shapes[0] == k, "projection: w must be %s [K=%lld, N]", dtype_name(x.dtype),
+                (long long)k);
+  PTO_CHECK_ARG(out.shapes[0] == m && out.shapes[1] == n, "projection: out must be [M, N]");
+  const void* res = nullptr;
+  int res_dt = 0;
+  if (nt == 4) {
+    PTO_CHECK_ARG(numel(t[2]) == m * n, "projection: residual must be [M, N]");
+    res = tptr(t[2]);
+    res_dt = (int)t[2].dtype;
+  }
+  return pto_hip_projection(tptr(x), tptr(w), res, tptr_mut(out), m, k, n, (int)x.dtype, res_dt, (int)out.dtype,
+                            stream);
+}
+
 int run_w8a16_swiglu(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
   PTO_CHECK_ARG(nt == 6 && ns == 0, "w8a16_swiglu: expected x, wg_q, wg_scale, wu_q, wu_scale, out, got %d + %d", nt, ns);
   for (int i = 0; i < nt; ++i) {
@@ -486,6 +511,7 @@ int dispatch(int kind, const PtoHipChipTensor* t, int nt, const uint64_t* s, int
     case kFfnSwiglu: return run_ffn(t, nt, s, ns, stream, false);
     case kFfnBlock: return run_ffn(t, nt, s, ns, stream, true);
     case kW8a16Matmul: return run_w8a16_matmul(t, nt, s, ns, stream);
+    case kProjection: return run_projection(t, nt, s, ns, stream);
     case kW8a16Swiglu: return run_w8a16_swiglu(t, nt, s, ns, stream);
     case kRopeKvCacheUpdate: return run_rope_kv(t, nt, s, ns, stream);
     case kRopeKvCacheUpdateFp8: return run_rope_kv_fp8(t, nt, s, ns, stream);

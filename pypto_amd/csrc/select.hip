@@ -83,6 +83,8 @@ extern "C" int pto_hip_select_program(const char* orchestration_name, const PtoH
     else if (r.matmul >= 1 && r.swiglu == 1 && ffn == n_kernels &&
              dirs_are(orch_dirs, n_orch_tensors, {IN, IN, IN, IN, OUT}))
       found = "ffn_swiglu";       // examples/models/01_ffn.py:111-131
+    else if (r.matmul >= 1 && r.matmul == n_kernels && dirs_are(orch_dirs, n_orch_tensors, {IN, IN, OUT}))
+      found = "projection";       // examples/models/qwen3_jit/kernels/projection.py:35-57 (x @ W, W [in, out])
     else if (r.rms == 1 && n_kernels == 1 && dirs_are(orch_dirs, n_orch_tensors, {IN, IN, OUT}))
       found = "rms_norm";         // examples/intermediate/03_normalization.py:33-65
     else if (r.gather >= 1 && r.gather == n_kernels && dirs_are(orch_dirs, n_orch_tensors, {IN, IN, IN, OUT}))

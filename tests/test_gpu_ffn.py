@@ -137,3 +137,44 @@ def test_ffn_swiglu_decode_size_without_norm(worker):
         hd(inp.x, inp.w_gate, inp.w_up, inp.w_down, inp.out)
     ref = oracle.ffn_swiglu(inp.x, inp.w_gate, inp.w_up, inp.w_down, h_dtype=torch.bfloat16)
     validate_golden({"out": inp.out.float()}, {"out": ref.float()}, rtol=2e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,n", [(1, 512, 1024), (16, 1024, 2816), (32, 2816, 1024), (33, 1024, 1000),
+                                   (200, 2048, 512), (700, 512, 1536)])
+def test_projection_matches_oracle(worker, dtype, m, k, n):
+    """x @ W with W [in, out] in both regimes (weights streamed once up to 32 rows, tiled GEMM above,
+    with and without k split), plain fp32 result and residual + cast forms."""
+    from pypto_amd.runtime import projection, projection_residual
+    g = torch.Generator().manual_seed(m + k)
+    x = (torch.randn(m, k, generator=g) / k ** 0.5).to(dtype)
+    w = torch.randn(k, n, generator=g).to(dtype)
+    res = torch.randn(m, n, generator=g)
+    out = torch.zeros(m, n)
+    with worker.register(projection) as h:
+        h(x, w, out)
+    ref = oracle.projection(x, w)
+    validate_golden({"out": out}, {"out": ref}, rtol=2e-3, atol=2e-3)
+    out16 = torch.zeros(m, n, dtype=dtype)
+    with worker.register(projection_residual) as h:
+        h(x, w, res, out16)
+    want = oracle.projection(x, w, res).to(dtype)
+    validate_golden({"out": out16.float()}, {"out": want.float()}, rtol=1e-2, atol=1e-2)
+    res16 = res.to(dtype)
+    with worker.register(projection_residual) as h:
+        h(x, w, res16, out)
+    validate_golden({"out": out}, {"out": oracle.projection(x, w, res16)}, rtol=2e-3, atol=2e-3)
+
+
+def test_projection_argument_rules(worker):
+    from pypto_amd.runtime import projection
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="w must be BF16"):
+        with worker.register(projection) as h:
+            h(x, torch.zeros(64, 64, dtype=torch.float16), torch.zeros(4, 64))
+    with pytest.raises(ValueError, match="multiples of 8"):
+        with worker.register(projection) as h:
+            h(torch.zeros(4, 60, dtype=torch.bfloat16), torch.zeros(60, 64, dtype=torch.bfloat16), torch.zeros(4, 64))
+    with pytest.raises(ValueError, match="out must be"):
+        with worker.register(projection) as h:
+            h(x, torch.zeros(64, 64, dtype=torch.bfloat16), torch.zeros(4, 32))

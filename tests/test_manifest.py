@@ -72,6 +72,12 @@ def test_ffn_manifest(tmp_path):
     assert prog.name == "ffn_swiglu" and prog.signature == (IN, IN, IN, IN, OUT)
 
 
+def test_matmul_only_manifest_is_a_projection(tmp_path):
+    kernels = [("matmul_kernel", "aic", ["IN", "IN", "OUT"])]
+    prog, _, _ = mf.compile_and_assemble(_write(tmp_path, "matmul_orch", ["IN", "IN", "OUT"], kernels))
+    assert prog.name == "projection" and prog.signature == (IN, IN, OUT)
+
+
 def test_unknown_kernel_sets_are_rejected(tmp_path):
     # gelu FFN of the same example file: no fused program here
     kernels = [("matmul_kernel", "aic", None), ("gelu_kernel", "aiv", None)]
