@@ -45,7 +45,7 @@ def main() -> int:
     ap.add_argument("--no-ffn", action="store_true", help="skip the FFN measurement")
     ap.add_argument("--no-extra", action="store_true",
                     help="skip the other workloads of the path: long-context e4m3 attention, decoder layer, "
-                         "the layer with bf16 weights, FFN at 16 tokens, 64-head MQA attention")
+                         "the layer with bf16 weights, FFN at 16 tokens, vocabulary projection, 64-head MQA attention")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy, a known-size reference for HBM byte counters")
     args = ap.parse_args()
@@ -57,7 +57,7 @@ def main() -> int:
 
     from pypto_amd import workloads
     from pypto_amd.runtime import (ChipWorker, RunConfig, benchmark, decoder_layer_decode, decoder_layer_decode_w16,
-                                   ffn_block, paged_attention)
+                                   ffn_block, paged_attention, projection)
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -233,6 +233,29 @@ def main() -> int:
             "bound": "hbm",
         }
         del fd, fdargs
+        torch.cuda.empty_cache()
+        # vocabulary projection of a decode step: the largest single weight stream of the model
+        lm_m, lm_k, lm_n = 16, 5120, 151936
+        lx = (torch.randn(lm_m, lm_k, device="cuda") / lm_k ** 0.5).to(torch.bfloat16)
+        lw = torch.randn(lm_k, lm_n, device="cuda").to(torch.bfloat16)
+        lo = torch.zeros(lm_m, lm_n, device="cuda")
+        torch.cuda.synchronize()
+        with worker.register(projection) as ph:
+            benchmark(ph, [(lx, lw, lo)], rounds=5, warmup=0)
+            pstats = benchmark(ph, [(lx, lw, lo)], rounds=20, warmup=0)
+        pbytes = lm_k * lm_n * 2 + lm_m * lm_k * 2 + lm_m * lm_n * 4
+        result["projection_vocab"] = {
+            "workload": "projection x[16,5120] @ W[5120,151936] bf16 -> fp32 (qwen3-14B vocabulary projection at the "
+                        "reference's decode batch), weights streamed once",
+            "algorithmic_bytes_per_step": pbytes,
+            "us_per_step": round(pstats.device_wall_us, 1),
+            "achieved": round(pbytes / pstats.device_wall_us / 1e3, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(pbytes / pstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "bound": "hbm",
+        }
+        del lx, lw, lo
         torch.cuda.empty_cache()
         # 64 query heads on one KV head (the reference's q_tile 64 shape at a serving size)
         mq = workloads.paged_attention_inputs(batch=256, num_heads=64, kv_head_num=1, head_dim=128, block_size=128,
