@@ -310,7 +310,7 @@ PTO_HIP_API int pto_hip_select_program(const char* orchestration_name, const Pto
  *                               partition partials unmerged (kernel timing aid; output invalid)
  *  "attn_variant"               0 = one wavefront per (sequence, KV head, partition), 1 = one pinned
  *                               workgroup per CU and the chunk list cut evenly over their wavefronts,
- *                               -1 = by launch size (default)
+ *                               -1 = by launch size and table capacity (default)
  *  "attn_group_tiles"           cap on the 16-head query tiles one wavefront carries: 0 = the whole KV
  *                               group up to 64 heads (32 at head_dim 256), the cache read once per
  *                               group (default); 1, 2, 4 = at most that many, read once per wavefront

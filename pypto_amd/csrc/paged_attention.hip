@@ -729,15 +729,21 @@ __global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(A
   long long s = (w * total + wtot - 1) / wtot;
   const long long s_end = ((w + 1) * total + wtot - 1) / wtot;
 
-  while (s < s_end) {  // one iteration per (sequence, head, tile) the run touches
-    int b, chunks;
+  // The run's first item is found with a prefix scan over the sequences; after that the position
+  // advances without another scan: next (head, tile) of the sequence, then the next sequence
+  // that has tokens.
+  int b, chunks, hg, chunk;
+  {
     long long first_item;
     lean_locate(p, lane, hg_count, s, b, first_item, chunks);
-    if (b < 0) break;  // cannot happen for s < total; keeps the loop finite whatever the data
+    if (b < 0) return;  // cannot happen for s < total
     b = __builtin_amdgcn_readfirstlane(b);
     chunks = __builtin_amdgcn_readfirstlane(chunks);
     const long long local = s - first_item;
-    const int hg = (int)(local / chunks), chunk = (int)(local % chunks);
+    hg = (int)(local / chunks);
+    chunk = (int)(local % chunks);
+  }
+  while (s < s_end) {  // one iteration per (sequence, head, tile) the run touches
     const long long left = s_end - s;
     const int run = (int)(left < (long long)(chunks - chunk) ? left : (long long)(chunks - chunk));
     const int h = hg / p.gtiles, gt = hg % p.gtiles;
@@ -765,6 +771,20 @@ __global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(A
       }
     }
     s += run;
+    chunk += run;
+    if (chunk == chunks && s < s_end) {
+      chunk = 0;
+      if (++hg == hg_count) {
+        hg = 0;
+        // s < s_end <= total: a later sequence with tokens exists; the bound on b keeps the
+        // loop finite whatever the lengths say
+        do {
+          ++b;
+          chunks = b < p.batch ? __builtin_amdgcn_readfirstlane(seq_chunks(p, p.ctx_lens[b])) : 0;
+        } while (b < p.batch && chunks == 0);
+        if (b >= p.batch) return;
+      }
+    }
   }
 }
 
@@ -1008,7 +1028,10 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   // 2.8 GB of e4m3 cache with contexts of 8K-32K, +13 % on 2.7 GB at head_dim 256, within 3 % either
   // way when all contexts are equal, nothing on 150 MB).  "attn_variant" 0/1 forces the choice.
   const int64_t kv_bound = batch * hkv * p.gtiles * max_ctx * 2 * d * (fp8 ? 1 : 2);
-  const bool lean = cx.attn_variant >= 0 ? cx.attn_variant == 1 : kv_bound >= (1ll << 30);
+  // Many short sequences are the exception (512 sequences of 100-1000 tokens: 280 us against 239 us
+  // for the grid, whose single-partition workgroups write final rows and need no merge), so the
+  // table must also allow contexts of 4096 tokens.
+  const bool lean = cx.attn_variant >= 0 ? cx.attn_variant == 1 : (kv_bound >= (1ll << 30) && max_ctx >= 4096);
   if (p.n_part > 1 && !lean) {
     const size_t rows = (size_t)batch * hq;
     const size_t o_bytes = rows * p.n_part * d * sizeof(float);
