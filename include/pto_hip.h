@@ -164,7 +164,9 @@ PTO_HIP_API int pto_hip_benchmark(int callable_id, const PtoHipChipTensor* tenso
 /* ---- typed entry points (what pto_hip_run dispatches to) ------------------------------- */
 
 /* Paged-attention decode.  config is HOST memory; kv_dtype/q_dtype are PtoHipDataType;
- * k_scale/v_scale are NULL unless kv_dtype == PTO_HIP_FP8E4M3FN. */
+ * k_scale/v_scale are NULL unless kv_dtype == PTO_HIP_FP8E4M3FN.  This entry takes bare
+ * pointers: block_table entries are used as given (the size of the caches is not known here); the
+ * same program through pto_hip_run checks them against the cache tensors. */
 PTO_HIP_API int pto_hip_paged_attention(const void* query, const void* key_cache,
                                         const void* value_cache, const int32_t* block_table,
                                         const int32_t* context_lens, float* out,

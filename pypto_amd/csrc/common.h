@@ -116,11 +116,13 @@ int cast_from_f32(const float* in, void* out, size_t n, int out_dtype, hipStream
 // pto_hip_paged_attention with an optional second output: the result rounded to the query dtype.
 // want_blocked asks for the copy as [Hq*D/8][32][8] over the batch rows (batch <= 32);
 // *wrote_blocked says whether that is how it was written (only a launch with a merge kernel can).
+// pool_blocks > 0: the number of physical blocks in the caches; a table entry beyond it that a
+// sequence uses reads block 0 instead and is reported by the next pto_hip_sync.
 int paged_attention(const void* query, const void* key_cache, const void* value_cache,
                     const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
                     bool want_blocked, bool* wrote_blocked,
                     const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
-                    const float* v_scale, void* stream);
+                    const float* v_scale, int64_t pool_blocks, void* stream);
 
 inline int dtype_bytes(int dt) {
   switch (dt) {

@@ -129,7 +129,7 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
   bool blk_attn = false;  // the 16-bit copy is blocked only when the merge kernel wrote it
   if ((rc = paged_attention(q16, a->key_cache, a->value_cache, a->block_table, a->seq_lens, attn, attn16, blk,
                             &blk_attn, cfg, dt, fp8kv ? PTO_HIP_FP8E4M3FN : dt, fp8kv ? a->k_scale : nullptr,
-                            fp8kv ? a->v_scale : nullptr, stream)))
+                            fp8kv ? a->v_scale : nullptr, a->pool_rows / (hkv * a->block_size), stream)))
     return rc;
   // 5. o_proj; 6. its finish + residual -> fp32, post-attention RMSNorm -> activation dtype
   if ((rc = w8a16_partials(attn16, blk_attn, a->wo_q, nullptr, b, hq * d, h, dt, st, &parts, w16))) return rc;

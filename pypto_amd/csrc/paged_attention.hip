@@ -47,6 +47,8 @@ struct AttnParams {
   const float* k_scale;  // [pool_blocks, Hkv] for an e4m3 cache, else null
   const float* v_scale;
   int batch, hq, hkv, group, gtiles, bs, max_blocks, tpp, n_part;
+  int pool_blocks; // physical blocks in the cache when the caller knows it, else 0 (table entries unchecked)
+  int* error_flag; // set when a table entry a sequence uses addresses a block outside the cache
   int gt_rows;     // query rows one wavefront covers: 16 x its tile count; gtiles = ceil(group / gt_rows)
   int n_wg;        // evenly split form: resident workgroups (one per CU); 0 = partition grid
   int lean_waves;  // ... and wavefronts in each
@@ -359,10 +361,17 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
   // per-chunk look-ups below are register reads, not memory round trips on the load path.
   int win_base = 0, win_blk = 0;
   float win_ks = 1.f, win_vs = 1.f;
+  bool bad_entry = false;
   auto load_window = [&](int first_block, bool preloaded) {
     win_base = first_block;
     const int idx = min(first_block + lane, p.max_blocks - 1);
     win_blk = preloaded ? first_window : table[idx];
+    if (p.pool_blocks > 0 && (unsigned)win_blk >= (unsigned)p.pool_blocks) {
+      // A block outside the cache: read block 0 instead of faulting, and report it if the
+      // sequence really uses this entry (entries past its end may hold anything).
+      bad_entry |= (first_block + lane) * p.bs < tok_end;
+      win_blk = 0;
+    }
     if constexpr (FP8) {
       // table entries past the end of the range may hold anything: do not dereference them
       const bool ok = (first_block + lane) * p.bs < tok_end;
@@ -454,6 +463,7 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
     }
   }
 
+  if (bad_entry) *p.error_flag = 1;
   // Row sum over the four k-groups of a column.
 #pragma unroll
   for (int t = 0; t < GT; ++t) {
@@ -933,7 +943,7 @@ namespace pto_hip {
 int paged_attention(const void* query, const void* key_cache, const void* value_cache,
                     const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
                     bool want_blocked, bool* wrote_blocked, const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
-                    const float* v_scale, void* stream) {
+                    const float* v_scale, int64_t pool_blocks, void* stream) {
   Context& cx = ctx();
   if (!cx.initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(config != nullptr, "paged_attention: config is null");
@@ -983,6 +993,8 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   if (wrote_blocked) *wrote_blocked = false;
   p.k_scale = k_scale;
   p.v_scale = v_scale;
+  p.pool_blocks = pool_blocks > 0 && pool_blocks < (1ll << 31) ? (int)pool_blocks : 0;
+  p.error_flag = cx.flags + 2;
   p.batch = (int)batch;
   p.hq = (int)hq;
   p.hkv = (int)hkv;
@@ -1090,6 +1102,7 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
                                        const int32_t* context_lens, float* out,
                                        const int64_t* config, int q_dtype, int kv_dtype,
                                        const float* k_scale, const float* v_scale, void* stream) {
+  // The size of the caches is not part of this signature: table entries are used as given.
   return pto_hip::paged_attention(query, key_cache, value_cache, block_table, context_lens, out, nullptr, false, nullptr, config,
-                                  q_dtype, kv_dtype, k_scale, v_scale, stream);
+                                  q_dtype, kv_dtype, k_scale, v_scale, 0, stream);
 }

@@ -187,11 +187,11 @@ int run_paged_attention(const PtoHipChipTensor* t, int nt, const uint64_t*, int 
     ks = reinterpret_cast<const float*>(tptr(t[7]));
     vs = reinterpret_cast<const float*>(tptr(t[8]));
   }
-  return pto_hip_paged_attention(tptr(t[0]), tptr(t[1]), tptr(t[2]),
-                                 reinterpret_cast<const int32_t*>(tptr(t[3])),
-                                 reinterpret_cast<const int32_t*>(tptr(t[4])),
-                                 reinterpret_cast<float*>(tptr_mut(t[5])), cfg, (int)t[0].dtype,
-                                 (int)t[1].dtype, ks, vs, stream);
+  // The tensor view says how many blocks the caches hold: table entries beyond that are caught.
+  return paged_attention(tptr(t[0]), tptr(t[1]), tptr(t[2]), reinterpret_cast<const int32_t*>(tptr(t[3])),
+                         reinterpret_cast<const int32_t*>(tptr(t[4])), reinterpret_cast<float*>(tptr_mut(t[5])),
+                         nullptr, false, nullptr, cfg, (int)t[0].dtype, (int)t[1].dtype, ks, vs,
+                         numel(t[1]) / (hkv * bs * d), stream);
 }
 
 int run_paged_gather(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns,
@@ -641,15 +641,18 @@ int pto_hip_sync(void* stream) {
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
   // Device-side argument errors of launches that do not block are reported here.
-  int flags[2] = {0, 0};
+  int flags[3] = {0, 0, 0};
   PTO_CHECK_HIP(hipMemcpy(flags, ctx().flags, sizeof(flags), hipMemcpyDeviceToHost));
-  if (flags[0] || flags[1]) {
+  if (flags[0] || flags[1] || flags[2]) {
     PTO_CHECK_HIP(hipMemset(ctx().flags, 0, sizeof(flags)));
     if (flags[0])
       return fail(PTO_HIP_ERR_INVALID_VALUE,
                   "paged_gather: an index addresses a block outside block_table or a row outside src");
+    if (flags[1])
+      return fail(PTO_HIP_ERR_INVALID_VALUE,
+                  "rope_kv_cache_update: a decode position lies outside the rope table, the block table or the cache");
     return fail(PTO_HIP_ERR_INVALID_VALUE,
-                "rope_kv_cache_update: a decode position lies outside the rope table, the block table or the cache");
+                "paged_attention: a block_table entry a sequence uses addresses a block outside the cache");
   }
   return PTO_HIP_OK;
 }

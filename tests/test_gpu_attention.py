@@ -320,3 +320,31 @@ def test_many_sequences_with_gaps(worker):
         _check(out, ref)
         empty = (ctxs == 0).repeat_interleave(8)
         assert (out[empty] == 0).all()
+
+
+def test_block_table_entry_outside_the_cache_is_caught(worker):
+    """Through the tensor interface the size of the caches is known: an entry beyond it that a
+    sequence uses is replaced by block 0 (no wild read) and reported by the next sync; entries
+    past a sequence's length may hold anything."""
+    inp = workloads.paged_attention_inputs(batch=3, num_heads=16, kv_head_num=4, block_size=64,
+                                           context_lens=[300, 64, 1000], ctx_range=(1, 1024), seed=23)
+    max_blocks = inp.block_table.numel() // 3
+    table = inp.block_table.clone().reshape(3, max_blocks)
+    table[1, 1:] = 2 ** 30                      # sequence 1 uses only its first block
+    table[0, 5:] = -7                           # sequence 0 uses blocks 0..4
+    args = list(inp.args())
+    args[3] = table.flatten().contiguous()
+    for tpp in (0, 128, -4):
+        out = _run(worker, dataclass_replace(inp, args[3]), tpp)
+        _check(out, _golden(inp))               # unused entries changed nothing
+    table[2, 3] = 2 ** 30                       # sequence 2 does use logical block 3
+    bad = dataclass_replace(inp, table.flatten().contiguous())
+    for tpp in (128, -4):
+        with pytest.raises(ValueError, match="outside the cache"):
+            _run(worker, bad, tpp)
+        worker.sync()                           # the report clears the flag
+
+
+def dataclass_replace(inp, table):
+    import dataclasses
+    return dataclasses.replace(inp, block_table=table)
