@@ -113,7 +113,8 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *      tensors: src[rows,hidden], indices[n] i32, block_table[nblk] i32, out[n,size]
  *      scalars: block_size, col_offset
  *  "rms_norm"          examples/intermediate/03_normalization.py:33-65
- *      tensors: x[T,H], gamma[1,H] fp32, out[T,H] (dtype of x or fp32);  scalars: eps (f32 bits)
+ *      tensors: x[T,H], [gamma[1,H] fp32,] out[T,H] (dtype of x or fp32);  scalars: eps (f32 bits)
+ *               (without gamma: the unweighted form of examples/models/08_llama_mini.py:93-118)
  *  "ffn_swiglu"        examples/models/01_ffn.py:111-131
  *      tensors: hidden_states[T,H], gate_proj_weight[H,I], up_proj_weight[H,I],
  *               down_proj_weight[I,H], output[T,H] (fp32 or dtype of x)

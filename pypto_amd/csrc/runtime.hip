@@ -219,19 +219,25 @@ int run_paged_gather(const PtoHipChipTensor* t, int nt, const uint64_t* s, int n
 }
 
 int run_rms_norm(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream) {
-  PTO_CHECK_ARG(nt == 3 && ns == 1, "rms_norm: expected 3 tensors + 1 scalar (eps), got %d + %d", nt, ns);
-  static const char* names[3] = {"x", "gamma", "out"};
-  for (int i = 0; i < 3; ++i) {
-    int rc = check_tensor("rms_norm", names[i], t[i], 1, 2);
+  // x, gamma, out - or x, out for the form without a weight (examples/models/08_llama_mini.py:93-118)
+  PTO_CHECK_ARG((nt == 3 || nt == 2) && ns == 1,
+                "rms_norm: expected x, [gamma,] out + 1 scalar (eps), got %d + %d", nt, ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor("rms_norm", i == 0 ? "x" : i == nt - 1 ? "out" : "gamma", t[i], 1, 2);
     if (rc) return rc;
   }
   PTO_CHECK_ARG(t[0].ndims == 2, "rms_norm: x must be 2-D");
   const int64_t rows = t[0].shapes[0], hidden = t[0].shapes[1];
-  PTO_CHECK_ARG(t[1].dtype == PTO_HIP_FP32 && numel(t[1]) == hidden,
-                "rms_norm: gamma must be FP32 with %lld elements", (long long)hidden);
-  PTO_CHECK_ARG(numel(t[2]) == rows * hidden, "rms_norm: out shape differs from x");
-  return pto_hip_rms_norm(tptr(t[0]), reinterpret_cast<const float*>(tptr(t[1])), tptr_mut(t[2]),
-                          rows, hidden, scalar_f32(s[0]), (int)t[0].dtype, (int)t[2].dtype, stream);
+  const float* gamma = nullptr;
+  if (nt == 3) {
+    PTO_CHECK_ARG(t[1].dtype == PTO_HIP_FP32 && numel(t[1]) == hidden,
+                  "rms_norm: gamma must be FP32 with %lld elements", (long long)hidden);
+    gamma = reinterpret_cast<const float*>(tptr(t[1]));
+  }
+  const PtoHipChipTensor& out = t[nt - 1];
+  PTO_CHECK_ARG(numel(out) == rows * hidden, "rms_norm: out shape differs from x");
+  return pto_hip_rms_norm(tptr(t[0]), gamma, tptr_mut(out), rows, hidden, scalar_f32(s[0]), (int)t[0].dtype,
+                          (int)out.dtype, stream);
 }
 
 int run_ffn(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream,

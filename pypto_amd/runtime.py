@@ -66,6 +66,7 @@ class HipProgram:
 paged_attention = HipProgram("paged_attention", (IN, IN, IN, IN, IN, OUT, HOST, IN, IN), optional=2)
 paged_gather = HipProgram("paged_gather", (IN, IN, IN, OUT), scalars=("block_size", "col_offset"))
 rms_norm = HipProgram("rms_norm", (IN, IN, OUT), scalars=("eps",))
+rms_norm_unweighted = HipProgram("rms_norm", (IN, OUT), scalars=("eps",))  # 08_llama_mini.py:93-118
 ffn_swiglu = HipProgram("ffn_swiglu", (IN, IN, IN, IN, OUT))
 ffn_block = HipProgram("ffn_block", (IN, IN, IN, IN, IN, OUT), scalars=("eps",))
 

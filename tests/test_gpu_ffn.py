@@ -25,6 +25,22 @@ def test_rms_norm(worker, dtype, rows, hidden):
     validate_golden({"out": out.float()}, {"out": ref.float()}, rtol=tol, atol=tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rms_norm_without_weight(worker, dtype):
+    """The unweighted form: x / sqrt(mean(x^2) + eps) (examples/models/08_llama_mini.py:93-118)."""
+    from pypto_amd.runtime import rms_norm_unweighted
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn((7, 1024), generator=g).to(dtype)
+    out = torch.zeros_like(x)
+    with worker.register(rms_norm_unweighted) as h:
+        h(x, out, 1e-6)
+    want = (x.float() / torch.sqrt(x.float().pow(2).mean(dim=-1, keepdim=True) + 1e-6)).to(dtype)
+    tol = {torch.float32: 2e-6, torch.bfloat16: 8e-3}[dtype]
+    validate_golden({"out": out.float()}, {"out": want.float()}, rtol=tol, atol=tol)
+    assert torch.equal(oracle.rms_norm(x, None, 1e-6, out_dtype=dtype), want) or torch.allclose(
+        oracle.rms_norm(x, None, 1e-6, out_dtype=dtype).float(), want.float(), rtol=tol, atol=tol)
+
+
 def test_ffn_reference_example_fp32(worker):
     """The reference's own case: 64x64 fp32, seed 0, rtol=atol=3e-3 (examples/models/01_ffn.py:155-179)."""
     torch.manual_seed(0)
