@@ -126,7 +126,7 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *  "w8a16_swiglu"      examples/models/qwen3_jit/kernels/mlp.py:22-61 with int8 weights
  *      tensors: x[M,K], wg_q[K,N] i8, wg_scale[N], wu_q[K,N] i8, wu_scale[N], out[M,N]
  *  "rope_kv_cache_update"  examples/models/qwen3_jit/kernels/attention.py:39-102
- *      tensors: qkv[B,(Hq+2Hkv)*D] fp32, seq_lens[B] i32, rope_cos[max_pos,D/2], rope_sin,
+ *      tensors: qkv[B,(Hq+2Hkv)*D] fp32, seq_lens[B] i32, rope_cos[max_pos,D/2] or [max_pos,D], rope_sin,
  *               block_table[B*max_blocks] i32, key_cache (INOUT), value_cache (INOUT), q_out[B*Hq,D]
  *      scalars: num_heads, kv_head_num, head_dim, block_size
  *  "rope_kv_cache_update_fp8"  the same with FP8E4M3FN caches, quantised on write
@@ -222,7 +222,8 @@ PTO_HIP_API int pto_hip_w8a16_swiglu(const void* x, const void* wg_q, const floa
 
 /* RoPE at pos = seq_len - 1, K/V rows appended to the paged cache, rotated Q cast to `dtype`
  * (examples/models/qwen3_jit/kernels/attention.py:39-102).  qkv is FP32 [B, (Hq+2Hkv)*D] laid out
- * q heads, then k heads, then v heads; rope_cos/rope_sin are FP32 [max_pos, D/2].  A position
+ * q heads, then k heads, then v heads; rope_cos/rope_sin are FP32 [max_pos, D/2] here (through
+ * pto_hip_run a [max_pos, D] table, the reference's form, is recognised by its shape).  A position
  * outside the tables is skipped and reported by the next pto_hip_sync. */
 PTO_HIP_API int pto_hip_rope_kv_cache_update(const float* qkv, const int32_t* seq_lens,
                                              const float* rope_cos, const float* rope_sin,
@@ -258,7 +259,7 @@ typedef struct PtoHipDecoderLayerArgs {
   const int32_t* block_table; /* [B, max_num_blocks_per_req] */
   void* key_cache;            /* [pool_rows, D] dtype, updated in place */
   void* value_cache;
-  const float* rope_cos;      /* [max_pos, D/2] */
+  const float* rope_cos;      /* [max_pos, D/2], or [max_pos, D] with rope_table_width = D */
   const float* rope_sin;
   const float* gamma_in;      /* [H] */
   const float* gamma_post;    /* [H] */
@@ -278,7 +279,8 @@ typedef struct PtoHipDecoderLayerArgs {
   float eps;
   int32_t dtype;              /* PTO_HIP_BF16 or PTO_HIP_FP16 */
   int32_t kv_dtype;           /* 0 = caches hold `dtype`; PTO_HIP_FP8E4M3FN = e4m3 caches, quantised on write */
-  int32_t reserved;
+  int32_t rope_table_width;   /* columns of rope_cos / rope_sin: 0 or D/2 = one angle per pair; D = the reference's
+                                 [max_pos, D] tables (low-half and high-half factors side by side) */
   float* k_scale;             /* [pool_blocks, Hkv] FP32, updated in place (e4m3 caches only) */
   float* v_scale;
 } PtoHipDecoderLayerArgs;

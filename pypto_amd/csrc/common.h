@@ -96,18 +96,19 @@ int w8a16_finish_norm(const W8Partials& parts, const float* scale, const void* r
 
 // RoPE + K/V append reading either final fp32 projections (qkv_scale null, splits 1) or the
 // partial sums of the q/k/v projection (summed in split order and scaled per channel).
+// rope_width: columns of the cos/sin tables, head_dim / 2 or head_dim.
 int rope_kv_cache_update(const float* qkv, const float* qkv_scale, int splits, int64_t split_stride,
                          const int32_t* seq_lens, const float* rope_cos, const float* rope_sin,
                          const int32_t* block_table, void* key_cache, void* value_cache, void* q_out,
                          int64_t batch, int64_t num_heads, int64_t kv_head_num, int64_t head_dim,
-                         int64_t block_size, int64_t max_num_blocks_per_req, int64_t max_pos,
+                         int64_t block_size, int64_t max_num_blocks_per_req, int64_t max_pos, int rope_width,
                          int64_t pool_rows, int dtype, void* stream);
 int rope_kv_cache_update_fp8(const float* qkv, const float* qkv_scale, int splits, int64_t split_stride,
                              const int32_t* seq_lens, const float* rope_cos, const float* rope_sin,
                              const int32_t* block_table, void* key_cache, void* value_cache, float* k_scale,
                              float* v_scale, void* q_out, int64_t batch, int64_t num_heads, int64_t kv_head_num,
                              int64_t head_dim, int64_t block_size, int64_t max_num_blocks_per_req,
-                             int64_t max_pos, int64_t pool_blocks, int q_dtype, void* stream);
+                             int64_t max_pos, int rope_width, int64_t pool_blocks, int q_dtype, void* stream);
 // RMSNorm of at most 32 rows written in the blocked activation layout [H/8][32][8].
 bool rms_norm_blocked_fits(int64_t rows, int64_t hidden);
 int rms_norm_blocked(const void* x, const float* gamma, void* out, int64_t rows, int64_t hidden, float eps,

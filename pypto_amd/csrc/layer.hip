@@ -55,6 +55,9 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
                 (long long)h, (long long)inter);
   PTO_CHECK_ARG(a->block_size > 0 && a->block_size % 16 == 0 && a->max_num_blocks_per_req > 0 && a->max_pos > 0,
                 "decoder_layer_decode: block_size must be a positive multiple of 16, the table and RoPE tables non-empty");
+  const int rope_w = a->rope_table_width ? a->rope_table_width : (int)(d / 2);
+  PTO_CHECK_ARG(rope_w == d / 2 || rope_w == d, "decoder_layer_decode: rope_table_width %d must be 0, %lld or %lld",
+                a->rope_table_width, (long long)d / 2, (long long)d);
   const bool fp8kv = a->kv_dtype == PTO_HIP_FP8E4M3FN;
   PTO_CHECK_ARG(a->kv_dtype == 0 || a->kv_dtype == a->dtype || fp8kv,
                 "decoder_layer_decode: cache dtype %s must be the activation dtype or FP8E4M3FN",
@@ -114,11 +117,12 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
     rc = rope_kv_cache_update_fp8(parts.part[0], a->wqkv_s, parts.splits, (int64_t)kW8MaxM * qkv_n, a->seq_lens,
                                   a->rope_cos, a->rope_sin, a->block_table, a->key_cache, a->value_cache, a->k_scale,
                                   a->v_scale, q16, b, hq, hkv, d, a->block_size, a->max_num_blocks_per_req,
-                                  a->max_pos, pool_blocks, dt, stream);
+                                  a->max_pos, rope_w, pool_blocks, dt, stream);
   } else {
     rc = rope_kv_cache_update(parts.part[0], a->wqkv_s, parts.splits, (int64_t)kW8MaxM * qkv_n, a->seq_lens,
                               a->rope_cos, a->rope_sin, a->block_table, a->key_cache, a->value_cache, q16, b, hq,
-                              hkv, d, a->block_size, a->max_num_blocks_per_req, a->max_pos, a->pool_rows, dt, stream);
+                              hkv, d, a->block_size, a->max_num_blocks_per_req, a->max_pos, rope_w, a->pool_rows, dt,
+                              stream);
   }
   if (rc) return rc;
   // 4. paged attention over seq_len tokens (including the one just written)

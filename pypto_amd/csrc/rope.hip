@@ -18,8 +18,9 @@ struct RopeParams {
   int splits;              // partial slabs to sum (1 when qkv is final)
   int64_t split_stride;    // elements between consecutive partial slabs
   const int32_t* seq_lens; // [B]
-  const float* cos;        // [max_pos, D/2]
-  const float* sin;
+  const float* cos;        // [max_pos, rope_w]: rope_w = D/2 (one angle per pair) or D (the
+  const float* sin;        // reference's tables: columns 0..D/2 rotate the low half, the rest the high half)
+  int rope_w;
   const int32_t* block_table;  // [B, max_blocks]
   void* key_cache;
   void* value_cache;
@@ -73,9 +74,9 @@ __global__ __launch_bounds__(128) void rope_kv_kernel(RopeParams p) {
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     const float lo = fetch(i), hi = fetch(i + half);
     if (is_q || is_k) {
-      const float c = p.cos[(size_t)cpos * half + i], s = p.sin[(size_t)cpos * half + i];
-      dst[i] = (T)(lo * c - hi * s);
-      dst[i + half] = (T)(hi * c + lo * s);
+      const size_t t_lo = (size_t)cpos * p.rope_w + i, t_hi = p.rope_w == p.d ? t_lo + half : t_lo;
+      dst[i] = (T)(lo * p.cos[t_lo] - hi * p.sin[t_lo]);
+      dst[i + half] = (T)(hi * p.cos[t_hi] + lo * p.sin[t_hi]);
     } else {
       dst[i] = (T)lo;
       dst[i + half] = (T)hi;
@@ -145,9 +146,9 @@ __global__ __launch_bounds__(64) void rope_kv_fp8_kernel(RopeFp8Params pp) {
     TQ* dst = reinterpret_cast<TQ*>(p.q_out) + ((size_t)b * p.hq + head) * p.d;
     for (int i = lane; i < half; i += 64) {
       const float lo = fetch(i), hi = fetch(i + half);
-      const float c = p.cos[(size_t)cpos * half + i], s = p.sin[(size_t)cpos * half + i];
-      dst[i] = (TQ)(lo * c - hi * s);
-      dst[i + half] = (TQ)(hi * c + lo * s);
+      const size_t t_lo = (size_t)cpos * p.rope_w + i, t_hi = p.rope_w == p.d ? t_lo + half : t_lo;
+      dst[i] = (TQ)(lo * p.cos[t_lo] - hi * p.sin[t_lo]);
+      dst[i + half] = (TQ)(hi * p.cos[t_hi] + lo * p.sin[t_hi]);
     }
     return;
   }
@@ -182,8 +183,8 @@ __global__ __launch_bounds__(64) void rope_kv_fp8_kernel(RopeFp8Params pp) {
         if (is_k) {
           const int i = e < half ? e : e - half;
           const float lo = fetch(i), hi = fetch(i + half);
-          const float c = p.cos[(size_t)cpos * half + i], s = p.sin[(size_t)cpos * half + i];
-          v = e < half ? lo * c - hi * s : hi * c + lo * s;
+          const size_t t_lo = (size_t)cpos * p.rope_w + i, t_hi = p.rope_w == p.d ? t_lo + half : t_lo;
+          v = e < half ? lo * p.cos[t_lo] - hi * p.sin[t_lo] : hi * p.cos[t_hi] + lo * p.sin[t_hi];
         } else {
           v = fetch(e);
         }
@@ -250,7 +251,7 @@ int rope_kv_cache_update(const float* qkv, const float* qkv_scale, int splits, i
                          const int32_t* seq_lens, const float* rope_cos, const float* rope_sin,
                          const int32_t* block_table, void* key_cache, void* value_cache, void* q_out,
                          int64_t batch, int64_t num_heads, int64_t kv_head_num, int64_t head_dim,
-                         int64_t block_size, int64_t max_num_blocks_per_req, int64_t max_pos,
+                         int64_t block_size, int64_t max_num_blocks_per_req, int64_t max_pos, int rope_width,
                          int64_t pool_rows, int dtype, void* stream) {
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(batch >= 0 && batch < 65536, "rope_kv_cache_update: batch %lld out of range", (long long)batch);
@@ -273,6 +274,10 @@ int rope_kv_cache_update(const float* qkv, const float* qkv_scale, int splits, i
   p.seq_lens = seq_lens;
   p.cos = rope_cos;
   p.sin = rope_sin;
+  PTO_CHECK_ARG(rope_width == head_dim / 2 || rope_width == head_dim,
+                "rope_kv_cache_update: rope tables must be [max_pos, %lld] or [max_pos, %lld], got width %d",
+                (long long)head_dim / 2, (long long)head_dim, rope_width);
+  p.rope_w = rope_width;
   p.block_table = block_table;
   p.key_cache = key_cache;
   p.value_cache = value_cache;
@@ -301,7 +306,7 @@ int rope_kv_cache_update_fp8(const float* qkv, const float* qkv_scale, int split
                              const int32_t* block_table, void* key_cache, void* value_cache, float* k_scale,
                              float* v_scale, void* q_out, int64_t batch, int64_t num_heads, int64_t kv_head_num,
                              int64_t head_dim, int64_t block_size, int64_t max_num_blocks_per_req,
-                             int64_t max_pos, int64_t pool_blocks, int q_dtype, void* stream) {
+                             int64_t max_pos, int rope_width, int64_t pool_blocks, int q_dtype, void* stream) {
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(batch >= 0 && batch < 65536, "rope_kv_cache_update_fp8: batch %lld out of range", (long long)batch);
   if (batch == 0) return PTO_HIP_OK;
@@ -327,6 +332,10 @@ int rope_kv_cache_update_fp8(const float* qkv, const float* qkv_scale, int split
   p.seq_lens = seq_lens;
   p.cos = rope_cos;
   p.sin = rope_sin;
+  PTO_CHECK_ARG(rope_width == head_dim / 2 || rope_width == head_dim,
+                "rope_kv_cache_update: rope tables must be [max_pos, %lld] or [max_pos, %lld], got width %d",
+                (long long)head_dim / 2, (long long)head_dim, rope_width);
+  p.rope_w = rope_width;
   p.block_table = block_table;
   p.key_cache = key_cache;
   p.value_cache = value_cache;
@@ -361,8 +370,8 @@ extern "C" int pto_hip_rope_kv_cache_update_fp8(const float* qkv, const int32_t*
                                                 int64_t pool_blocks, int q_dtype, void* stream) {
   return pto_hip::rope_kv_cache_update_fp8(qkv, nullptr, 1, 0, seq_lens, rope_cos, rope_sin, block_table, key_cache,
                                            value_cache, k_scale, v_scale, q_out, batch, num_heads, kv_head_num,
-                                           head_dim, block_size, max_num_blocks_per_req, max_pos, pool_blocks,
-                                           q_dtype, stream);
+                                           head_dim, block_size, max_num_blocks_per_req, max_pos, (int)(head_dim / 2),
+                                           pool_blocks, q_dtype, stream);
 }
 
 extern "C" int pto_hip_rope_kv_cache_update(const float* qkv, const int32_t* seq_lens, const float* rope_cos,
@@ -373,5 +382,5 @@ extern "C" int pto_hip_rope_kv_cache_update(const float* qkv, const int32_t* seq
                                             int64_t max_pos, int64_t pool_rows, int dtype, void* stream) {
   return pto_hip::rope_kv_cache_update(qkv, nullptr, 1, 0, seq_lens, rope_cos, rope_sin, block_table, key_cache,
                                        value_cache, q_out, batch, num_heads, kv_head_num, head_dim, block_size,
-                                       max_num_blocks_per_req, max_pos, pool_rows, dtype, stream);
+                                       max_num_blocks_per_req, max_pos, (int)(head_dim / 2), pool_rows, dtype, stream);
 }

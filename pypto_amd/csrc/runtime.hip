@@ -343,6 +343,12 @@ int run_w8a16_swiglu(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns,
                               (int)t[5].dtype, stream);
 }
 
+// Columns of a cos/sin table: [max_pos, D] (the reference's tables, low-half and high-half
+// factors side by side) when the tensor says so, else D/2 (one angle per rotated pair).
+inline int rope_table_width(const PtoHipChipTensor& table, int64_t d) {
+  return table.ndims == 2 && table.shapes[1] == (uint32_t)d ? (int)d : (int)(d / 2);
+}
+
 int run_rope_kv_fp8(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream) {
   PTO_CHECK_ARG(nt == 10 && ns == 4,
                 "rope_kv_cache_update_fp8: expected qkv, seq_lens, rope_cos, rope_sin, block_table, key_cache, "
@@ -361,7 +367,8 @@ int run_rope_kv_fp8(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns
                 "rope_kv_cache_update_fp8: seq_lens and block_table must be INT32");
   PTO_CHECK_ARG(t[2].dtype == PTO_HIP_FP32 && t[3].dtype == PTO_HIP_FP32 && numel(t[2]) == numel(t[3]) &&
                     d % 2 == 0 && numel(t[2]) % (d / 2) == 0,
-                "rope_kv_cache_update_fp8: rope_cos/rope_sin must be FP32 [max_pos, D/2]");
+                "rope_kv_cache_update_fp8: rope_cos/rope_sin must be FP32 [max_pos, D/2] or [max_pos, D]");
+  const int rope_w = rope_table_width(t[2], d);
   PTO_CHECK_ARG(batch > 0 ? numel(t[4]) % batch == 0 : true,
                 "rope_kv_cache_update_fp8: block_table must be [B, max_blocks]");
   PTO_CHECK_ARG(t[5].dtype == PTO_HIP_FP8E4M3FN && t[6].dtype == PTO_HIP_FP8E4M3FN && numel(t[5]) == numel(t[6]) &&
@@ -373,12 +380,12 @@ int run_rope_kv_fp8(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns
                 "rope_kv_cache_update_fp8: k_scale/v_scale must be FP32 [pool_blocks, Hkv]");
   PTO_CHECK_ARG((t[9].dtype == PTO_HIP_BF16 || t[9].dtype == PTO_HIP_FP16) && numel(t[9]) == batch * hq * d,
                 "rope_kv_cache_update_fp8: q_out must be BF16 or FP16 [B*Hq, D]");
-  return pto_hip_rope_kv_cache_update_fp8(
-      reinterpret_cast<const float*>(tptr(t[0])), reinterpret_cast<const int32_t*>(tptr(t[1])),
+  return rope_kv_cache_update_fp8(
+      reinterpret_cast<const float*>(tptr(t[0])), nullptr, 1, 0, reinterpret_cast<const int32_t*>(tptr(t[1])),
       reinterpret_cast<const float*>(tptr(t[2])), reinterpret_cast<const float*>(tptr(t[3])),
       reinterpret_cast<const int32_t*>(tptr(t[4])), tptr_mut(t[5]), tptr_mut(t[6]),
       reinterpret_cast<float*>(tptr_mut(t[7])), reinterpret_cast<float*>(tptr_mut(t[8])), tptr_mut(t[9]), batch, hq,
-      hkv, d, bs, batch ? numel(t[4]) / batch : 1, numel(t[2]) / (d / 2), pool_blocks, (int)t[9].dtype, stream);
+      hkv, d, bs, batch ? numel(t[4]) / batch : 1, numel(t[2]) / rope_w, rope_w, pool_blocks, (int)t[9].dtype, stream);
 }
 
 int run_rope_kv(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream) {
@@ -398,18 +405,19 @@ int run_rope_kv(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hi
                 "rope_kv_cache_update: seq_lens and block_table must be INT32");
   PTO_CHECK_ARG(t[2].dtype == PTO_HIP_FP32 && t[3].dtype == PTO_HIP_FP32 && numel(t[2]) == numel(t[3]) &&
                     numel(t[2]) % (d / 2) == 0,
-                "rope_kv_cache_update: rope_cos/rope_sin must be FP32 [max_pos, D/2]");
+                "rope_kv_cache_update: rope_cos/rope_sin must be FP32 [max_pos, D/2] or [max_pos, D]");
+  const int rope_w = rope_table_width(t[2], d);
   PTO_CHECK_ARG(batch > 0 ? numel(t[4]) % batch == 0 : true, "rope_kv_cache_update: block_table must be [B, max_blocks]");
   PTO_CHECK_ARG(t[5].dtype == t[6].dtype && t[5].dtype == t[7].dtype && numel(t[5]) == numel(t[6]) &&
                     numel(t[5]) % d == 0 && numel(t[7]) == batch * hq * d,
                 "rope_kv_cache_update: caches and q_out must share a dtype; caches [rows, D], q_out [B*Hq, D]");
-  return pto_hip_rope_kv_cache_update(reinterpret_cast<const float*>(tptr(t[0])),
+  return rope_kv_cache_update(reinterpret_cast<const float*>(tptr(t[0])), nullptr, 1, 0,
                                       reinterpret_cast<const int32_t*>(tptr(t[1])),
                                       reinterpret_cast<const float*>(tptr(t[2])),
                                       reinterpret_cast<const float*>(tptr(t[3])),
                                       reinterpret_cast<const int32_t*>(tptr(t[4])), tptr_mut(t[5]), tptr_mut(t[6]),
                                       tptr_mut(t[7]), batch, hq, hkv, d, bs, batch ? numel(t[4]) / batch : 1,
-                                      numel(t[2]) / (d / 2), numel(t[5]) / d, (int)t[5].dtype, stream);
+                                      numel(t[2]) / rope_w, rope_w, numel(t[5]) / d, (int)t[5].dtype, stream);
 }
 
 int run_decoder_layer(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream) {
@@ -474,7 +482,8 @@ int run_decoder_layer(const PtoHipChipTensor* t, int nt, const uint64_t* s, int 
   PTO_CHECK_ARG(w[2]->ndims == 2, "decoder_layer_decode: w_gate must be [H, I]");
   a.intermediate = w[2]->shapes[1];
   a.max_num_blocks_per_req = a.batch ? numel(t[2]) / a.batch : 1;
-  a.max_pos = numel(t[5 + o]) / (a.head_dim / 2);
+  a.rope_table_width = rope_table_width(t[5 + o], a.head_dim);
+  a.max_pos = numel(t[5 + o]) / a.rope_table_width;
   a.pool_rows = numel(t[3]) / a.head_dim;
   a.dtype = (int)t[0].dtype;
   const int64_t qkv_n = (a.num_heads + 2 * a.kv_head_num) * a.head_dim;

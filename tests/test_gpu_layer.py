@@ -82,6 +82,41 @@ def test_w8a16_more_than_one_row_pass(worker, m):
     validate_golden({"out": out2.float()}, {"out": ref2.float()}, rtol=1e-2, atol=1e-3)
 
 
+def test_rope_tables_of_full_head_width(worker):
+    """The reference's tables are [max_pos, D]: columns 0..D/2 multiply the low half, the rest the
+    high half (examples/models/qwen3_jit/kernels/attention.py:57-70).  Duplicated half-width tables
+    give the same bits as the half-width call; tables whose halves differ follow the four-factor form."""
+    b, hq, hkv, d, bs = 3, 8, 2, 128, 16
+    seq = [17, 1, 40]
+    inp = workloads.decoder_layer_inputs(batch=b, hidden=256, num_heads=hq, kv_head_num=hkv, head_dim=d,
+                                         intermediate=512, block_size=bs, context_lens=seq, seed=3)
+    g = torch.Generator().manual_seed(4)
+    qkv = torch.randn(b, (hq + 2 * hkv) * d, generator=g)
+
+    def run(cos, sin, program=rope_kv_cache_update, extra=()):
+        kc, vc = inp.key_cache.clone(), inp.value_cache.clone()
+        q_out = torch.zeros(b * hq, d, dtype=torch.bfloat16)
+        with worker.register(program) as h:
+            h(qkv, inp.seq_lens, cos, sin, inp.block_table, kc, vc, *extra, q_out, hq, hkv, d, bs)
+        return q_out, kc, vc
+
+    half = run(inp.rope_cos, inp.rope_sin)
+    full = run(torch.cat([inp.rope_cos, inp.rope_cos], dim=1), torch.cat([inp.rope_sin, inp.rope_sin], dim=1))
+    assert all(torch.equal(a, c) for a, c in zip(half, full))
+    # halves that differ: lo' = lo*cos_lo - hi*sin_lo, hi' = hi*cos_hi + lo*sin_hi
+    cos2 = torch.cat([inp.rope_cos, 0.5 * inp.rope_cos], dim=1).contiguous()
+    sin2 = torch.cat([inp.rope_sin, -inp.rope_sin], dim=1).contiguous()
+    q_out, kc, _ = run(cos2, sin2)
+    pos = torch.tensor(seq) - 1
+    q = qkv[:, :hq * d].reshape(b, hq, d)
+    lo, hi = q[..., :d // 2], q[..., d // 2:]
+    c_lo, c_hi = cos2[pos, :d // 2].unsqueeze(1), cos2[pos, d // 2:].unsqueeze(1)
+    s_lo, s_hi = sin2[pos, :d // 2].unsqueeze(1), sin2[pos, d // 2:].unsqueeze(1)
+    want = torch.cat([lo * c_lo - hi * s_lo, hi * c_hi + lo * s_hi], dim=-1).to(torch.bfloat16).reshape(b * hq, d)
+    assert torch.allclose(q_out.float(), want.float(), atol=2e-2, rtol=1e-2)
+    assert not torch.equal(q_out, half[0])
+
+
 def test_rope_kv_cache_update(worker):
     b, hq, hkv, d, bs = 3, 8, 2, 128, 16
     seq = [17, 1, 40]
