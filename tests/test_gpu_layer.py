@@ -117,6 +117,31 @@ def test_rope_tables_of_full_head_width(worker):
     assert not torch.equal(q_out, half[0])
 
 
+def test_contiguous_per_sequence_cache_is_the_one_block_case(worker):
+    """The reference's decode example keeps K/V per sequence at row b*Hkv*MAX_SEQ + h*MAX_SEQ + pos
+    (examples/models/qwen3_jit/kernels/attention.py:72-80): the paged layout with one block of MAX_SEQ
+    tokens per sequence and block_table[b] = b."""
+    b, hq, hkv, d, max_seq = 3, 8, 2, 128, 64
+    seq = [17, 1, 64]
+    g = torch.Generator().manual_seed(8)
+    qkv = torch.randn(b, (hq + 2 * hkv) * d, generator=g)
+    cos, sin = oracle.rope_cos_sin(max_seq, d)
+    kc = torch.zeros(b * hkv * max_seq, d, dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    q_out = torch.zeros(b * hq, d, dtype=torch.bfloat16)
+    with worker.register(rope_kv_cache_update) as h:
+        h(qkv, torch.tensor(seq, dtype=torch.int32), cos, sin, torch.arange(b, dtype=torch.int32), kc, vc, q_out,
+          hq, hkv, d, max_seq)
+    v = qkv[:, (hq + hkv) * d:].reshape(b, hkv, d).to(torch.bfloat16)
+    written = torch.zeros(b * hkv * max_seq, dtype=torch.bool)
+    for bi in range(b):
+        for hh in range(hkv):
+            row = bi * hkv * max_seq + hh * max_seq + seq[bi] - 1
+            assert torch.equal(vc[row], v[bi, hh])
+            written[row] = True
+    assert (vc[~written] == 0).all() and (kc[~written] == 0).all() and (kc[written] != 0).any()
+
+
 def test_rope_kv_cache_update(worker):
     b, hq, hkv, d, bs = 3, 8, 2, 128, 16
     seq = [17, 1, 40]
