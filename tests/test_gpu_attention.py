@@ -348,3 +348,22 @@ def test_block_table_entry_outside_the_cache_is_caught(worker):
 def dataclass_replace(inp, table):
     import dataclasses
     return dataclasses.replace(inp, block_table=table)
+
+
+@pytest.mark.parametrize("context_len", [8192, 8100])
+def test_reference_end_to_end_configs(worker, context_len):
+    """The reference's two whole-program cases: batch 64, 16 heads on one KV head, block 128, context
+    8192 and the unaligned 8100, table sized for 32768 tokens, scale 1.0 and a block table drawn
+    with replacement (tests/st/runtime/framework_and_models/test_paged_attention.py:843-901,
+    examples/models/04_paged_attention.py:560-575).  The pool holds the blocks in use only."""
+    batch, hq, d, bs, max_model_len = 64, 16, 128, 128, 32768
+    inp = workloads.paged_attention_inputs(batch=batch, num_heads=hq, kv_head_num=1, head_dim=d, block_size=bs,
+                                           context_lens=[context_len] * batch, ctx_range=(1, context_len),
+                                           max_num_blocks_per_req=max_model_len // bs, scale=1.0, seed=29)
+    pool_blocks = inp.key_cache.shape[0] // bs
+    g = torch.Generator().manual_seed(30)
+    table = torch.randint(0, pool_blocks, (batch * (max_model_len // bs),), generator=g, dtype=torch.int32)
+    inp = dataclass_replace(inp, table)
+    ref = _golden(inp)
+    for tpp in (0, -4):
+        _check(_run(worker, inp, tpp), ref)
