@@ -135,6 +135,8 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *      scalars: num_heads, kv_head_num, head_dim, block_size
  *  "projection"            examples/models/qwen3_jit/kernels/projection.py:35-57,118-177
  *      tensors: x[M,K], w[K,N] (dtype of x), [residual[M,N],] out[M,N] (fp32 or dtype of x)
+ *  "gate_up_swiglu"        examples/models/qwen3_jit/kernels/mlp.py:22-61
+ *      tensors: x[M,K], w_gate[K,N], w_up[K,N], out[M,N], all of one 16-bit dtype
  *  "decoder_layer_decode"  examples/models/qwen3_jit/qwen3_decode.py:47-113
  *      tensors: hidden_states[B,H], seq_lens, block_table, key_cache (INOUT), value_cache (INOUT),
  *               rope_cos, rope_sin, gamma_in[H], gamma_post[H], wqkv_q, wqkv_s, wo_q, wo_s, wg_q, wg_s,
@@ -204,6 +206,12 @@ PTO_HIP_API int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void
  * weights once (HBM-bound), more rows run as an MFMA-tiled GEMM. */
 PTO_HIP_API int pto_hip_projection(const void* x, const void* w, const void* residual, void* out, int64_t m,
                                    int64_t k, int64_t n, int dtype, int res_dtype, int out_dtype, void* stream);
+
+/* out[M, N] = SiLU(x @ w_gate) * (x @ w_up) rounded to `dtype`: the gate/up half of the FFN with the
+ * reference's 16-bit weights (examples/models/qwen3_jit/kernels/mlp.py:22-61).  Regimes and shape
+ * rules as pto_hip_projection. */
+PTO_HIP_API int pto_hip_gate_up_swiglu(const void* x, const void* w_gate, const void* w_up, void* out, int64_t m,
+                                       int64_t k, int64_t n, int dtype, void* stream);
 
 /* W8A16 decode projection (no counterpart in the reference, which has no quantised weights; the
  * contract is its projection kernel's, examples/models/qwen3_jit/kernels/projection.py:145-177,

@@ -25,6 +25,7 @@ EXPORTS = (
     "pto_hip_w8a16_matmul", "pto_hip_w8a16_swiglu", "pto_hip_rope_kv_cache_update",
     "pto_hip_rope_kv_cache_update_fp8",
     "pto_hip_decoder_layer_decode", "pto_hip_select_program", "pto_hip_projection",
+    "pto_hip_gate_up_swiglu",
 )
 
 
@@ -97,6 +98,7 @@ def load() -> C.CDLL:
         "pto_hip_w8a16_matmul": [vp, vp, vp, vp, vp, i64, i64, i64, C.c_int, C.c_int, C.c_int, vp],
         "pto_hip_w8a16_swiglu": [vp, vp, vp, vp, vp, vp, i64, i64, i64, C.c_int, C.c_int, vp],
         "pto_hip_projection": [vp, vp, vp, vp, i64, i64, i64, C.c_int, C.c_int, C.c_int, vp],
+        "pto_hip_gate_up_swiglu": [vp, vp, vp, vp, i64, i64, i64, C.c_int, vp],
         "pto_hip_rope_kv_cache_update": [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64,
                                          C.c_int, vp],
         "pto_hip_rope_kv_cache_update_fp8": [vp] * 10 + [i64] * 8 + [C.c_int, vp],

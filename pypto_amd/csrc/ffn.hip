@@ -659,3 +659,41 @@ extern "C" int pto_hip_projection(const void* x, const void* w, const void* resi
   p.res_dtype = res_dtype;
   return launch_typed<false>(p, dtype, out_dtype, st);
 }
+
+// out[M, N] = SiLU(x @ w_gate) * (x @ w_up), rounded to the activation type: the gate/up half of
+// the FFN as the reference's mlp_block writes it (examples/models/qwen3_jit/kernels/mlp.py:22-61).
+// Same two regimes as pto_hip_projection.
+extern "C" int pto_hip_gate_up_swiglu(const void* x, const void* w_gate, const void* w_up, void* out, int64_t m,
+                                      int64_t k, int64_t n, int dtype, void* stream) {
+  using namespace pto_hip;
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(m >= 0 && k > 0 && n > 0 && m < (1 << 30) && k < (1 << 30) && n < (1 << 30),
+                "gate_up_swiglu: bad shape M=%lld K=%lld N=%lld", (long long)m, (long long)k, (long long)n);
+  if (m == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(dtype == PTO_HIP_BF16 || dtype == PTO_HIP_FP16, "gate_up_swiglu: dtype %s not in {BF16, FP16}",
+                dtype_name(dtype));
+  PTO_CHECK_ARG(x && w_gate && w_up && out, "gate_up_swiglu: null tensor pointer");
+  PTO_CHECK_ARG(k % 8 == 0 && n % 8 == 0, "gate_up_swiglu: K = %lld and N = %lld must be multiples of 8",
+                (long long)k, (long long)n);
+  PTO_CHECK_ARG(((uintptr_t)x | (uintptr_t)w_gate | (uintptr_t)w_up | (uintptr_t)out) % 16 == 0,
+                "gate_up_swiglu: operand pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  if (m <= kSkinnyMaxTokens && ctx().gemm_variant == 0 && k % 16 == 0 && k >= 32) {
+    W8Partials parts{};
+    int rc = w8a16_partials(x, false, w_gate, w_up, m, k, n, dtype, st, &parts, true);
+    if (rc) return rc;
+    return w8a16_finish(parts, nullptr, nullptr, nullptr, 0, out, dtype, false, m, n, st);
+  }
+  GemmParams p{};
+  p.a = reinterpret_cast<const uint16_t*>(x);
+  p.b0 = reinterpret_cast<const uint16_t*>(w_gate);
+  p.b1 = reinterpret_cast<const uint16_t*>(w_up);
+  p.c = out;
+  p.lda = k;
+  p.ldb = n;
+  p.ldc = n;
+  p.m = (int)m;
+  p.n = (int)n;
+  p.k = (int)k;
+  return launch_typed<true>(p, dtype, dtype, st);
+}

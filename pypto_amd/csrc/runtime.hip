@@ -80,13 +80,14 @@ enum ProgramKind {
   kRopeKvCacheUpdateFp8,
   kDecoderLayerDecode,
   kProjection,
+  kGateUpSwiglu,
   kNumPrograms
 };
 
 const char* const kProgramNames[kNumPrograms] = {
     "paged_attention", "paged_gather",  "rms_norm",           "ffn_swiglu",          "ffn_block",
     "w8a16_matmul",    "w8a16_swiglu",  "rope_kv_cache_update", "rope_kv_cache_update_fp8",
-    "decoder_layer_decode", "projection"};
+    "decoder_layer_decode", "projection", "gate_up_swiglu"};
 
 std::mutex g_mu;
 std::vector<int> g_callables;  // callable id -> ProgramKind, -1 once unregistered
@@ -323,6 +324,23 @@ int run_projection(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, h
                             stream);
 }
 
+int run_gate_up_swiglu(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
+  PTO_CHECK_ARG(nt == 4 && ns == 0, "gate_up_swiglu: expected x, w_gate, w_up, out and no scalars, got %d + %d", nt,
+                ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor("gate_up_swiglu", "operand", t[i], 2, 2);
+    if (rc) return rc;
+  }
+  const PtoHipChipTensor &x = t[0], &wg = t[1], &wu = t[2], &out = t[3];
+  const int64_t m = x.shapes[0], k = x.shapes[1], n = wg.shapes[1];
+  PTO_CHECK_ARG(wg.dtype == x.dtype && wu.dtype == x.dtype && out.dtype == x.dtype,
+                "gate_up_swiglu: weights and out must have the dtype of x (%s)", dtype_name(x.dtype));
+  PTO_CHECK_ARG(wg.shapes[0] == k && wu.shapes[0] == k && wu.shapes[1] == n,
+                "gate_up_swiglu: w_gate and w_up must be [K=%lld, N]", (long long)k);
+  PTO_CHECK_ARG(out.shapes[0] == m && out.shapes[1] == n, "gate_up_swiglu: out must be [M, N]");
+  return pto_hip_gate_up_swiglu(tptr(x), tptr(wg), tptr(wu), tptr_mut(out), m, k, n, (int)x.dtype, stream);
+}
+
 int run_w8a16_swiglu(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
   PTO_CHECK_ARG(nt == 6 && ns == 0, "w8a16_swiglu: expected x, wg_q, wg_scale, wu_q, wu_scale, out, got %d + %d", nt, ns);
   for (int i = 0; i < nt; ++i) {
@@ -527,6 +545,7 @@ int dispatch(int kind, const PtoHipChipTensor* t, int nt, const uint64_t* s, int
     case kFfnBlock: return run_ffn(t, nt, s, ns, stream, true);
     case kW8a16Matmul: return run_w8a16_matmul(t, nt, s, ns, stream);
     case kProjection: return run_projection(t, nt, s, ns, stream);
+    case kGateUpSwiglu: return run_gate_up_swiglu(t, nt, s, ns, stream);
     case kW8a16Swiglu: return run_w8a16_swiglu(t, nt, s, ns, stream);
     case kRopeKvCacheUpdate: return run_rope_kv(t, nt, s, ns, stream);
     case kRopeKvCacheUpdateFp8: return run_rope_kv_fp8(t, nt, s, ns, stream);

@@ -72,6 +72,7 @@ ffn_block = HipProgram("ffn_block", (IN, IN, IN, IN, IN, OUT), scalars=("eps",))
 
 projection = HipProgram("projection", (IN, IN, OUT))
 projection_residual = HipProgram("projection", (IN, IN, IN, OUT))
+gate_up_swiglu = HipProgram("gate_up_swiglu", (IN, IN, IN, OUT))
 w8a16_matmul = HipProgram("w8a16_matmul", (IN, IN, IN, OUT))
 w8a16_matmul_residual = HipProgram("w8a16_matmul", (IN, IN, IN, IN, OUT))
 w8a16_swiglu = HipProgram("w8a16_swiglu", (IN, IN, IN, IN, IN, OUT))
@@ -98,7 +99,8 @@ decoder_layer_decode_w16_fp8kv = HipProgram(
     "decoder_layer_decode", (IN, IN, IN, INOUT, INOUT, INOUT, INOUT) + (IN,) * 9 + (OUT,),
     scalars=("num_heads", "kv_head_num", "head_dim", "block_size", "eps"))
 
-PROGRAMS = {p.name: p for p in (paged_attention, paged_gather, rms_norm, ffn_swiglu, ffn_block, projection, w8a16_matmul,
+PROGRAMS = {p.name: p for p in (paged_attention, paged_gather, rms_norm, ffn_swiglu, ffn_block, projection, gate_up_swiglu,
+                                w8a16_matmul,
                                 w8a16_swiglu, rope_kv_cache_update, rope_kv_cache_update_fp8,
                                 decoder_layer_decode)}
 

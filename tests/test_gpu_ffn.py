@@ -194,3 +194,60 @@ def test_projection_argument_rules(worker):
     with pytest.raises(ValueError, match="out must be"):
         with worker.register(projection) as h:
             h(x, torch.zeros(64, 64, dtype=torch.bfloat16), torch.zeros(4, 32))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,n", [(16, 1024, 2816), (32, 512, 1000), (100, 1024, 2816), (300, 512, 1536)])
+def test_gate_up_swiglu_matches_oracle(worker, dtype, m, k, n):
+    from pypto_amd.runtime import gate_up_swiglu
+    g = torch.Generator().manual_seed(m + n)
+    x = torch.randn(m, k, generator=g).to(dtype)
+    wg = (torch.randn(k, n, generator=g) / k ** 0.5).to(dtype)
+    wu = (torch.randn(k, n, generator=g) / k ** 0.5).to(dtype)
+    out = torch.zeros(m, n, dtype=dtype)
+    with worker.register(gate_up_swiglu) as h:
+        h(x, wg, wu, out)
+    want = oracle.swiglu(oracle.projection(x, wg), oracle.projection(x, wu)).to(dtype)
+    validate_golden({"out": out.float()}, {"out": want.float()}, rtol=2e-2, atol=1e-2)
+
+
+def test_reference_scope3_from_the_public_programs(worker):
+    """Scope 3 of the reference's qwen3 decode layer at its own configuration (batch 16, hidden 5120,
+    intermediate 25600, inputs randn / sqrt(fan_in); tests/st/runtime/framework_and_models/
+    test_qwen3_decode_scope3_mixed.py:45-47,255-336) composed from the programs that stand in for its
+    kernels: out_projection_residual, post_rmsnorm, mlp_block, down_projection_residual
+    (examples/models/qwen3_jit/qwen3_decode.py:100-110).  Checked against its golden, written out
+    below, at its tolerance rtol 2e-2 / atol 1e-3."""
+    from pypto_amd.runtime import gate_up_swiglu, projection_residual
+    batch, hidden, inter = 16, 5120, 25600
+    g = torch.Generator().manual_seed(0)
+    rn = lambda shape, fan_in: torch.randn(shape, generator=g) / fan_in ** 0.5
+    attn_out = rn([batch, hidden], hidden).to(torch.bfloat16).cuda()
+    hidden_states = rn([batch, hidden], hidden).to(torch.bfloat16).cuda()
+    wo = rn([hidden, hidden], hidden).to(torch.bfloat16).cuda()
+    post_rms_weight = rn([1, hidden], hidden).cuda()
+    w_gate = rn([hidden, inter], inter).to(torch.bfloat16).cuda()
+    w_up = rn([hidden, inter], inter).to(torch.bfloat16).cuda()
+    w_down = rn([inter, hidden], hidden).to(torch.bfloat16).cuda()
+    resid1 = torch.zeros(batch, hidden, device="cuda")
+    post_norm = torch.zeros(batch, hidden, dtype=torch.bfloat16, device="cuda")
+    mlp = torch.zeros(batch, inter, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros(batch, hidden, dtype=torch.bfloat16, device="cuda")
+    with worker.register(projection_residual) as h:
+        h(attn_out, wo, hidden_states, resid1)
+    with worker.register(rms_norm) as h:
+        h(resid1, post_rms_weight, post_norm, 1e-6)
+    with worker.register(gate_up_swiglu) as h:
+        h(post_norm, w_gate, w_up, mlp)
+    with worker.register(projection_residual) as h:
+        h(mlp, w_down, resid1, out)
+    worker.sync()
+    # the reference's golden, on the GPU in fp32 (same steps, same rounding points)
+    o_proj = attn_out.float() @ wo.float()
+    r1 = o_proj + hidden_states.float()
+    inv_rms = torch.rsqrt(r1.pow(2).mean(dim=-1, keepdim=True) + 1e-6)
+    normed_bf16 = (r1 * inv_rms * post_rms_weight).bfloat16()
+    gate, up = normed_bf16.float() @ w_gate.float(), normed_bf16.float() @ w_up.float()
+    mlp_bf16 = (gate * torch.sigmoid(gate) * up).bfloat16()
+    want = (mlp_bf16.float() @ w_down.float() + r1).bfloat16()
+    validate_golden({"out": out.float().cpu()}, {"out": want.float().cpu()}, rtol=2e-2, atol=1e-3)
