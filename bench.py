@@ -214,6 +214,30 @@ def main() -> int:
         }
         del dw, dwargs
         torch.cuda.empty_cache()
+        # the reference's CI perf-guard workload: one qwen3-14B decoder layer, batch 16, sequences at
+        # max_seq 4096 (.github/perf_baselines/qwen3_14b_decode.json: 1016.66 us on its own hardware)
+        dq = workloads.decoder_layer_inputs(batch=16, hidden=5120, num_heads=40, kv_head_num=8, head_dim=128,
+                                            intermediate=17408, context=4096, theta=1e6, device="cuda",
+                                            int8_weights=False)
+        torch.cuda.synchronize()
+        with worker.register(decoder_layer_decode_w16) as dh:
+            dqargs = [dq.args()]
+            benchmark(dh, dqargs, rounds=5, warmup=0)
+            dqstats = benchmark(dh, dqargs, rounds=20, warmup=0)
+        dqbytes = dq.algorithmic_bytes()
+        result["decoder_layer_qwen3_14b"] = {
+            "workload": "qwen3-14B decoder layer decode step, bf16 weights: H5120 Hq40 Hkv8 D128 I17408 B16 ctx4096 "
+                        "(the shape of the reference's CI perf guard, 1016.66 us there on other hardware)",
+            "algorithmic_bytes_per_step": dqbytes,
+            "us_per_step": round(dqstats.device_wall_us, 1),
+            "achieved": round(dqbytes / dqstats.device_wall_us / 1e3, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(dqbytes / dqstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "bound": "hbm",
+        }
+        del dq, dqargs
+        torch.cuda.empty_cache()
         # FFN block at a decode-size token count: bound by reading the 16-bit weights once
         fd = [workloads.ffn_inputs(tokens=16, hidden=4096, intermediate=11008, seed=s, device="cuda") for s in (0, 1)]
         torch.cuda.synchronize()
