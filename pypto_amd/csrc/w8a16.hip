@@ -382,18 +382,35 @@ int check_common(const char* what, int64_t m, int64_t k, int64_t n, int x_dtype,
   return PTO_HIP_OK;
 }
 
-// k splits: a few workgroups per compute unit, each wavefront with at least a few steps when k
-// allows, split boundaries on multiples of the rows one round of the wavefronts covers.
-void choose_splits(int64_t k, int64_t slabs_total, int waves, int* splits, int* k_per_split) {
+// k splits.  A CU pulls its weight bytes at a bounded rate (about its 1/num_cu share of the HBM
+// rate), so a launch lasts as long as the CU with the most bytes: 272 workgroups on 256 CUs leave
+// 16 CUs with twice the work and ran 1.5x longer than 256 would.  The split count is the one
+// that minimises   rounds x (steps per wavefront + ramp) + splits x partial-sum cost,
+// rounds = ceil(workgroups / (wgs_per_cu x num_cu)); the constants are fitted to measured
+// launches (ramp 2.5 steps; one split's partial sums cost about n_total / 10000 steps).
+// Split boundaries fall on multiples of the rows one round of the wavefronts covers, and a
+// wavefront keeps at least min_steps steps when k allows.
+void choose_splits(int64_t k, int64_t slabs_total, int64_t n_total, int waves, int* splits, int* k_per_split) {
   const int kUnit = kStep * waves;  // k rows one round of the wavefronts covers
   const pto_hip::Context& cx = pto_hip::ctx();
   const int64_t units = (k + kUnit - 1) / kUnit;
-  int64_t want = (cx.w8a16_wgs_per_cu * cx.num_cu) / slabs_total;
-  if (want < 1) want = 1;
-  int64_t per = (units + want - 1) / want;
-  if (per < cx.w8a16_min_steps) per = units >= cx.w8a16_min_steps ? cx.w8a16_min_steps : units;
-  *splits = (int)((units + per - 1) / per);
-  *k_per_split = (int)(per * kUnit);
+  const int64_t capacity = std::max<int64_t>(1, cx.w8a16_wgs_per_cu * cx.num_cu);
+  const double ramp = 2.5, partial_cost = (double)n_total / 10000.0;
+  int64_t best_per = units;
+  double best_cost = 1e30;
+  for (int64_t want = 1; want <= std::min<int64_t>(units, 16); ++want) {
+    const int64_t per = (units + want - 1) / want;
+    if (want > 1 && per < cx.w8a16_min_steps) break;
+    const int64_t real = (units + per - 1) / per;
+    const int64_t rounds = (slabs_total * real + capacity - 1) / capacity;
+    const double cost = (double)rounds * ((double)per + ramp) + (real > 1 ? (double)real * partial_cost : 0.0);
+    if (cost < best_cost) {
+      best_cost = cost;
+      best_per = per;
+    }
+  }
+  *splits = (int)((units + best_per - 1) / best_per);
+  *k_per_split = (int)(best_per * kUnit);
 }
 
 }  // namespace
@@ -412,7 +429,7 @@ int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* w
   p.slabs = (int)((n + kSlab - 1) / kSlab);
   p.n_mats = wq1 ? 2 : 1;
   p.x_blocked = x_blocked ? 1 : 0;
-  choose_splits(k, (int64_t)p.slabs * p.n_mats, kWavesPerWg, &p.splits, &p.k_per_split);
+  choose_splits(k, (int64_t)p.slabs * p.n_mats, n * p.n_mats, kWavesPerWg, &p.splits, &p.k_per_split);
   const size_t one = (size_t)p.splits * kMaxM * n * sizeof(float);
   void* ws = nullptr;
   int rc = workspace(one * p.n_mats, &ws);
