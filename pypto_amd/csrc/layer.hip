@@ -80,10 +80,13 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
 
   // Layer-private intermediates (the kernels' own scratch lives in the shared workspace).
   auto up = [](size_t n) { return (n + 255) / 256 * 256; };
-  const size_t sz_normed = up((size_t)b * h * 2),
+  // The 16-bit activations may be kept in the blocked layout [K/8][32][8], which spans 32 row
+  // slots whatever the batch: those buffers are sized for 32 rows.
+  const size_t rows16 = kW8MaxM;
+  const size_t sz_normed = up(rows16 * h * 2),
                sz_q = up((size_t)b * hq * d * 2), sz_attn = up((size_t)b * hq * d * 4),
-               sz_attn16 = up((size_t)b * hq * d * 2), sz_resid = up((size_t)b * h * 4),
-               sz_h = up((size_t)b * inter * 2);
+               sz_attn16 = up(rows16 * hq * d * 2), sz_resid = up((size_t)b * h * 4),
+               sz_h = up(rows16 * inter * 2);
   const size_t total = sz_normed + sz_q + sz_attn + sz_attn16 + sz_resid + sz_normed + sz_h;
   void* lws = nullptr;
   {

@@ -301,6 +301,20 @@ def test_decoder_layer_decode_16bit_weights(worker, dtype, batch):
     assert torch.allclose(inp.value_cache.float(), ref_v.float(), atol=2e-2, rtol=1e-2)
 
 
+def test_decoder_layer_small_batch_odd_sizes(worker):
+    """Batch 16 with hidden 576 and intermediate 544 (k not a multiple of the 128 rows one round of
+    the projection wavefronts covers, partial 128-column slabs): the blocked 16-bit activations span
+    32 row slots whatever the batch, and their buffers must be sized for that."""
+    ctxs = [49, 15, 1, 357, 128, 1, 1, 1, 1, 128, 1, 128, 392, 128, 128, 128]
+    inp = workloads.decoder_layer_inputs(batch=16, hidden=576, num_heads=4, kv_head_num=4, head_dim=128,
+                                         intermediate=544, block_size=128, context_lens=ctxs, seed=5,
+                                         int8_weights=False)
+    ref_out, _, _ = _oracle_layer(inp)
+    with worker.register(decoder_layer_decode_w16) as h:
+        h(*inp.args())
+    validate_golden({"out": inp.out.float()}, {"out": ref_out.float()}, rtol=2e-2, atol=2e-2)
+
+
 def test_decoder_layer_16bit_weights_second_half_matches_reference_golden(worker):
     """With an identity-like first half the layer's output is the reference's scope-3 golden
     (o_proj + residual, post RMSNorm, SwiGLU MLP, residual;
