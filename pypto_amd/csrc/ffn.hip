@@ -419,11 +419,13 @@ int launch_variant(GemmParams p, hipStream_t st) {
   p.splits = 1;
   p.k_per_split = p.k;
   p.slabs = nullptr;
-  // variant 0 (default): eight wavefronts (two per SIMD) on a 256x256 tile, or on a 128x256 tile
-  // when the large one would leave CUs without a workgroup (measured on the LLaMA-7B down pass:
-  // 183 us against 223 us for the large tile with k split in two); when even the small tile
-  // covers at most half of the CUs (a few hundred tokens), k is split over up to eight
-  // workgroups per tile, each writing an fp32 slab that a second kernel sums in split order.
+  // variant 0 (default): eight wavefronts (two per SIMD) on a 256x256 tile; when that would leave
+  // CUs without a workgroup, either the 128x256 tile, with k split over up to 16 workgroups per
+  // tile while even the short tiles cover at most half of the CUs (a few hundred tokens), or -
+  // beyond 1024 rows, where the tall tile is well filled - the 256x256 tile with k split in up
+  // to four, whichever needs the fewest rounds of workgroups over the CUs (LLaMA-7B down pass at
+  // 2048 tokens: 128 tall tiles split in two 192 us, 256 short tiles 204 us).  Splits write fp32 slabs that a second kernel sums in
+  // split order.
   // variants 1-3 keep four wavefronts (one per SIMD): 1 = 256x256 tile, 2 = 128x256 tile,
   // 3 = 256x256 tile with k split in two.  4 = eight wavefronts, 256x256 tile, k split in two
   // when CUs would idle.  5 = eight wavefronts, 128x256 tile.
@@ -432,8 +434,25 @@ int launch_variant(GemmParams p, hipStream_t st) {
   const int64_t small_tiles = (int64_t)((p.m + 127) / 128) * tiles_n;
   const bool few = big_tiles < num_cu;
   int want = 1;
+  bool small_tile = variant == 5 || (variant == 0 && few);
   if (variant == 3 || (variant == 4 && few)) want = 2;
-  if (variant == 0 && few && small_tiles * 2 <= num_cu) want = (int)std::min<int64_t>(kMaxSplits, num_cu / small_tiles);
+  if (variant == 0 && few) {
+    if (small_tiles * 2 <= num_cu) {
+      want = (int)std::min<int64_t>(kMaxSplits, num_cu / small_tiles);
+    } else if (p.m > 1024) {
+      // Time in units of one tall tile: rounds of workgroups over the CUs, a short tile costing
+      // 0.5 / 0.86 of a tall one (measured), a split launch about 0.05 more for its slabs.
+      double best = (double)((small_tiles + num_cu - 1) / num_cu) * (0.5 / 0.86);
+      for (int s = 1; s <= 4; ++s) {
+        const double cost = (double)((big_tiles * s + num_cu - 1) / num_cu) / s + (s > 1 ? 0.05 : 0.0);
+        if (cost < best) {
+          best = cost;
+          small_tile = false;
+          want = s;
+        }
+      }
+    }
+  }
   if (want > 1 && p.k >= 4 * BK * want && p.n % 4 == 0) {
     p.k_per_split = ((p.k + want * BK - 1) / (want * BK)) * BK;
     p.splits = (p.k + p.k_per_split - 1) / p.k_per_split;
@@ -445,7 +464,7 @@ int launch_variant(GemmParams p, hipStream_t st) {
     }
   }
   int rc;
-  if (variant == 5 || (variant == 0 && few)) rc = launch_gemm<2, 2, 4, DUAL, BF16, OutT>(p, st);
+  if (small_tile) rc = launch_gemm<2, 2, 4, DUAL, BF16, OutT>(p, st);
   else if (variant == 2) rc = launch_gemm<2, 2, 2, DUAL, BF16, OutT>(p, st);
   else if (variant == 0 || variant == 4) rc = launch_gemm<4, 2, 4, DUAL, BF16, OutT>(p, st);
   else rc = launch_gemm<4, 2, 2, DUAL, BF16, OutT>(p, st);
