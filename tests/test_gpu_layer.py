@@ -315,6 +315,20 @@ def test_decoder_layer_small_batch_odd_sizes(worker):
     validate_golden({"out": inp.out.float()}, {"out": ref_out.float()}, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("hidden,int8", [(12288, True), (9216, False)])
+def test_decoder_layer_wide_hidden(worker, hidden, int8):
+    """Hidden sizes beyond the fused residual + RMSNorm finish (8192 channels): that step falls back
+    to a plain finish followed by the stand-alone RMSNorm, and activations stay row-major."""
+    batch = 3
+    inp = workloads.decoder_layer_inputs(batch=batch, hidden=hidden, num_heads=8, kv_head_num=2, head_dim=128,
+                                         intermediate=1024, block_size=64, context_lens=[100, 137, 174], seed=7,
+                                         int8_weights=int8)
+    ref_out, _, _ = _oracle_layer(inp)
+    with worker.register(decoder_layer_decode if int8 else decoder_layer_decode_w16) as h:
+        h(*inp.args())
+    validate_golden({"out": inp.out.float()}, {"out": ref_out.float()}, rtol=2e-2, atol=2e-2)
+
+
 def test_decoder_layer_16bit_weights_second_half_matches_reference_golden(worker):
     """With an identity-like first half the layer's output is the reference's scope-3 golden
     (o_proj + residual, post RMSNorm, SwiGLU MLP, residual;
