@@ -259,7 +259,9 @@ PTO_HIP_API int pto_hip_rope_kv_cache_update_fp8(const float* qkv, const int32_t
  * RMSNorm -> QKV -> RoPE + K/V append -> paged attention -> o_proj + residual -> RMSNorm ->
  * SwiGLU FFN + residual.  Projection weights are [in, out]: either the reference's 16-bit weights
  * (all *_s pointers NULL; golden tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:255-287)
- * or INT8 codes with FP32 per-output scales.
+ * or INT8 codes with FP32 per-output scales.  Up to 32 sequences stream the weights once through
+ * skinny projections; more run the projections as tiled GEMMs (16-bit weights) or as consecutive groups
+ * of 32 sequences (INT8 weights).
  * With e4m3 caches pool_rows is still the row count of each cache (pool_blocks * Hkv * block_size). */
 typedef struct PtoHipDecoderLayerArgs {
   const void* hidden_states;  /* [B, H] dtype */

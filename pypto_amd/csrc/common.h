@@ -44,7 +44,11 @@ struct Context {
   // Intermediates of the composed decoder layer (grow-only).
   void* layer_ws = nullptr;
   size_t layer_ws_bytes = 0;
-  // Buffers the two scratch areas outgrew.  They stay allocated until pto_hip_close: launches
+  // Split-K slabs of the tiled GEMM (grow-only), apart from the two above so that a caller's
+  // intermediates in either of them survive a GEMM launch.
+  void* gemm_ws = nullptr;
+  size_t gemm_ws_bytes = 0;
+  // Buffers the scratch areas outgrew.  They stay allocated until pto_hip_close: launches
   // recorded into a HIP graph keep the address they were recorded with.
   std::vector<void*> retired;
   // 256 bytes of device flags written by kernels that report bad indices to the host.
@@ -85,6 +89,8 @@ int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* w
                    int64_t n, int x_dtype, hipStream_t st, W8Partials* out, bool w16 = false);
 // Grow-only device scratch for intermediates that must survive calls which use workspace().
 int layer_workspace(size_t bytes, void** ptr);
+// Grow-only device scratch for the split-K slabs of the tiled GEMM.
+int gemm_workspace(size_t bytes, void** ptr);
 // out = cast(sum_s(part0) * scale0 [-> SiLU(.) * (sum_s(part1) * scale1)] [+ residual]).
 int w8a16_finish(const W8Partials& parts, const float* scale0, const float* scale1, const void* residual,
                  int res_dtype, void* out, int out_dtype, bool out_blocked, int64_t m, int64_t n, hipStream_t st);

@@ -458,7 +458,7 @@ int launch_variant(GemmParams p, hipStream_t st) {
     p.splits = (p.k + p.k_per_split - 1) / p.k_per_split;
     if (p.splits > 1) {
       void* ws = nullptr;
-      const int rc = pto_hip::layer_workspace((size_t)p.splits * (DUAL ? 2 : 1) * p.m * p.n * sizeof(float), &ws);
+      const int rc = pto_hip::gemm_workspace((size_t)p.splits * (DUAL ? 2 : 1) * p.m * p.n * sizeof(float), &ws);
       if (rc) return rc;
       p.slabs = reinterpret_cast<float*>(ws);
     }

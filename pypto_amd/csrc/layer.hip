@@ -14,6 +14,65 @@
 
 #include "common.h"
 
+namespace {
+
+// The layer for more than 32 sequences with 16-bit weights: the same steps, each projection as a
+// tiled GEMM (k split while the tiles alone leave CUs idle), so that the weights are read once
+// for the whole batch instead of once per 32 sequences.  Activations are row-major.
+int layer_large_batch(const PtoHipDecoderLayerArgs* a, int rope_w, void* stream) {
+  using namespace pto_hip;
+  const int64_t b = a->batch, h = a->hidden, hq = a->num_heads, hkv = a->kv_head_num, d = a->head_dim,
+                inter = a->intermediate;
+  const int dt = a->dtype;
+  const bool fp8kv = a->kv_dtype == PTO_HIP_FP8E4M3FN;
+  const int64_t qkv_n = (hq + 2 * hkv) * d;
+  auto up = [](size_t n) { return (n + 255) / 256 * 256; };
+  const size_t sz_normed = up((size_t)b * h * 2), sz_qkv = up((size_t)b * qkv_n * 4),
+               sz_q = up((size_t)b * hq * d * 2), sz_attn = up((size_t)b * hq * d * 4),
+               sz_attn16 = up((size_t)b * hq * d * 2), sz_resid = up((size_t)b * h * 4),
+               sz_h = up((size_t)b * inter * 2);
+  void* lws = nullptr;
+  int rc = layer_workspace(sz_normed + sz_qkv + sz_q + sz_attn + sz_attn16 + sz_resid + sz_normed + sz_h, &lws);
+  if (rc) return rc;
+  char* w = reinterpret_cast<char*>(lws);
+  void* normed = w;              w += sz_normed;
+  float* qkv = (float*)w;        w += sz_qkv;
+  void* q16 = w;                 w += sz_q;
+  float* attn = (float*)w;       w += sz_attn;
+  void* attn16 = w;              w += sz_attn16;
+  float* resid1 = (float*)w;     w += sz_resid;
+  void* normed2 = w;             w += sz_normed;
+  void* hbuf = w;
+
+  if ((rc = pto_hip_rms_norm(a->hidden_states, a->gamma_in, normed, b, h, a->eps, dt, dt, stream))) return rc;
+  if ((rc = pto_hip_projection(normed, a->wqkv_q, nullptr, qkv, b, h, qkv_n, dt, 0, PTO_HIP_FP32, stream))) return rc;
+  const int64_t pool_blocks = a->pool_rows / (hkv * a->block_size);
+  if (fp8kv)
+    rc = rope_kv_cache_update_fp8(qkv, nullptr, 1, 0, a->seq_lens, a->rope_cos, a->rope_sin, a->block_table,
+                                  a->key_cache, a->value_cache, a->k_scale, a->v_scale, q16, b, hq, hkv, d,
+                                  a->block_size, a->max_num_blocks_per_req, a->max_pos, rope_w, pool_blocks, dt, stream);
+  else
+    rc = rope_kv_cache_update(qkv, nullptr, 1, 0, a->seq_lens, a->rope_cos, a->rope_sin, a->block_table, a->key_cache,
+                              a->value_cache, q16, b, hq, hkv, d, a->block_size, a->max_num_blocks_per_req, a->max_pos,
+                              rope_w, a->pool_rows, dt, stream);
+  if (rc) return rc;
+  float scale = 1.0f / sqrtf((float)d);
+  uint32_t scale_bits;
+  __builtin_memcpy(&scale_bits, &scale, 4);
+  const int64_t cfg[7] = {b, hq, hkv, d, a->block_size, a->max_num_blocks_per_req, (int64_t)scale_bits};
+  if ((rc = paged_attention(q16, a->key_cache, a->value_cache, a->block_table, a->seq_lens, attn, attn16, false, nullptr,
+                            cfg, dt, fp8kv ? PTO_HIP_FP8E4M3FN : dt, fp8kv ? a->k_scale : nullptr,
+                            fp8kv ? a->v_scale : nullptr, pool_blocks, stream)))
+    return rc;
+  if ((rc = pto_hip_projection(attn16, a->wo_q, a->hidden_states, resid1, b, hq * d, h, dt, dt, PTO_HIP_FP32, stream)))
+    return rc;
+  if ((rc = pto_hip_rms_norm(resid1, a->gamma_post, normed2, b, h, a->eps, PTO_HIP_FP32, dt, stream))) return rc;
+  if ((rc = pto_hip_gate_up_swiglu(normed2, a->wg_q, a->wu_q, hbuf, b, h, inter, dt, stream))) return rc;
+  return pto_hip_projection(hbuf, a->wd_q, resid1, a->out, b, inter, h, dt, PTO_HIP_FP32, dt, stream);
+}
+
+}  // namespace
+
 extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, void* stream) {
   using namespace pto_hip;
   Context& cx = ctx();
@@ -23,26 +82,6 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
                 inter = a->intermediate;
   PTO_CHECK_ARG(b >= 0 && b < (1 << 20), "decoder_layer_decode: batch %lld out of range", (long long)b);
   if (b == 0) return PTO_HIP_OK;
-  if (b > kW8MaxM) {
-    // The projections hold 32 rows per pass: larger batches run as consecutive groups of 32
-    // sequences in stream order (each group's rows of the block table, lengths and activations;
-    // the caches and weights are shared).
-    PTO_CHECK_ARG(a->hidden_states && a->out && a->seq_lens && a->block_table,
-                  "decoder_layer_decode: null tensor pointer");
-    PTO_CHECK_ARG(a->dtype == PTO_HIP_BF16 || a->dtype == PTO_HIP_FP16,
-                  "decoder_layer_decode: activation dtype %s not in {BF16, FP16}", dtype_name(a->dtype));
-    for (int64_t b0 = 0; b0 < b; b0 += kW8MaxM) {
-      PtoHipDecoderLayerArgs part = *a;
-      part.batch = std::min<int64_t>(kW8MaxM, b - b0);
-      part.hidden_states = reinterpret_cast<const char*>(a->hidden_states) + (size_t)b0 * h * 2;
-      part.out = reinterpret_cast<char*>(a->out) + (size_t)b0 * h * 2;
-      part.seq_lens = a->seq_lens + b0;
-      part.block_table = a->block_table + b0 * a->max_num_blocks_per_req;
-      const int rc = pto_hip_decoder_layer_decode(&part, stream);
-      if (rc) return rc;
-    }
-    return PTO_HIP_OK;
-  }
   PTO_CHECK_ARG(h > 0 && hq > 0 && hkv > 0 && d > 0 && inter > 0 && hq % hkv == 0,
                 "decoder_layer_decode: bad model dimensions");
   PTO_CHECK_ARG(a->dtype == PTO_HIP_BF16 || a->dtype == PTO_HIP_FP16,
@@ -74,6 +113,23 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
   PTO_CHECK_ARG(n_scales == 0 || n_scales == 5,
                 "decoder_layer_decode: weight scales must be given for all five projections or for none");
   const bool w16 = n_scales == 0;
+  if (b > kW8MaxM && w16) return layer_large_batch(a, rope_w, stream);
+  if (b > kW8MaxM) {
+    // The int8 projections hold 32 rows per pass: larger batches run as consecutive groups of 32
+    // sequences in stream order (each group's rows of the block table, lengths and activations;
+    // the caches and weights are shared).
+    for (int64_t b0 = 0; b0 < b; b0 += kW8MaxM) {
+      PtoHipDecoderLayerArgs part = *a;
+      part.batch = std::min<int64_t>(kW8MaxM, b - b0);
+      part.hidden_states = reinterpret_cast<const char*>(a->hidden_states) + (size_t)b0 * h * 2;
+      part.out = reinterpret_cast<char*>(a->out) + (size_t)b0 * h * 2;
+      part.seq_lens = a->seq_lens + b0;
+      part.block_table = a->block_table + b0 * a->max_num_blocks_per_req;
+      const int rc = pto_hip_decoder_layer_decode(&part, stream);
+      if (rc) return rc;
+    }
+    return PTO_HIP_OK;
+  }
   hipStream_t st = (hipStream_t)stream;
   const int dt = a->dtype;
   const int64_t qkv_n = (hq + 2 * hkv) * d;

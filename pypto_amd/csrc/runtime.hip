@@ -66,6 +66,13 @@ int layer_workspace(size_t bytes, void** ptr) {
   return rc;
 }
 
+int gemm_workspace(size_t bytes, void** ptr) {
+  Context& c = ctx();
+  const int rc = grow_scratch(&c.gemm_ws, &c.gemm_ws_bytes, bytes);
+  *ptr = c.gemm_ws;
+  return rc;
+}
+
 namespace {
 
 enum ProgramKind {
@@ -612,6 +619,9 @@ int pto_hip_close(void) {
   if (c.layer_ws) PTO_CHECK_HIP(hipFree(c.layer_ws));
   c.layer_ws = nullptr;
   c.layer_ws_bytes = 0;
+  if (c.gemm_ws) PTO_CHECK_HIP(hipFree(c.gemm_ws));
+  c.gemm_ws = nullptr;
+  c.gemm_ws_bytes = 0;
   for (void* old : c.retired) PTO_CHECK_HIP(hipFree(old));
   c.retired.clear();
   c.initialized = false;
