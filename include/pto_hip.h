@@ -336,6 +336,9 @@ PTO_HIP_API int pto_hip_select_program(const char* orchestration_name, const Pto
  *                               4 = 8 wavefronts, 256-row tile, k split when CUs would idle,
  *                               5 = 8 wavefronts, 128-row tile
  *  "w8a16_wgs_per_cu"           workgroups per CU the W8A16 k split aims at (default 1)
+ *  "w8a16_wide"                 1 = int8 codes of large matrices (>= 150 MB) are read 16 per lane
+ *                               (default), 0 = always 8 per lane, 2 = 16 per lane whenever the
+ *                               channel count is a multiple of 16
  *  "w8a16_min_steps"            fewest 32-row steps per wavefront before k is split further
  *                               (default 8)
  */

@@ -804,6 +804,9 @@ int pto_hip_set_option(const char* name, int64_t value) {
   } else if (!std::strcmp(name, "w8a16_wgs_per_cu")) {
     PTO_CHECK_ARG(value >= 1 && value <= 16, "w8a16_wgs_per_cu must be in [1, 16]");
     c.w8a16_wgs_per_cu = value;
+  } else if (!std::strcmp(name, "w8a16_wide")) {
+    PTO_CHECK_ARG(value >= 0 && value <= 2, "w8a16_wide must be 0, 1 or 2");
+    c.w8a16_wide = value;
   } else if (!std::strcmp(name, "w8a16_min_steps")) {
     PTO_CHECK_ARG(value >= 1 && value <= 1024, "w8a16_min_steps must be in [1, 1024]");
     c.w8a16_min_steps = value;
@@ -824,6 +827,7 @@ int pto_hip_get_option(const char* name, int64_t* value) {
   else if (!std::strcmp(name, "attn_group_tiles")) *value = c.attn_group_tiles;
   else if (!std::strcmp(name, "w8a16_wgs_per_cu")) *value = c.w8a16_wgs_per_cu;
   else if (!std::strcmp(name, "w8a16_min_steps")) *value = c.w8a16_min_steps;
+  else if (!std::strcmp(name, "w8a16_wide")) *value = c.w8a16_wide;
   else return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
   return PTO_HIP_OK;
 }

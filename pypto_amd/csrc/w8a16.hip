@@ -30,7 +30,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
 
-constexpr int kSlab = pto_hip::kW8Slab;  // output channels per workgroup
+constexpr int kSlab = pto_hip::kW8Slab;  // output channels per workgroup (8 per lane); twice that with 16 per lane
 constexpr int kStep = 32;                // k rows per step
 constexpr int kMaxM = pto_hip::kW8MaxM;
 constexpr int kWavesPerWg = 4;           // wavefronts per workgroup of the partial kernel
@@ -66,21 +66,28 @@ __device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
   }
 }
 
-// W8: int8 weight codes (8 bytes = 8 channels per row and lane); otherwise 16-bit weights of the
-// activation type (16 bytes = 8 channels).
-template <bool W8>
+typedef uint32_t u32x2 __attribute__((__vector_size__(2 * sizeof(uint32_t))));
+
+// One register stage of a lane: kCols channels of the k rows kg*8 .. kg*8+7, and the activations.
+// W8: int8 weight codes, 8 bytes (kCols 8) or 16 bytes (kCols 16) per row and lane; otherwise
+// 16-bit weights of the activation type (16 bytes = 8 channels).  A lane load of 16 bytes moves
+// twice the weights per request; the int8 form with 8-byte loads is kept for channel counts that
+// are not a multiple of 16.
+template <bool W8, int kCols>
 struct Stage {
-  typename std::conditional<W8, uint2, u32x4>::type w[8];  // 8 channels of k rows kg*8 .. kg*8+7
-  u32x4 xa[2];                                             // activations of rows c and c+16, k = kg*8 .. +8
+  typename std::conditional<(W8 && kCols == 8), u32x2, u32x4>::type w[8];
+  u32x4 xa[2];  // activations of rows c and c+16, k = kg*8 .. +8
 };
 
 // kWaves wavefronts per workgroup, kStages register stages per wavefront (kStages - 1 in flight),
 // kOcc wavefronts per SIMD the register budget is cut for.
-template <bool BF16, bool W8, int kWaves, int kStages, int kOcc>
+template <bool BF16, bool W8, int kCols, int kWaves, int kStages, int kOcc>
 __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOcc, kOcc))) void w8a16_partial_kernel(
     GemvParams p) {
+  static_assert(kCols == 8 || (W8 && kCols == 16), "16 channels per lane only with int8 codes");
   constexpr int kHalf = kWaves / 2;
-  __shared__ float red[kHalf * kMaxM * kSlab];  // 16 KiB per wavefront of the lower half
+  constexpr int kSlab = 16 * kCols;  // output channels per workgroup: 16 lanes of kCols channels
+  __shared__ float red[kHalf * kMaxM * kSlab];  // 16 or 32 KiB per wavefront of the lower half
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: row addresses stay scalar
   const int c = lane & 15, kg = lane >> 4;
@@ -92,7 +99,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
   const int k_end = min(p.k, k_begin + p.k_per_split);
   const int n_steps = (k_end - k_begin + kStep - 1) / kStep;
 
-  const int n0 = slab * kSlab + c * 8;
+  const int n0 = slab * kSlab + c * kCols;
   // Row-major x: lane (c, kg) reads 16 bytes of rows c and c+16 at k = kstep + 8*kg.  Blocked x
   // keeps the 32 rows of each 8-k group together, so the same two reads of a wavefront cover 2 KB
   // of consecutive bytes instead of 32 half cache lines.
@@ -103,9 +110,9 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
                                     : p.x + (size_t)min(c + 16, p.m - 1) * p.k + kg * 8;
   const bool m0_ok = c < p.m, m1_ok = c + 16 < p.m;
 
-  f32x4 acc[8][2];
+  f32x4 acc[kCols][2];
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+  for (int i = 0; i < kCols; ++i)
 #pragma unroll
     for (int h = 0; h < 2; ++h) acc[i][h] = f32x4{0.f, 0.f, 0.f, 0.f};
 
@@ -116,11 +123,11 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
   // per-lane offset that never changes.
   const int last_step = wave < n_steps ? wave + (n_steps - 1 - wave) / kWaves * kWaves : n_steps - 1;
   constexpr int kWBytes = W8 ? 1 : 2;  // bytes per weight
-  typedef typename std::conditional<W8, uint2, u32x4>::type wvec_t;
+  typedef typename std::conditional<(W8 && kCols == 8), u32x2, u32x4>::type wvec_t;
   const char* wbase = reinterpret_cast<const char*>(p.wq[mat]);
-  const uint32_t lane_off = (uint32_t)min(n0, p.n - 8) + (uint32_t)(kg * 8) * (uint32_t)p.n;
+  const uint32_t lane_off = (uint32_t)min(n0, p.n - kCols) + (uint32_t)(kg * 8) * (uint32_t)p.n;
   auto step_row = [&](int step) { return min(k_begin + step * kStep, p.k - kStep); };
-  auto load = [&](Stage<W8>& s, int step) {
+  auto load = [&](Stage<W8, kCols>& s, int step) {
     const int kstep = step_row(min(step, last_step));
     s.xa[0] = *reinterpret_cast<const u32x4*>(xp0 + (size_t)kstep * x_step);
     s.xa[1] = *reinterpret_cast<const u32x4*>(xp1 + (size_t)kstep * x_step);
@@ -130,21 +137,21 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
       s.w[e] = *reinterpret_cast<const wvec_t*>(row + (size_t)lane_off * kWBytes);
     }
   };
-  auto compute = [&](const Stage<W8>& s, int step) {
+  auto compute = [&](const Stage<W8, kCols>& s, int step) {
     const int row0 = step_row(step) + kg * 8;  // first of this lane's 8 rows
     const bool k_ok = row0 >= k_begin + step * kStep && row0 < k_end;
     const u32x4 z = {0u, 0u, 0u, 0u};
     const u32x4 a0 = (k_ok && m0_ok) ? s.xa[0] : z;
     const u32x4 a1 = (k_ok && m1_ok) ? s.xa[1] : z;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kCols; ++i) {
       // channel n0 + i: its 8 k-values, as packed pairs (k, k+1)
       u32x4 b;
       if constexpr (W8) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const uint32_t w0 = i < 4 ? s.w[2 * q].x : s.w[2 * q].y;
-          const uint32_t w1 = i < 4 ? s.w[2 * q + 1].x : s.w[2 * q + 1].y;
+          const uint32_t w0 = s.w[2 * q][i >> 2];
+          const uint32_t w1 = s.w[2 * q + 1][i >> 2];
           const float f0 = (float)(int8_t)(w0 >> ((i & 3) * 8));
           const float f1 = (float)(int8_t)(w1 >> ((i & 3) * 8));
           b[q] = pack_pair<BF16>(f0, f1);
@@ -164,7 +171,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
   // Wavefront w takes steps w, w + kWaves, ...; kStages register stages, all but the one being
   // consumed in flight.  The trip count is rounded up to whole rounds of kStages: surplus steps
   // multiply by zero.
-  Stage<W8> st[kStages];
+  Stage<W8, kCols> st[kStages];
 #pragma unroll
   for (int u = 0; u < kStages - 1; ++u) load(st[u], wave + u * kWaves);
   for (int s = wave; s < n_steps; s += kStages * kWaves) {
@@ -180,7 +187,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
   if (wave >= kHalf) {
     float* dst = red + (wave - kHalf) * (kMaxM * kSlab) + lane;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < kCols; ++i)
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -190,7 +197,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
   if (wave < kHalf) {
     const float* src = red + wave * (kMaxM * kSlab) + lane;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < kCols; ++i)
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -204,19 +211,20 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int m = h * 16 + 4 * kg + r;
-        float4 lo = {acc[0][h][r], acc[1][h][r], acc[2][h][r], acc[3][h][r]};
-        float4 hi = {acc[4][h][r], acc[5][h][r], acc[6][h][r], acc[7][h][r]};
-        float4* d4 = reinterpret_cast<float4*>(dst + m * kSlab + c * 8);
-        d4[0] = lo;
-        d4[1] = hi;
+        float4* d4 = reinterpret_cast<float4*>(dst + m * kSlab + c * kCols);
+#pragma unroll
+        for (int v = 0; v < kCols / 4; ++v)
+          d4[v] = float4{acc[4 * v][h][r], acc[4 * v + 1][h][r], acc[4 * v + 2][h][r], acc[4 * v + 3][h][r]};
       }
   }
   __syncthreads();
-  // thread t sums float4 chunk (t % 32) of rows t/32, t/32 + 8, ... over the remaining slices
-  constexpr int kRowsPerPass = kWaves * 64 / 32;
+  // thread t sums one float4 chunk of rows t / chunks, t / chunks + rows per pass, ... over the
+  // remaining slices (chunks = float4s per slab row)
+  constexpr int kChunks = kSlab / 4;
+  constexpr int kRowsPerPass = kWaves * 64 / kChunks;
 #pragma unroll
-  for (int m = tid >> 5; m < kMaxM; m += kRowsPerPass) {
-    const int ch = (tid & 31) * 4;
+  for (int m = tid / kChunks; m < kMaxM; m += kRowsPerPass) {
+    const int ch = (tid % kChunks) * 4;
     float4 a = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int w = 0; w < kHalf; ++w) {
@@ -426,7 +434,14 @@ int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* w
   p.m = (int)m;
   p.k = (int)k;
   p.n = (int)n;
-  p.slabs = (int)((n + kSlab - 1) / kSlab);
+  // int8 codes are read 16 per lane (a 256-channel slab per workgroup, half the requests per byte)
+  // for large matrices when rows and base addresses allow 16-byte loads, else 8 per lane like the
+  // 16-bit weights.  Measured: 235 MB of codes 3.6 -> 4.5 TB/s, 525 MB 4.2 -> 4.8 TB/s; but 59 MB
+  // 3.8 -> 3.2 TB/s (half the slabs, so twice the k splits and fewer wavefronts), hence the size bound.
+  const bool wide = !w16 && ctx().w8a16_wide != 0 && n % 16 == 0 && ((uintptr_t)wq0 | (uintptr_t)wq1) % 16 == 0 &&
+                    (ctx().w8a16_wide == 2 || k * n * (wq1 ? 2 : 1) >= (int64_t)150 * 1000 * 1000);
+  const int slab_cols = wide ? 2 * kSlab : kSlab;
+  p.slabs = (int)((n + slab_cols - 1) / slab_cols);
   p.n_mats = wq1 ? 2 : 1;
   p.x_blocked = x_blocked ? 1 : 0;
   choose_splits(k, (int64_t)p.slabs * p.n_mats, n * p.n_mats, kWavesPerWg, &p.splits, &p.k_per_split);
@@ -442,11 +457,14 @@ int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* w
   const dim3 block((unsigned)kWavesPerWg * 64);
   const bool bf = x_dtype == PTO_HIP_BF16;
   if (w16) {  // twice the bytes per stage: three wavefronts per SIMD
-    if (bf) hipLaunchKernelGGL((w8a16_partial_kernel<true, false, kWavesPerWg, 2, 3>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((w8a16_partial_kernel<false, false, kWavesPerWg, 2, 3>), grid, block, 0, st, p);
+    if (bf) hipLaunchKernelGGL((w8a16_partial_kernel<true, false, 8, kWavesPerWg, 2, 3>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((w8a16_partial_kernel<false, false, 8, kWavesPerWg, 2, 3>), grid, block, 0, st, p);
+  } else if (wide) {  // 32 accumulators per lane: two wavefronts per SIMD
+    if (bf) hipLaunchKernelGGL((w8a16_partial_kernel<true, true, 16, kWavesPerWg, 2, 2>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((w8a16_partial_kernel<false, true, 16, kWavesPerWg, 2, 2>), grid, block, 0, st, p);
   } else {
-    if (bf) hipLaunchKernelGGL((w8a16_partial_kernel<true, true, kWavesPerWg, 2, 4>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((w8a16_partial_kernel<false, true, kWavesPerWg, 2, 4>), grid, block, 0, st, p);
+    if (bf) hipLaunchKernelGGL((w8a16_partial_kernel<true, true, 8, kWavesPerWg, 2, 4>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((w8a16_partial_kernel<false, true, 8, kWavesPerWg, 2, 4>), grid, block, 0, st, p);
   }
   PTO_CHECK_HIP(hipGetLastError());
   out->part[0] = p.part[0];

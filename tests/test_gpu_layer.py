@@ -51,6 +51,36 @@ def test_w8a16_swiglu(worker):
     validate_golden({"out": out.float()}, {"out": ref.float()}, rtol=1e-2, atol=1e-3)
 
 
+@pytest.mark.parametrize("m,k,n", [(32, 512, 1024), (16, 1056, 272), (5, 4096, 2064), (32, 2048, 1000)])
+def test_w8a16_codes_read_16_per_lane(worker, m, k, n):
+    """Large int8 matrices are read with 16-byte lane loads (256-channel slabs); forced here at small
+    sizes.  A channel count that is not a multiple of 16 keeps the 8-byte form.  Same sums, same
+    order within a wavefront: the two forms agree to fp32 rounding."""
+    g = torch.Generator().manual_seed(n)
+    x = (torch.randn(m, k, generator=g) * 0.5).to(torch.bfloat16)
+    wq = torch.randint(-127, 128, (k, n), generator=g, dtype=torch.int8)
+    wu = torch.randint(-127, 128, (k, n), generator=g, dtype=torch.int8)
+    s1 = torch.rand(n, generator=g) * 0.01 + 0.001
+    s2 = torch.rand(n, generator=g) * 0.01 + 0.001
+    outs = []
+    for wide in (2, 0):
+        worker.set_option("w8a16_wide", wide)
+        try:
+            out = torch.zeros(m, n)
+            with worker.register(w8a16_matmul) as h:
+                h(x, wq, s1, out)
+            out2 = torch.zeros(m, n, dtype=torch.bfloat16)
+            with worker.register(w8a16_swiglu) as h:
+                h(x, wq, s1, wu, s2, out2)
+        finally:
+            worker.set_option("w8a16_wide", 1)
+        validate_golden({"out": out}, {"out": oracle.w8a16_matmul(x, wq, s1)}, rtol=1e-3, atol=1e-3)
+        ref2 = oracle.swiglu(oracle.w8a16_matmul(x, wq, s1), oracle.w8a16_matmul(x, wu, s2)).to(torch.bfloat16)
+        validate_golden({"out": out2.float()}, {"out": ref2.float()}, rtol=1e-2, atol=1e-3)
+        outs.append(out)
+    assert torch.allclose(outs[0], outs[1], rtol=1e-5, atol=1e-4)
+
+
 def test_w8a16_argument_rules(worker):
     wq = torch.zeros(40, 64, dtype=torch.int8)
     s = torch.ones(64)
