@@ -216,8 +216,10 @@ PTO_HIP_API int pto_hip_gate_up_swiglu(const void* x, const void* w_gate, const 
 /* W8A16 decode projection (no counterpart in the reference, which has no quantised weights; the
  * contract is its projection kernel's, examples/models/qwen3_jit/kernels/projection.py:145-177,
  * x @ W with W [in, out]):  out[M, N] = (x[M,K] @ w_q[K,N]) * w_scale[N] (+ residual[M,N]).
- * x is BF16/FP16, w_q INT8, accumulation fp32; residual may be NULL.  Built for decode: the
- * weights stream from HBM once per 32 rows of x, so M beyond a few dozen rows belongs to a GEMM. */
+ * x is BF16/FP16, w_q INT8, accumulation fp32; residual may be NULL.  Up to 32 rows the weights
+ * stream from HBM once through skinny kernels (decode); more rows run as one MFMA-tiled GEMM that
+ * widens the codes inside the kernel (N a multiple of 16, 16-byte aligned tensors, out FP32 or the
+ * type of x), and otherwise as consecutive 32-row passes. */
 PTO_HIP_API int pto_hip_w8a16_matmul(const void* x, const void* w_q, const float* w_scale,
                                      const void* residual, void* out, int64_t m, int64_t k, int64_t n,
                                      int x_dtype, int res_dtype, int out_dtype, void* stream);
@@ -341,6 +343,9 @@ PTO_HIP_API int pto_hip_select_program(const char* orchestration_name, const Pto
  *                               channel count is a multiple of 16
  *  "w8a16_min_steps"            fewest 32-row steps per wavefront before k is split further
  *                               (default 8)
+ *  "w8a16_gemm_rows"            rows from which the int8 projections run as one tiled GEMM (codes
+ *                               widened inside the kernel, weights read once) instead of 32-row
+ *                               passes (default 33; 0 = never)
  */
 PTO_HIP_API int pto_hip_set_option(const char* name, int64_t value);
 PTO_HIP_API int pto_hip_get_option(const char* name, int64_t* value);

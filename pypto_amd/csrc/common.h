@@ -63,6 +63,7 @@ struct Context {
   int64_t w8a16_wgs_per_cu = 1;  // workgroups of the W8A16 partial kernel aimed at per compute unit
   int64_t w8a16_wide = 1;        // int8 codes read 16 per lane: 0 never, 1 for large matrices, 2 whenever shapes allow
   int64_t w8a16_min_steps = 8;   // fewest 32-row steps per wavefront before k is split further
+  int64_t w8a16_gemm_rows = 33;  // rows from which int8 projections run as a tiled GEMM (0 = never)
 };
 
 Context& ctx();
@@ -97,6 +98,15 @@ int w8a16_finish(const W8Partials& parts, const float* scale0, const float* scal
                  int res_dtype, void* out, int out_dtype, bool out_blocked, int64_t m, int64_t n, hipStream_t st);
 // sum_out = sum_s(part) * scale + residual (fp32); normed_out = cast(RMSNorm(sum_out) * gamma).
 bool w8a16_finish_norm_fits(int64_t n);
+// The tiled GEMM with int8 weight codes (widened on their way into LDS, scales applied to the
+// accumulators): out = (x @ codes0) * scale0 (+ residual), or with codes1 / scale1 given
+// SiLU((x @ codes0) * scale0) * ((x @ codes1) * scale1).  gemm_w8_fits says whether the shapes,
+// types and addresses allow it; callers fall back to 32-row passes otherwise.
+bool gemm_w8_fits(const void* x, const void* wq0, const void* wq1, const void* residual, const void* out, int64_t m,
+                  int64_t k, int64_t n, int x_dtype, int out_dtype);
+int gemm_w8(const void* x, const void* wq0, const float* scale0, const void* wq1, const float* scale1,
+            const void* residual, int res_dtype, void* out, int64_t m, int64_t k, int64_t n, int x_dtype,
+            int out_dtype, hipStream_t st);
 int w8a16_finish_norm(const W8Partials& parts, const float* scale, const void* residual, int res_dtype,
                       float* sum_out, const float* gamma, void* normed_out, int out_dtype, bool out_blocked,
                       int64_t m, int64_t n, float eps, hipStream_t st);

@@ -56,6 +56,8 @@ struct GemmParams {
   float* slabs;             // [splits][DUAL ? 2 : 1][m][n] when splits > 1
   const void* residual;     // optional [m, n] added to the product (single-operand pass only)
   int res_dtype;
+  const float* scale0;      // int8 weight codes: one scale per output column of b0 (and b1); else null
+  const float* scale1;
 };
 
 __device__ __forceinline__ float load_residual(const void* r, int dt, int64_t i) {
@@ -81,6 +83,16 @@ __device__ __forceinline__ void store_out(OutT* p, float v) { *p = (OutT)v; }
 // Sigmoid in the device form of the reference, recip(1 + exp(-g)) (01_ffn.py:70-74).
 __device__ __forceinline__ float silu(float g) { return g * __frcp_rn(1.f + __expf(-g)); }
 
+// Two small integers held as fp32 -> packed pair of 16-bit floats, exact (|value| <= 128 has at most
+// 8 significant bits: the upper half of the fp32 pattern is its bf16).
+template <bool BF16>
+__device__ __forceinline__ uint32_t widen_pair(float lo, float hi) {
+  if constexpr (BF16)
+    return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo), 0x07060302u);
+  else
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+}
+
 // Workgroup id -> tile id such that ids congruent mod 8 (one XCD) get a contiguous tile range.
 __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
   const int x = pid % kXcds, local = pid / kXcds;
@@ -96,14 +108,18 @@ __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
 // as MT x NT accumulators, NT = 8 / WN.  2 x 2 wavefronts with 4 x 4 accumulators run one
 // wavefront per SIMD; 2 x 4 wavefronts with 4 x 2 accumulators run two per SIMD, so the MFMA pipe
 // has a second instruction stream to draw from while one waits on memory or a barrier.
-template <int MT, int WM, int WN, bool DUAL, bool BF16, int EDGE, typename OutT>
+// W8: B holds int8 codes (a 16-byte chunk is 16 columns); they are widened to the activation type,
+// exactly, on their way into LDS, and the per-column scales are applied to the accumulators.
+template <int MT, int WM, int WN, bool DUAL, bool BF16, int EDGE, typename OutT, bool W8>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   constexpr int NBUF = 2;
   constexpr int NT = (BN / 32) / WN;        // B fragments (32 columns each) per wavefront
   constexpr int T = 64 * WM * WN;           // threads
   constexpr int BM = 32 * MT * WM;
   constexpr int NA = BM * 8 / T;            // 16-byte A chunks per thread and tile
-  constexpr int NB = BK * 32 / T;           // 16-byte B chunks per thread and tile
+  constexpr int BCH = W8 ? 16 : 32;         // 16-byte B chunks per k row of the tile
+  constexpr int BCOLS = BN / BCH;           // columns per chunk: 8, or 16 int8 codes
+  constexpr int NB = BK * BCH / T;          // 16-byte B chunks per thread and tile
   static_assert(NT >= 1 && (!DUAL || NT % 2 == 0), "gate/up pass needs gate and up columns in every wavefront");
   constexpr int A_ELEMS = BM * LDK;
   constexpr int B_ELEMS = BK * LDN;
@@ -129,17 +145,18 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   const int a_chunk = tid & 7, a_row = tid >> 3;
   // B: thread owns 16-byte chunk (tid % 32) of k rows tid/32 + (T/32)*i; in the gate/up pass chunks
   // 0..15 come from the gate weights and 16..31 from the up weights (same output columns).
-  const int b_chunk = tid & 31, b_row = tid >> 5;
+  const int b_chunk = tid % BCH, b_row = tid / BCH;
   const uint16_t* bsrc;
   int b_col;  // global column of the chunk
   if (DUAL) {
-    bsrc = (b_chunk < 16) ? p.b0 : p.b1;
-    b_col = n0 + (b_chunk & 15) * 8;
+    bsrc = (b_chunk < BCH / 2) ? p.b0 : p.b1;
+    b_col = n0 + (b_chunk % (BCH / 2)) * BCOLS;
   } else {
     bsrc = p.b0;
-    b_col = n0 + b_chunk * 8;
+    b_col = n0 + b_chunk * BCOLS;
   }
-  if (EDGE == 2) b_col = min(b_col, p.n - 8);
+  if (EDGE == 2) b_col = min(b_col, p.n - BCOLS);
+  constexpr int BESZ = W8 ? 1 : 2;  // bytes per B element
   const uint16_t* a_ptr[NA];
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
@@ -147,7 +164,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
     if (EDGE != 0) r = min(r, p.m - 1);
     a_ptr[i] = p.a + (int64_t)r * p.lda + k_begin + a_chunk * 8;
   }
-  const uint16_t* b_ptr = bsrc + (int64_t)(k_begin + b_row) * p.ldb + b_col;
+  const char* b_ptr = reinterpret_cast<const char*>(bsrc) + ((int64_t)(k_begin + b_row) * p.ldb + b_col) * BESZ;
 
   u32x4 ra[NA];
   u32x4 rb[NB];
@@ -164,10 +181,36 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   };
   auto load_b = [&](int k0, int i) {
     if constexpr (EDGE == 2) {
-      const int kk = min(k0 + b_row + (T / 32) * i, klen - 1) - b_row;
-      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)kk * p.ldb);
+      const int kk = min(k0 + b_row + (T / BCH) * i, klen - 1) - b_row;
+      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)kk * p.ldb * BESZ);
     } else {
-      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)(k0 + (T / 32) * i) * p.ldb);
+      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)(k0 + (T / BCH) * i) * p.ldb * BESZ);
+    }
+  };
+  // One B chunk from its registers into the LDS tile `db`: 16-bit weights as they are, int8 codes
+  // widened (16 codes -> two 16-byte writes).
+  auto store_b = [&](uint16_t* db, int i) {
+    uint16_t* dst = db + (b_row + (T / BCH) * i) * LDN + b_chunk * BCOLS;
+    if constexpr (W8) {
+      u32x4 lo, hi;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const uint32_t codes = rb[i][w];
+        const float f0 = (float)(int8_t)(codes), f1 = (float)(int8_t)(codes >> 8);
+        const float f2 = (float)(int8_t)(codes >> 16), f3 = (float)(int8_t)(codes >> 24);
+        const uint32_t p01 = widen_pair<BF16>(f0, f1), p23 = widen_pair<BF16>(f2, f3);
+        if (w < 2) {
+          lo[2 * w] = p01;
+          lo[2 * w + 1] = p23;
+        } else {
+          hi[2 * (w - 2)] = p01;
+          hi[2 * (w - 2) + 1] = p23;
+        }
+      }
+      *reinterpret_cast<u32x4*>(dst) = lo;
+      *reinterpret_cast<u32x4*>(dst + 8) = hi;
+    } else {
+      *reinterpret_cast<u32x4*>(dst) = rb[i];
     }
   };
   auto load_tile = [&](int k0) {
@@ -183,8 +226,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
       *reinterpret_cast<u32x4*>(da + (a_row + (T / 8) * i) * LDK + a_chunk * 8) = ra[i];
     uint16_t* db = sb + buf * B_ELEMS;
 #pragma unroll
-    for (int i = 0; i < NB; ++i)
-      *reinterpret_cast<u32x4*>(db + (b_row + (T / 32) * i) * LDN + b_chunk * 8) = rb[i];
+    for (int i = 0; i < NB; ++i) store_b(db, i);
   };
 
   f32x16 acc[MT][NT];
@@ -264,8 +306,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
         }
         if (ks == 0 && q < NA)
           *reinterpret_cast<u32x4*>(da + (a_row + (T / 8) * q) * LDK + a_chunk * 8) = ra[q];
-        if (ks == 1 && q < NB)
-          *reinterpret_cast<u32x4*>(db + (b_row + (T / 32) * q) * LDN + b_chunk * 8) = rb[q];
+        if (ks == 1 && q < NB) store_b(db, q);
         if (ks == 2 && q < NA) load_a(k_next, q);
         if (ks == 3 && q < NB) load_b(k_next, q);
         __builtin_amdgcn_sched_barrier(0);
@@ -280,6 +321,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   // acc[i][jn][r]: row = m0 + wm*MT*32 + i*32 + (r/4)*8 + (lane/32)*4 + r%4, col = lane%32 + ...
   OutT* c = reinterpret_cast<OutT*>(p.c);
   const int row_base = m0 + wm * MT * 32 + (lane >> 5) * 4;
+  float sc[NT];  // int8 weight codes: the scale of each of this lane's columns
+  if constexpr (W8) {
+#pragma unroll
+    for (int jn = 0; jn < NT; ++jn) {
+      const int col = DUAL ? n0 + wn * (16 * NT) + (jn % (NT / 2)) * 32 + (lane & 31)
+                           : n0 + wn * (32 * NT) + jn * 32 + (lane & 31);
+      const float* s = (DUAL && jn >= NT / 2) ? p.scale1 : p.scale0;
+      sc[jn] = col < p.n ? s[col] : 0.f;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
 #pragma unroll
@@ -297,7 +348,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
               s[0] = acc[i][jn][r];
               s[mn] = acc[i][jn + NT / 2][r];
             } else {
-              store_out<OutT>(c + (int64_t)row * p.ldc + col, silu(acc[i][jn][r]) * acc[i][jn + NT / 2][r]);
+              float g = acc[i][jn][r], u = acc[i][jn + NT / 2][r];
+              if constexpr (W8) {
+                g *= sc[jn];
+                u *= sc[jn + NT / 2];
+              }
+              store_out<OutT>(c + (int64_t)row * p.ldc + col, silu(g) * u);
             }
           }
         }
@@ -310,6 +366,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
               p.slabs[(int64_t)split * mn + (int64_t)row * p.n + col] = acc[i][jn][r];
             } else {
               float v = acc[i][jn][r];
+              if constexpr (W8) v *= sc[jn];
               if (p.residual) v += load_residual(p.residual, p.res_dtype, (int64_t)row * p.n + col);
               store_out<OutT>(c + (int64_t)row * p.ldc + col, v);
             }
@@ -321,7 +378,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
 }
 
 
-template <int MT, int WM, int WN, bool DUAL, bool BF16, int EDGE, typename OutT>
+template <int MT, int WM, int WN, bool DUAL, bool BF16, int EDGE, typename OutT, bool W8>
 int launch_gemm_e(GemmParams p, hipStream_t st) {
   constexpr int BM = 32 * MT * WM;
   constexpr int NBUF = 2;
@@ -329,7 +386,7 @@ int launch_gemm_e(GemmParams p, hipStream_t st) {
   const int bn_out = DUAL ? BN / 2 : BN;
   p.tiles_n = (p.n + bn_out - 1) / bn_out;
   const size_t smem = (size_t)NBUF * (BM * LDK + BK * LDN) * sizeof(uint16_t);
-  auto kern = gemm_kernel<MT, WM, WN, DUAL, BF16, EDGE, OutT>;
+  auto kern = gemm_kernel<MT, WM, WN, DUAL, BF16, EDGE, OutT, W8>;
   static bool attr_set = false;  // per instantiation
   if (!attr_set) {
     PTO_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -341,13 +398,13 @@ int launch_gemm_e(GemmParams p, hipStream_t st) {
   return PTO_HIP_OK;
 }
 
-template <int MT, int WM, int WN, bool DUAL, bool BF16, typename OutT>
+template <int MT, int WM, int WN, bool DUAL, bool BF16, typename OutT, bool W8 = false>
 int launch_gemm(GemmParams p, hipStream_t st) {
   constexpr int BM_ = 32 * MT * WM;
   const bool edge = p.n % (DUAL ? BN / 2 : BN) != 0 || p.k % BK != 0 || (p.splits > 1 && p.k_per_split % BK != 0);
-  if (edge) return launch_gemm_e<MT, WM, WN, DUAL, BF16, 2, OutT>(p, st);
-  if (p.m % BM_ != 0) return launch_gemm_e<MT, WM, WN, DUAL, BF16, 1, OutT>(p, st);
-  return launch_gemm_e<MT, WM, WN, DUAL, BF16, 0, OutT>(p, st);
+  if (edge) return launch_gemm_e<MT, WM, WN, DUAL, BF16, 2, OutT, W8>(p, st);
+  if (p.m % BM_ != 0) return launch_gemm_e<MT, WM, WN, DUAL, BF16, 1, OutT, W8>(p, st);
+  return launch_gemm_e<MT, WM, WN, DUAL, BF16, 0, OutT, W8>(p, st);
 }
 
 // Sum of the split-K slabs in split order (so the result does not depend on which workgroup
@@ -356,7 +413,8 @@ constexpr int kMaxSplits = 16;
 constexpr int kSplitBatch = 8;  // slabs loaded before the first add
 template <bool DUAL, typename OutT>
 __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* slabs, OutT* c, int64_t ldc, int m, int n,
-                                                          int splits, const void* residual, int res_dtype) {
+                                                          int splits, const void* residual, int res_dtype,
+                                                          const float* scale0, const float* scale1) {
   const int nq = n / 4;
   const int64_t quads = (int64_t)m * nq, mn = (int64_t)m * n;
   constexpr int kMats = DUAL ? 2 : 1;
@@ -385,6 +443,14 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* slabs, Ou
             t[mat].w += v[sp][mat].w;
           }
     }
+    if (scale0) {  // int8 weight codes: per-column scales
+      const float4 s0 = *reinterpret_cast<const float4*>(scale0 + col);
+      t[0] = float4{t[0].x * s0.x, t[0].y * s0.y, t[0].z * s0.z, t[0].w * s0.w};
+      if constexpr (DUAL) {
+        const float4 s1 = *reinterpret_cast<const float4*>(scale1 + col);
+        t[1] = float4{t[1].x * s1.x, t[1].y * s1.y, t[1].z * s1.z, t[1].w * s1.w};
+      }
+    }
     float4 y = t[0];
     if constexpr (DUAL) y = float4{silu(t[0].x) * t[1].x, silu(t[0].y) * t[1].y, silu(t[0].z) * t[1].z, silu(t[0].w) * t[1].w};
     if (!DUAL && residual) {
@@ -407,12 +473,13 @@ int launch_finish(const GemmParams& p, hipStream_t st) {
   const int64_t quads = (int64_t)p.m * (p.n / 4);
   const unsigned blocks = (unsigned)std::min<int64_t>((quads + 255) / 256, 4096);
   hipLaunchKernelGGL((gemm_finish_kernel<DUAL, OutT>), dim3(blocks), dim3(256), 0, st, p.slabs,
-                     reinterpret_cast<OutT*>(p.c), p.ldc, p.m, p.n, p.splits, p.residual, p.res_dtype);
+                     reinterpret_cast<OutT*>(p.c), p.ldc, p.m, p.n, p.splits, p.residual, p.res_dtype, p.scale0,
+                     p.scale1);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
 }
 
-template <bool DUAL, bool BF16, typename OutT>
+template <bool DUAL, bool BF16, typename OutT, bool W8 = false>
 int launch_variant(GemmParams p, hipStream_t st) {
   const int64_t variant = pto_hip::ctx().gemm_variant;
   const int64_t num_cu = pto_hip::ctx().num_cu;
@@ -464,9 +531,11 @@ int launch_variant(GemmParams p, hipStream_t st) {
     }
   }
   int rc;
-  if (small_tile) rc = launch_gemm<2, 2, 4, DUAL, BF16, OutT>(p, st);
+  if (small_tile) rc = launch_gemm<2, 2, 4, DUAL, BF16, OutT, W8>(p, st);
+  else if (variant == 0 || variant == 4) rc = launch_gemm<4, 2, 4, DUAL, BF16, OutT, W8>(p, st);
+  else if constexpr (W8) return pto_hip::fail(PTO_HIP_ERR_UNSUPPORTED, "gemm_variant %lld has no int8-weight form",
+                                              (long long)variant);
   else if (variant == 2) rc = launch_gemm<2, 2, 2, DUAL, BF16, OutT>(p, st);
-  else if (variant == 0 || variant == 4) rc = launch_gemm<4, 2, 4, DUAL, BF16, OutT>(p, st);
   else rc = launch_gemm<4, 2, 2, DUAL, BF16, OutT>(p, st);
   if (rc || p.splits == 1) return rc;
   return launch_finish<DUAL, OutT>(p, st);
@@ -475,6 +544,12 @@ int launch_variant(GemmParams p, hipStream_t st) {
 template <bool DUAL>
 int launch_typed(const GemmParams& p, int dtype, int out_dtype, hipStream_t st) {
   const bool bf16 = dtype == PTO_HIP_BF16;
+  if (p.scale0) {  // int8 weight codes
+    if (out_dtype == PTO_HIP_FP32)
+      return bf16 ? launch_variant<DUAL, true, float, true>(p, st) : launch_variant<DUAL, false, float, true>(p, st);
+    if (out_dtype == PTO_HIP_BF16 && bf16) return launch_variant<DUAL, true, __bf16, true>(p, st);
+    if (out_dtype == PTO_HIP_FP16 && !bf16) return launch_variant<DUAL, false, _Float16, true>(p, st);
+  }
   if (out_dtype == PTO_HIP_FP32)
     return bf16 ? launch_variant<DUAL, true, float>(p, st) : launch_variant<DUAL, false, float>(p, st);
   if (out_dtype == PTO_HIP_BF16 && bf16) return launch_variant<DUAL, true, __bf16>(p, st);
@@ -544,6 +619,39 @@ int ffn_skinny(const void* x, const float* gamma, const void* w_gate, const void
 }
 
 }  // namespace
+
+namespace pto_hip {
+
+bool gemm_w8_fits(const void* x, const void* wq0, const void* wq1, const void* residual, const void* out, int64_t m,
+                  int64_t k, int64_t n, int x_dtype, int out_dtype) {
+  const int64_t from = ctx().w8a16_gemm_rows, variant = ctx().gemm_variant;
+  return from > 0 && m >= from && (variant == 0 || variant == 4 || variant == 5) && k % 8 == 0 && n % 16 == 0 &&
+         ((uintptr_t)x | (uintptr_t)wq0 | (uintptr_t)wq1 | (uintptr_t)residual | (uintptr_t)out) % 16 == 0 &&
+         (x_dtype == PTO_HIP_BF16 || x_dtype == PTO_HIP_FP16) && (out_dtype == PTO_HIP_FP32 || out_dtype == x_dtype);
+}
+
+int gemm_w8(const void* x, const void* wq0, const float* scale0, const void* wq1, const float* scale1,
+            const void* residual, int res_dtype, void* out, int64_t m, int64_t k, int64_t n, int x_dtype,
+            int out_dtype, hipStream_t st) {
+  GemmParams p{};
+  p.a = reinterpret_cast<const uint16_t*>(x);
+  p.b0 = reinterpret_cast<const uint16_t*>(wq0);
+  p.b1 = reinterpret_cast<const uint16_t*>(wq1);
+  p.scale0 = scale0;
+  p.scale1 = scale1;
+  p.c = out;
+  p.lda = k;
+  p.ldb = n;
+  p.ldc = n;
+  p.m = (int)m;
+  p.n = (int)n;
+  p.k = (int)k;
+  p.residual = residual;
+  p.res_dtype = res_dtype;
+  return wq1 ? launch_typed<true>(p, x_dtype, out_dtype, st) : launch_typed<false>(p, x_dtype, out_dtype, st);
+}
+
+}  // namespace pto_hip
 
 extern "C" int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void* w_gate,
                                   const void* w_up, const void* w_down, void* out, int64_t tokens,

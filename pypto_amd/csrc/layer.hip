@@ -16,9 +16,16 @@
 
 namespace {
 
-// The layer for more than 32 sequences with 16-bit weights: the same steps, each projection as a
-// tiled GEMM (k split while the tiles alone leave CUs idle), so that the weights are read once
-// for the whole batch instead of once per 32 sequences.  Activations are row-major.
+// One projection of the large-batch layer: 16-bit weights (scale null) or int8 codes.
+int project(const void* x, const void* w, const float* scale, const void* residual, void* out, int64_t m, int64_t k,
+            int64_t n, int dt, int res_dt, int out_dt, void* stream) {
+  if (!scale) return pto_hip_projection(x, w, residual, out, m, k, n, dt, res_dt, out_dt, stream);
+  return pto_hip_w8a16_matmul(x, w, scale, residual, out, m, k, n, dt, res_dt, out_dt, stream);
+}
+
+// The layer for more than 32 sequences (16-bit weights, or int8 codes with the tiled GEMM on): the same steps, each projection as a tiled GEMM (k split
+// while the tiles alone leave CUs idle), so that the weights are read once for the whole batch
+// instead of once per 32 sequences.  Activations are row-major.
 int layer_large_batch(const PtoHipDecoderLayerArgs* a, int rope_w, void* stream) {
   using namespace pto_hip;
   const int64_t b = a->batch, h = a->hidden, hq = a->num_heads, hkv = a->kv_head_num, d = a->head_dim,
@@ -45,7 +52,7 @@ int layer_large_batch(const PtoHipDecoderLayerArgs* a, int rope_w, void* stream)
   void* hbuf = w;
 
   if ((rc = pto_hip_rms_norm(a->hidden_states, a->gamma_in, normed, b, h, a->eps, dt, dt, stream))) return rc;
-  if ((rc = pto_hip_projection(normed, a->wqkv_q, nullptr, qkv, b, h, qkv_n, dt, 0, PTO_HIP_FP32, stream))) return rc;
+  if ((rc = project(normed, a->wqkv_q, a->wqkv_s, nullptr, qkv, b, h, qkv_n, dt, 0, PTO_HIP_FP32, stream))) return rc;
   const int64_t pool_blocks = a->pool_rows / (hkv * a->block_size);
   if (fp8kv)
     rc = rope_kv_cache_update_fp8(qkv, nullptr, 1, 0, a->seq_lens, a->rope_cos, a->rope_sin, a->block_table,
@@ -64,11 +71,13 @@ int layer_large_batch(const PtoHipDecoderLayerArgs* a, int rope_w, void* stream)
                             cfg, dt, fp8kv ? PTO_HIP_FP8E4M3FN : dt, fp8kv ? a->k_scale : nullptr,
                             fp8kv ? a->v_scale : nullptr, pool_blocks, stream)))
     return rc;
-  if ((rc = pto_hip_projection(attn16, a->wo_q, a->hidden_states, resid1, b, hq * d, h, dt, dt, PTO_HIP_FP32, stream)))
+  if ((rc = project(attn16, a->wo_q, a->wo_s, a->hidden_states, resid1, b, hq * d, h, dt, dt, PTO_HIP_FP32, stream)))
     return rc;
   if ((rc = pto_hip_rms_norm(resid1, a->gamma_post, normed2, b, h, a->eps, PTO_HIP_FP32, dt, stream))) return rc;
-  if ((rc = pto_hip_gate_up_swiglu(normed2, a->wg_q, a->wu_q, hbuf, b, h, inter, dt, stream))) return rc;
-  return pto_hip_projection(hbuf, a->wd_q, resid1, a->out, b, inter, h, dt, PTO_HIP_FP32, dt, stream);
+  if (a->wg_s) rc = pto_hip_w8a16_swiglu(normed2, a->wg_q, a->wg_s, a->wu_q, a->wu_s, hbuf, b, h, inter, dt, dt, stream);
+  else rc = pto_hip_gate_up_swiglu(normed2, a->wg_q, a->wu_q, hbuf, b, h, inter, dt, stream);
+  if (rc) return rc;
+  return project(hbuf, a->wd_q, a->wd_s, resid1, a->out, b, inter, h, dt, PTO_HIP_FP32, dt, stream);
 }
 
 }  // namespace
@@ -113,11 +122,16 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
   PTO_CHECK_ARG(n_scales == 0 || n_scales == 5,
                 "decoder_layer_decode: weight scales must be given for all five projections or for none");
   const bool w16 = n_scales == 0;
-  if (b > kW8MaxM && w16) return layer_large_batch(a, rope_w, stream);
+  // int8 codes: the tiled GEMM wants 16-byte aligned matrices, and can be switched off.
+  const bool gemm8 = cx.w8a16_gemm_rows > 0 && b >= cx.w8a16_gemm_rows &&
+                     (cx.gemm_variant == 0 || cx.gemm_variant == 4 || cx.gemm_variant == 5) &&
+                     ((uintptr_t)a->wqkv_q | (uintptr_t)a->wo_q | (uintptr_t)a->wg_q | (uintptr_t)a->wu_q |
+                      (uintptr_t)a->wd_q) % 16 == 0;
+  if (b > kW8MaxM && (w16 || gemm8)) return layer_large_batch(a, rope_w, stream);
   if (b > kW8MaxM) {
-    // The int8 projections hold 32 rows per pass: larger batches run as consecutive groups of 32
-    // sequences in stream order (each group's rows of the block table, lengths and activations;
-    // the caches and weights are shared).
+    // Otherwise the int8 projections hold 32 rows per pass: larger batches run as consecutive
+    // groups of 32 sequences in stream order (each group's rows of the block table, lengths and
+    // activations; the caches and weights are shared).
     for (int64_t b0 = 0; b0 < b; b0 += kW8MaxM) {
       PtoHipDecoderLayerArgs part = *a;
       part.batch = std::min<int64_t>(kW8MaxM, b - b0);

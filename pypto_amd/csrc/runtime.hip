@@ -810,6 +810,9 @@ int pto_hip_set_option(const char* name, int64_t value) {
   } else if (!std::strcmp(name, "w8a16_min_steps")) {
     PTO_CHECK_ARG(value >= 1 && value <= 1024, "w8a16_min_steps must be in [1, 1024]");
     c.w8a16_min_steps = value;
+  } else if (!std::strcmp(name, "w8a16_gemm_rows")) {
+    PTO_CHECK_ARG(value >= 0 && value <= (1 << 20), "w8a16_gemm_rows must be in [0, 2^20]");
+    c.w8a16_gemm_rows = value;
   } else {
     return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
   }
@@ -828,6 +831,7 @@ int pto_hip_get_option(const char* name, int64_t* value) {
   else if (!std::strcmp(name, "w8a16_wgs_per_cu")) *value = c.w8a16_wgs_per_cu;
   else if (!std::strcmp(name, "w8a16_min_steps")) *value = c.w8a16_min_steps;
   else if (!std::strcmp(name, "w8a16_wide")) *value = c.w8a16_wide;
+  else if (!std::strcmp(name, "w8a16_gemm_rows")) *value = c.w8a16_gemm_rows;
   else return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
   return PTO_HIP_OK;
 }

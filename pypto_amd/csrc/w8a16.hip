@@ -534,6 +534,9 @@ extern "C" int pto_hip_w8a16_matmul(const void* x, const void* w_q, const float*
     PTO_CHECK_ARG(res_dtype == PTO_HIP_FP32 || res_dtype == PTO_HIP_BF16 || res_dtype == PTO_HIP_FP16,
                   "w8a16_matmul: residual dtype %s not in {FP32, BF16, FP16}", dtype_name(res_dtype));
   hipStream_t st = (hipStream_t)stream;
+  // Many rows: one tiled GEMM that reads the codes once.
+  if (gemm_w8_fits(x, w_q, nullptr, residual, out, m, k, n, x_dtype, out_dtype))
+    return gemm_w8(x, w_q, w_scale, nullptr, nullptr, residual, res_dtype, out, m, k, n, x_dtype, out_dtype, st);
   // The kernel holds 32 rows of x per pass; more rows stream the weights once per pass, in order
   // on the stream (the partial buffer is reused).
   for (int64_t r0 = 0; r0 < m; r0 += kMaxM) {
@@ -562,6 +565,8 @@ extern "C" int pto_hip_w8a16_swiglu(const void* x, const void* wg_q, const float
                     ((uintptr_t)wg_scale % 16 == 0) && ((uintptr_t)wu_scale % 16 == 0) && ((uintptr_t)out % 16 == 0),
                 "w8a16_swiglu: misaligned operand");
   hipStream_t st = (hipStream_t)stream;
+  if (gemm_w8_fits(x, wg_q, wu_q, nullptr, out, m, k, n, x_dtype, out_dtype))
+    return gemm_w8(x, wg_q, wg_scale, wu_q, wu_scale, nullptr, 0, out, m, k, n, x_dtype, out_dtype, st);
   for (int64_t r0 = 0; r0 < m; r0 += kMaxM) {  // 32 rows per pass, as in w8a16_matmul
     const int64_t rows = std::min<int64_t>(kMaxM, m - r0);
     W8Partials parts{};

@@ -89,9 +89,11 @@ def test_w8a16_argument_rules(worker):
             h(torch.zeros(4, 40, dtype=torch.bfloat16), wq, s, torch.zeros(4, 64))
 
 
+@pytest.mark.parametrize("gemm_rows", [0, 33])
 @pytest.mark.parametrize("m", [33, 64, 75])
-def test_w8a16_more_than_one_row_pass(worker, m):
-    """Row counts beyond one 32-row pass: every pass reuses the partial buffer in stream order."""
+def test_w8a16_more_than_one_row_pass(worker, m, gemm_rows):
+    """Row counts beyond one 32-row pass, as consecutive passes that reuse the partial buffer in
+    stream order (gemm_rows 0) and as one tiled GEMM over the int8 codes (the default)."""
     torch.manual_seed(m)
     k, n = 512, 384
     x = (torch.randn(m, k) * 0.5).to(torch.bfloat16)
@@ -101,15 +103,51 @@ def test_w8a16_more_than_one_row_pass(worker, m):
     su = torch.rand(n) * 0.01 + 0.001
     res = torch.randn(m, n)
     out = torch.zeros(m, n)
-    with worker.register(w8a16_matmul_residual) as h:
-        h(x, wq, s, res, out)
+    out2 = torch.zeros(m, n, dtype=torch.bfloat16)
+    worker.set_option("w8a16_gemm_rows", gemm_rows)
+    try:
+        with worker.register(w8a16_matmul_residual) as h:
+            h(x, wq, s, res, out)
+        with worker.register(w8a16_swiglu) as h:
+            h(x, wq, s, wu, su, out2)
+    finally:
+        worker.set_option("w8a16_gemm_rows", 33)
     ref = oracle.w8a16_matmul(x, wq, s) + res
     validate_golden({"out": out}, {"out": ref}, rtol=1e-3, atol=1e-3)
-    out2 = torch.zeros(m, n, dtype=torch.bfloat16)
-    with worker.register(w8a16_swiglu) as h:
-        h(x, wq, s, wu, su, out2)
     ref2 = oracle.swiglu(oracle.w8a16_matmul(x, wq, s), oracle.w8a16_matmul(x, wu, su)).to(torch.bfloat16)
     validate_golden({"out": out2.float()}, {"out": ref2.float()}, rtol=1e-2, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,n", [(300, 4096, 1040), (64, 11008, 4096), (129, 528, 272), (2048, 1024, 768),
+                                   (40, 256, 16), (96, 2048, 1000)])
+def test_w8a16_tiled_gemm_over_int8_codes(worker, dtype, m, k, n):
+    """More than 32 rows: the codes go through the tiled GEMM (widened exactly inside the kernel,
+    scales on the accumulators) - ragged tiles in every dimension, k split over workgroups with
+    the scales applied after the slabs are summed, and a channel count that is not a multiple of
+    16 (1000), which keeps the 32-row passes."""
+    g = torch.Generator().manual_seed(m + n)
+    x = (torch.randn(m, k, generator=g) * 0.5).to(dtype)
+    wq = torch.randint(-127, 128, (k, n), generator=g, dtype=torch.int8)
+    wu = torch.randint(-127, 128, (k, n), generator=g, dtype=torch.int8)
+    s = torch.rand(n, generator=g) * 0.01 + 0.001
+    su = torch.rand(n, generator=g) * 0.01 + 0.001
+    res = torch.randn(m, n, generator=g).to(dtype)
+    out = torch.zeros(m, n)
+    with worker.register(w8a16_matmul) as h:
+        h(x, wq, s, out)
+    ref = oracle.w8a16_matmul(x, wq, s)
+    validate_golden({"out": out}, {"out": ref}, rtol=1e-4, atol=1e-4 * float(ref.abs().max()))
+    out16 = torch.zeros(m, n, dtype=dtype)
+    with worker.register(w8a16_matmul_residual) as h:
+        h(x, wq, s, res, out16)
+    validate_golden({"out": out16.float()}, {"out": (ref + res.float()).to(dtype).float()}, rtol=1e-2,
+                    atol=1e-2 * max(1.0, float(ref.abs().max()) / 16))
+    out2 = torch.zeros(m, n, dtype=dtype)
+    with worker.register(w8a16_swiglu) as h:
+        h(x, wq, s, wu, su, out2)
+    ref2 = oracle.swiglu(ref, oracle.w8a16_matmul(x, wu, su)).to(dtype)
+    validate_golden({"out": out2.float()}, {"out": ref2.float()}, rtol=1e-2, atol=1e-2 * max(1.0, float(ref2.float().abs().max()) / 16))
 
 
 def test_rope_tables_of_full_head_width(worker):
@@ -311,6 +349,26 @@ def test_decoder_layer_decode(worker, batch, ctxs):
     assert torch.allclose(inp.value_cache.float(), ref_v.float(), atol=2e-2, rtol=1e-2)
     changed = (inp.key_cache != kc0).any(dim=1).sum().item()
     assert changed <= batch * 2
+
+
+@pytest.mark.parametrize("batch,gemm_rows", [(45, 0), (100, 0), (100, 33), (300, 33)])
+def test_decoder_layer_decode_int8_weights_many_sequences(worker, batch, gemm_rows):
+    """More than 32 sequences with int8 weights: as groups of 32 through the skinny projections
+    (gemm_rows 0) and with every projection as one tiled GEMM over the codes (the default)."""
+    g = torch.Generator().manual_seed(batch)
+    ctxs = torch.randint(1, 300, (batch,), generator=g).tolist()
+    inp = workloads.decoder_layer_inputs(batch=batch, hidden=1024, num_heads=8, kv_head_num=2, head_dim=128,
+                                         intermediate=2816, block_size=64, context_lens=ctxs, seed=batch + 1)
+    ref_out, ref_k, ref_v = _oracle_layer(inp)
+    worker.set_option("w8a16_gemm_rows", gemm_rows)
+    try:
+        with worker.register(decoder_layer_decode) as h:
+            h(*inp.args())
+    finally:
+        worker.set_option("w8a16_gemm_rows", 33)
+    validate_golden({"out": inp.out.float()}, {"out": ref_out.float()}, rtol=2e-2, atol=2e-2)
+    assert torch.allclose(inp.key_cache.float(), ref_k.float(), atol=2e-2, rtol=1e-2)
+    assert torch.allclose(inp.value_cache.float(), ref_v.float(), atol=2e-2, rtol=1e-2)
 
 
 @pytest.mark.parametrize("dtype,batch", [(torch.bfloat16, 16), (torch.float16, 5), (torch.bfloat16, 40)])
