@@ -336,7 +336,8 @@ PTO_HIP_API int pto_hip_select_program(const char* orchestration_name, const Pto
  *                               skinny projections up to 32 tokens), 1..3 = 4-wavefront alternatives
  *                               (256-row tile, 128-row tile, 256-row tile with k split in two),
  *                               4 = 8 wavefronts, 256-row tile, k split when CUs would idle,
- *                               5 = 8 wavefronts, 128-row tile
+ *                               5 = 8 wavefronts, 128-row tile, 6 = 8 wavefronts, 64-row tile, k split
+ *                               while CUs would idle (the default choice for 33..64 rows)
  *  "w8a16_wgs_per_cu"           workgroups per CU the W8A16 k split aims at (default 1)
  *  "w8a16_wide"                 1 = int8 codes of large matrices (>= 150 MB) are read 16 per lane
  *                               (default), 0 = always 8 per lane, 2 = 16 per lane whenever the

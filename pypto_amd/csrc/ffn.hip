@@ -270,7 +270,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   };
   constexpr int kReads = MT + 2 * NT;                         // LDS reads per k-step
   constexpr int kSlots = MT * NT;                             // MFMAs per k-step
-  static_assert(kSlots >= NA && kSlots >= NB, "one LDS write / global load per MFMA slot");
+  constexpr int kMovesPerSlot = ((NA > NB ? NA : NB) + kSlots - 1) / kSlots;  // LDS writes / global loads per slot
   constexpr int kReadsPerSlot = (kReads + kSlots - 1) / kSlots;
   constexpr int kSteps = BK / 16;
 
@@ -304,11 +304,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
           for (int r = q * kReadsPerSlot; r < (q + 1) * kReadsPerSlot; ++r)
             if (r < kReads) read_one(buf, ks + 1, (ks + 1) & 1, r);
         }
-        if (ks == 0 && q < NA)
-          *reinterpret_cast<u32x4*>(da + (a_row + (T / 8) * q) * LDK + a_chunk * 8) = ra[q];
-        if (ks == 1 && q < NB) store_b(db, q);
-        if (ks == 2 && q < NA) load_a(k_next, q);
-        if (ks == 3 && q < NB) load_b(k_next, q);
+#pragma unroll
+        for (int e = q * kMovesPerSlot; e < (q + 1) * kMovesPerSlot; ++e) {
+          if (ks == 0 && e < NA)
+            *reinterpret_cast<u32x4*>(da + (a_row + (T / 8) * e) * LDK + a_chunk * 8) = ra[e];
+          if (ks == 1 && e < NB) store_b(db, e);
+          if (ks == 2 && e < NA) load_a(k_next, e);
+          if (ks == 3 && e < NB) load_b(k_next, e);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -495,7 +498,7 @@ int launch_variant(GemmParams p, hipStream_t st) {
   // split order.
   // variants 1-3 keep four wavefronts (one per SIMD): 1 = 256x256 tile, 2 = 128x256 tile,
   // 3 = 256x256 tile with k split in two.  4 = eight wavefronts, 256x256 tile, k split in two
-  // when CUs would idle.  5 = eight wavefronts, 128x256 tile.
+  // when CUs would idle.  5 = eight wavefronts, 128x256 tile.  6 = eight wavefronts, 64x256 tile, k split while CUs would idle.
   const int64_t tiles_n = (p.n + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256);
   const int64_t big_tiles = (int64_t)((p.m + 255) / 256) * tiles_n;
   const int64_t small_tiles = (int64_t)((p.m + 127) / 128) * tiles_n;
@@ -520,6 +523,15 @@ int launch_variant(GemmParams p, hipStream_t st) {
       }
     }
   }
+  // Up to 64 rows: a 64-row tile.  With the 128-row tile the MFMA work on its padding rows, not
+  // the weight stream, set the time for int8 codes (half the bytes of 16-bit weights: decoder
+  // layer at batch 64 205 -> 177 us) and still cost 2-5 % with 16-bit weights.
+  const bool tiny_tile = variant == 6 || (variant == 0 && p.m <= 64);
+  if (tiny_tile) {
+    const int64_t tiny_tiles = (int64_t)((p.m + 63) / 64) * tiles_n;
+    small_tile = false;
+    want = tiny_tiles * 2 <= num_cu ? (int)std::min<int64_t>(kMaxSplits, num_cu / tiny_tiles) : 1;
+  }
   if (want > 1 && p.k >= 4 * BK * want && p.n % 4 == 0) {
     p.k_per_split = ((p.k + want * BK - 1) / (want * BK)) * BK;
     p.splits = (p.k + p.k_per_split - 1) / p.k_per_split;
@@ -531,7 +543,8 @@ int launch_variant(GemmParams p, hipStream_t st) {
     }
   }
   int rc;
-  if (small_tile) rc = launch_gemm<2, 2, 4, DUAL, BF16, OutT, W8>(p, st);
+  if (tiny_tile) rc = launch_gemm<1, 2, 4, DUAL, BF16, OutT, W8>(p, st);
+  else if (small_tile) rc = launch_gemm<2, 2, 4, DUAL, BF16, OutT, W8>(p, st);
   else if (variant == 0 || variant == 4) rc = launch_gemm<4, 2, 4, DUAL, BF16, OutT, W8>(p, st);
   else if constexpr (W8) return pto_hip::fail(PTO_HIP_ERR_UNSUPPORTED, "gemm_variant %lld has no int8-weight form",
                                               (long long)variant);
@@ -625,7 +638,7 @@ namespace pto_hip {
 bool gemm_w8_fits(const void* x, const void* wq0, const void* wq1, const void* residual, const void* out, int64_t m,
                   int64_t k, int64_t n, int x_dtype, int out_dtype) {
   const int64_t from = ctx().w8a16_gemm_rows, variant = ctx().gemm_variant;
-  return from > 0 && m >= from && (variant == 0 || variant == 4 || variant == 5) && k % 8 == 0 && n % 16 == 0 &&
+  return from > 0 && m >= from && (variant == 0 || variant >= 4) && k % 8 == 0 && n % 16 == 0 &&
          ((uintptr_t)x | (uintptr_t)wq0 | (uintptr_t)wq1 | (uintptr_t)residual | (uintptr_t)out) % 16 == 0 &&
          (x_dtype == PTO_HIP_BF16 || x_dtype == PTO_HIP_FP16) && (out_dtype == PTO_HIP_FP32 || out_dtype == x_dtype);
 }

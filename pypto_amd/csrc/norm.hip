@@ -51,23 +51,26 @@ __global__ __launch_bounds__(kThreads) void rms_norm_kernel(const TI* __restrict
   }
 }
 
-// 16-bit rows whose length is a multiple of 8 and at most 8 * kThreads * kVecPerThread: each
-// thread keeps its 16-byte chunks in registers, so the row is read from memory once.
+// Rows whose length is a multiple of 8 and at most 8 * kThreads * kVecPerThread, 16-bit output
+// (input of the same type, or fp32 - the residual stream between the two halves of a decoder
+// layer): each thread keeps its groups of 8 elements in registers, so the row is read from memory
+// once.
 constexpr int kVecPerThread = 4;
 // BLOCKED writes the output as [hidden/8][32][8] (at most 32 rows): the activation layout the
 // W8A16 projections of the decoder layer read.
-template <typename T, bool BLOCKED>
-__global__ __launch_bounds__(kThreads) void rms_norm_vec_kernel(const T* __restrict__ x,
+template <typename TI, typename T, bool BLOCKED>
+__global__ __launch_bounds__(kThreads) void rms_norm_vec_kernel(const TI* __restrict__ x,
                                                                 const float* __restrict__ gamma,
                                                                 T* __restrict__ out, int64_t hidden,
                                                                 float eps) {
   typedef __attribute__((__vector_size__(8 * sizeof(T)))) T vec8;
+  typedef __attribute__((__vector_size__(8 * sizeof(TI)))) TI vec8i;
   const int64_t row = blockIdx.x;
-  const vec8* xr = reinterpret_cast<const vec8*>(x + row * hidden);
+  const vec8i* xr = reinterpret_cast<const vec8i*>(x + row * hidden);
   vec8* orow = BLOCKED ? reinterpret_cast<vec8*>(out) + row : reinterpret_cast<vec8*>(out + row * hidden);
   constexpr int kOutStride = BLOCKED ? 32 : 1;  // vec8 units between consecutive 8-element groups
   const int nvec = (int)(hidden / 8);
-  vec8 v[kVecPerThread];
+  vec8i v[kVecPerThread];
   float ss = 0.f;
 #pragma unroll
   for (int u = 0; u < kVecPerThread; ++u) {
@@ -144,10 +147,10 @@ int rms_norm_blocked(const void* x, const float* gamma, void* out, int64_t rows,
   if (rows == 0) return PTO_HIP_OK;
   dim3 grid((unsigned)rows), block(kThreads);
   if (dtype == PTO_HIP_BF16)
-    hipLaunchKernelGGL((rms_norm_vec_kernel<__bf16, true>), grid, block, 0, st, (const __bf16*)x, gamma, (__bf16*)out,
-                       hidden, eps);
+    hipLaunchKernelGGL((rms_norm_vec_kernel<__bf16, __bf16, true>), grid, block, 0, st, (const __bf16*)x, gamma,
+                       (__bf16*)out, hidden, eps);
   else
-    hipLaunchKernelGGL((rms_norm_vec_kernel<_Float16, true>), grid, block, 0, st, (const _Float16*)x, gamma,
+    hipLaunchKernelGGL((rms_norm_vec_kernel<_Float16, _Float16, true>), grid, block, 0, st, (const _Float16*)x, gamma,
                        (_Float16*)out, hidden, eps);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
@@ -163,17 +166,25 @@ extern "C" int pto_hip_rms_norm(const void* x, const float* gamma, void* out, in
   if (rows == 0) return PTO_HIP_OK;
   PTO_CHECK_ARG(x && out, "rms_norm: null tensor pointer");
   hipStream_t st = (hipStream_t)stream;
-  const bool vec_ok = x_dtype == out_dtype && (x_dtype == PTO_HIP_BF16 || x_dtype == PTO_HIP_FP16) &&
-                      hidden % 8 == 0 && hidden <= 8 * kThreads * kVecPerThread &&
+  const bool vec_ok = (out_dtype == PTO_HIP_BF16 || out_dtype == PTO_HIP_FP16) &&
+                      (x_dtype == out_dtype || x_dtype == PTO_HIP_FP32) && hidden % 8 == 0 &&
+                      hidden <= 8 * kThreads * kVecPerThread &&
                       ((uintptr_t)x | (uintptr_t)out | (uintptr_t)gamma) % 16 == 0;
   if (vec_ok) {
     dim3 grid((unsigned)rows), block(kThreads);
-    if (x_dtype == PTO_HIP_BF16)
-      hipLaunchKernelGGL((rms_norm_vec_kernel<__bf16, false>), grid, block, 0, st, (const __bf16*)x, gamma,
+    const bool bf = out_dtype == PTO_HIP_BF16;
+    if (x_dtype == PTO_HIP_FP32 && bf)
+      hipLaunchKernelGGL((rms_norm_vec_kernel<float, __bf16, false>), grid, block, 0, st, (const float*)x, gamma,
+                         (__bf16*)out, hidden, eps);
+    else if (x_dtype == PTO_HIP_FP32)
+      hipLaunchKernelGGL((rms_norm_vec_kernel<float, _Float16, false>), grid, block, 0, st, (const float*)x, gamma,
+                         (_Float16*)out, hidden, eps);
+    else if (bf)
+      hipLaunchKernelGGL((rms_norm_vec_kernel<__bf16, __bf16, false>), grid, block, 0, st, (const __bf16*)x, gamma,
                          (__bf16*)out, hidden, eps);
     else
-      hipLaunchKernelGGL((rms_norm_vec_kernel<_Float16, false>), grid, block, 0, st, (const _Float16*)x, gamma,
-                         (_Float16*)out, hidden, eps);
+      hipLaunchKernelGGL((rms_norm_vec_kernel<_Float16, _Float16, false>), grid, block, 0, st, (const _Float16*)x,
+                         gamma, (_Float16*)out, hidden, eps);
     PTO_CHECK_HIP(hipGetLastError());
     return PTO_HIP_OK;
   }

@@ -789,6 +789,7 @@ int pto_hip_set_option(const char* name, int64_t value) {
     PTO_CHECK_ARG(value >= 0, "attn_tokens_per_partition must be >= 0");
     c.attn_tokens_per_partition = value;
   } else if (!std::strcmp(name, "gemm_variant")) {
+    PTO_CHECK_ARG(value >= 0 && value <= 6, "gemm_variant must be in [0, 6]");
     c.gemm_variant = value;
   } else if (!std::strcmp(name, "attn_group_tiles")) {
     PTO_CHECK_ARG(value == 0 || value == 1 || value == 2 || value == 4, "attn_group_tiles must be 0, 1, 2 or 4");

@@ -25,6 +25,23 @@ def test_rms_norm(worker, dtype, rows, hidden):
     validate_golden({"out": out.float()}, {"out": ref.float()}, rtol=tol, atol=tol)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,hidden", [(64, 4096), (3, 8192), (5, 1000), (2, 8200)])
+def test_rms_norm_of_fp32_rows_to_16_bit(worker, out_dtype, rows, hidden):
+    """The post-attention norm of a decoder layer: fp32 residual stream in, activation type out
+    (tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:278-280).  Row lengths
+    inside and outside the form that keeps the row in registers."""
+    g = torch.Generator().manual_seed(hidden)
+    x = torch.randn((rows, hidden), generator=g) * 3
+    gamma = 1 + 0.02 * torch.randn((1, hidden), generator=g)
+    out = torch.zeros((rows, hidden), dtype=out_dtype)
+    with worker.register(rms_norm) as h:
+        h(x, gamma, out, 1e-6)
+    ref = oracle.rms_norm(x, gamma, 1e-6, out_dtype=out_dtype)
+    tol = {torch.bfloat16: 8e-3, torch.float16: 1e-3}[out_dtype]
+    validate_golden({"out": out.float()}, {"out": ref.float()}, rtol=tol, atol=tol)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rms_norm_without_weight(worker, dtype):
     """The unweighted form: x / sqrt(mean(x^2) + eps) (examples/models/08_llama_mini.py:93-118)."""
@@ -57,7 +74,7 @@ def test_ffn_reference_example_fp32(worker):
     assert torch.allclose(out, oracle.ffn_swiglu(x, wg, wu, wd), rtol=3e-3, atol=3e-3)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
 def test_ffn_tiny_fp16(worker, variant):
     """x[128,512] fp16, I=1024, weights N(0,0.02), seed 0; max-abs 1e-2 / rel 2e-2."""
     inp = workloads.ffn_tiny(seed=0)
@@ -72,7 +89,7 @@ def test_ffn_tiny_fp16(worker, variant):
     validate_golden({"out": inp.out}, {"out": ref32}, rtol=2e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("t,h,i", [(256, 512, 1024), (100, 264, 520), (512, 1024, 2816)])
 def test_ffn_block_bf16(worker, variant, t, h, i):
     """RMSNorm prologue + SwiGLU FFN, bf16, incl. shapes that are not tile multiples."""
