@@ -76,11 +76,15 @@ int workspace(size_t bytes, void** ptr);
 // ---- W8A16 decode projections, shared with the composed decoder layer -------------------
 constexpr int kW8Slab = 128;  // output channels per workgroup of the partial kernel
 constexpr int kW8MaxM = 32;   // rows of a partial slab (activation rows are at most this many)
-// fp32 partial sums of a projection, one [32, N] slab per k split: element (s, m, n) of
-// projection i is part[i][(s * 32 + m) * N + n].  They live in the shared workspace.
+// fp32 partial sums of a projection, one slab per k split: element (s, m, n) of projection i is
+// part[i][s * slab_stride + m * N + n].  The skinny kernels write [32, N] slabs into the shared
+// workspace; the tiled GEMM writes [M, N] slabs into its own scratch area (or, with one split, the
+// finished product into the caller's buffer: `scaled` then says the channel scales are in).
 struct W8Partials {
   float* part[2];
   int splits;
+  int64_t slab_stride;
+  bool scaled;
 };
 // Launches the partial kernel for x[M, K] @ wq0[K, N] (and wq1 when non-null).  x_blocked: x is
 // stored [K/8][32][8] - element (m, k) at ((k/8)*32 + m)*8 + k%8 - the layout the layer's own
@@ -98,6 +102,9 @@ int w8a16_finish(const W8Partials& parts, const float* scale0, const float* scal
                  int res_dtype, void* out, int out_dtype, bool out_blocked, int64_t m, int64_t n, hipStream_t st);
 // sum_out = sum_s(part) * scale + residual (fp32); normed_out = cast(RMSNorm(sum_out) * gamma).
 bool w8a16_finish_norm_fits(int64_t n);
+int w8a16_finish_norm(const W8Partials& parts, const float* scale, const void* residual, int res_dtype,
+                      float* sum_out, const float* gamma, void* normed_out, int out_dtype, bool out_blocked,
+                      int64_t m, int64_t n, float eps, hipStream_t st);
 // The tiled GEMM with int8 weight codes (widened on their way into LDS, scales applied to the
 // accumulators): out = (x @ codes0) * scale0 (+ residual), or with codes1 / scale1 given
 // SiLU((x @ codes0) * scale0) * ((x @ codes1) * scale1).  gemm_w8_fits says whether the shapes,
@@ -107,9 +114,11 @@ bool gemm_w8_fits(const void* x, const void* wq0, const void* wq1, const void* r
 int gemm_w8(const void* x, const void* wq0, const float* scale0, const void* wq1, const float* scale1,
             const void* residual, int res_dtype, void* out, int64_t m, int64_t k, int64_t n, int x_dtype,
             int out_dtype, hipStream_t st);
-int w8a16_finish_norm(const W8Partials& parts, const float* scale, const void* residual, int res_dtype,
-                      float* sum_out, const float* gamma, void* normed_out, int out_dtype, bool out_blocked,
-                      int64_t m, int64_t n, float eps, hipStream_t st);
+// x[M, K] @ w[K, N] through the tiled GEMM, left as k-split partial sums for a fused consumer
+// (scale null: 16-bit weights).  With one split the product, scales applied, is written to
+// `direct` (fp32 [M, N]) and returned as a single slab.
+int gemm_partials(const void* x, const void* w, const float* scale, int64_t m, int64_t k, int64_t n, int x_dtype,
+                  float* direct, hipStream_t st, W8Partials* out);
 
 // RoPE + K/V append reading either final fp32 projections (qkv_scale null, splits 1) or the
 // partial sums of the q/k/v projection (summed in split order and scaled per channel).

@@ -58,6 +58,7 @@ struct GemmParams {
   int res_dtype;
   const float* scale0;      // int8 weight codes: one scale per output column of b0 (and b1); else null
   const float* scale1;
+  pto_hip::W8Partials* partials_out;  // non-null: leave the k-split slabs unsummed and describe them here
 };
 
 __device__ __forceinline__ float load_residual(const void* r, int dt, int64_t i) {
@@ -550,7 +551,17 @@ int launch_variant(GemmParams p, hipStream_t st) {
                                               (long long)variant);
   else if (variant == 2) rc = launch_gemm<2, 2, 2, DUAL, BF16, OutT>(p, st);
   else rc = launch_gemm<4, 2, 2, DUAL, BF16, OutT>(p, st);
-  if (rc || p.splits == 1) return rc;
+  if (rc) return rc;
+  if (p.partials_out) {  // a fused consumer sums the slabs (one split: the product is in p.c, scales applied)
+    pto_hip::W8Partials& o = *p.partials_out;
+    o.part[0] = p.splits > 1 ? p.slabs : reinterpret_cast<float*>(p.c);
+    o.part[1] = nullptr;
+    o.splits = p.splits;
+    o.slab_stride = (int64_t)p.m * p.n;
+    o.scaled = p.splits == 1;
+    return PTO_HIP_OK;
+  }
+  if (p.splits == 1) return rc;
   return launch_finish<DUAL, OutT>(p, st);
 }
 
@@ -662,6 +673,27 @@ int gemm_w8(const void* x, const void* wq0, const float* scale0, const void* wq1
   p.residual = residual;
   p.res_dtype = res_dtype;
   return wq1 ? launch_typed<true>(p, x_dtype, out_dtype, st) : launch_typed<false>(p, x_dtype, out_dtype, st);
+}
+
+int gemm_partials(const void* x, const void* w, const float* scale, int64_t m, int64_t k, int64_t n, int x_dtype,
+                  float* direct, hipStream_t st, W8Partials* out) {
+  PTO_CHECK_ARG(m > 0 && k % 8 == 0 && n % (scale ? 16 : 8) == 0 &&
+                    ((uintptr_t)x | (uintptr_t)w | (uintptr_t)direct) % 16 == 0,
+                "gemm_partials: unsupported shape [%lld, %lld] @ [%lld, %lld] or misaligned operand", (long long)m,
+                (long long)k, (long long)k, (long long)n);
+  GemmParams p{};
+  p.a = reinterpret_cast<const uint16_t*>(x);
+  p.b0 = reinterpret_cast<const uint16_t*>(w);
+  p.scale0 = scale;
+  p.c = direct;
+  p.lda = k;
+  p.ldb = n;
+  p.ldc = n;
+  p.m = (int)m;
+  p.n = (int)n;
+  p.k = (int)k;
+  p.partials_out = out;
+  return launch_typed<false>(p, x_dtype, PTO_HIP_FP32, st);
 }
 
 }  // namespace pto_hip

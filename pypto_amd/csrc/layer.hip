@@ -34,7 +34,7 @@ int layer_large_batch(const PtoHipDecoderLayerArgs* a, int rope_w, void* stream)
   const bool fp8kv = a->kv_dtype == PTO_HIP_FP8E4M3FN;
   const int64_t qkv_n = (hq + 2 * hkv) * d;
   auto up = [](size_t n) { return (n + 255) / 256 * 256; };
-  const size_t sz_normed = up((size_t)b * h * 2), sz_qkv = up((size_t)b * qkv_n * 4),
+  const size_t sz_normed = up((size_t)b * h * 2), sz_qkv = up((size_t)b * std::max(qkv_n, h) * 4),  // also holds an unsplit o_proj product
                sz_q = up((size_t)b * hq * d * 2), sz_attn = up((size_t)b * hq * d * 4),
                sz_attn16 = up((size_t)b * hq * d * 2), sz_resid = up((size_t)b * h * 4),
                sz_h = up((size_t)b * inter * 2);
@@ -51,17 +51,23 @@ int layer_large_batch(const PtoHipDecoderLayerArgs* a, int rope_w, void* stream)
   void* normed2 = w;             w += sz_normed;
   void* hbuf = w;
 
+  hipStream_t st = (hipStream_t)stream;
   if ((rc = pto_hip_rms_norm(a->hidden_states, a->gamma_in, normed, b, h, a->eps, dt, dt, stream))) return rc;
-  if ((rc = project(normed, a->wqkv_q, a->wqkv_s, nullptr, qkv, b, h, qkv_n, dt, 0, PTO_HIP_FP32, stream))) return rc;
+  // The k-split slabs of the q/k/v and o projections go unsummed to the kernels that follow them
+  // (RoPE + append; residual + RMSNorm), as the partial sums of the skinny projections do.
+  W8Partials parts{};
+  if ((rc = gemm_partials(normed, a->wqkv_q, a->wqkv_s, b, h, qkv_n, dt, qkv, st, &parts))) return rc;
+  const float* qkv_scale = parts.scaled ? nullptr : a->wqkv_s;
   const int64_t pool_blocks = a->pool_rows / (hkv * a->block_size);
   if (fp8kv)
-    rc = rope_kv_cache_update_fp8(qkv, nullptr, 1, 0, a->seq_lens, a->rope_cos, a->rope_sin, a->block_table,
-                                  a->key_cache, a->value_cache, a->k_scale, a->v_scale, q16, b, hq, hkv, d,
-                                  a->block_size, a->max_num_blocks_per_req, a->max_pos, rope_w, pool_blocks, dt, stream);
+    rc = rope_kv_cache_update_fp8(parts.part[0], qkv_scale, parts.splits, parts.slab_stride, a->seq_lens, a->rope_cos,
+                                  a->rope_sin, a->block_table, a->key_cache, a->value_cache, a->k_scale, a->v_scale,
+                                  q16, b, hq, hkv, d, a->block_size, a->max_num_blocks_per_req, a->max_pos, rope_w,
+                                  pool_blocks, dt, stream);
   else
-    rc = rope_kv_cache_update(qkv, nullptr, 1, 0, a->seq_lens, a->rope_cos, a->rope_sin, a->block_table, a->key_cache,
-                              a->value_cache, q16, b, hq, hkv, d, a->block_size, a->max_num_blocks_per_req, a->max_pos,
-                              rope_w, a->pool_rows, dt, stream);
+    rc = rope_kv_cache_update(parts.part[0], qkv_scale, parts.splits, parts.slab_stride, a->seq_lens, a->rope_cos,
+                              a->rope_sin, a->block_table, a->key_cache, a->value_cache, q16, b, hq, hkv, d,
+                              a->block_size, a->max_num_blocks_per_req, a->max_pos, rope_w, a->pool_rows, dt, stream);
   if (rc) return rc;
   float scale = 1.0f / sqrtf((float)d);
   uint32_t scale_bits;
@@ -71,9 +77,17 @@ int layer_large_batch(const PtoHipDecoderLayerArgs* a, int rope_w, void* stream)
                             cfg, dt, fp8kv ? PTO_HIP_FP8E4M3FN : dt, fp8kv ? a->k_scale : nullptr,
                             fp8kv ? a->v_scale : nullptr, pool_blocks, stream)))
     return rc;
-  if ((rc = project(attn16, a->wo_q, a->wo_s, a->hidden_states, resid1, b, hq * d, h, dt, dt, PTO_HIP_FP32, stream)))
-    return rc;
-  if ((rc = pto_hip_rms_norm(resid1, a->gamma_post, normed2, b, h, a->eps, PTO_HIP_FP32, dt, stream))) return rc;
+  if (w8a16_finish_norm_fits(h)) {
+    // o_proj into the buffer the q/k/v product no longer needs, then sum + residual + RMSNorm in one kernel
+    if ((rc = gemm_partials(attn16, a->wo_q, a->wo_s, b, hq * d, h, dt, qkv, st, &parts))) return rc;
+    if ((rc = w8a16_finish_norm(parts, parts.scaled ? nullptr : a->wo_s, a->hidden_states, dt, resid1, a->gamma_post,
+                                normed2, dt, false, b, h, a->eps, st)))
+      return rc;
+  } else {
+    if ((rc = project(attn16, a->wo_q, a->wo_s, a->hidden_states, resid1, b, hq * d, h, dt, dt, PTO_HIP_FP32, stream)))
+      return rc;
+    if ((rc = pto_hip_rms_norm(resid1, a->gamma_post, normed2, b, h, a->eps, PTO_HIP_FP32, dt, stream))) return rc;
+  }
   if (a->wg_s) rc = pto_hip_w8a16_swiglu(normed2, a->wg_q, a->wg_s, a->wu_q, a->wu_s, hbuf, b, h, inter, dt, dt, stream);
   else rc = pto_hip_gate_up_swiglu(normed2, a->wg_q, a->wu_q, hbuf, b, h, inter, dt, stream);
   if (rc) return rc;
@@ -127,7 +141,7 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
                      (cx.gemm_variant == 0 || cx.gemm_variant >= 4) &&
                      ((uintptr_t)a->wqkv_q | (uintptr_t)a->wo_q | (uintptr_t)a->wg_q | (uintptr_t)a->wu_q |
                       (uintptr_t)a->wd_q) % 16 == 0;
-  if (b > kW8MaxM && (w16 || gemm8)) return layer_large_batch(a, rope_w, stream);
+  if (w16 ? b > kW8MaxM : gemm8) return layer_large_batch(a, rope_w, stream);
   if (b > kW8MaxM) {
     // Otherwise the int8 projections hold 32 rows per pass: larger batches run as consecutive
     // groups of 32 sequences in stream order (each group's rows of the block table, lengths and

@@ -237,7 +237,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
 }
 
 struct FinishParams {
-  const float* part0;   // [splits, 32, N]
+  const float* part0;   // [splits, 32 or M, N]: `stride` elements between splits
   const float* part1;   // second projection for SwiGLU, or null
   const float* scale0;  // [N]
   const float* scale1;
@@ -245,6 +245,7 @@ struct FinishParams {
   void* out;            // [M, N]
   int m, n, splits, res_dtype, out_dtype;
   int out_blocked;  // write out as [N/8][32][8] for the next projection
+  int64_t stride;
 };
 
 // Element index of (row m, channel n) in the blocked activation layout [N/8][32][8].
@@ -275,10 +276,9 @@ __device__ __forceinline__ void store4_from_f32(void* p, size_t i, int dt, float
 
 // Sum of the k splits of four channels, in split order, times the channel scales.  Loads go out
 // four at a time; the additions keep the order.
-__device__ __forceinline__ float4 sum_splits(const float* part, const float* scale, int splits, int m, int n,
-                                             int nn) {
+__device__ __forceinline__ float4 sum_splits(const float* part, const float* scale, int splits, size_t stride, int m,
+                                             int n, int nn) {
   float4 a = {0.f, 0.f, 0.f, 0.f};
-  const size_t stride = (size_t)kMaxM * nn;
   const float* src = part + (size_t)m * nn + n;
   int s = 0;
   for (; s + 4 <= splits; s += 4) {
@@ -305,9 +305,9 @@ __global__ __launch_bounds__(256) void w8a16_finish_kernel(FinishParams p) {
   const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
   const int m = blockIdx.y;
   if (n >= p.n) return;
-  float4 a = sum_splits(p.part0, p.scale0, p.splits, m, n, p.n);
+  float4 a = sum_splits(p.part0, p.scale0, p.splits, (size_t)p.stride, m, n, p.n);
   if (p.part1) {
-    const float4 u = sum_splits(p.part1, p.scale1, p.splits, m, n, p.n);
+    const float4 u = sum_splits(p.part1, p.scale1, p.splits, (size_t)p.stride, m, n, p.n);
     a = float4{silu_mul(a.x, u.x), silu_mul(a.y, u.y), silu_mul(a.z, u.z), silu_mul(a.w, u.w)};
   }
   const size_t idx = (size_t)m * p.n + n;
@@ -333,6 +333,7 @@ struct FinishNormParams {
   int n, splits, res_dtype, out_dtype;
   int out_blocked;
   float eps;
+  int64_t stride;  // elements between splits
 };
 
 __global__ __launch_bounds__(kNormThreads) void w8a16_finish_norm_kernel(FinishNormParams p) {
@@ -343,7 +344,7 @@ __global__ __launch_bounds__(kNormThreads) void w8a16_finish_norm_kernel(FinishN
   for (int u = 0; u < kNormVec; ++u) {
     const int n = (threadIdx.x + u * kNormThreads) * 4;
     if (n < p.n) {
-      float4 a = sum_splits(p.part, p.scale, p.splits, m, n, p.n);
+      float4 a = sum_splits(p.part, p.scale, p.splits, (size_t)p.stride, m, n, p.n);
       const float4 r = load4_as_f32(p.residual, (size_t)m * p.n + n, p.res_dtype);
       a.x += r.x; a.y += r.y; a.z += r.z; a.w += r.w;
       v[u] = a;
@@ -470,6 +471,8 @@ int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* w
   out->part[0] = p.part[0];
   out->part[1] = wq1 ? p.part[1] : nullptr;
   out->splits = p.splits;
+  out->slab_stride = (int64_t)kMaxM * n;
+  out->scaled = false;
   return PTO_HIP_OK;
 }
 
@@ -488,6 +491,7 @@ int w8a16_finish(const W8Partials& parts, const float* scale0, const float* scal
   f.res_dtype = res_dtype;
   f.out_dtype = out_dtype;
   f.out_blocked = out_blocked ? 1 : 0;
+  f.stride = parts.slab_stride;
   hipLaunchKernelGGL(w8a16_finish_kernel, dim3((unsigned)((n / 4 + 255) / 256), (unsigned)m), dim3(256), 0, st, f);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
@@ -511,6 +515,7 @@ int w8a16_finish_norm(const W8Partials& parts, const float* scale, const void* r
   f.out_dtype = out_dtype;
   f.out_blocked = out_blocked ? 1 : 0;
   f.eps = eps;
+  f.stride = parts.slab_stride;
   hipLaunchKernelGGL(w8a16_finish_norm_kernel, dim3((unsigned)m), dim3(kNormThreads), 0, st, f);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
