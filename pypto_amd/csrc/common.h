@@ -60,6 +60,7 @@ struct Context {
   int64_t attn_skip_merge = 0;
   int64_t attn_group_tiles = 0;  // cap on the query tiles one wavefront carries (0 = by group size)
   int64_t gemm_variant = 0;
+  int64_t gemm_splits = 0;       // k splits of the tiled GEMM: 0 = by shape, 1..16 = as given (when k allows)
   int64_t w8a16_wgs_per_cu = 1;  // workgroups of the W8A16 partial kernel aimed at per compute unit
   int64_t w8a16_wide = 1;        // int8 codes read 16 per lane: 0 never, 1 for large matrices, 2 whenever shapes allow
   int64_t w8a16_min_steps = 8;   // fewest 32-row steps per wavefront before k is split further

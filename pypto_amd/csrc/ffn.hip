@@ -490,13 +490,10 @@ int launch_variant(GemmParams p, hipStream_t st) {
   p.splits = 1;
   p.k_per_split = p.k;
   p.slabs = nullptr;
-  // variant 0 (default): eight wavefronts (two per SIMD) on a 256x256 tile; when that would leave
-  // CUs without a workgroup, either the 128x256 tile, with k split over up to 16 workgroups per
-  // tile while even the short tiles cover at most half of the CUs (a few hundred tokens), or -
-  // beyond 1024 rows, where the tall tile is well filled - the 256x256 tile with k split in up
-  // to four, whichever needs the fewest rounds of workgroups over the CUs (LLaMA-7B down pass at
-  // 2048 tokens: 128 tall tiles split in two 192 us, 256 short tiles 204 us).  Splits write fp32 slabs that a second kernel sums in
-  // split order.
+  // variant 0 (default): eight wavefronts (two per SIMD); up to 64 rows a 64x256 tile with k split
+  // over up to 16 workgroups per tile while CUs would idle, beyond that the 256x256 or the 128x256
+  // tile and the k split count with the least estimated time (below).  Splits write fp32 slabs
+  // that a second kernel sums in split order.
   // variants 1-3 keep four wavefronts (one per SIMD): 1 = 256x256 tile, 2 = 128x256 tile,
   // 3 = 256x256 tile with k split in two.  4 = eight wavefronts, 256x256 tile, k split in two
   // when CUs would idle.  5 = eight wavefronts, 128x256 tile.  6 = eight wavefronts, 64x256 tile, k split while CUs would idle.
@@ -505,20 +502,33 @@ int launch_variant(GemmParams p, hipStream_t st) {
   const int64_t small_tiles = (int64_t)((p.m + 127) / 128) * tiles_n;
   const bool few = big_tiles < num_cu;
   int want = 1;
-  bool small_tile = variant == 5 || (variant == 0 && few);
+  bool small_tile = variant == 5;
   if (variant == 3 || (variant == 4 && few)) want = 2;
-  if (variant == 0 && few) {
-    if (small_tiles * 2 <= num_cu) {
-      want = (int)std::min<int64_t>(kMaxSplits, num_cu / small_tiles);
-    } else if (p.m > 1024) {
-      // Time in units of one tall tile: rounds of workgroups over the CUs, a short tile costing
-      // 0.5 / 0.86 of a tall one (measured), a split launch about 0.05 more for its slabs.
-      double best = (double)((small_tiles + num_cu - 1) / num_cu) * (0.5 / 0.86);
-      for (int s = 1; s <= 4; ++s) {
-        const double cost = (double)((big_tiles * s + num_cu - 1) / num_cu) / s + (s > 1 ? 0.05 : 0.0);
-        if (cost < best) {
-          best = cost;
-          small_tile = false;
+  if (variant == 0 && p.m > 64) {
+    // Estimated time of each (tile height, k splits) pair, in microseconds, fitted to measured
+    // launches: rounds of workgroups over the CUs x the k rows one workgroup walks x the time per
+    // k row (a 256-row tile 18 ns when few CUs are busy up to 27.5 ns when all are, a 128-row
+    // tile 11 to 17.5 ns), not less than the weights take to stream from HBM; with k split, plus
+    // the finish launch and the slab traffic (slower once the slabs outgrow the last-level cache).
+    double best = 1e30;
+    const int mats = DUAL ? 2 : 1;
+    const double stream_us = (double)p.k * p.n * mats * (W8 ? 1 : 2) / 5.5e6;
+    for (int tall = 1; tall >= 0; --tall) {
+      const int64_t tiles = tall ? big_tiles : small_tiles;
+      for (int s = 1; s <= kMaxSplits; ++s) {
+        if (s > 1 && (p.k < 4 * BK * s || p.n % 4 != 0)) break;
+        const int64_t kps = ((p.k + s * BK - 1) / (s * BK)) * BK;
+        const int64_t real = (p.k + kps - 1) / kps;
+        if (real != s) continue;
+        const int64_t wgs = tiles * real, rounds = (wgs + num_cu - 1) / num_cu;
+        const double load = std::min(1.0, (double)wgs / (double)num_cu);
+        const double ns_row = tall ? 18.1 + 9.4 * load : 11.0 + 6.5 * load;
+        const double slab_mb = (double)real * p.m * p.n * mats * 4.0 / 1e6;  // written, then read back
+        const double t = std::max((double)rounds * (double)kps * ns_row * 1e-3, stream_us) +
+                         (real > 1 ? 7.0 + 2.0 * slab_mb / (slab_mb <= 128.0 ? 8.0 : 4.0) : 0.0);
+        if (t < best) {
+          best = t;
+          small_tile = !tall;
           want = s;
         }
       }
@@ -533,6 +543,7 @@ int launch_variant(GemmParams p, hipStream_t st) {
     small_tile = false;
     want = tiny_tiles * 2 <= num_cu ? (int)std::min<int64_t>(kMaxSplits, num_cu / tiny_tiles) : 1;
   }
+  if (pto_hip::ctx().gemm_splits > 0) want = (int)pto_hip::ctx().gemm_splits;
   if (want > 1 && p.k >= 4 * BK * want && p.n % 4 == 0) {
     p.k_per_split = ((p.k + want * BK - 1) / (want * BK)) * BK;
     p.splits = (p.k + p.k_per_split - 1) / p.k_per_split;

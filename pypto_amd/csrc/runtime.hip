@@ -791,6 +791,9 @@ int pto_hip_set_option(const char* name, int64_t value) {
   } else if (!std::strcmp(name, "gemm_variant")) {
     PTO_CHECK_ARG(value >= 0 && value <= 6, "gemm_variant must be in [0, 6]");
     c.gemm_variant = value;
+  } else if (!std::strcmp(name, "gemm_splits")) {
+    PTO_CHECK_ARG(value >= 0 && value <= 16, "gemm_splits must be in [0, 16]");
+    c.gemm_splits = value;
   } else if (!std::strcmp(name, "attn_group_tiles")) {
     PTO_CHECK_ARG(value == 0 || value == 1 || value == 2 || value == 4, "attn_group_tiles must be 0, 1, 2 or 4");
     c.attn_group_tiles = value;
@@ -825,6 +828,7 @@ int pto_hip_get_option(const char* name, int64_t* value) {
   Context& c = ctx();
   if (!std::strcmp(name, "attn_tokens_per_partition")) *value = c.attn_tokens_per_partition;
   else if (!std::strcmp(name, "gemm_variant")) *value = c.gemm_variant;
+  else if (!std::strcmp(name, "gemm_splits")) *value = c.gemm_splits;
   else if (!std::strcmp(name, "attn_waves_per_cu")) *value = c.attn_waves_per_cu;
   else if (!std::strcmp(name, "attn_skip_merge")) *value = c.attn_skip_merge;
   else if (!std::strcmp(name, "attn_variant")) *value = c.attn_variant;
