@@ -508,7 +508,7 @@ int launch_variant(GemmParams p, hipStream_t st) {
     // Estimated time of each (tile height, k splits) pair, in microseconds, fitted to measured
     // launches: rounds of workgroups over the CUs x the k rows one workgroup walks x the time per
     // k row (a 256-row tile 18 ns when few CUs are busy up to 27.5 ns when all are, a 128-row
-    // tile 11 to 17.5 ns), not less than the weights take to stream from HBM; with k split, plus
+    // tile 11 to 17.5 ns, int8 codes up to 4.5 ns more), not less than the weights take to stream from HBM; with k split, plus
     // the finish launch and the slab traffic (slower once the slabs outgrow the last-level cache).
     double best = 1e30;
     const int mats = DUAL ? 2 : 1;
@@ -522,7 +522,11 @@ int launch_variant(GemmParams p, hipStream_t st) {
         if (real != s) continue;
         const int64_t wgs = tiles * real, rounds = (wgs + num_cu - 1) / num_cu;
         const double load = std::min(1.0, (double)wgs / (double)num_cu);
-        const double ns_row = tall ? 18.1 + 9.4 * load : 11.0 + 6.5 * load;
+        // int8 codes: the widening is the same VALU work per k row for both heights; it shows once
+        // the launch is MFMA-bound (more than one round), and hides less well behind the short
+        // tile's fewer MFMAs
+        const double ns_row =
+            (tall ? 18.1 + 9.4 * load : 11.0 + 6.5 * load) + (W8 && rounds > 1 ? (tall ? 2.5 : 4.5) : 0.0);
         const double slab_mb = (double)real * p.m * p.n * mats * 4.0 / 1e6;  // written, then read back
         const double t = std::max((double)rounds * (double)kps * ns_row * 1e-3, stream_us) +
                          (real > 1 ? 7.0 + 2.0 * slab_mb / (slab_mb <= 128.0 ? 8.0 : 4.0) : 0.0);
