@@ -199,6 +199,34 @@ def test_projection_matches_oracle(worker, dtype, m, k, n):
     validate_golden({"out": out}, {"out": oracle.projection(x, w, res16)}, rtol=2e-3, atol=2e-3)
 
 
+@pytest.mark.parametrize("variant,splits", [(4, 1), (4, 3), (5, 1), (5, 5), (6, 2), (6, 16), (0, 7)])
+def test_every_tile_height_and_split_count_gives_the_same_product(worker, variant, splits):
+    """The launcher picks tile height and k splits from an estimated time; whatever it picks, the
+    result is the same product: each height with forced split counts (incl. more splits than k
+    allows, which falls back to fewer) on a shape ragged in every dimension."""
+    from pypto_amd.runtime import gate_up_swiglu, projection
+    m, k, n = 300, 1096, 1000
+    g = torch.Generator().manual_seed(variant * 31 + splits)
+    x = (torch.randn(m, k, generator=g) / k ** 0.5).to(torch.bfloat16)
+    w = torch.randn(k, n, generator=g).to(torch.bfloat16)
+    wu = torch.randn(k, n, generator=g).to(torch.bfloat16)
+    out = torch.zeros(m, n)
+    out16 = torch.zeros(m, n, dtype=torch.bfloat16)
+    worker.set_option("gemm_variant", variant)
+    worker.set_option("gemm_splits", splits)
+    try:
+        with worker.register(projection) as h:
+            h(x, w, out)
+        with worker.register(gate_up_swiglu) as h:
+            h(x, w, wu, out16)
+    finally:
+        worker.set_option("gemm_variant", 0)
+        worker.set_option("gemm_splits", 0)
+    validate_golden({"out": out}, {"out": oracle.projection(x, w)}, rtol=2e-3, atol=2e-3)
+    want = oracle.swiglu(oracle.projection(x, w), oracle.projection(x, wu)).to(torch.bfloat16)
+    validate_golden({"out": out16.float()}, {"out": want.float()}, rtol=1e-2, atol=1e-2)
+
+
 def test_projection_argument_rules(worker):
     from pypto_amd.runtime import projection
     x = torch.zeros(4, 64, dtype=torch.bfloat16)
