@@ -32,10 +32,17 @@ def _capture(worker, program, args, stream):
     return graph
 
 
-def test_decoder_layer_replays_follow_growing_sequences(worker):
-    batch = 6
+@pytest.mark.parametrize("batch", [6, 40])
+def test_decoder_layer_replays_follow_growing_sequences(worker, batch):
+    """Batch 6 takes the skinny projections, batch 40 the tiled GEMMs whose k-split slabs feed the
+    RoPE and RMSNorm kernels directly (a scratch area of their own)."""
+    if batch == 6:
+        ctxs = [100, 1, 250, 33, 60, 129]  # four more tokens stay inside each last block
+    else:
+        g0 = torch.Generator().manual_seed(21)
+        ctxs = (torch.randint(0, 5, (batch,), generator=g0) * 64 + torch.randint(1, 59, (batch,), generator=g0)).tolist()
     inp = workloads.decoder_layer_inputs(batch=batch, hidden=1024, num_heads=8, kv_head_num=2, head_dim=128,
-                                         intermediate=2816, block_size=64, context_lens=[100, 1, 250, 33, 60, 129], seed=11)  # four more tokens stay inside each last block
+                                         intermediate=2816, block_size=64, context_lens=ctxs, seed=11)
     args = _cuda(inp.args())
     hidden, seq_lens, key_cache, value_cache, out = args[0], args[1], args[3], args[4], args[19]
     assert out.shape == hidden.shape
@@ -64,7 +71,7 @@ def test_decoder_layer_replays_follow_growing_sequences(worker):
         assert torch.isfinite(out.float()).all()
         assert torch.equal(out, twin[19]), f"replay {step} differs from the eager step"
         assert torch.equal(key_cache, twin[3]) and torch.equal(value_cache, twin[4])
-    assert int(seq_lens[0]) == 104
+    assert int(seq_lens[0]) == ctxs[0] + 4
 
 
 def test_attention_and_ffn_replays(worker):
