@@ -41,7 +41,6 @@ FLAGS = [
 # (they are rescaled by VALU code every chunk); the GEMM keeps the default AGPR form.
 EXTRA_FLAGS = {
     "paged_attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
-    "paged_attention_fp8.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
 }
 
 

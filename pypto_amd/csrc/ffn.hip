@@ -29,572 +29,19 @@
 
 #include "common.h"
 
+#include "gemm.h"
+
 namespace {
 
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
-typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
-typedef short v4s __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) v4s lds_v4s;
-
-constexpr int BK = 64;        // k extent of one LDS tile
-constexpr int LDK = BK + 8;   // padded LDS row, in 16-bit elements (144 bytes)
-constexpr int BN = 256;       // LDS columns per tile
-constexpr int LDN = BN + 32;  // padded LDS row of the B tile, in elements (576 bytes)
-constexpr int kXcds = 8;
-
-struct GemmParams {
-  const uint16_t* a;   // [M, K]
-  const uint16_t* b0;  // [K, N]
-  const uint16_t* b1;  // [K, N] second operand of the gate/up pass
-  void* c;             // [M, N]
-  int64_t lda, ldb, ldc;
-  int m, n, k;
-  int tiles_m, tiles_n;
-  int splits, k_per_split;  // split-K: each split writes its own fp32 slab, a second kernel sums them
-  float* slabs;             // [splits][DUAL ? 2 : 1][m][n] when splits > 1
-  const void* residual;     // optional [m, n] added to the product (single-operand pass only)
-  int res_dtype;
-  const float* scale0;      // int8 weight codes: one scale per output column of b0 (and b1); else null
-  const float* scale1;
-  pto_hip::W8Partials* partials_out;  // non-null: leave the k-split slabs unsummed and describe them here
-};
-
-__device__ __forceinline__ float load_residual(const void* r, int dt, int64_t i) {
-  if (dt == PTO_HIP_FP32) return reinterpret_cast<const float*>(r)[i];
-  if (dt == PTO_HIP_BF16) return (float)reinterpret_cast<const __bf16*>(r)[i];
-  return (float)reinterpret_cast<const _Float16*>(r)[i];
-}
-
-template <bool BF16>
-__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
-  if constexpr (BF16) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-  } else {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-  }
-}
-
-template <typename OutT>
-__device__ __forceinline__ void store_out(OutT* p, float v) { *p = (OutT)v; }
-
-// Sigmoid in the device form of the reference, recip(1 + exp(-g)) (01_ffn.py:70-74).
-__device__ __forceinline__ float silu(float g) { return g * __frcp_rn(1.f + __expf(-g)); }
-
-// Two small integers held as fp32 -> packed pair of 16-bit floats, exact (|value| <= 128 has at most
-// 8 significant bits: the upper half of the fp32 pattern is its bf16).
-template <bool BF16>
-__device__ __forceinline__ uint32_t widen_pair(float lo, float hi) {
-  if constexpr (BF16)
-    return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, hi), __builtin_bit_cast(uint32_t, lo), 0x07060302u);
-  else
-    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
-}
-
-// Workgroup id -> tile id such that ids congruent mod 8 (one XCD) get a contiguous tile range.
-__device__ __forceinline__ int xcd_remap(int pid, int nwg) {
-  const int x = pid % kXcds, local = pid / kXcds;
-  const int full = nwg / kXcds, rem = nwg % kXcds;
-  const int base = x < rem ? x * (full + 1) : rem * (full + 1) + (x - rem) * full;
-  return base + local;
-}
-
-// EDGE = 0 assumes m, n, k are multiples of the tile.  EDGE = 1: only m is ragged - the A row
-// pointers are clamped once, the loop is the same.  EDGE = 2 clamps every address into the
-// operands (so all loads stay unconditional) and zeroes the A chunks that lie past k.
-// Wavefront grid WM x WN over the (32*MT*WM) x 256 tile: each wavefront owns (32*MT) x (32*NT)
-// as MT x NT accumulators, NT = 8 / WN.  2 x 2 wavefronts with 4 x 4 accumulators run one
-// wavefront per SIMD; 2 x 4 wavefronts with 4 x 2 accumulators run two per SIMD, so the MFMA pipe
-// has a second instruction stream to draw from while one waits on memory or a barrier.
-// W8: B holds int8 codes (a 16-byte chunk is 16 columns); they are widened to the activation type,
-// exactly, on their way into LDS, and the per-column scales are applied to the accumulators.
-template <int MT, int WM, int WN, bool DUAL, bool BF16, int EDGE, typename OutT, bool W8>
-__global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
-  constexpr int NBUF = 2;
-  constexpr int NT = (BN / 32) / WN;        // B fragments (32 columns each) per wavefront
-  constexpr int T = 64 * WM * WN;           // threads
-  constexpr int BM = 32 * MT * WM;
-  constexpr int NA = BM * 8 / T;            // 16-byte A chunks per thread and tile
-  constexpr int BCH = W8 ? 16 : 32;         // 16-byte B chunks per k row of the tile
-  constexpr int BCOLS = BN / BCH;           // columns per chunk: 8, or 16 int8 codes
-  constexpr int NB = BK * BCH / T;          // 16-byte B chunks per thread and tile
-  static_assert(NT >= 1 && (!DUAL || NT % 2 == 0), "gate/up pass needs gate and up columns in every wavefront");
-  constexpr int A_ELEMS = BM * LDK;
-  constexpr int B_ELEMS = BK * LDN;
-  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-  uint16_t* sa = smem;                      // [NBUF][BM][LDK]  rows = m, k contiguous
-  uint16_t* sb = smem + NBUF * A_ELEMS;     // [NBUF][BK][LDN]  rows = k, n contiguous (as in memory)
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int wm = wave % WM, wn = wave / WM;
-
-  const int ntiles = p.tiles_m * p.tiles_n;
-  const int logical = xcd_remap(blockIdx.x, ntiles * p.splits);
-  const int split = logical / ntiles, tile = logical % ntiles;
-  const int tm = tile % p.tiles_m, tn = tile / p.tiles_m;
-  const int k_begin = split * p.k_per_split;
-  const int klen = min(p.k, k_begin + p.k_per_split) - k_begin;  // this workgroup's k extent
-  const int m0 = tm * BM;
-  const int n0 = tn * (DUAL ? BN / 2 : BN);
-
-  // ---- global -> register staging ---------------------------------------------------
-  // A: thread owns 16-byte chunk (tid % 8) of rows tid/8 + (T/8)*i.
-  const int a_chunk = tid & 7, a_row = tid >> 3;
-  // B: thread owns 16-byte chunk (tid % 32) of k rows tid/32 + (T/32)*i; in the gate/up pass chunks
-  // 0..15 come from the gate weights and 16..31 from the up weights (same output columns).
-  const int b_chunk = tid % BCH, b_row = tid / BCH;
-  const uint16_t* bsrc;
-  int b_col;  // global column of the chunk
-  if (DUAL) {
-    bsrc = (b_chunk < BCH / 2) ? p.b0 : p.b1;
-    b_col = n0 + (b_chunk % (BCH / 2)) * BCOLS;
-  } else {
-    bsrc = p.b0;
-    b_col = n0 + b_chunk * BCOLS;
-  }
-  if (EDGE == 2) b_col = min(b_col, p.n - BCOLS);
-  constexpr int BESZ = W8 ? 1 : 2;  // bytes per B element
-  const uint16_t* a_ptr[NA];
-#pragma unroll
-  for (int i = 0; i < NA; ++i) {
-    int r = m0 + a_row + (T / 8) * i;
-    if (EDGE != 0) r = min(r, p.m - 1);
-    a_ptr[i] = p.a + (int64_t)r * p.lda + k_begin + a_chunk * 8;
-  }
-  const char* b_ptr = reinterpret_cast<const char*>(bsrc) + ((int64_t)(k_begin + b_row) * p.ldb + b_col) * BESZ;
-
-  u32x4 ra[NA];
-  u32x4 rb[NB];
-  auto load_a = [&](int k0, int i) {
-    if constexpr (EDGE == 2) {
-      const int ka = min(k0 + a_chunk * 8, klen - 8) - a_chunk * 8;  // clamped tile origin for A
-      const bool a_ok = k0 + a_chunk * 8 < klen;
-      u32x4 v = *reinterpret_cast<const u32x4*>(a_ptr[i] + ka);
-      u32x4 z = {0u, 0u, 0u, 0u};
-      ra[i] = a_ok ? v : z;
-    } else {
-      ra[i] = *reinterpret_cast<const u32x4*>(a_ptr[i] + k0);
-    }
-  };
-  auto load_b = [&](int k0, int i) {
-    if constexpr (EDGE == 2) {
-      const int kk = min(k0 + b_row + (T / BCH) * i, klen - 1) - b_row;
-      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)kk * p.ldb * BESZ);
-    } else {
-      rb[i] = *reinterpret_cast<const u32x4*>(b_ptr + (int64_t)(k0 + (T / BCH) * i) * p.ldb * BESZ);
-    }
-  };
-  // One B chunk from its registers into the LDS tile `db`: 16-bit weights as they are, int8 codes
-  // widened (16 codes -> two 16-byte writes).
-  auto store_b = [&](uint16_t* db, int i) {
-    uint16_t* dst = db + (b_row + (T / BCH) * i) * LDN + b_chunk * BCOLS;
-    if constexpr (W8) {
-      u32x4 lo, hi;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const uint32_t codes = rb[i][w];
-        const float f0 = (float)(int8_t)(codes), f1 = (float)(int8_t)(codes >> 8);
-        const float f2 = (float)(int8_t)(codes >> 16), f3 = (float)(int8_t)(codes >> 24);
-        const uint32_t p01 = widen_pair<BF16>(f0, f1), p23 = widen_pair<BF16>(f2, f3);
-        if (w < 2) {
-          lo[2 * w] = p01;
-          lo[2 * w + 1] = p23;
-        } else {
-          hi[2 * (w - 2)] = p01;
-          hi[2 * (w - 2) + 1] = p23;
-        }
-      }
-      *reinterpret_cast<u32x4*>(dst) = lo;
-      *reinterpret_cast<u32x4*>(dst + 8) = hi;
-    } else {
-      *reinterpret_cast<u32x4*>(dst) = rb[i];
-    }
-  };
-  auto load_tile = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < NA; ++i) load_a(k0, i);
-#pragma unroll
-    for (int i = 0; i < NB; ++i) load_b(k0, i);
-  };
-  auto store_tile = [&](int buf) {
-    uint16_t* da = sa + buf * A_ELEMS;
-#pragma unroll
-    for (int i = 0; i < NA; ++i)
-      *reinterpret_cast<u32x4*>(da + (a_row + (T / 8) * i) * LDK + a_chunk * 8) = ra[i];
-    uint16_t* db = sb + buf * B_ELEMS;
-#pragma unroll
-    for (int i = 0; i < NB; ++i) store_b(db, i);
-  };
-
-  f32x16 acc[MT][NT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int jn = 0; jn < NT; ++jn)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][jn][r] = 0.f;
-
-  // Operand fragments of v_mfma_f32_32x32x16: lane l holds row/column l%32, k = 8*(l/32)..+8.
-  //  A: one 16-byte read from its m-row.
-  //  B: two transposing reads.  In each group of 16 lanes, lane s supplies the address of 4
-  //     consecutive n of k-row s/4 (columns (s%4)*4..); the hardware hands lane c of the group
-  //     the four k-values of column c.  Lanes 16..31 take the next 16 columns, lanes 32..63 the
-  //     next 8 k-rows.
-  const int a_frag = (wm * MT * 32 + (lane & 31)) * LDK + (lane >> 5) * 8;
-  const int grp = lane >> 4, sub = lane & 15;
-  int b_frag[NT];
-#pragma unroll
-  for (int jn = 0; jn < NT; ++jn) {
-    // gate/up pass: the first NT/2 fragments are gate columns, the rest the up columns of the same outputs
-    const int col = DUAL ? ((jn / (NT / 2)) * (BN / 2) + wn * (16 * NT) + (jn % (NT / 2)) * 32)
-                         : (wn * (32 * NT) + jn * 32);
-    b_frag[jn] = ((grp >> 1) * 8 + (sub >> 2)) * LDN + col + (grp & 1) * 16 + (sub & 3) * 4;
-  }
-
-  // One LDS read of the fragment set for k-step `ks` of buffer `buf`: r < MT reads A fragment r,
-  // the rest read half (4 k-rows) of a B fragment.
-  u32x4 fa[2][MT], fb[2][NT];
-  auto read_one = [&](int buf, int ks, int set, int r) {
-    if (r < MT) {
-      fa[set][r] = *reinterpret_cast<const u32x4*>(sa + buf * A_ELEMS + a_frag + ks * 16 + r * 32 * LDK);
-    } else {
-      const int jn = (r - MT) >> 1, half = (r - MT) & 1;
-      const uint16_t* src = sb + buf * B_ELEMS + (ks * 16 + half * 4) * LDN + b_frag[jn];
-      const uint2 v = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)src));
-      fb[set][jn][half * 2 + 0] = v.x;
-      fb[set][jn][half * 2 + 1] = v.y;
-    }
-  };
-  constexpr int kReads = MT + 2 * NT;                         // LDS reads per k-step
-  constexpr int kSlots = MT * NT;                             // MFMAs per k-step
-  constexpr int kMovesPerSlot = ((NA > NB ? NA : NB) + kSlots - 1) / kSlots;  // LDS writes / global loads per slot
-  constexpr int kReadsPerSlot = (kReads + kSlots - 1) / kSlots;
-  constexpr int kSteps = BK / 16;
-
-  // Main loop, one iteration per k-tile.  Registers ra/rb hold tile kt+1 on entry.  The MFMAs of
-  // k-step ks are interleaved with the LDS reads of the fragments for ks+1 and, in turn, with
-  // the LDS writes of tile kt+1 (k-steps 0-1) and the global loads of tile kt+2 (k-steps 2-3),
-  // so each MFMA issues next to at most a few memory instructions.  sched_barrier pins that
-  // order.  All loads are unconditional (past the end they re-read the last tile, a cache hit)
-  // so the number of requests outstanding at each wait is known at compile time.
-  const int nk = (klen + BK - 1) / BK;
-  load_tile(0);
-  store_tile(0);
-  load_tile(min(1, nk - 1) * BK);
-  __syncthreads();
-#pragma unroll
-  for (int r = 0; r < kReads; ++r) read_one(0, 0, 0, r);
-
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    const int k_next = min(kt + 2, nk - 1) * BK;
-    uint16_t* da = sa + (buf ^ 1) * A_ELEMS;
-    uint16_t* db = sb + (buf ^ 1) * B_ELEMS;
-#pragma unroll
-    for (int ks = 0; ks < kSteps; ++ks) {
-#pragma unroll
-      for (int q = 0; q < kSlots; ++q) {
-        const int i = q / NT, jn = q % NT;
-        acc[i][jn] = mfma32<BF16>(fa[ks & 1][i], fb[ks & 1][jn], acc[i][jn]);
-        if (ks + 1 < kSteps) {
-#pragma unroll
-          for (int r = q * kReadsPerSlot; r < (q + 1) * kReadsPerSlot; ++r)
-            if (r < kReads) read_one(buf, ks + 1, (ks + 1) & 1, r);
-        }
-#pragma unroll
-        for (int e = q * kMovesPerSlot; e < (q + 1) * kMovesPerSlot; ++e) {
-          if (ks == 0 && e < NA)
-            *reinterpret_cast<u32x4*>(da + (a_row + (T / 8) * e) * LDK + a_chunk * 8) = ra[e];
-          if (ks == 1 && e < NB) store_b(db, e);
-          if (ks == 2 && e < NA) load_a(k_next, e);
-          if (ks == 3 && e < NB) load_b(k_next, e);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < kReads; ++r) read_one(buf ^ 1, 0, 0, r);
-  }
-
-  // ---- epilogue ------------------------------------------------------------------------
-  // acc[i][jn][r]: row = m0 + wm*MT*32 + i*32 + (r/4)*8 + (lane/32)*4 + r%4, col = lane%32 + ...
-  OutT* c = reinterpret_cast<OutT*>(p.c);
-  const int row_base = m0 + wm * MT * 32 + (lane >> 5) * 4;
-  float sc[NT];  // int8 weight codes: the scale of each of this lane's columns
-  if constexpr (W8) {
-#pragma unroll
-    for (int jn = 0; jn < NT; ++jn) {
-      const int col = DUAL ? n0 + wn * (16 * NT) + (jn % (NT / 2)) * 32 + (lane & 31)
-                           : n0 + wn * (32 * NT) + jn * 32 + (lane & 31);
-      const float* s = (DUAL && jn >= NT / 2) ? p.scale1 : p.scale0;
-      sc[jn] = col < p.n ? s[col] : 0.f;
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < MT; ++i) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = row_base + i * 32 + (r >> 2) * 8 + (r & 3);
-      if (row >= p.m) continue;
-      const int64_t mn = (int64_t)p.m * p.n;
-      if constexpr (DUAL) {
-#pragma unroll
-        for (int jn = 0; jn < NT / 2; ++jn) {
-          const int col = n0 + wn * (16 * NT) + jn * 32 + (lane & 31);
-          if (col < p.n) {
-            if (p.splits > 1) {
-              float* s = p.slabs + (int64_t)split * 2 * mn + (int64_t)row * p.n + col;
-              s[0] = acc[i][jn][r];
-              s[mn] = acc[i][jn + NT / 2][r];
-            } else {
-              float g = acc[i][jn][r], u = acc[i][jn + NT / 2][r];
-              if constexpr (W8) {
-                g *= sc[jn];
-                u *= sc[jn + NT / 2];
-              }
-              store_out<OutT>(c + (int64_t)row * p.ldc + col, silu(g) * u);
-            }
-          }
-        }
-      } else {
-#pragma unroll
-        for (int jn = 0; jn < NT; ++jn) {
-          const int col = n0 + wn * (32 * NT) + jn * 32 + (lane & 31);
-          if (col < p.n) {
-            if (p.splits > 1) {
-              p.slabs[(int64_t)split * mn + (int64_t)row * p.n + col] = acc[i][jn][r];
-            } else {
-              float v = acc[i][jn][r];
-              if constexpr (W8) v *= sc[jn];
-              if (p.residual) v += load_residual(p.residual, p.res_dtype, (int64_t)row * p.n + col);
-              store_out<OutT>(c + (int64_t)row * p.ldc + col, v);
-            }
-          }
-        }
-      }
-    }
-  }
-}
-
-
-template <int MT, int WM, int WN, bool DUAL, bool BF16, int EDGE, typename OutT, bool W8>
-int launch_gemm_e(GemmParams p, hipStream_t st) {
-  constexpr int BM = 32 * MT * WM;
-  constexpr int NBUF = 2;
-  p.tiles_m = (p.m + BM - 1) / BM;
-  const int bn_out = DUAL ? BN / 2 : BN;
-  p.tiles_n = (p.n + bn_out - 1) / bn_out;
-  const size_t smem = (size_t)NBUF * (BM * LDK + BK * LDN) * sizeof(uint16_t);
-  auto kern = gemm_kernel<MT, WM, WN, DUAL, BF16, EDGE, OutT, W8>;
-  static bool attr_set = false;  // per instantiation
-  if (!attr_set) {
-    PTO_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    attr_set = true;
-  }
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(64 * WM * WN), smem, st, p);
-  PTO_CHECK_HIP(hipGetLastError());
-  return PTO_HIP_OK;
-}
-
-template <int MT, int WM, int WN, bool DUAL, bool BF16, typename OutT, bool W8 = false>
-int launch_gemm(GemmParams p, hipStream_t st) {
-  constexpr int BM_ = 32 * MT * WM;
-  const bool edge = p.n % (DUAL ? BN / 2 : BN) != 0 || p.k % BK != 0 || (p.splits > 1 && p.k_per_split % BK != 0);
-  if (edge) return launch_gemm_e<MT, WM, WN, DUAL, BF16, 2, OutT, W8>(p, st);
-  if (p.m % BM_ != 0) return launch_gemm_e<MT, WM, WN, DUAL, BF16, 1, OutT, W8>(p, st);
-  return launch_gemm_e<MT, WM, WN, DUAL, BF16, 0, OutT, W8>(p, st);
-}
-
-// Sum of the split-K slabs in split order (so the result does not depend on which workgroup
-// finished first), then SwiGLU for the gate/up pass, cast and store.  n is a multiple of 4.
-constexpr int kMaxSplits = 16;
-constexpr int kSplitBatch = 8;  // slabs loaded before the first add
-template <bool DUAL, typename OutT>
-__global__ __launch_bounds__(256) void gemm_finish_kernel(const float* slabs, OutT* c, int64_t ldc, int m, int n,
-                                                          int splits, const void* residual, int res_dtype,
-                                                          const float* scale0, const float* scale1) {
-  const int nq = n / 4;
-  const int64_t quads = (int64_t)m * nq, mn = (int64_t)m * n;
-  constexpr int kMats = DUAL ? 2 : 1;
-  for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < quads; q += (int64_t)gridDim.x * 256) {
-    const int64_t row = q / nq;
-    const int col = (int)(q % nq) * 4;
-    const float* src = slabs + row * n + col;
-    float4 t[kMats];
-#pragma unroll
-    for (int mat = 0; mat < kMats; ++mat) t[mat] = float4{0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < splits; s0 += kSplitBatch) {
-      float4 v[kSplitBatch][kMats];
-#pragma unroll
-      for (int sp = 0; sp < kSplitBatch; ++sp)
-#pragma unroll
-        for (int mat = 0; mat < kMats; ++mat)
-          v[sp][mat] = *reinterpret_cast<const float4*>(src + ((int64_t)min(s0 + sp, splits - 1) * kMats + mat) * mn);
-#pragma unroll
-      for (int mat = 0; mat < kMats; ++mat)
-#pragma unroll
-        for (int sp = 0; sp < kSplitBatch; ++sp)
-          if (s0 + sp < splits) {
-            t[mat].x += v[sp][mat].x;
-            t[mat].y += v[sp][mat].y;
-            t[mat].z += v[sp][mat].z;
-            t[mat].w += v[sp][mat].w;
-          }
-    }
-    if (scale0) {  // int8 weight codes: per-column scales
-      const float4 s0 = *reinterpret_cast<const float4*>(scale0 + col);
-      t[0] = float4{t[0].x * s0.x, t[0].y * s0.y, t[0].z * s0.z, t[0].w * s0.w};
-      if constexpr (DUAL) {
-        const float4 s1 = *reinterpret_cast<const float4*>(scale1 + col);
-        t[1] = float4{t[1].x * s1.x, t[1].y * s1.y, t[1].z * s1.z, t[1].w * s1.w};
-      }
-    }
-    float4 y = t[0];
-    if constexpr (DUAL) y = float4{silu(t[0].x) * t[1].x, silu(t[0].y) * t[1].y, silu(t[0].z) * t[1].z, silu(t[0].w) * t[1].w};
-    if (!DUAL && residual) {
-      const int64_t r0 = row * n + col;
-      y.x += load_residual(residual, res_dtype, r0);
-      y.y += load_residual(residual, res_dtype, r0 + 1);
-      y.z += load_residual(residual, res_dtype, r0 + 2);
-      y.w += load_residual(residual, res_dtype, r0 + 3);
-    }
-    OutT* dst = c + row * ldc + col;
-    store_out<OutT>(dst + 0, y.x);
-    store_out<OutT>(dst + 1, y.y);
-    store_out<OutT>(dst + 2, y.z);
-    store_out<OutT>(dst + 3, y.w);
-  }
-}
-
-template <bool DUAL, typename OutT>
-int launch_finish(const GemmParams& p, hipStream_t st) {
-  const int64_t quads = (int64_t)p.m * (p.n / 4);
-  const unsigned blocks = (unsigned)std::min<int64_t>((quads + 255) / 256, 4096);
-  hipLaunchKernelGGL((gemm_finish_kernel<DUAL, OutT>), dim3(blocks), dim3(256), 0, st, p.slabs,
-                     reinterpret_cast<OutT*>(p.c), p.ldc, p.m, p.n, p.splits, p.residual, p.res_dtype, p.scale0,
-                     p.scale1);
-  PTO_CHECK_HIP(hipGetLastError());
-  return PTO_HIP_OK;
-}
-
-template <bool DUAL, bool BF16, typename OutT, bool W8 = false>
-int launch_variant(GemmParams p, hipStream_t st) {
-  const int64_t variant = pto_hip::ctx().gemm_variant;
-  const int64_t num_cu = pto_hip::ctx().num_cu;
-  p.splits = 1;
-  p.k_per_split = p.k;
-  p.slabs = nullptr;
-  // variant 0 (default): eight wavefronts (two per SIMD); up to 64 rows a 64x256 tile with k split
-  // over up to 16 workgroups per tile while CUs would idle, beyond that the 256x256 or the 128x256
-  // tile and the k split count with the least estimated time (below).  Splits write fp32 slabs
-  // that a second kernel sums in split order.
-  // variants 1-3 keep four wavefronts (one per SIMD): 1 = 256x256 tile, 2 = 128x256 tile,
-  // 3 = 256x256 tile with k split in two.  4 = eight wavefronts, 256x256 tile, k split in two
-  // when CUs would idle.  5 = eight wavefronts, 128x256 tile.  6 = eight wavefronts, 64x256 tile, k split while CUs would idle.
-  const int64_t tiles_n = (p.n + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256);
-  const int64_t big_tiles = (int64_t)((p.m + 255) / 256) * tiles_n;
-  const int64_t small_tiles = (int64_t)((p.m + 127) / 128) * tiles_n;
-  const bool few = big_tiles < num_cu;
-  int want = 1;
-  bool small_tile = variant == 5;
-  if (variant == 3 || (variant == 4 && few)) want = 2;
-  if (variant == 0 && p.m > 64) {
-    // Estimated time of each (tile height, k splits) pair, in microseconds, fitted to measured
-    // launches: rounds of workgroups over the CUs x the k rows one workgroup walks x the time per
-    // k row (a 256-row tile 18 ns when few CUs are busy up to 27.5 ns when all are, a 128-row
-    // tile 11 to 17.5 ns, int8 codes up to 4.5 ns more), not less than the weights take to stream from HBM; with k split, plus
-    // the finish launch and the slab traffic (slower once the slabs outgrow the last-level cache).
-    double best = 1e30;
-    const int mats = DUAL ? 2 : 1;
-    const double stream_us = (double)p.k * p.n * mats * (W8 ? 1 : 2) / 5.5e6;
-    for (int tall = 1; tall >= 0; --tall) {
-      const int64_t tiles = tall ? big_tiles : small_tiles;
-      for (int s = 1; s <= kMaxSplits; ++s) {
-        if (s > 1 && (p.k < 4 * BK * s || p.n % 4 != 0)) break;
-        const int64_t kps = ((p.k + s * BK - 1) / (s * BK)) * BK;
-        const int64_t real = (p.k + kps - 1) / kps;
-        if (real != s) continue;
-        const int64_t wgs = tiles * real, rounds = (wgs + num_cu - 1) / num_cu;
-        const double load = std::min(1.0, (double)wgs / (double)num_cu);
-        // int8 codes: the widening is the same VALU work per k row for both heights; it shows once
-        // the launch is MFMA-bound (more than one round), and hides less well behind the short
-        // tile's fewer MFMAs
-        const double ns_row =
-            (tall ? 18.1 + 9.4 * load : 11.0 + 6.5 * load) + (W8 && rounds > 1 ? (tall ? 2.5 : 4.5) : 0.0);
-        const double slab_mb = (double)real * p.m * p.n * mats * 4.0 / 1e6;  // written, then read back
-        const double t = std::max((double)rounds * (double)kps * ns_row * 1e-3, stream_us) +
-                         (real > 1 ? 7.0 + 2.0 * slab_mb / (slab_mb <= 128.0 ? 8.0 : 4.0) : 0.0);
-        if (t < best) {
-          best = t;
-          small_tile = !tall;
-          want = s;
-        }
-      }
-    }
-  }
-  // Up to 64 rows: a 64-row tile.  With the 128-row tile the MFMA work on its padding rows, not
-  // the weight stream, set the time for int8 codes (half the bytes of 16-bit weights: decoder
-  // layer at batch 64 205 -> 177 us) and still cost 2-5 % with 16-bit weights.
-  const bool tiny_tile = variant == 6 || (variant == 0 && p.m <= 64);
-  if (tiny_tile) {
-    const int64_t tiny_tiles = (int64_t)((p.m + 63) / 64) * tiles_n;
-    small_tile = false;
-    want = tiny_tiles * 2 <= num_cu ? (int)std::min<int64_t>(kMaxSplits, num_cu / tiny_tiles) : 1;
-  }
-  if (pto_hip::ctx().gemm_splits > 0) want = (int)pto_hip::ctx().gemm_splits;
-  if (want > 1 && p.k >= 4 * BK * want && p.n % 4 == 0) {
-    p.k_per_split = ((p.k + want * BK - 1) / (want * BK)) * BK;
-    p.splits = (p.k + p.k_per_split - 1) / p.k_per_split;
-    if (p.splits > 1) {
-      void* ws = nullptr;
-      const int rc = pto_hip::gemm_workspace((size_t)p.splits * (DUAL ? 2 : 1) * p.m * p.n * sizeof(float), &ws);
-      if (rc) return rc;
-      p.slabs = reinterpret_cast<float*>(ws);
-    }
-  }
-  int rc;
-  if (tiny_tile) rc = launch_gemm<1, 2, 4, DUAL, BF16, OutT, W8>(p, st);
-  else if (small_tile) rc = launch_gemm<2, 2, 4, DUAL, BF16, OutT, W8>(p, st);
-  else if (variant == 0 || variant == 4) rc = launch_gemm<4, 2, 4, DUAL, BF16, OutT, W8>(p, st);
-  else if constexpr (W8) return pto_hip::fail(PTO_HIP_ERR_UNSUPPORTED, "gemm_variant %lld has no int8-weight form",
-                                              (long long)variant);
-  else if (variant == 2) rc = launch_gemm<2, 2, 2, DUAL, BF16, OutT>(p, st);
-  else rc = launch_gemm<4, 2, 2, DUAL, BF16, OutT>(p, st);
-  if (rc) return rc;
-  if (p.partials_out) {  // a fused consumer sums the slabs (one split: the product is in p.c, scales applied)
-    pto_hip::W8Partials& o = *p.partials_out;
-    o.part[0] = p.splits > 1 ? p.slabs : reinterpret_cast<float*>(p.c);
-    o.part[1] = nullptr;
-    o.splits = p.splits;
-    o.slab_stride = (int64_t)p.m * p.n;
-    o.scaled = p.splits == 1;
-    return PTO_HIP_OK;
-  }
-  if (p.splits == 1) return rc;
-  return launch_finish<DUAL, OutT>(p, st);
-}
+using namespace pto_hip::gemm;
 
 template <bool DUAL>
 int launch_typed(const GemmParams& p, int dtype, int out_dtype, hipStream_t st) {
-  const bool bf16 = dtype == PTO_HIP_BF16;
-  if (p.scale0) {  // int8 weight codes
-    if (out_dtype == PTO_HIP_FP32)
-      return bf16 ? launch_variant<DUAL, true, float, true>(p, st) : launch_variant<DUAL, false, float, true>(p, st);
-    if (out_dtype == PTO_HIP_BF16 && bf16) return launch_variant<DUAL, true, __bf16, true>(p, st);
-    if (out_dtype == PTO_HIP_FP16 && !bf16) return launch_variant<DUAL, false, _Float16, true>(p, st);
-  }
-  if (out_dtype == PTO_HIP_FP32)
-    return bf16 ? launch_variant<DUAL, true, float>(p, st) : launch_variant<DUAL, false, float>(p, st);
-  if (out_dtype == PTO_HIP_BF16 && bf16) return launch_variant<DUAL, true, __bf16>(p, st);
-  if (out_dtype == PTO_HIP_FP16 && !bf16) return launch_variant<DUAL, false, _Float16>(p, st);
-  return pto_hip::fail(PTO_HIP_ERR_INVALID_VALUE, "ffn: output dtype %s must be FP32 or the input dtype %s",
-                       pto_hip::dtype_name(out_dtype), pto_hip::dtype_name(dtype));
+  if (p.scale0)  // int8 weight codes
+    return DUAL ? pto_hip::gemm_launch_w8_dual(p, dtype, out_dtype, st)
+                : pto_hip::gemm_launch_w8_single(p, dtype, out_dtype, st);
+  return DUAL ? pto_hip::gemm_launch_w16_dual(p, dtype, out_dtype, st)
+              : pto_hip::gemm_launch_w16_single(p, dtype, out_dtype, st);
 }
 
 // ---- fp32 operands: the reference's 64x64 teaching example (01_ffn.py:155-160) ---------------
