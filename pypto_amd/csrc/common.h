@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -68,6 +69,13 @@ struct Context {
 };
 
 Context& ctx();
+// Host-side state (the scratch areas and their growth, the options, launch attributes set on first
+// use) is shared by every caller, and a program's launches use the shared scratch areas in stream
+// order.  Every entry point that sizes scratch or launches holds this lock for the duration of the
+// call, so host threads take turns; it is recursive because pto_hip_run dispatches to the typed
+// entry points.  The lock orders host work only: two streams still share one scratch area.
+std::recursive_mutex& dispatch_mutex();
+#define PTO_DISPATCH_LOCK() std::lock_guard<std::recursive_mutex> pto_dispatch_lock_(::pto_hip::dispatch_mutex())
 // Returns a workspace of at least `bytes`.  A request beyond the current size allocates a new
 // buffer of at least twice the old size and retires the old one without freeing it, so that
 // queued work and launches recorded into a HIP graph stay valid; it fails while a stream is

@@ -164,6 +164,7 @@ extern "C" int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void*
                                   const void* w_up, const void* w_down, void* out, int64_t tokens,
                                   int64_t hidden, int64_t intermediate, float eps, int dtype,
                                   int out_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
   using namespace pto_hip;
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(tokens >= 0 && hidden > 0 && intermediate > 0, "ffn: bad shape T=%lld H=%lld I=%lld",
@@ -253,6 +254,7 @@ extern "C" int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void*
 // skinny projection kernels; more rows go through the tiled GEMM.
 extern "C" int pto_hip_projection(const void* x, const void* w, const void* residual, void* out, int64_t m,
                                   int64_t k, int64_t n, int dtype, int res_dtype, int out_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
   using namespace pto_hip;
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(m >= 0 && k > 0 && n > 0 && m < (1 << 30) && k < (1 << 30) && n < (1 << 30),
@@ -299,6 +301,7 @@ extern "C" int pto_hip_projection(const void* x, const void* w, const void* resi
 // Same two regimes as pto_hip_projection.
 extern "C" int pto_hip_gate_up_swiglu(const void* x, const void* w_gate, const void* w_up, void* out, int64_t m,
                                       int64_t k, int64_t n, int dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
   using namespace pto_hip;
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(m >= 0 && k > 0 && n > 0 && m < (1 << 30) && k < (1 << 30) && n < (1 << 30),

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 
 #include "common.h"
 
@@ -371,11 +372,11 @@ int launch_gemm_e(GemmParams p, hipStream_t st) {
   p.tiles_n = (p.n + bn_out - 1) / bn_out;
   const size_t smem = (size_t)NBUF * (BM * LDK + BK * LDN) * sizeof(uint16_t);
   auto kern = gemm_kernel<MT, WM, WN, DUAL, BF16, EDGE, OutT, W8>;
-  static bool attr_set = false;  // per instantiation
-  if (!attr_set) {
+  static std::atomic<bool> attr_set{false};  // per instantiation; callers hold the dispatch lock
+  if (!attr_set.load(std::memory_order_acquire)) {
     PTO_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    attr_set = true;
+    attr_set.store(true, std::memory_order_release);
   }
   hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(64 * WM * WN), smem, st, p);
   PTO_CHECK_HIP(hipGetLastError());

@@ -97,6 +97,7 @@ int layer_large_batch(const PtoHipDecoderLayerArgs* a, int rope_w, void* stream)
 }  // namespace
 
 extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, void* stream) {
+  PTO_DISPATCH_LOCK();
   using namespace pto_hip;
   Context& cx = ctx();
   if (!cx.initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");

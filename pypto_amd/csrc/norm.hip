@@ -159,6 +159,7 @@ int rms_norm_blocked(const void* x, const float* gamma, void* out, int64_t rows,
 
 extern "C" int pto_hip_rms_norm(const void* x, const float* gamma, void* out, int64_t rows,
                                 int64_t hidden, float eps, int x_dtype, int out_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
   using namespace pto_hip;
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(rows >= 0 && hidden > 0, "rms_norm: bad shape [%lld, %lld]", (long long)rows, (long long)hidden);

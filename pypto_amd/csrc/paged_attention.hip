@@ -16,7 +16,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
-
+#include <atomic>
 #include <type_traits>
 
 #include "common.h"
@@ -901,11 +901,12 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
     const size_t lean_lds = std::max<size_t>((size_t)p.lean_waves * KStage<D, FP8>::kBytes, 84 * 1024);
     dim3 lgrid(p.n_wg), lblock(p.lean_waves * 64);
     auto go = [&](auto kern) -> int {
-      static bool attr_set = false;  // per instantiation
-      if (!attr_set) {
+      // per instantiation; setting the attribute twice from two threads is harmless
+      static std::atomic<bool> attr_set{false};
+      if (!attr_set.load(std::memory_order_acquire)) {
         PTO_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
       }
       hipLaunchKernelGGL(kern, lgrid, lblock, lean_lds, stream, p);
       return PTO_HIP_OK;
@@ -1102,6 +1103,7 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
                                        const int32_t* context_lens, float* out,
                                        const int64_t* config, int q_dtype, int kv_dtype,
                                        const float* k_scale, const float* v_scale, void* stream) {
+  PTO_DISPATCH_LOCK();
   // The size of the caches is not part of this signature: table entries are used as given.
   return pto_hip::paged_attention(query, key_cache, value_cache, block_table, context_lens, out, nullptr, false, nullptr, config,
                                   q_dtype, kv_dtype, k_scale, v_scale, 0, stream);

@@ -78,6 +78,7 @@ extern "C" int pto_hip_paged_gather(const void* src, const int32_t* indices,
                                     int64_t src_rows, int64_t src_hidden, int64_t table_len,
                                     int64_t block_size, int64_t col_offset, int64_t size,
                                     int elem_bytes, void* stream) {
+  PTO_DISPATCH_LOCK();
   using namespace pto_hip;
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   // Argument rules of the op's type deduction (paged_gather.cpp:129-147).

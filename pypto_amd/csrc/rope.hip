@@ -368,6 +368,7 @@ extern "C" int pto_hip_rope_kv_cache_update_fp8(const float* qkv, const int32_t*
                                                 int64_t kv_head_num, int64_t head_dim, int64_t block_size,
                                                 int64_t max_num_blocks_per_req, int64_t max_pos,
                                                 int64_t pool_blocks, int q_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
   return pto_hip::rope_kv_cache_update_fp8(qkv, nullptr, 1, 0, seq_lens, rope_cos, rope_sin, block_table, key_cache,
                                            value_cache, k_scale, v_scale, q_out, batch, num_heads, kv_head_num,
                                            head_dim, block_size, max_num_blocks_per_req, max_pos, (int)(head_dim / 2),
@@ -380,6 +381,7 @@ extern "C" int pto_hip_rope_kv_cache_update(const float* qkv, const int32_t* seq
                                             int64_t num_heads, int64_t kv_head_num, int64_t head_dim,
                                             int64_t block_size, int64_t max_num_blocks_per_req,
                                             int64_t max_pos, int64_t pool_rows, int dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
   return pto_hip::rope_kv_cache_update(qkv, nullptr, 1, 0, seq_lens, rope_cos, rope_sin, block_table, key_cache,
                                        value_cache, q_out, batch, num_heads, kv_head_num, head_dim, block_size,
                                        max_num_blocks_per_req, max_pos, (int)(head_dim / 2), pool_rows, dtype, stream);

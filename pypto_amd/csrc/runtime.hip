@@ -7,6 +7,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -33,6 +34,11 @@ int fail(int status, const char* fmt, ...) {
 Context& ctx() {
   static Context c;
   return c;
+}
+
+std::recursive_mutex& dispatch_mutex() {
+  static std::recursive_mutex mu;
+  return mu;
 }
 
 namespace {
@@ -117,8 +123,10 @@ inline float scalar_f32(uint64_t bits) {
   return f;
 }
 
+// align: bytes the first element's address must be a multiple of; 0 = by type (index tensors their
+// element size, data tensors the 16 bytes of the kernels' vector accesses).
 int check_tensor(const char* prog, const char* name, const PtoHipChipTensor& t, int ndims_min,
-                 int ndims_max) {
+                 int ndims_max, int align = 0) {
   PTO_CHECK_ARG(t.ndims >= (uint32_t)ndims_min && t.ndims <= (uint32_t)ndims_max &&
                     t.ndims <= PTO_HIP_MAX_DIMS,
                 "%s: tensor '%s' has %u dims, expected %d..%d", prog, name, t.ndims, ndims_min,
@@ -127,6 +135,17 @@ int check_tensor(const char* prog, const char* name, const PtoHipChipTensor& t, 
                 name, t.dtype);
   PTO_CHECK_ARG(t.buffer.addr != 0 || numel(t) == 0, "%s: tensor '%s' has a null buffer", prog,
                 name);
+  // A view (start_offset in elements, pto_backend.py:578-606) must lie inside its buffer when the
+  // buffer's size is given, and must keep the alignment the kernels' accesses assume.
+  const uint64_t eb = (uint64_t)dtype_bytes(t.dtype);
+  if (align == 0) align = (t.dtype == PTO_HIP_INT32 || t.dtype == PTO_HIP_INT64) ? (int)eb : 16;
+  PTO_CHECK_ARG(t.buffer.size == 0 || (t.start_offset + (uint64_t)numel(t)) * eb <= t.buffer.size,
+                "%s: tensor '%s' (start_offset %llu + %lld elements of %llu bytes) reaches past its %llu-byte buffer",
+                prog, name, (unsigned long long)t.start_offset, (long long)numel(t), (unsigned long long)eb,
+                (unsigned long long)t.buffer.size);
+  PTO_CHECK_ARG(numel(t) == 0 || (t.buffer.addr + t.start_offset * eb) % (uint64_t)align == 0,
+                "%s: tensor '%s' starts at an address that is not a multiple of %d bytes (base 0x%llx, start_offset %llu)",
+                prog, name, align, (unsigned long long)t.buffer.addr, (unsigned long long)t.start_offset);
   return PTO_HIP_OK;
 }
 
@@ -209,7 +228,8 @@ int run_paged_gather(const PtoHipChipTensor* t, int nt, const uint64_t* s, int n
                 nt, ns);
   static const char* names[4] = {"src", "indices", "block_table", "out"};
   for (int i = 0; i < 4; ++i) {
-    int rc = check_tensor("paged_gather", names[i], t[i], 1, 2);
+    // rows are copied 16 bytes at a time where their addresses allow and bytewise otherwise
+    int rc = check_tensor("paged_gather", names[i], t[i], 1, 2, dtype_bytes(t[i].dtype) ? dtype_bytes(t[i].dtype) : 1);
     if (rc) return rc;
   }
   PTO_CHECK_ARG(t[0].ndims == 2 && t[3].ndims == 2, "paged_gather: src and out must be 2-D");
@@ -217,7 +237,9 @@ int run_paged_gather(const PtoHipChipTensor* t, int nt, const uint64_t* s, int n
                 "paged_gather: indices and block_table must be INT32");
   PTO_CHECK_ARG(t[0].dtype == t[3].dtype, "paged_gather: out dtype %s differs from src dtype %s",
                 dtype_name(t[3].dtype), dtype_name(t[0].dtype));
-  PTO_CHECK_ARG(t[3].shapes[0] == numel(t[1]), "paged_gather: out has %u rows for %lld indices",
+  // The reference's output is the static [max_indices, size] buffer; the runtime index count says
+  // how many rows are filled and the rest stays untouched (paged_gather.cpp:176-189).
+  PTO_CHECK_ARG(t[3].shapes[0] >= numel(t[1]), "paged_gather: out has %u rows for %lld indices",
                 t[3].shapes[0], (long long)numel(t[1]));
   return pto_hip_paged_gather(tptr(t[0]), reinterpret_cast<const int32_t*>(tptr(t[1])),
                               reinterpret_cast<const int32_t*>(tptr(t[2])), tptr_mut(t[3]),
@@ -385,6 +407,7 @@ int run_rope_kv_fp8(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns
   }
   const int64_t hq = (int64_t)s[0], hkv = (int64_t)s[1], d = (int64_t)s[2], bs = (int64_t)s[3];
   PTO_CHECK_ARG(hq > 0 && hkv > 0 && d > 0 && bs > 0, "rope_kv_cache_update_fp8: non-positive scalar");
+  PTO_CHECK_ARG(d >= 2 && d % 2 == 0, "rope_kv_cache_update_fp8: head_dim %lld must be even and at least 2", (long long)d);
   const int64_t batch = numel(t[1]);
   PTO_CHECK_ARG(t[0].dtype == PTO_HIP_FP32 && numel(t[0]) == batch * (hq + 2 * hkv) * d,
                 "rope_kv_cache_update_fp8: qkv must be FP32 [B, (Hq+2Hkv)*D]");
@@ -423,6 +446,7 @@ int run_rope_kv(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hi
   }
   const int64_t hq = (int64_t)s[0], hkv = (int64_t)s[1], d = (int64_t)s[2], bs = (int64_t)s[3];
   PTO_CHECK_ARG(hq > 0 && hkv > 0 && d > 0 && bs > 0, "rope_kv_cache_update: non-positive scalar");
+  PTO_CHECK_ARG(d >= 2 && d % 2 == 0, "rope_kv_cache_update: head_dim %lld must be even and at least 2", (long long)d);
   const int64_t batch = numel(t[1]);
   PTO_CHECK_ARG(t[0].dtype == PTO_HIP_FP32 && numel(t[0]) == batch * (hq + 2 * hkv) * d,
                 "rope_kv_cache_update: qkv must be FP32 [B, (Hq+2Hkv)*D]");
@@ -502,8 +526,8 @@ int run_decoder_layer(const PtoHipChipTensor* t, int nt, const uint64_t* s, int 
   a.head_dim = (int64_t)s[2];
   a.block_size = (int64_t)s[3];
   a.eps = scalar_f32(s[4]);
-  PTO_CHECK_ARG(a.num_heads > 0 && a.kv_head_num > 0 && a.head_dim > 1 && a.block_size > 0,
-                "decoder_layer_decode: non-positive scalar");
+  PTO_CHECK_ARG(a.num_heads > 0 && a.kv_head_num > 0 && a.head_dim > 1 && a.head_dim % 2 == 0 && a.block_size > 0,
+                "decoder_layer_decode: non-positive scalar or odd head_dim");
   PTO_CHECK_ARG(w[2]->ndims == 2, "decoder_layer_decode: w_gate must be [H, I]");
   a.intermediate = w[2]->shapes[1];
   a.max_num_blocks_per_req = a.batch ? numel(t[2]) / a.batch : 1;
@@ -579,6 +603,7 @@ extern "C" {
 const char* pto_hip_last_error(void) { return last_error().c_str(); }
 
 int pto_hip_init(int device_id) {
+  PTO_DISPATCH_LOCK();
   Context& c = ctx();
   int n = 0;
   PTO_CHECK_HIP(hipGetDeviceCount(&n));
@@ -606,28 +631,44 @@ int pto_hip_init(int device_id) {
 }
 
 int pto_hip_close(void) {
+  PTO_DISPATCH_LOCK();
   Context& c = ctx();
   if (!c.initialized) return PTO_HIP_OK;
   if (--c.refcount > 0) return PTO_HIP_OK;  // another worker still holds the device
   c.refcount = 0;
-  PTO_CHECK_HIP(hipDeviceSynchronize());
-  if (c.workspace) PTO_CHECK_HIP(hipFree(c.workspace));
+  // Everything is released whatever fails on the way; the first failure is what the call reports.
+  hipError_t first = hipDeviceSynchronize();
+  const char* what = "hipDeviceSynchronize";
+  auto release = [&](void* ptr, const char* name) {
+    if (!ptr) return;
+    const hipError_t e = hipFree(ptr);
+    if (e != hipSuccess && first == hipSuccess) {
+      first = e;
+      what = name;
+    }
+  };
+  release(c.workspace, "hipFree(workspace)");
   c.workspace = nullptr;
   c.workspace_bytes = 0;
-  if (c.flags) PTO_CHECK_HIP(hipFree(c.flags));
+  release(c.flags, "hipFree(flags)");
   c.flags = nullptr;
-  if (c.layer_ws) PTO_CHECK_HIP(hipFree(c.layer_ws));
+  release(c.layer_ws, "hipFree(layer workspace)");
   c.layer_ws = nullptr;
   c.layer_ws_bytes = 0;
-  if (c.gemm_ws) PTO_CHECK_HIP(hipFree(c.gemm_ws));
+  release(c.gemm_ws, "hipFree(GEMM workspace)");
   c.gemm_ws = nullptr;
   c.gemm_ws_bytes = 0;
-  for (void* old : c.retired) PTO_CHECK_HIP(hipFree(old));
+  for (void* old : c.retired) release(old, "hipFree(retired workspace)");
   c.retired.clear();
   c.initialized = false;
   {
     std::lock_guard<std::mutex> lk(g_mu);
     g_callables.clear();
+  }
+  if (first != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(PTO_HIP_ERR_RUNTIME, "close: %s failed: %s (all device memory of the library was released)", what,
+                hipGetErrorString(first));
   }
   return PTO_HIP_OK;
 }
@@ -682,6 +723,7 @@ int pto_hip_copy_from(void* dst_host_ptr, uint64_t src_dev_ptr, size_t nbytes) {
 }
 
 int pto_hip_sync(void* stream) {
+  PTO_DISPATCH_LOCK();
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
   // Device-side argument errors of launches that do not block are reported here.
@@ -726,6 +768,7 @@ int pto_hip_unregister(int callable_id) {
 
 int pto_hip_run(int callable_id, const PtoHipChipTensor* tensors, int n_tensors,
                 const uint64_t* scalars, int n_scalars, void* stream) {
+  PTO_DISPATCH_LOCK();
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   int kind;
   int rc = lookup(callable_id, &kind);
@@ -737,6 +780,7 @@ int pto_hip_run(int callable_id, const PtoHipChipTensor* tensors, int n_tensors,
 }
 
 int pto_hip_kernel_entry(int callable_id, int64_t* args, int n_tensors, int n_scalars, void* stream) {
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(args || (n_tensors + n_scalars) == 0, "kernel_entry: null args");
   PTO_CHECK_ARG(n_tensors >= 0 && n_tensors <= 64 && n_scalars >= 0 && n_scalars <= 64,
                 "kernel_entry: argument counts out of range");
@@ -753,6 +797,7 @@ int pto_hip_kernel_entry(int callable_id, int64_t* args, int n_tensors, int n_sc
 int pto_hip_benchmark(int callable_id, const PtoHipChipTensor* tensors, int n_sets, int n_tensors,
                       const uint64_t* scalars, int n_scalars, int rounds, int warmup, void* stream,
                       float* avg_us) {
+  PTO_DISPATCH_LOCK();
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(n_sets >= 1 && rounds >= 1 && warmup >= 0 && avg_us, "benchmark: bad arguments");
   hipStream_t st = (hipStream_t)stream;
@@ -784,6 +829,7 @@ int pto_hip_benchmark(int callable_id, const PtoHipChipTensor* tensors, int n_se
 
 int pto_hip_set_option(const char* name, int64_t value) {
   PTO_CHECK_ARG(name != nullptr, "set_option: null name");
+  PTO_DISPATCH_LOCK();
   Context& c = ctx();
   if (!std::strcmp(name, "attn_tokens_per_partition")) {
     PTO_CHECK_ARG(value >= 0, "attn_tokens_per_partition must be >= 0");
@@ -825,6 +871,7 @@ int pto_hip_set_option(const char* name, int64_t value) {
 
 int pto_hip_get_option(const char* name, int64_t* value) {
   PTO_CHECK_ARG(name && value, "get_option: null argument");
+  PTO_DISPATCH_LOCK();
   Context& c = ctx();
   if (!std::strcmp(name, "attn_tokens_per_partition")) *value = c.attn_tokens_per_partition;
   else if (!std::strcmp(name, "gemm_variant")) *value = c.gemm_variant;

@@ -526,6 +526,7 @@ int w8a16_finish_norm(const W8Partials& parts, const float* scale, const void* r
 extern "C" int pto_hip_w8a16_matmul(const void* x, const void* w_q, const float* w_scale,
                                     const void* residual, void* out, int64_t m, int64_t k, int64_t n,
                                     int x_dtype, int res_dtype, int out_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
   using namespace pto_hip;
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   int rc = check_common("w8a16_matmul", m, k, n, x_dtype, out_dtype);
@@ -560,6 +561,7 @@ extern "C" int pto_hip_w8a16_matmul(const void* x, const void* w_q, const float*
 extern "C" int pto_hip_w8a16_swiglu(const void* x, const void* wg_q, const float* wg_scale,
                                     const void* wu_q, const float* wu_scale, void* out, int64_t m,
                                     int64_t k, int64_t n, int x_dtype, int out_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
   using namespace pto_hip;
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   int rc = check_common("w8a16_swiglu", m, k, n, x_dtype, out_dtype);

@@ -274,8 +274,9 @@ def test_fp8_rejects_small_blocks(worker):
 
 def test_full_size_long_fp8_config_properties(worker):
     """B64 Hq64 Hkv8 ctx~U[8192,32768] e4m3 (2.8 GB of cache, built on the GPU): the two launch
-    forms cut the work differently (fixed partitions vs even chunk runs) and must agree; three
-    whole sequences are checked against the oracle on the CPU."""
+    forms cut the work differently (fixed partitions vs even chunk runs) and must agree; sixteen
+    whole sequences (a quarter of the batch, the shortest and the longest among them) are checked
+    against the oracle on the CPU."""
     inp = workloads.attention_long_fp8(seed=0, device="cuda")
     outs = {}
     for name, variant in (("grid", 0), ("split", 1), ("auto", -1)):
@@ -292,7 +293,11 @@ def test_full_size_long_fp8_config_properties(worker):
     cfg = inp.config.tolist()
     b, hq, hkv, d, bs, mb = cfg[:6]
     table = inp.block_table.reshape(b, mb)
-    for seq in (0, 17, 63):
+    order = torch.argsort(inp.context_lens.cpu()).tolist()
+    picked = [order[0], order[-1]]
+    picked += [s for s in range(64) if s not in picked][::4][:14]
+    assert len(set(picked)) == 16
+    for seq in picked:
         nblk = (int(inp.context_lens[seq]) + bs - 1) // bs
         blocks = table[seq, :nblk].long()
         rows = (blocks[:, None, None] * hkv * bs + torch.arange(hkv, device="cuda")[None, :, None] * bs

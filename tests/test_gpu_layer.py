@@ -185,6 +185,21 @@ def test_rope_tables_of_full_head_width(worker):
     assert not torch.equal(q_out, half[0])
 
 
+@pytest.mark.parametrize("head_dim", [1, 7])
+def test_rope_head_dim_must_be_even(worker, head_dim):
+    """head_dim 1 once divided by zero on the host (table width D/2 = 0); an odd head_dim has no rotate-half."""
+    b, hq, hkv, bs = 2, 2, 1, 16
+    qkv = torch.zeros(b, (hq + 2 * hkv) * head_dim)
+    table = torch.zeros(b, dtype=torch.int32)
+    cache = torch.zeros(b * hkv * bs, head_dim, dtype=torch.bfloat16)
+    q_out = torch.zeros(b * hq, head_dim, dtype=torch.bfloat16)
+    cos = torch.ones(bs, max(head_dim // 2, 1))
+    with pytest.raises(ValueError, match="head_dim"):
+        with worker.register(rope_kv_cache_update) as h:
+            h(qkv, torch.ones(b, dtype=torch.int32), cos, cos.clone(), table, cache, cache.clone(), q_out,
+              hq, hkv, head_dim, bs)
+
+
 def test_contiguous_per_sequence_cache_is_the_one_block_case(worker):
     """The reference's decode example keeps K/V per sequence at row b*Hkv*MAX_SEQ + h*MAX_SEQ + pos
     (examples/models/qwen3_jit/kernels/attention.py:72-80): the paged layout with one block of MAX_SEQ
@@ -349,6 +364,59 @@ def test_decoder_layer_decode(worker, batch, ctxs):
     assert torch.allclose(inp.value_cache.float(), ref_v.float(), atol=2e-2, rtol=1e-2)
     changed = (inp.key_cache != kc0).any(dim=1).sum().item()
     assert changed <= batch * 2
+
+
+def test_decoder_layer_full_configuration(worker):
+    """The decoder-layer configuration at its full shape: hidden 4096, 32 query / 8 KV heads of 128,
+    intermediate 14336, batch 32, contexts of 4096, block 128, RoPE theta 5e5, int8 weights with
+    per-channel scales (218 MB of codes, 537 MB of bf16 cache, built on the GPU).  Six whole sequences
+    are checked against the oracle: their cache blocks are gathered to the host into a compact pool with
+    an identity block table, the oracle runs the layer on those sequences, and the layer's output rows
+    and the K/V rows it appended must agree; every other cache row must be untouched."""
+    inp = workloads.decoder_layer_inputs(device="cuda", seed=0)
+    batch, hkv, d, bs, mb = 32, inp.kv_head_num, inp.head_dim, inp.block_size, inp.max_num_blocks_per_req
+    assert inp.hidden.shape == (32, 4096) and inp.weights["gate"][0].shape == (4096, 14336)
+    assert inp.weights["qkv"][0].dtype == torch.int8 and mb == 32 and int(inp.seq_lens[0]) == 4096
+    seqs = [0, 5, 13, 21, 30, 31]
+    table = inp.block_table.reshape(batch, mb)
+
+    def sub_pool(cache):
+        """Rows of the blocks of `seqs`, block after block in table order: [len(seqs)*mb*Hkv*bs, D] on the host."""
+        blocks = table[seqs].reshape(-1).long()
+        rows = (blocks[:, None] * (hkv * bs) + torch.arange(hkv * bs, device="cuda")[None, :]).reshape(-1)
+        return cache[rows].cpu()
+
+    k0, v0 = sub_pool(inp.key_cache), sub_pool(inp.value_cache)
+    kc_before, vc_before = inp.key_cache.clone(), inp.value_cache.clone()
+    with worker.register(decoder_layer_decode) as h:
+        h(*inp.args())
+    worker.sync()
+
+    cpu = lambda t: None if t is None else t.cpu()
+    w = {name: (cpu(c), cpu(sc)) for name, (c, sc) in inp.weights.items()}
+    ref_out, ref_k, ref_v = oracle.decoder_layer_decode(
+        inp.hidden[seqs].cpu(), inp.seq_lens[seqs].cpu(), torch.arange(len(seqs) * mb, dtype=torch.int32), k0, v0,
+        inp.rope_cos.cpu(), inp.rope_sin.cpu(), inp.gamma_in.cpu(), inp.gamma_post.cpu(),
+        *w["qkv"], *w["o"], *w["gate"], *w["up"], *w["down"],
+        num_heads=inp.num_heads, kv_head_num=hkv, head_dim=d, block_size=bs, max_num_blocks_per_req=mb, eps=inp.eps)
+    got = inp.out[seqs].float().cpu()
+    print("max_abs_err", (got - ref_out.float()).abs().max().item(), "ref_max", ref_out.float().abs().max().item(),
+          flush=True)
+    assert torch.isfinite(inp.out.float()).all()
+    validate_golden({"out": got}, {"out": ref_out.float()}, rtol=2e-2, atol=2e-2)
+    k1, v1 = sub_pool(inp.key_cache), sub_pool(inp.value_cache)
+    assert torch.allclose(k1.float(), ref_k.float(), atol=2e-2, rtol=2e-2)
+    assert torch.allclose(v1.float(), ref_v.float(), atol=2e-2, rtol=2e-2)
+    # the oracle changed exactly one row per (sequence, KV head) of the compact pool, and so did the layer
+    assert int((ref_k != k0).any(dim=1).sum()) == len(seqs) * hkv
+    assert torch.equal((k1 != k0).any(dim=1), (ref_k != k0).any(dim=1))
+    # over the whole cache: at most batch * Hkv rows differ from before, the ones at position 4095
+    k_changed = (inp.key_cache != kc_before).any(dim=1)
+    v_changed = (inp.value_cache != vc_before).any(dim=1)
+    assert int(k_changed.sum()) == batch * hkv and int(v_changed.sum()) == batch * hkv
+    last_blocks = table[:, mb - 1].long()
+    want_rows = ((last_blocks[:, None] * hkv + torch.arange(hkv, device="cuda")[None, :]) * bs + bs - 1).reshape(-1)
+    assert torch.equal(torch.nonzero(k_changed).flatten().sort().values, want_rows.sort().values)
 
 
 @pytest.mark.parametrize("batch,gemm_rows", [(45, 0), (100, 0), (100, 33), (300, 33)])

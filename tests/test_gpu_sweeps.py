@@ -1,0 +1,250 @@
+"""Seeded randomised parity sweeps over the supported shapes, each case against the CPU oracle.
+
+A bounded subset (about 200 cases in all, sized to run in well under a minute of GPU time plus the
+oracle's CPU time) of the shape space the hand-picked tests sample: head sizes, group widths, block
+sizes, ragged and empty sequences, 16-bit and e4m3 caches, every launch form; FFN / projection
+shapes that are odd multiples of 8 on every GEMM tiling; int8 weight codes through the skinny and
+the tiled path; the composed layer with either weight and cache type; bit-exact gathers.
+
+Every case prints its full description before it runs (so a fault names its case) and the sweep
+stops at its first mismatch.
+"""
+
+import random
+
+import pytest
+import torch
+
+import oracle
+from pypto_amd import workloads
+from pypto_amd.runtime import (decoder_layer_decode, decoder_layer_decode_fp8kv, decoder_layer_decode_w16,
+                               decoder_layer_decode_w16_fp8kv, ffn_block, ffn_swiglu, gate_up_swiglu, paged_attention,
+                               paged_gather, projection, projection_residual, w8a16_matmul, w8a16_matmul_residual,
+                               w8a16_swiglu)
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(name, out, ref, rtol, atol):
+    out, ref = out.float(), ref.float()
+    assert torch.isfinite(out).all(), f"{name}: non-finite output"
+    err = (out - ref).abs()
+    over = err > atol + rtol * ref.abs()
+    assert not over.any(), (f"{name}: {int(over.sum())} elements off, max err {err.max().item():.4g}, "
+                            f"ref max {ref.abs().max().item():.4g}")
+
+
+def test_attention_sweep(worker):
+    rng = random.Random(20240)
+    try:
+        for case in range(70):
+            d = rng.choice([128, 128, 128, 256])
+            hkv = rng.choice([1, 1, 2, 4, 8])
+            group = rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16, 17, 24, 32, 40, 64])
+            if d == 256 and group > 32:
+                group = 32
+            hq = hkv * group
+            fp8 = rng.random() < 0.35
+            bs = rng.choice([32, 64, 128, 256] if fp8 else [16, 32, 48, 64, 128, 256])
+            batch = rng.randint(1, 5)
+            top = rng.choice([40, 300, 1200, 2500])
+            ctxs = [rng.choice([0, 1, bs - 1, bs, bs + 1, rng.randint(1, top), rng.randint(1, top)]) for _ in range(batch)]
+            dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float16
+            mb = (max(max(ctxs), 1) + bs - 1) // bs + rng.choice([0, 0, 3])
+            inp = workloads.paged_attention_inputs(
+                batch=batch, num_heads=hq, kv_head_num=hkv, head_dim=d, block_size=bs, context_lens=ctxs,
+                ctx_range=(1, max(max(ctxs), 1)), dtype=dtype, fp8_kv=fp8, max_num_blocks_per_req=mb,
+                seed=rng.randint(0, 10 ** 6), scale=rng.choice([None, None, 1.0, 0.0884]))
+            align = bs if bs >= 32 else 32
+            variant, tpp, waves, gt = rng.choice([(-1, 0, 0, 0), (0, align * rng.randint(1, 8), 0, 0),
+                                                  (1, 0, rng.choice([0, 1, 2, 4, 8]), 0), (0, 0, 0, rng.choice([1, 2])),
+                                                  (1, 0, 0, 1)])
+            print(f"attention case {case}: B{batch} Hq{hq} Hkv{hkv} D{d} bs{bs} ctx{ctxs} {dtype} e4m3={fp8} mb={mb} "
+                  f"variant={variant} tpp={tpp} waves={waves} tiles={gt}", flush=True)
+            ref = oracle.paged_attention_golden(inp.query, inp.key_cache, inp.value_cache, inp.block_table,
+                                                inp.context_lens, inp.config, inp.k_scale, inp.v_scale)
+            worker.set_option("attn_variant", variant)
+            worker.set_option("attn_tokens_per_partition", tpp)
+            worker.set_option("attn_waves_per_cu", waves)
+            worker.set_option("attn_group_tiles", gt)
+            dev = [t.cuda() if isinstance(t, torch.Tensor) and i != 6 else t for i, t in enumerate(inp.args())]
+            dev[5].fill_(float("nan"))
+            torch.cuda.synchronize()
+            with worker.register(paged_attention) as h:
+                h(*dev)
+            worker.sync()
+            out = dev[5].cpu()
+            assert torch.isfinite(out).all()
+            err = (out - ref).abs().max().item()
+            assert err <= 1e-2 + 2e-2 * ref.abs().max().item(), f"case {case}: max err {err}"
+    finally:
+        for name, value in (("attn_variant", -1), ("attn_tokens_per_partition", 0), ("attn_waves_per_cu", 0),
+                            ("attn_group_tiles", 0)):
+            worker.set_option(name, value)
+
+
+def test_ffn_and_projection_sweep(worker):
+    rng = random.Random(20241)
+    try:
+        for case in range(50):
+            t = rng.choice([1, 2, 7, 16, 31, 32, 33, 48, 64, 65, 100, 128, 129, 200, 256, 300, 512, 700])
+            h = 8 * rng.randint(8, 160)
+            i = 8 * rng.randint(8, 320)
+            dtype = rng.choice([torch.bfloat16, torch.float16])
+            variant = rng.choice([0, 0, 0, 1, 2, 3, 4, 5, 6])
+            splits = rng.choice([0, 0, 0, 2, 3])
+            kind = rng.choice(["ffn_block", "ffn_swiglu", "projection", "projection_residual", "gate_up"])
+            out_fp32 = rng.random() < 0.4
+            seed = rng.randint(0, 10 ** 6)
+            print(f"ffn case {case}: {kind} T{t} H{h} I{i} {dtype} variant={variant} splits={splits} "
+                  f"out_fp32={out_fp32} seed={seed}", flush=True)
+            worker.set_option("gemm_variant", variant)
+            worker.set_option("gemm_splits", splits)
+            g = torch.Generator().manual_seed(seed)
+            if kind in ("ffn_block", "ffn_swiglu"):
+                inp = workloads.ffn_inputs(tokens=t, hidden=h, intermediate=i, seed=seed, dtype=dtype,
+                                           with_norm=kind == "ffn_block")
+                out = torch.zeros(t, h, dtype=torch.float32 if out_fp32 else dtype)
+                if kind == "ffn_block":
+                    with worker.register(ffn_block) as hd:
+                        hd(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, out, inp.eps)
+                    ref = oracle.ffn_block(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, inp.eps)
+                else:
+                    with worker.register(ffn_swiglu) as hd:
+                        hd(inp.x, inp.w_gate, inp.w_up, inp.w_down, out)
+                    ref = oracle.ffn_swiglu(inp.x, inp.w_gate, inp.w_up, inp.w_down, h_dtype=dtype)
+                _close(f"case {case}", out, ref, 2e-2, 1e-2)
+                continue
+            x = (torch.randn(t, h, generator=g) / h ** 0.5).to(dtype)
+            wa = torch.randn(h, i, generator=g).to(dtype)
+            if kind == "gate_up":
+                wb = torch.randn(h, i, generator=g).to(dtype)
+                out = torch.zeros(t, i, dtype=dtype)
+                with worker.register(gate_up_swiglu) as hd:
+                    hd(x, wa, wb, out)
+                ref = oracle.swiglu(oracle.projection(x, wa), oracle.projection(x, wb)).to(dtype)
+                _close(f"case {case}", out, ref, 2e-2, 1e-2)
+                continue
+            out = torch.zeros(t, i, dtype=torch.float32 if out_fp32 else dtype)
+            if kind == "projection":
+                with worker.register(projection) as hd:
+                    hd(x, wa, out)
+                ref = oracle.projection(x, wa)
+            else:
+                res = torch.randn(t, i, generator=g).to(rng.choice([torch.float32, dtype]))
+                with worker.register(projection_residual) as hd:
+                    hd(x, wa, res, out)
+                ref = oracle.projection(x, wa, res)
+            _close(f"case {case}", out, ref.to(out.dtype), 1e-2, 1e-2)
+    finally:
+        worker.set_option("gemm_variant", 0)
+        worker.set_option("gemm_splits", 0)
+
+
+def test_w8a16_sweep(worker):
+    rng = random.Random(20242)
+    try:
+        for case in range(40):
+            m = rng.choice([1, 5, 16, 32, 33, 48, 64, 65, 100, 128, 129, 200, 256, 300, 512, 700, 1025])
+            k = 16 * rng.randint(2, 200)
+            n = 8 * rng.randint(1, 300)
+            if rng.random() < 0.7:
+                n = (n + 15) // 16 * 16
+            dtype = rng.choice([torch.bfloat16, torch.float16])
+            variant = rng.choice([0, 0, 0, 4, 5, 6, 6])
+            wide = rng.choice([1, 1, 0, 2])
+            kind = rng.choice(["matmul", "residual", "swiglu"])
+            out_dt = rng.choice([torch.float32, dtype])
+            seed = rng.randint(0, 10 ** 6)
+            print(f"w8a16 case {case}: {kind} m{m} k{k} n{n} {dtype} out {out_dt} variant={variant} wide={wide} "
+                  f"seed={seed}", flush=True)
+            g = torch.Generator().manual_seed(seed)
+            x = (torch.randn(m, k, generator=g) * 0.5).to(dtype)
+            wq = torch.randint(-127, 128, (k, n), generator=g, dtype=torch.int8)
+            wu = torch.randint(-127, 128, (k, n), generator=g, dtype=torch.int8)
+            s = torch.rand(n, generator=g) * 0.01 + 0.001
+            su = torch.rand(n, generator=g) * 0.01 + 0.001
+            out = torch.zeros(m, n, dtype=out_dt)
+            worker.set_option("gemm_variant", variant)
+            worker.set_option("w8a16_wide", wide)
+            ref = oracle.w8a16_matmul(x, wq, s)
+            if kind == "matmul":
+                with worker.register(w8a16_matmul) as h:
+                    h(x, wq, s, out)
+            elif kind == "residual":
+                res = torch.randn(m, n, generator=g).to(rng.choice([torch.float32, dtype]))
+                with worker.register(w8a16_matmul_residual) as h:
+                    h(x, wq, s, res, out)
+                ref = ref + res.float()
+            else:
+                with worker.register(w8a16_swiglu) as h:
+                    h(x, wq, s, wu, su, out)
+                ref = oracle.swiglu(ref, oracle.w8a16_matmul(x, wu, su))
+            ref = ref.to(out_dt).float()
+            tol = 1e-4 if out_dt == torch.float32 else 1e-2
+            _close(f"case {case}", out, ref, tol, tol * max(1.0, float(ref.abs().max())))
+    finally:
+        worker.set_option("gemm_variant", 0)
+        worker.set_option("w8a16_wide", 1)
+
+
+def test_decoder_layer_and_gather_sweep(worker):
+    rng = random.Random(20243)
+    for case in range(24):
+        d = rng.choice([128, 128, 256])
+        hkv = rng.choice([1, 2, 4])
+        hq = hkv * rng.choice([1, 2, 4, 5, 8])
+        hidden = 16 * rng.randint(4, 64)
+        inter = 16 * rng.randint(4, 128)
+        batch = rng.choice([1, 2, 5, 16, 32, 33, 40, 64, 100])
+        fp8 = rng.random() < 0.4
+        bs = rng.choice([32, 64, 128] if fp8 else [16, 32, 64, 128])
+        int8 = rng.random() < 0.5
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        ctxs = [rng.choice([1, bs, bs + 1, rng.randint(1, 400)]) for _ in range(batch)]
+        seed = rng.randint(0, 10 ** 6)
+        print(f"layer case {case}: B{batch} H{hidden} Hq{hq} Hkv{hkv} D{d} I{inter} bs{bs} {dtype} int8={int8} "
+              f"e4m3={fp8} seed={seed} ctx{ctxs}", flush=True)
+        inp = workloads.decoder_layer_inputs(batch=batch, hidden=hidden, num_heads=hq, kv_head_num=hkv, head_dim=d,
+                                             intermediate=inter, block_size=bs, context_lens=ctxs, seed=seed,
+                                             dtype=dtype, int8_weights=int8)
+        kw = dict(num_heads=hq, kv_head_num=hkv, head_dim=d, block_size=bs,
+                  max_num_blocks_per_req=inp.max_num_blocks_per_req, eps=inp.eps)
+        flat = [t for name in ("qkv", "o", "gate", "up", "down") for t in inp.weights[name]]
+        args = list(inp.args())
+        if fp8:
+            pool_blocks = inp.key_cache.shape[0] // (hkv * bs)
+            kc, ks = oracle.quantize_kv_fp8(inp.key_cache, pool_blocks, hkv, bs)
+            vc, vs = oracle.quantize_kv_fp8(inp.value_cache, pool_blocks, hkv, bs)
+            ref = oracle.decoder_layer_decode(inp.hidden, inp.seq_lens, inp.block_table, kc, vc, inp.rope_cos,
+                                              inp.rope_sin, inp.gamma_in, inp.gamma_post, *flat, k_scale=ks,
+                                              v_scale=vs, **kw)[0]
+            args[3:5] = [kc.clone(), vc.clone(), ks.clone(), vs.clone()]
+            prog = decoder_layer_decode_fp8kv if int8 else decoder_layer_decode_w16_fp8kv
+        else:
+            ref = oracle.decoder_layer_decode(inp.hidden, inp.seq_lens, inp.block_table, inp.key_cache,
+                                              inp.value_cache, inp.rope_cos, inp.rope_sin, inp.gamma_in,
+                                              inp.gamma_post, *flat, **kw)[0]
+            prog = decoder_layer_decode if int8 else decoder_layer_decode_w16
+        with worker.register(prog) as h:
+            h(*args)
+        _close(f"layer case {case}", inp.out, ref, 2e-2, 2e-2)
+
+        # a gather beside each layer case: bit-exact, fewer indices than output rows now and then
+        rows, hid = rng.randint(1, 40) * bs, 8 * rng.randint(1, 64)
+        gdt = rng.choice([torch.float16, torch.bfloat16, torch.float32, torch.int8])
+        src = torch.randint(-100, 100, (rows, hid)).to(gdt)
+        nblk = rows // bs
+        table = torch.randint(0, nblk, (nblk,), dtype=torch.int32)
+        idx = torch.randint(0, rows, (rng.randint(1, 300),), dtype=torch.int32)
+        size = 8 * rng.randint(1, hid // 8)
+        off = 8 * rng.randint(0, (hid - size) // 8)
+        spare = rng.choice([0, 0, 5])
+        print(f"gather case {case}: rows{rows} hid{hid} {gdt} n{idx.numel()} size{size} off{off} spare{spare}", flush=True)
+        gout = torch.full((idx.numel() + spare, size), 7).to(gdt).cuda()  # resident: spare rows must stay as they are
+        with worker.register(paged_gather) as h:
+            h(src, idx, table, gout, bs, off)
+        worker.sync()
+        gout = gout.cpu()
+        assert torch.equal(gout[:idx.numel()], oracle.paged_gather(src, idx, table, bs, size, off))
+        assert (gout[idx.numel():] == 7).all()
