@@ -176,6 +176,30 @@ PTO_HIP_API int pto_hip_paged_attention(const void* query, const void* key_cache
                                         const int64_t* config, int q_dtype, int kv_dtype,
                                         const float* k_scale, const float* v_scale, void* stream);
 
+/* pto_hip_paged_attention for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, same kernels and partitioning, bit-identical results; the
+ * per-partition partial results (m, l, o) go to a fixed device array of
+ * PTO_HIP_NOALLOC_SCRATCH_BYTES that the library's code object carries (every GPU the library runs
+ * on holds its copy until the process ends) instead of the grow-only workspace, and the call makes
+ * no hipMalloc / hipFree.  The partials take
+ *     batch * num_heads * partitions * (head_dim + 2) * 4 bytes   (partitions <= 8 in the default choice
+ *                                                                  while batch * kv_head_num <= 4 * CUs), or
+ *     (batch * kv_head_num * tiles + 4 * CUs) * 16 * tiles_per_wavefront * (head_dim + 2) * 4 bytes
+ *                                      for launches that may stream a gigabyte of cache or more;
+ * both benchmark configurations fit (2.1 MB and 12.8 MB).  A launch that needs more is refused with
+ * PTO_HIP_ERR_INVALID_VALUE before anything is launched.  Every call on a GPU shares that GPU's
+ * array: calls that overlap in time on one GPU (two streams, two threads) race.  Nothing in the array
+ * has to start at zero: each launch writes every slot it later reads.  pto_hip_init looks up the
+ * array's device address, so the entry point needs no set-up of its own. */
+#define PTO_HIP_NOALLOC_SCRATCH_BYTES (32u << 20)
+PTO_HIP_API int pto_hip_paged_attention_noalloc(const void* query, const void* key_cache,
+                                                const void* value_cache, const int32_t* block_table,
+                                                const int32_t* context_lens, float* out,
+                                                const int64_t* config, int q_dtype, int kv_dtype,
+                                                const float* k_scale, const float* v_scale,
+                                                void* stream);
+
 /* out[i, :] = src[block_table[idx / bs] * bs + idx % bs, col_offset : col_offset + size]
  * (src/ir/op/tensor_ops/paged_gather.cpp:74-199), bit-exact, asynchronous on the stream.  An index
  * that addresses a block outside block_table or a row outside src is skipped and reported by

@@ -25,7 +25,7 @@ EXPORTS = (
     "pto_hip_w8a16_matmul", "pto_hip_w8a16_swiglu", "pto_hip_rope_kv_cache_update",
     "pto_hip_rope_kv_cache_update_fp8",
     "pto_hip_decoder_layer_decode", "pto_hip_select_program", "pto_hip_projection",
-    "pto_hip_gate_up_swiglu",
+    "pto_hip_gate_up_swiglu", "pto_hip_paged_attention_noalloc",
 )
 
 
@@ -92,6 +92,7 @@ def load() -> C.CDLL:
         "pto_hip_benchmark": [C.c_int, C.POINTER(ChipTensor), C.c_int, C.c_int, C.POINTER(u64),
                               C.c_int, C.c_int, C.c_int, vp, C.POINTER(C.c_float)],
         "pto_hip_paged_attention": [vp, vp, vp, vp, vp, vp, C.POINTER(i64), C.c_int, C.c_int, vp, vp, vp],
+        "pto_hip_paged_attention_noalloc": [vp, vp, vp, vp, vp, vp, C.POINTER(i64), C.c_int, C.c_int, vp, vp, vp],
         "pto_hip_paged_gather": [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, C.c_int, vp],
         "pto_hip_rms_norm": [vp, vp, vp, i64, i64, C.c_float, C.c_int, C.c_int, vp],
         "pto_hip_ffn_swiglu": [vp, vp, vp, vp, vp, vp, i64, i64, i64, C.c_float, C.c_int, C.c_int, vp],

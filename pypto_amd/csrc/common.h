@@ -158,7 +158,14 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
                     const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
                     bool want_blocked, bool* wrote_blocked,
                     const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
-                    const float* v_scale, int64_t pool_blocks, void* stream);
+                    const float* v_scale, int64_t pool_blocks, void* stream, void* fixed_scratch = nullptr,
+                    size_t fixed_scratch_bytes = 0);
+// fixed_scratch != null: the partition partials go there instead of the grow-only workspace, and a
+// launch that needs more than fixed_scratch_bytes is refused (nothing is allocated either way).
+//
+// Looks up, for `device` (which must be current), the address of the file-scope device array that
+// backs pto_hip_paged_attention_noalloc.  Called by pto_hip_init; idempotent per device.
+int attn_static_scratch_init(int device);
 
 inline int dtype_bytes(int dt) {
   switch (dt) {

@@ -944,7 +944,8 @@ namespace pto_hip {
 int paged_attention(const void* query, const void* key_cache, const void* value_cache,
                     const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
                     bool want_blocked, bool* wrote_blocked, const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
-                    const float* v_scale, int64_t pool_blocks, void* stream) {
+                    const float* v_scale, int64_t pool_blocks, void* stream, void* fixed_scratch,
+                    size_t fixed_scratch_bytes) {
   Context& cx = ctx();
   if (!cx.initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(config != nullptr, "paged_attention: config is null");
@@ -1013,6 +1014,17 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
 
   const int64_t max_ctx = max_blocks * bs;
   const bool bf16 = q_dtype == PTO_HIP_BF16;
+  // Where the partition partials live: the caller's fixed area (never grown) or the workspace.
+  auto partials_area = [&](size_t bytes, void** ws) -> int {
+    if (!fixed_scratch) return workspace(bytes, ws);
+    if (bytes > fixed_scratch_bytes)
+      return fail(PTO_HIP_ERR_INVALID_VALUE,
+                  "paged_attention_noalloc: this launch needs %zu bytes of partition partials, the fixed scratch "
+                  "area holds %zu; use pto_hip_paged_attention for launches of this size",
+                  bytes, fixed_scratch_bytes);
+    *ws = fixed_scratch;
+    return PTO_HIP_OK;
+  };
 
   // Context partitions: about one wavefront per SIMD when every sequence is at its maximum
   // length (measured best for short launches, where the spread of finishing times matters more
@@ -1050,7 +1062,7 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     const size_t o_bytes = rows * p.n_part * d * sizeof(float);
     const size_t ml_bytes = rows * p.n_part * 2 * sizeof(float);
     void* ws = nullptr;
-    int rc = workspace(o_bytes + ml_bytes, &ws);
+    int rc = partials_area(o_bytes + ml_bytes, &ws);
     if (rc != PTO_HIP_OK) return rc;
     p.part_o = reinterpret_cast<float*>(ws);
     p.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + o_bytes);
@@ -1068,7 +1080,7 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     const size_t slots = (size_t)batch * hkv * p.gtiles + (size_t)p.n_wg * waves;
     const size_t o_bytes = slots * p.gt_rows * d * sizeof(float), ml_bytes = slots * p.gt_rows * 2 * sizeof(float);
     void* ws = nullptr;
-    int rc = workspace(o_bytes + ml_bytes, &ws);
+    int rc = partials_area(o_bytes + ml_bytes, &ws);
     if (rc != PTO_HIP_OK) return rc;
     p.part_o = reinterpret_cast<float*>(ws);
     p.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + o_bytes);
@@ -1097,6 +1109,49 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   return cast_from_f32(out, out16, (size_t)batch * hq * d, q_dtype, (hipStream_t)stream);
 }
 }  // namespace pto_hip
+
+// ---------------------------------------------------------------------------------------------
+// Entry point that allocates nothing: the partition partials live in a file-scope device array
+// instead of the grow-only workspace.  In host code the array's name is only a stand-in for the
+// symbol; its device address is looked up once per device (each GPU holds its own copy of the
+// array at its own address) and host code uses that pointer from then on.
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[PTO_HIP_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, null until looked up
+}  // namespace
+
+namespace pto_hip {
+int attn_static_scratch_init(int device) {
+  PTO_CHECK_ARG(device >= 0 && device < kMaxDevices, "device id %d beyond the %d this library keeps state for", device,
+                kMaxDevices);
+  if (g_scratch_ptr[device]) return PTO_HIP_OK;
+  void* ptr = nullptr;
+  PTO_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  PTO_CHECK_ARG(ptr != nullptr, "the static scratch array has no address on device %d", device);
+  g_scratch_ptr[device] = ptr;
+  return PTO_HIP_OK;
+}
+}  // namespace pto_hip
+
+extern "C" int pto_hip_paged_attention_noalloc(const void* query, const void* key_cache, const void* value_cache,
+                                               const int32_t* block_table, const int32_t* context_lens, float* out,
+                                               const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
+                                               const float* v_scale, void* stream) {
+  PTO_DISPATCH_LOCK();
+  pto_hip::Context& cx = pto_hip::ctx();
+  if (!cx.initialized)
+    return pto_hip::fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  void* area = cx.device >= 0 && cx.device < kMaxDevices ? g_scratch_ptr[cx.device] : nullptr;
+  if (!area)
+    return pto_hip::fail(PTO_HIP_ERR_NOT_INITIALIZED, "the static scratch area of device %d was not set up by pto_hip_init",
+                         cx.device);
+  return pto_hip::paged_attention(query, key_cache, value_cache, block_table, context_lens, out, nullptr, false, nullptr,
+                                  config, q_dtype, kv_dtype, k_scale, v_scale, 0, stream, area,
+                                  PTO_HIP_NOALLOC_SCRATCH_BYTES);
+}
 
 extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
                                        const void* value_cache, const int32_t* block_table,

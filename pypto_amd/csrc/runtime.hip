@@ -621,6 +621,10 @@ int pto_hip_init(int device_id) {
                 device_id, prop.gcnArchName);
   c.device = device_id;
   c.num_cu = prop.multiProcessorCount;
+  {
+    const int rc = attn_static_scratch_init(device_id);  // address of the no-allocation entry's device array
+    if (rc) return rc;
+  }
   if (!c.flags) {
     PTO_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&c.flags), 256));
     PTO_CHECK_HIP(hipMemset(c.flags, 0, 256));
