@@ -322,16 +322,22 @@ typedef struct PtoHipDecoderLayerArgs {
 } PtoHipDecoderLayerArgs;
 PTO_HIP_API int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* args, void* stream);
 
-/* ---- manifest -> program ------------------------------------------------------------------
+/* ---- compile side: manifest -> program, manifest writer, target description ---------------
+ * None of these needs a device; all are callable before pto_hip_init.
+ *
  * The reference describes a compiled program by a kernel_config.py manifest (ORCHESTRATION +
  * KERNELS[{func_id, name, core_type, signature}], python/pypto/backend/pto_backend.py:933-1045)
  * and runs it by compiling every kernel (python/pypto/runtime/device_runner.py:505-664).  Here a
- * recognised manifest maps to one fused program name for pto_hip_register: the 4-kernel
- * paged-attention set (qk_matmul/pv_matmul on aic, softmax_prepare/online_update and the optional
- * init_inplace on aiv), the
- * matmul + swiglu FFN chain, a single rms_norm kernel, paged_gather.  orch_dirs may be null when
- * the manifest carries no signature.  PTO_HIP_ERR_NOT_FOUND when nothing matches.  Needs no
- * device: callable before pto_hip_init.  *program_name points at a static string. */
+ * recognised manifest maps to one fused program name for pto_hip_register.  Recognition is exact:
+ * the orchestration function's name and every kernel name must be ones the reference's own
+ * programs use for that program (kernel_qk_matmul, kernel_softmax_prepare[_unaligned],
+ * kernel_pv_matmul, kernel_online_update and the optional kernel_init_inplace under
+ * paged_attention; one to three matmul_kernel plus one swiglu_kernel under ffn_swiglu; a single
+ * matmul / matmul_kernel; a single rms_norm kernel; paged_gather), every kernel must sit on the
+ * core type of its role (matrix work aic, vector work aiv) and the orchestration's directions
+ * must be the program's.  A kernel called matmul_btranspose or matmul_bias is not a plain matmul:
+ * such manifests are PTO_HIP_ERR_NOT_FOUND.  orch_dirs may be null when the manifest carries no
+ * signature.  *program_name points at a static string. */
 enum { PTO_HIP_CORE_AIC = 0, PTO_HIP_CORE_AIV = 1 };
 enum { PTO_HIP_DIR_IN = 0, PTO_HIP_DIR_OUT = 1, PTO_HIP_DIR_INOUT = 2 };
 typedef struct PtoHipManifestKernel {
@@ -342,6 +348,59 @@ typedef struct PtoHipManifestKernel {
 PTO_HIP_API int pto_hip_select_program(const char* orchestration_name, const PtoHipManifestKernel* kernels,
                                        int32_t n_kernels, const int32_t* orch_dirs, int32_t n_orch_tensors,
                                        const char** program_name);
+
+/* The text of kernel_config.py for a fused program, in the format of the reference's generator
+ * (_generate_config_file, python/pypto/backend/pto_backend.py:933-1045): RUNTIME_CONFIG,
+ * ORCHESTRATION with its signature, one KERNELS entry per kernel of the reference program.
+ * runtime_name NULL = "tensormap_and_ringbuffer".  *needed (may be NULL) receives the size with
+ * the terminator; buf NULL only asks for it.  Programs without a manifest form (the fused layer,
+ * the W8A16 entries) are PTO_HIP_ERR_NOT_FOUND. */
+PTO_HIP_API int pto_hip_write_manifest(const char* program_name, const char* runtime_name, char* buf, size_t cap,
+                                       size_t* needed);
+
+/* The gfx950 target as the reference's backend plug-in describes a target: class Backend (SoC
+ * model, op registry; include/pypto/backend/common/backend.h:173-371) and class BackendHandler
+ * (include/pypto/backend/common/backend_handler.h:130-475).  Memory spaces are indexed
+ * DDR 0, Vec 1, Mat 2, Left 3, Right 4, Acc 5, Bias 6 (include/pypto/ir/memory_space.h:35-46). */
+typedef struct PtoHipBackendInfo {
+  char type_name[16];     /* Backend::GetTypeName(): "gfx950" */
+  char backend_type[16];  /* BackendTypeToString(): "HipGfx950" */
+  char target_arch[16];   /* BackendHandler::GetPtoTargetArch() */
+  int32_t cube_cores;     /* Backend::GetCoreCount(CUBE): MFMA pipes = compute units */
+  int32_t vector_cores;   /* Backend::GetCoreCount(VECTOR) */
+  int32_t dies;           /* XCDs */
+  int32_t wavefront_size;
+  int32_t n_ops;          /* registered tile / tensor ops */
+  int32_t n_programs;     /* fused programs with a manifest form */
+  uint64_t mem_bytes[7];      /* Backend::GetMemSize per memory space */
+  uint64_t mem_alignment[7];  /* Backend::GetMemAlignment */
+  uint64_t l2_bytes_per_die;
+  uint64_t last_level_cache_bytes;
+} PtoHipBackendInfo;
+PTO_HIP_API int pto_hip_backend_info(PtoHipBackendInfo* info);
+/* Registered op names in sorted order, index 0 .. n_ops - 1. */
+PTO_HIP_API int pto_hip_backend_op_name(int32_t index, const char** name);
+/* Backend::GetOpInfo: the pipe that carries the op ("M", "V", "MTE2", ...), the fused programs that
+ * realise it (comma separated) and how.  An unregistered op is PTO_HIP_ERR_NOT_FOUND with the
+ * reference's message "No codegen registered for operation: <name>". */
+PTO_HIP_API int pto_hip_backend_op_info(const char* op_name, char* pipe, size_t pipe_cap, char* programs,
+                                        size_t programs_cap, char* how, size_t how_cap);
+/* Runs the op's registered codegen callback (BackendCodegenFunc, backend.h:78) on a call
+ * result = op(args...) and returns the lines it emitted. */
+PTO_HIP_API int pto_hip_backend_codegen(const char* op_name, const char* const* args, int32_t n_args,
+                                        const char* result, char* buf, size_t cap);
+/* Whether the fused program realises every op of a tile program: PTO_HIP_OK, or the first op that
+ * is unregistered (PTO_HIP_ERR_NOT_FOUND, the message above) or realised only by other programs
+ * (PTO_HIP_ERR_UNSUPPORTED). */
+PTO_HIP_API int pto_hip_backend_check_ops(const char* program_name, const char* const* ops, int32_t n_ops);
+/* The ops the reference writes the program in, comma separated. */
+PTO_HIP_API int pto_hip_backend_program_ops(const char* program_name, char* buf, size_t cap, size_t* needed);
+/* Backend::FindMemPath: shortest path through the memory hierarchy, *n = 0 when unreachable. */
+PTO_HIP_API int pto_hip_backend_mem_path(int32_t from, int32_t to, int32_t* path, int32_t cap, int32_t* n);
+/* A BackendHandler hook by its method name ("GetPtoTargetArch", "RequiresGMPipeBuffer",
+ * "GetL0cCapacityBytes", ...); the value as text, booleans as 0 / 1.  arg: the element-type code
+ * for hooks that take a DataType. */
+PTO_HIP_API int pto_hip_backend_handler_query(const char* hook, int32_t arg, char* buf, size_t cap);
 
 /* ---- tuning knobs (integers by name; unknown names are PTO_HIP_ERR_NOT_FOUND) ------------
  *  "attn_tokens_per_partition"  0 = choose from the device's CU count (default)

@@ -26,6 +26,9 @@ EXPORTS = (
     "pto_hip_rope_kv_cache_update_fp8",
     "pto_hip_decoder_layer_decode", "pto_hip_select_program", "pto_hip_projection",
     "pto_hip_gate_up_swiglu", "pto_hip_paged_attention_noalloc",
+    "pto_hip_write_manifest", "pto_hip_backend_info", "pto_hip_backend_op_name", "pto_hip_backend_op_info",
+    "pto_hip_backend_codegen", "pto_hip_backend_check_ops", "pto_hip_backend_program_ops",
+    "pto_hip_backend_mem_path", "pto_hip_backend_handler_query",
 )
 
 
@@ -46,6 +49,24 @@ class ChipTensor(C.Structure):
 
 class ManifestKernel(C.Structure):
     _fields_ = [("func_id", C.c_int32), ("core_type", C.c_int32), ("name", C.c_char_p)]
+
+
+class BackendInfo(C.Structure):
+    _fields_ = [
+        ("type_name", C.c_char * 16),
+        ("backend_type", C.c_char * 16),
+        ("target_arch", C.c_char * 16),
+        ("cube_cores", C.c_int32),
+        ("vector_cores", C.c_int32),
+        ("dies", C.c_int32),
+        ("wavefront_size", C.c_int32),
+        ("n_ops", C.c_int32),
+        ("n_programs", C.c_int32),
+        ("mem_bytes", C.c_uint64 * 7),
+        ("mem_alignment", C.c_uint64 * 7),
+        ("l2_bytes_per_die", C.c_uint64),
+        ("last_level_cache_bytes", C.c_uint64),
+    ]
 
 
 class DeviceInfo(C.Structure):
@@ -106,6 +127,15 @@ def load() -> C.CDLL:
         "pto_hip_decoder_layer_decode": [vp, vp],
         "pto_hip_select_program": [C.c_char_p, C.POINTER(ManifestKernel), C.c_int32, C.POINTER(C.c_int32),
                                    C.c_int32, C.POINTER(C.c_char_p)],
+        "pto_hip_write_manifest": [C.c_char_p, C.c_char_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)],
+        "pto_hip_backend_info": [C.POINTER(BackendInfo)],
+        "pto_hip_backend_op_name": [C.c_int32, C.POINTER(C.c_char_p)],
+        "pto_hip_backend_op_info": [C.c_char_p, C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t],
+        "pto_hip_backend_codegen": [C.c_char_p, C.POINTER(C.c_char_p), C.c_int32, C.c_char_p, C.c_char_p, C.c_size_t],
+        "pto_hip_backend_check_ops": [C.c_char_p, C.POINTER(C.c_char_p), C.c_int32],
+        "pto_hip_backend_program_ops": [C.c_char_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)],
+        "pto_hip_backend_mem_path": [C.c_int32, C.c_int32, C.POINTER(C.c_int32), C.c_int32, C.POINTER(C.c_int32)],
+        "pto_hip_backend_handler_query": [C.c_char_p, C.c_int32, C.c_char_p, C.c_size_t],
         "pto_hip_set_option": [C.c_char_p, i64],
         "pto_hip_get_option": [C.c_char_p, C.POINTER(i64)],
     }

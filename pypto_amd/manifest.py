@@ -143,6 +143,30 @@ def read_kernel_config(work_dir: str | Path) -> Manifest:
         kernels=tuple(kernels))
 
 
+def kernel_config_text(program: str, runtime: str = DEFAULT_RUNTIME) -> str:
+    """``kernel_config.py`` text for a fused program, in the reference generator's format
+    (``_generate_config_file``, python/pypto/backend/pto_backend.py:933-1045), from the native
+    backend's program table.  ValueError for a program without a manifest form."""
+    lib = _lib.load()
+    need = C.c_size_t(0)
+    _lib.check(lib.pto_hip_write_manifest(program.encode(), runtime.encode(), None, 0, C.byref(need)))
+    buf = C.create_string_buffer(need.value)
+    _lib.check(lib.pto_hip_write_manifest(program.encode(), runtime.encode(), buf, need.value, None))
+    return buf.value.decode()
+
+
+def write_kernel_config(work_dir: str | Path, program: str, runtime: str = DEFAULT_RUNTIME) -> Path:
+    """Writes ``<work_dir>/kernel_config.py`` for ``program`` and returns its path: the manifest half
+    of the reference's artifact tree (docs/en/dev/codegen/00-pto_codegen.md:721-743).  The tree's
+    ``kernels/`` and ``orchestration/`` sources have no counterpart here - one fused kernel stands
+    for the whole task graph - so the manifest's source paths name files that are not written."""
+    work_dir = Path(work_dir)
+    work_dir.mkdir(parents=True, exist_ok=True)
+    path = work_dir / "kernel_config.py"
+    path.write_text(kernel_config_text(program, runtime), encoding="utf-8")
+    return path
+
+
 def select_program_name(manifest: Manifest) -> str:
     """Name of the fused HIP program the manifest's kernel set describes (native matcher)."""
     lib = _lib.load()
