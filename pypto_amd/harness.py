@@ -27,9 +27,18 @@ import torch
 from .runtime import ChipWorker, HipProgram, RunConfig, validate_golden
 
 
+_FACTORIES = (torch.randn, torch.rand, torch.zeros, torch.ones)
+
+
 @dataclass
 class TensorSpec:
-    """One tensor of a test case (tensor_spec.py:30-77)."""
+    """One tensor of a test case: name, shape, dtype, how to fill it, whether it is an output.
+
+    Same fields as the reference's spec (tensor_spec.py:30-77).  ``init_value`` may be nothing
+    (zeros), a number (constant fill), a tensor (converted to ``dtype``), one of torch's shape
+    factories (``torch.randn`` / ``rand`` / ``zeros`` / ``ones``, called with the shape) or any other
+    callable returning array-like data.
+    """
 
     name: str
     shape: list[int]
@@ -38,25 +47,26 @@ class TensorSpec:
     is_output: bool = False
 
     def create_tensor(self) -> torch.Tensor:
-        if self.init_value is None:
+        init = self.init_value
+        if init is None:
             return torch.zeros(self.shape, dtype=self.dtype)
-        if isinstance(self.init_value, (int, float)):
-            return torch.full(self.shape, self.init_value, dtype=self.dtype)
-        if isinstance(self.init_value, torch.Tensor):
-            return self.init_value.to(dtype=self.dtype)
-        if callable(self.init_value):
-            fn = self.init_value
-            if fn in (torch.randn, torch.rand, torch.zeros, torch.ones):
-                if not self.dtype.is_floating_point or self.dtype.itemsize < 2:
-                    return fn(self.shape).to(self.dtype)
-                return fn(self.shape, dtype=self.dtype)
-            return torch.as_tensor(fn(), dtype=self.dtype)
-        raise TypeError(f"Unsupported init_value type {type(self.init_value)!r} for tensor {self.name!r}")
+        if isinstance(init, torch.Tensor):
+            return init.to(dtype=self.dtype)
+        if isinstance(init, (int, float)):
+            return torch.full(self.shape, init, dtype=self.dtype)
+        if not callable(init):
+            raise TypeError(f"Unsupported init_value type {type(init)!r} for tensor {self.name!r}")
+        if any(init is f for f in _FACTORIES):
+            # the random factories only produce wide floating types: draw in fp32, then convert
+            wide = self.dtype.is_floating_point and self.dtype.itemsize >= 2
+            return init(self.shape, dtype=self.dtype) if wide else init(self.shape).to(self.dtype)
+        return torch.as_tensor(init(), dtype=self.dtype)
 
 
 @dataclass
 class RunResult:
-    """Outcome of one test-case run (runner.py:530-566)."""
+    """Outcome of one test-case run; prints as ``PASS: name (1.23s)`` / ``FAIL: name - error``
+    (the reference's form, runner.py:530-566)."""
 
     __test__ = False  # not a pytest class
 
@@ -67,13 +77,14 @@ class RunResult:
     profile: dict[str, Any] | None = None
 
     def __str__(self) -> str:
-        time_str = f" ({self.execution_time:.2f}s)" if self.execution_time else ""
-        if self.passed:
-            return (f"PASS: {self.test_name}" if self.test_name else "PASS") + time_str
-        msg = f"FAIL: {self.test_name}" if self.test_name else "FAIL"
-        if self.error:
-            msg += f" - {self.error}"
-        return msg + time_str
+        parts = ["PASS" if self.passed else "FAIL"]
+        if self.test_name:
+            parts[0] += f": {self.test_name}"
+        if not self.passed and self.error:
+            parts.append(f"- {self.error}")
+        if self.execution_time:
+            parts.append(f"({self.execution_time:.2f}s)")
+        return " ".join(parts)
 
 
 class PTOTestCase(ABC):

@@ -21,6 +21,7 @@ from __future__ import annotations
 
 import contextvars
 import ctypes as C
+import math
 import struct
 from dataclasses import dataclass
 from typing import Any, Sequence
@@ -121,35 +122,52 @@ class RunConfig:
             raise ValueError(f"device_id must be a non-negative int, got {self.device_id!r}")
 
 
+def _element_size(dtype: torch.dtype) -> int:
+    return torch.empty(0, dtype=dtype).element_size()
+
+
+def _require_plain_int(value: Any) -> bool:
+    """True for an int that is not a bool (bool is an int subclass and never a size or an address)."""
+    return isinstance(value, int) and not isinstance(value, bool)
+
+
 class DeviceTensor:
-    """Handle to a buffer already resident on a worker (device_tensor.py:43-110)."""
+    """Handle to a buffer already resident on a worker: address, shape and element type.
+
+    The contract is the reference's (device_tensor.py:43-110): the address is a positive integer,
+    the shape a non-empty sequence of positive integers, the dtype a ``torch.dtype``; the memory
+    belongs to whoever allocated it.
+    """
+
+    __slots__ = ("data_ptr", "shape", "dtype")
 
     def __init__(self, data_ptr: int, shape: Sequence[int], dtype: torch.dtype) -> None:
-        if isinstance(data_ptr, bool) or not isinstance(data_ptr, int) or data_ptr <= 0:
-            raise ValueError(f"DeviceTensor.data_ptr must be a positive int, got {data_ptr!r}")
-        raw_shape = tuple(shape)
-        for d in raw_shape:
-            if isinstance(d, bool) or not isinstance(d, int):
-                raise TypeError(f"DeviceTensor.shape must contain ints, got {raw_shape!r}")
-        if not raw_shape:
-            raise ValueError("DeviceTensor.shape must be non-empty")
-        if any(d <= 0 for d in raw_shape):
-            raise ValueError(f"DeviceTensor.shape must be all positive, got {raw_shape}")
-        if not isinstance(dtype, torch.dtype):
-            raise TypeError(f"DeviceTensor.dtype must be torch.dtype, got {type(dtype).__name__}")
-        self.data_ptr = data_ptr
-        self.shape = raw_shape
-        self.dtype = dtype
+        dims = tuple(shape)
+        problem: Exception | None = None
+        if not _require_plain_int(data_ptr) or data_ptr <= 0:
+            problem = ValueError(f"DeviceTensor.data_ptr must be a positive int, got {data_ptr!r}")
+        elif not all(_require_plain_int(d) for d in dims):
+            problem = TypeError(f"DeviceTensor.shape must contain ints, got {dims!r}")
+        elif len(dims) == 0:
+            problem = ValueError("DeviceTensor.shape must be non-empty")
+        elif min(dims) <= 0:
+            problem = ValueError(f"DeviceTensor.shape must be all positive, got {dims}")
+        elif not isinstance(dtype, torch.dtype):
+            problem = TypeError(f"DeviceTensor.dtype must be torch.dtype, got {type(dtype).__name__}")
+        if problem is not None:
+            raise problem
+        self.data_ptr, self.shape, self.dtype = data_ptr, dims, dtype
+
+    @property
+    def numel(self) -> int:
+        return math.prod(self.shape)
 
     @property
     def nbytes(self) -> int:
-        n = torch.tensor([], dtype=self.dtype).element_size()
-        for d in self.shape:
-            n *= d
-        return n
+        return self.numel * _element_size(self.dtype)
 
     def __repr__(self) -> str:
-        return f"DeviceTensor(data_ptr=0x{self.data_ptr:x}, shape={self.shape}, dtype={self.dtype})"
+        return f"DeviceTensor(data_ptr={self.data_ptr:#x}, shape={self.shape}, dtype={self.dtype})"
 
 
 def scalar_to_uint64(value: Any) -> int:
@@ -198,10 +216,8 @@ class ChipWorker:
 
     def __init__(self, config: RunConfig | None = None, *, level: int = 2, auto_init: bool = True) -> None:
         if level != 2:
-            raise ValueError(
-                f"ChipWorker only supports level=2; got level={level}. "
-                f"L3+ runtimes go through DistributedWorker."
-            )
+            # one GPU is the reference's level 2 (a single chip); higher levels are its multi-chip workers
+            raise ValueError(f"ChipWorker only supports level=2 (one device), got level={level}")
         self._config = config or RunConfig()
         self._lib = _lib.load()
         self._initialized = False
@@ -536,25 +552,26 @@ def validate_golden(
     rtol: float = 1e-5,
     atol: float = 1e-5,
 ) -> None:
-    """``torch.isclose`` comparison where NaN in the golden marks a don't-care element.
+    """Compares every tensor of ``outputs`` with its namesake in ``golden``.
 
-    Same contract as device_runner.py:850-899.
+    The rule is the reference's (device_runner.py:850-899): an element passes when
+    ``|actual - expected| <= atol + rtol * |expected|``; a NaN in the golden marks an element nobody
+    cares about and always passes.  The first failing tensor raises AssertionError with the count
+    of mismatches and up to 20 of them.
     """
-    for name, actual_tensor in outputs.items():
-        actual = actual_tensor.cpu()
-        expected = golden[name].cpu()
-        care = ~torch.isnan(expected)
-        close = torch.isclose(actual, expected, rtol=rtol, atol=atol) | ~care
-        if not bool(close.all()):
-            bad = torch.where(~close.flatten())[0]
-            fa, fe = actual.flatten(), expected.flatten()
-            n_show = min(20, bad.numel())
-            lines = [f"    [{i.item()}] actual={fa[i].item()}, expected={fe[i].item()}" for i in bad[:n_show]]
-            n_dc = int((~care).sum().item())
-            skipped = f" ({n_dc} don't-care skipped)" if n_dc else ""
-            raise AssertionError(
-                f"Output '{name}' does not match golden.\n"
-                f"Mismatched elements: {bad.numel()}/{actual.numel()}{skipped}\n"
-                f"rtol={rtol}, atol={atol}\n"
-                f"First {n_show} mismatches:\n" + "\n".join(lines)
-            )
+    limit = 20
+    for name, produced in outputs.items():
+        got, want = produced.detach().cpu().reshape(-1), golden[name].detach().cpu().reshape(-1)
+        ignored = want.isnan()
+        wrong = ~(torch.isclose(got, want, rtol=rtol, atol=atol) | ignored)
+        n_wrong = int(wrong.sum())
+        if n_wrong == 0:
+            continue
+        where = wrong.nonzero().flatten()[:limit].tolist()
+        report = [f"Output '{name}' does not match golden.",
+                  f"Mismatched elements: {n_wrong}/{got.numel()}"
+                  + (f" ({int(ignored.sum())} don't-care skipped)" if bool(ignored.any()) else ""),
+                  f"rtol={rtol}, atol={atol}",
+                  f"First {len(where)} mismatches:"]
+        report += [f"    [{i}] actual={got[i].item()}, expected={want[i].item()}" for i in where]
+        raise AssertionError("\n".join(report))
