@@ -7,10 +7,15 @@ A step is one paged-attention decode pass over one batch of the "small" configur
 (batch 16, 32 query heads, 8 KV heads, head_dim 128, block 128, context ~U[512,4096], bf16 KV in
 a pool of 1024 blocks, permutation block table).  The step rotates through several identical KV
 pools so the working set stays larger than the 256 MB last-level cache.  The printed JSON line
-carries the whole-step throughput (`value`), the roofline of the dominant kernel, the FFN block
-at LLaMA-7B shape as a second measurement, two more HBM-bound workloads of the same path (the
-long-context e4m3 attention configuration and one W8A16 decoder-layer decode step), and the CPU
-oracle timed on this machine's host cores.
+carries the whole-step throughput (`value`), the roofline of the dominant kernel, and one block
+per other configuration of the path: the FFN at LLaMA-7B shape, the long-context e4m3 attention
+configuration and one W8A16 decoder-layer decode step.  Every block has a `cpu_baseline` beside
+it: the CPU oracle timed on this machine's host cores on a bounded sample of the same workload.
+
+The HBM traffic of the dominant kernel and its traced duration are read from
+profiles/bench_attention_small_ffn_llama7b.json, which `python -m pypto_amd.profile_summary` writes
+from rocprofv3 runs of this script; the in-run duration comes from HIP events that the library
+records around the kernel on its stream ("attn_kernel_timing").
 """
 
 from __future__ import annotations
@@ -21,19 +26,49 @@ import os
 import statistics
 import sys
 import time
+from pathlib import Path
 
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 KV_POOLS = 4                   # 4 x 537 MB of K+V, cycled
+ROOT = Path(__file__).resolve().parent
+PROFILE = ROOT / "profiles" / "bench_attention_small_ffn_llama7b.json"
+DOMINANT_KERNEL = "attn_partition_kernel<128, true, false, 1>"
 
-# HBM bytes one launch of the dominant kernel moves, from hardware counters: rocprofv3 --pmc
-# FETCH_SIZE and --pmc WRITE_SIZE (KiB per dispatch) of this script, each scaled by what the same
-# counter reads for a plain 1 GiB device copy (FETCH_SIZE reads 0.5 KiB per KiB copied, WRITE_SIZE
-# 1.0).  The counter runs and their figures are in profiles/bench_attention_small_ffn_llama7b.md.
-PMC_FETCH_KIB = 74372.5
-PMC_FETCH_SCALE = 1048576.0 / 524321.0
-PMC_WRITE_KIB = 1284.8
-PMC_WRITE_SCALE = 1.0
+
+def _profile_figures() -> dict:
+    """Counter traffic and traced duration of the dominant kernel from the tracked profile data."""
+    from pypto_amd.profile_summary import hbm_traffic_bytes
+
+    if not PROFILE.exists():
+        return {"traffic": None, "kernel_us_rocprof": None, "source": f"{PROFILE.name} not found"}
+    prof = json.loads(PROFILE.read_text())
+    key = next((k for k in prof.get("kernels", {}) if k.endswith(DOMINANT_KERNEL)), None)
+    if key is None:
+        return {"traffic": None, "kernel_us_rocprof": None, "source": f"{PROFILE.name} has no {DOMINANT_KERNEL}"}
+    return {"traffic": hbm_traffic_bytes(prof, key),
+            "kernel_us_rocprof": round(prof["kernels"][key]["avg_us"], 2),
+            "source": f"profiles/{PROFILE.name}: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this script scaled by a "
+                      "plain copy of known size; --kernel-trace --stats average duration"}
+
+
+def _time_cpu(fn, budget_s: float, min_runs: int = 3, max_runs: int = 400):
+    """Median wall time of fn() over as many runs as fit the budget (at least min_runs), after one warm-up."""
+    fn()
+    times = []
+    t_begin = time.perf_counter()
+    while len(times) < min_runs or (time.perf_counter() - t_begin < budget_s and len(times) < max_runs):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return statistics.median(times), len(times)
+
+
+def _hbm_block(workload: str, nbytes: int, us: float) -> dict:
+    gbps = nbytes / us / 1e3
+    return {"workload": workload, "algorithmic_bytes_per_step": nbytes, "us_per_step": round(us, 1),
+            "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
+            "bound": "hbm"}
 
 
 def main() -> int:
@@ -41,11 +76,13 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timings")
     ap.add_argument("--no-ffn", action="store_true", help="skip the FFN measurement")
     ap.add_argument("--no-extra", action="store_true",
-                    help="skip the other workloads of the path: long-context e4m3 attention, decoder layer, "
-                         "the layer with bf16 weights, FFN at 16 tokens, vocabulary projection, 64-head MQA attention")
+                    help="skip the long-context e4m3 attention configuration and the decoder layer")
+    ap.add_argument("--more", action="store_true",
+                    help="also time shapes outside the benchmark configurations: the layer with bf16 weights, a "
+                         "qwen3-14B layer, the FFN at 16 tokens, a vocabulary projection, 64-head MQA attention")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy, a known-size reference for HBM byte counters")
     args = ap.parse_args()
@@ -56,8 +93,8 @@ def main() -> int:
     import torch
 
     from pypto_amd import workloads
-    from pypto_amd.runtime import (ChipWorker, RunConfig, benchmark, decoder_layer_decode, decoder_layer_decode_w16,
-                                   ffn_block, paged_attention, projection)
+    from pypto_amd.runtime import (ChipWorker, PreparedBenchmark, RunConfig, benchmark, decoder_layer_decode,
+                                   decoder_layer_decode_w16, ffn_block, paged_attention, projection)
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -65,31 +102,34 @@ def main() -> int:
 
     worker = ChipWorker(RunConfig(platform="mi355x", device_id=0))
     info = worker.device_info()
+    cores = torch.get_num_threads()
+    cpu = not args.no_cpu_baseline
+    if cpu:
+        import oracle
 
     # ---- paged-attention decode, small configuration ------------------------------------
     pools = [workloads.attention_small(seed=0, device="cuda") for _ in range(KV_POOLS)]
     torch.cuda.synchronize()
     step_bytes = pools[0].algorithmic_bytes()
-    arg_sets = [p.args() for p in pools]
     handle = worker.register(paged_attention)
+    prepared = PreparedBenchmark(handle, [p.args() for p in pools])
 
-    benchmark(handle, arg_sets, rounds=max(args.warmup, 1), warmup=0)  # untimed warm-up steps
+    prepared.run(max(args.warmup, 1))       # W untimed warm-up steps
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    stats = benchmark(handle, arg_sets, rounds=args.steps, warmup=0)   # exactly K timed steps
+    stats = prepared.run(args.steps)        # exactly K timed steps, issued by the library's register-once loop
     torch.cuda.synchronize()
     wall_s = time.perf_counter() - t0
     ms_per_step = wall_s * 1e3 / args.steps
     value = step_bytes / (wall_s / args.steps) / 1e9
-    step_us_events = stats.device_wall_us
 
-    # Dominant kernel alone (streaming kernel, partials left unmerged), HIP events on its stream.
-    worker.set_option("attn_skip_merge", 1)
-    benchmark(handle, arg_sets, rounds=10, warmup=0)
-    kstats = benchmark(handle, arg_sets, rounds=args.steps, warmup=0)
-    worker.set_option("attn_skip_merge", 0)
-    kernel_us = kstats.device_wall_us
+    # The dominant kernel alone: the library brackets it with HIP events on its stream in every launch.
+    worker.set_option("attn_kernel_timing", 1)
+    prepared.run(max(args.steps, 50))
+    kernel_us = worker.get_option("attn_kernel_time_ns") / 1e3
+    worker.set_option("attn_kernel_timing", 0)
     achieved = step_bytes / kernel_us / 1e3  # GB/s
+    prof = _profile_figures()
 
     result = {
         "metric": "paged-attn decode HBM GB/s + FFN TFLOP/s, % of MI355X roofline, 1 GPU",
@@ -109,24 +149,34 @@ def main() -> int:
                         "pool 1024 blocks, permutation table, scale 1/sqrt(128), fp32 softmax",
             "kv_pools_rotated": KV_POOLS,
             "algorithmic_bytes_per_step": step_bytes,
-            "step_us_hip_events": round(step_us_events, 2),
+            "step_us_hip_events": round(stats.device_wall_us, 2),
             "device": info["arch"],
             "compute_units": info["compute_units"],
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "attn_partition_kernel<128, true, false, 1>",
+            "kernel": DOMINANT_KERNEL,
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "kernel_us": round(kernel_us, 2),
-            "traffic": round((PMC_FETCH_KIB * PMC_FETCH_SCALE + PMC_WRITE_KIB * PMC_WRITE_SCALE) * 1024),
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this script, scaled by a 1 GiB copy",
+            "kernel_us_rocprof": prof["kernel_us_rocprof"],
+            "traffic": prof["traffic"],
+            "traffic_source": prof["source"],
         },
     }
+    if cpu:
+        p = pools[0]
+        host = [t.cpu() for t in (p.query, p.key_cache, p.value_cache, p.block_table, p.context_lens, p.config)]
+        med, n = _time_cpu(lambda: oracle.paged_attention_golden(*host), 8.0, min_runs=5)
+        result["cpu_baseline"] = {
+            "value": round(step_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"full steps of the same workload (torch block-loop golden): median of {n} steps, "
+                      f"{med * 1e3:.1f} ms per step, os.cpu_count()={os.cpu_count()}"}
+        del host
     handle.unregister()
-    del pools[1:], arg_sets
+    del pools, prepared
 
     # ---- FFN block at LLaMA-7B shape (second half of the metric) ------------------------------
     if not args.no_ffn:
@@ -149,9 +199,21 @@ def main() -> int:
             "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
             "bound": "mfma",
         }
-        del f
+        if cpu:
+            rows = 256  # of the 2048 token rows; the weights are the full ones
+            hx, hg = f.x[:rows].cpu(), f.gamma.cpu()
+            hw = [w.cpu() for w in (f.w_gate, f.w_up, f.w_down)]
+            med, n = _time_cpu(lambda: oracle.ffn_block(hx, hg, *hw, f.eps), 6.0)
+            sample_flops = f.flops() * rows // f.x.shape[0]
+            result["ffn"]["cpu_baseline"] = {
+                "value": round(sample_flops / med / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                "sample": f"{rows} of the {f.x.shape[0]} token rows through the oracle's ffn_block with the full weights: "
+                          f"median of {n} runs, {med * 1e3:.0f} ms per run"}
+            del hx, hw
+        del f, fargs
+        torch.cuda.empty_cache()
 
-    # ---- the path's other HBM-bound workloads ---------------------------------------------------
+    # ---- the path's other configurations --------------------------------------------------------
     if not args.no_extra:
         lf = workloads.attention_long_fp8(seed=0, device="cuda")
         torch.cuda.synchronize()
@@ -159,20 +221,32 @@ def main() -> int:
             largs = [lf.args()]
             benchmark(lh, largs, rounds=3, warmup=0)
             lstats = benchmark(lh, largs, rounds=10, warmup=0)
-        lbytes = lf.algorithmic_bytes()
-        result["attention_long_fp8"] = {
-            "workload": "paged-attention decode long: B64 Hq64 Hkv8 D128 bs128 ctx~U[8192,32768], e4m3 KV with "
-                        "one fp32 scale per (block, KV head), dequantised in-kernel",
-            "algorithmic_bytes_per_step": lbytes,
-            "us_per_step": round(lstats.device_wall_us, 1),
-            "achieved": round(lbytes / lstats.device_wall_us / 1e3, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": round(lbytes / lstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
-            "bound": "hbm",
-        }
+        result["attention_long_fp8"] = _hbm_block(
+            "paged-attention decode long: B64 Hq64 Hkv8 D128 bs128 ctx~U[8192,32768], e4m3 KV with one fp32 scale per "
+            "(block, KV head), dequantised in-kernel", lf.algorithmic_bytes(), lstats.device_wall_us)
+        if cpu:
+            # one whole sequence of the batch: its blocks gathered into a compact pool with an identity table
+            cfg = lf.config.tolist()
+            b, hq, hkv, d, bs, mb = cfg[:6]
+            seq = 0
+            ctx = int(lf.context_lens[seq])
+            nblk = (ctx + bs - 1) // bs
+            blocks = lf.block_table.reshape(b, mb)[seq, :nblk].long()
+            rows = (blocks[:, None] * (hkv * bs) + torch.arange(hkv * bs, device="cuda")[None, :]).reshape(-1)
+            sub = (lf.query[seq * hq:(seq + 1) * hq].cpu(), lf.key_cache[rows].cpu(), lf.value_cache[rows].cpu(),
+                   torch.arange(nblk, dtype=torch.int32), lf.context_lens[seq:seq + 1].cpu(),
+                   torch.tensor([1, hq, hkv, d, bs, nblk, cfg[6]], dtype=torch.int64),
+                   lf.k_scale[blocks].cpu(), lf.v_scale[blocks].cpu())
+            med, n = _time_cpu(lambda: oracle.paged_attention_golden(*sub), 5.0)
+            sub_bytes = ctx * hkv * d * 2 + nblk * hkv * 8 + hq * d * 6
+            result["attention_long_fp8"]["cpu_baseline"] = {
+                "value": round(sub_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+                "sample": f"one of the 64 sequences (context {ctx}) through the torch block-loop golden, codes "
+                          f"dequantised on the host: median of {n} runs, {med * 1e3:.0f} ms per run"}
+            del sub
         del lf, largs
         torch.cuda.empty_cache()
+
         dl = workloads.decoder_layer_inputs(device="cuda")
         torch.cuda.synchronize()
         with worker.register(decoder_layer_decode) as dh:
@@ -180,152 +254,92 @@ def main() -> int:
             benchmark(dh, dargs, rounds=5, warmup=0)
             dstats = benchmark(dh, dargs, rounds=20, warmup=0)
         dbytes = dl.algorithmic_bytes()
-        result["decoder_layer"] = {
-            "workload": "decoder-layer decode step: H4096 Hq32 Hkv8 D128 I14336 B32 ctx4096, int8 weights with "
-                        "per-channel scales, bf16 activations and paged KV",
-            "algorithmic_bytes_per_step": dbytes,
-            "us_per_step": round(dstats.device_wall_us, 1),
-            "achieved": round(dbytes / dstats.device_wall_us / 1e3, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": round(dbytes / dstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
-            "bound": "hbm",
-        }
+        result["decoder_layer"] = _hbm_block(
+            "decoder-layer decode step: H4096 Hq32 Hkv8 D128 I14336 B32 ctx4096, int8 weights with per-channel "
+            "scales, bf16 activations and paged KV", dbytes, dstats.device_wall_us)
+        if cpu:
+            # four of the 32 sequences: their blocks in a compact pool; the weights are the full ones
+            seqs = [0, 9, 18, 27]
+            mb, hkv, bs = dl.max_num_blocks_per_req, dl.kv_head_num, dl.block_size
+            blocks = dl.block_table.reshape(-1, mb)[seqs].reshape(-1).long()
+            rows = (blocks[:, None] * (hkv * bs) + torch.arange(hkv * bs, device="cuda")[None, :]).reshape(-1)
+            hw = [t.cpu() for name in ("qkv", "o", "gate", "up", "down") for t in dl.weights[name]]
+            hargs = (dl.hidden[seqs].cpu(), dl.seq_lens[seqs].cpu(), torch.arange(len(seqs) * mb, dtype=torch.int32),
+                     dl.key_cache[rows].cpu(), dl.value_cache[rows].cpu(), dl.rope_cos.cpu(), dl.rope_sin.cpu(),
+                     dl.gamma_in.cpu(), dl.gamma_post.cpu(), *hw)
+            kw = dict(num_heads=dl.num_heads, kv_head_num=hkv, head_dim=dl.head_dim, block_size=bs,
+                      max_num_blocks_per_req=mb, eps=dl.eps)
+            med, n = _time_cpu(lambda: oracle.decoder_layer_decode(*hargs, **kw), 6.0, min_runs=2)
+            wbytes = sum(c.numel() * c.element_size() for c, _ in dl.weights.values())
+            sub_bytes = wbytes + (dbytes - wbytes) * len(seqs) // dl.hidden.shape[0]
+            result["decoder_layer"]["cpu_baseline"] = {
+                "value": round(sub_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+                "sample": f"{len(seqs)} of the 32 sequences through the oracle's decoder_layer_decode with the full "
+                          f"weights (bytes = all weights + those sequences' K/V): median of {n} runs, "
+                          f"{med * 1e3:.0f} ms per run"}
+            del hw, hargs
         del dl, dargs
         torch.cuda.empty_cache()
-        # the same layer with the reference's 16-bit weights
+
+    # ---- shapes outside the benchmark configurations (on request) ---------------------------------
+    if args.more:
+        more = {}
         dw = workloads.decoder_layer_inputs(device="cuda", int8_weights=False)
-        torch.cuda.synchronize()
         with worker.register(decoder_layer_decode_w16) as dh:
-            dwargs = [dw.args()]
-            benchmark(dh, dwargs, rounds=5, warmup=0)
-            dwstats = benchmark(dh, dwargs, rounds=20, warmup=0)
-        dwbytes = dw.algorithmic_bytes()
-        result["decoder_layer_w16"] = {
-            "workload": "decoder-layer decode step with bf16 weights (the reference's layer): H4096 Hq32 Hkv8 D128 "
-                        "I14336 B32 ctx4096, bf16 activations and paged KV",
-            "algorithmic_bytes_per_step": dwbytes,
-            "us_per_step": round(dwstats.device_wall_us, 1),
-            "achieved": round(dwbytes / dwstats.device_wall_us / 1e3, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": round(dwbytes / dwstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
-            "bound": "hbm",
-        }
-        del dw, dwargs
+            benchmark(dh, [dw.args()], rounds=5, warmup=0)
+            st = benchmark(dh, [dw.args()], rounds=20, warmup=0)
+        more["decoder_layer_w16"] = _hbm_block(
+            "decoder-layer decode step with bf16 weights (the reference's layer): H4096 Hq32 Hkv8 D128 I14336 B32 "
+            "ctx4096", dw.algorithmic_bytes(), st.device_wall_us)
+        del dw
         torch.cuda.empty_cache()
         # the reference's CI perf-guard workload: one qwen3-14B decoder layer, batch 16, sequences at
         # max_seq 4096 (.github/perf_baselines/qwen3_14b_decode.json: 1016.66 us on its own hardware)
         dq = workloads.decoder_layer_inputs(batch=16, hidden=5120, num_heads=40, kv_head_num=8, head_dim=128,
                                             intermediate=17408, context=4096, theta=1e6, device="cuda",
                                             int8_weights=False)
-        torch.cuda.synchronize()
         with worker.register(decoder_layer_decode_w16) as dh:
-            dqargs = [dq.args()]
-            benchmark(dh, dqargs, rounds=5, warmup=0)
-            dqstats = benchmark(dh, dqargs, rounds=20, warmup=0)
-        dqbytes = dq.algorithmic_bytes()
-        result["decoder_layer_qwen3_14b"] = {
-            "workload": "qwen3-14B decoder layer decode step, bf16 weights: H5120 Hq40 Hkv8 D128 I17408 B16 ctx4096 "
-                        "(the shape of the reference's CI perf guard, 1016.66 us there on other hardware)",
-            "algorithmic_bytes_per_step": dqbytes,
-            "us_per_step": round(dqstats.device_wall_us, 1),
-            "achieved": round(dqbytes / dqstats.device_wall_us / 1e3, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": round(dqbytes / dqstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
-            "bound": "hbm",
-        }
-        del dq, dqargs
+            benchmark(dh, [dq.args()], rounds=5, warmup=0)
+            st = benchmark(dh, [dq.args()], rounds=20, warmup=0)
+        more["decoder_layer_qwen3_14b"] = _hbm_block(
+            "qwen3-14B decoder layer decode step, bf16 weights: H5120 Hq40 Hkv8 D128 I17408 B16 ctx4096 (the shape of "
+            "the reference's CI perf guard, 1016.66 us there on other hardware)", dq.algorithmic_bytes(),
+            st.device_wall_us)
+        del dq
         torch.cuda.empty_cache()
-        # FFN block at a decode-size token count: bound by reading the 16-bit weights once
         fd = [workloads.ffn_inputs(tokens=16, hidden=4096, intermediate=11008, seed=s, device="cuda") for s in (0, 1)]
-        torch.cuda.synchronize()
         with worker.register(ffn_block) as fh:
             fdargs = [(f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.out, f.eps) for f in fd]
             benchmark(fh, fdargs, rounds=10, warmup=0)
-            fdstats = benchmark(fh, fdargs, rounds=40, warmup=0)
-        wbytes = 3 * 4096 * 11008 * 2 + 2 * 16 * 4096 * 2
-        result["ffn_decode"] = {
-            "workload": "FFN LLaMA-7B at 16 tokens: H4096 I11008 bf16 weights streamed once, RMSNorm prologue, SwiGLU",
-            "algorithmic_bytes_per_step": wbytes,
-            "us_per_step": round(fdstats.device_wall_us, 1),
-            "achieved": round(wbytes / fdstats.device_wall_us / 1e3, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": round(wbytes / fdstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
-            "bound": "hbm",
-        }
+            st = benchmark(fh, fdargs, rounds=40, warmup=0)
+        more["ffn_decode"] = _hbm_block(
+            "FFN LLaMA-7B at 16 tokens: H4096 I11008 bf16 weights streamed once, RMSNorm prologue, SwiGLU",
+            3 * 4096 * 11008 * 2 + 2 * 16 * 4096 * 2, st.device_wall_us)
         del fd, fdargs
         torch.cuda.empty_cache()
-        # vocabulary projection of a decode step: the largest single weight stream of the model
         lm_m, lm_k, lm_n = 16, 5120, 151936
         lx = (torch.randn(lm_m, lm_k, device="cuda") / lm_k ** 0.5).to(torch.bfloat16)
         lw = torch.randn(lm_k, lm_n, device="cuda").to(torch.bfloat16)
         lo = torch.zeros(lm_m, lm_n, device="cuda")
-        torch.cuda.synchronize()
         with worker.register(projection) as ph:
             benchmark(ph, [(lx, lw, lo)], rounds=5, warmup=0)
-            pstats = benchmark(ph, [(lx, lw, lo)], rounds=20, warmup=0)
-        pbytes = lm_k * lm_n * 2 + lm_m * lm_k * 2 + lm_m * lm_n * 4
-        result["projection_vocab"] = {
-            "workload": "projection x[16,5120] @ W[5120,151936] bf16 -> fp32 (qwen3-14B vocabulary projection at the "
-                        "reference's decode batch), weights streamed once",
-            "algorithmic_bytes_per_step": pbytes,
-            "us_per_step": round(pstats.device_wall_us, 1),
-            "achieved": round(pbytes / pstats.device_wall_us / 1e3, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": round(pbytes / pstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
-            "bound": "hbm",
-        }
+            st = benchmark(ph, [(lx, lw, lo)], rounds=20, warmup=0)
+        more["projection_vocab"] = _hbm_block(
+            "projection x[16,5120] @ W[5120,151936] bf16 -> fp32 (qwen3-14B vocabulary projection), weights streamed "
+            "once", lm_k * lm_n * 2 + lm_m * lm_k * 2 + lm_m * lm_n * 4, st.device_wall_us)
         del lx, lw, lo
         torch.cuda.empty_cache()
-        # 64 query heads on one KV head (the reference's q_tile 64 shape at a serving size)
         mq = workloads.paged_attention_inputs(batch=256, num_heads=64, kv_head_num=1, head_dim=128, block_size=128,
                                               ctx_range=(2048, 4096), seed=0, device="cuda")
-        torch.cuda.synchronize()
         with worker.register(paged_attention) as mh:
-            margs = [mq.args()]
-            benchmark(mh, margs, rounds=5, warmup=0)
-            mstats = benchmark(mh, margs, rounds=20, warmup=0)
-        mbytes = mq.algorithmic_bytes()
-        result["attention_mqa64"] = {
-            "workload": "paged-attention decode, 64 query heads per KV head: B256 Hq64 Hkv1 D128 bs128 "
-                        "ctx~U[2048,4096] bf16 KV; the cache is counted once",
-            "algorithmic_bytes_per_step": mbytes,
-            "us_per_step": round(mstats.device_wall_us, 1),
-            "achieved": round(mbytes / mstats.device_wall_us / 1e3, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": round(mbytes / mstats.device_wall_us / 1e3 / HBM_PEAK_GBPS, 4),
-            "bound": "hbm",
-        }
-        del mq, margs
+            benchmark(mh, [mq.args()], rounds=5, warmup=0)
+            st = benchmark(mh, [mq.args()], rounds=20, warmup=0)
+        more["attention_mqa64"] = _hbm_block(
+            "paged-attention decode, 64 query heads per KV head: B256 Hq64 Hkv1 D128 bs128 ctx~U[2048,4096] bf16 KV; "
+            "the cache is counted once", mq.algorithmic_bytes(), st.device_wall_us)
+        del mq
         torch.cuda.empty_cache()
-
-    # ---- CPU baseline: the oracle on this machine's host cores --------------------------------
-    if not args.no_cpu_baseline:
-        import oracle
-
-        p = pools[0]
-        host = [t.cpu() for t in (p.query, p.key_cache, p.value_cache, p.block_table, p.context_lens, p.config)]
-        times = []
-        oracle.paged_attention_golden(*host)  # warm-up
-        t_begin = time.perf_counter()
-        while len(times) < 5 or (time.perf_counter() - t_begin < 10.0 and len(times) < 400):
-            t0 = time.perf_counter()
-            oracle.paged_attention_golden(*host)
-            times.append(time.perf_counter() - t0)
-        med = statistics.median(times)
-        result["cpu_baseline"] = {
-            "value": round(step_bytes / med / 1e9, 3),
-            "unit": "GB/s",
-            "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": f"full steps of the same workload (torch block-loop golden) for ~10 s after 1 warm-up: median of "
-                      f"{len(times)} steps, {med * 1e3:.1f} ms per step, os.cpu_count()={os.cpu_count()}",
-        }
+        result["more"] = more
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")

@@ -406,8 +406,11 @@ PTO_HIP_API int pto_hip_backend_handler_query(const char* hook, int32_t arg, cha
  *  "attn_tokens_per_partition"  0 = choose from the device's CU count (default)
  *  "attn_waves_per_cu"          cap on resident attention wavefronts per CU, 0 = none (default); for
  *                               the evenly split form the wavefronts per CU (0 = 4, at most 8)
- *  "attn_skip_merge"            1 = launch only the streaming attention kernel and leave the
- *                               partition partials unmerged (kernel timing aid; output invalid)
+ *  "attn_kernel_timing"         1 = every paged-attention launch gives its streaming kernel a start and a stop
+ *                               HIP event that take the dispatch's own timestamps (results are unaffected;
+ *                               not for launches under graph capture)
+ *  "attn_kernel_time_ns"        read only: mean interval of the pairs recorded since the last read, in
+ *                               nanoseconds (0 when there are none); waits for the last recorded launch
  *  "attn_variant"               0 = one wavefront per (sequence, KV head, partition), 1 = one pinned
  *                               workgroup per CU and the chunk list cut evenly over their wavefronts,
  *                               -1 = by launch size and table capacity (default)

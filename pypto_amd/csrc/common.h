@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <mutex>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "pto_hip.h"
@@ -58,7 +59,10 @@ struct Context {
   int64_t attn_tokens_per_partition = 0;
   int64_t attn_waves_per_cu = 0;
   int64_t attn_variant = -1;  // -1 by launch size, 0 partition grid, 1 evenly split form
-  int64_t attn_skip_merge = 0;
+  // "attn_kernel_timing": the streaming attention kernel of every launch is bracketed by a pair of
+  // HIP events on its stream; "attn_kernel_time_ns" reads the mean interval and drops the pairs.
+  int64_t attn_kernel_timing = 0;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> attn_timed;
   int64_t attn_group_tiles = 0;  // cap on the query tiles one wavefront carries (0 = by group size)
   int64_t gemm_variant = 0;
   int64_t gemm_splits = 0;       // k splits of the tiled GEMM: 0 = by shape, 1..16 = as given (when k allows)

@@ -13,6 +13,7 @@
 //     registers with v_perm_b32 and fed as the A operand of O^T = V^T P^T, so P never
 //     leaves the accumulator layout it was produced in.
 //   * the query group of a KV head (padded to 16 rows) stays in registers as B operand.
+#include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -888,6 +889,26 @@ __global__ __launch_bounds__(256) void attn_lean_reduce_kernel(AttnParams p, lon
   }
 }
 
+// Launches the streaming kernel.  With "attn_kernel_timing" set the launch carries a start and a stop
+// event that take the dispatch's own begin and end timestamps (what a kernel trace reports), not
+// the time of event markers queued around it; pto_hip_get_option("attn_kernel_time_ns") turns the
+// recorded pairs into a mean.
+template <typename Kernel>
+int launch_streaming(Kernel kern, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const AttnParams& p) {
+  pto_hip::Context& cx = pto_hip::ctx();
+  if (cx.attn_kernel_timing) {
+    hipEvent_t e0, e1;
+    PTO_CHECK_HIP(hipEventCreate(&e0));
+    PTO_CHECK_HIP(hipEventCreate(&e1));
+    cx.attn_timed.emplace_back(e0, e1);
+    hipExtLaunchKernelGGL(kern, grid, block, lds, stream, e0, e1, 0, p);
+  } else {
+    hipLaunchKernelGGL(kern, grid, block, lds, stream, p);
+  }
+  PTO_CHECK_HIP(hipGetLastError());
+  return PTO_HIP_OK;
+}
+
 template <int D, bool FP8, int GT>
 int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   dim3 grid((unsigned)(p.n_part * p.hkv * p.gtiles * batch));
@@ -908,29 +929,22 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         attr_set.store(true, std::memory_order_release);
       }
-      hipLaunchKernelGGL(kern, lgrid, lblock, lean_lds, stream, p);
-      return PTO_HIP_OK;
+      return launch_streaming(kern, lgrid, lblock, lean_lds, stream, p);
     };
     int rc = PTO_HIP_OK;
     if (bf16) rc = go(attn_lean_kernel<D, true, FP8, GT>);
     else rc = go(attn_lean_kernel<D, false, FP8, GT>);
     if (rc) return rc;
+    hipLaunchKernelGGL((attn_lean_reduce_kernel<D>), dim3((unsigned)((batch * p.hq + 3) / 4)), dim3(256), 0, stream,
+                       p, (long long)p.n_wg * p.lean_waves);
     PTO_CHECK_HIP(hipGetLastError());
-    if (!pto_hip::ctx().attn_skip_merge) {
-      hipLaunchKernelGGL((attn_lean_reduce_kernel<D>), dim3((unsigned)((batch * p.hq + 3) / 4)), dim3(256), 0, stream,
-                         p, (long long)p.n_wg * p.lean_waves);
-      PTO_CHECK_HIP(hipGetLastError());
-    }
     return PTO_HIP_OK;
-  } else if (bf16) {
-    hipLaunchKernelGGL((attn_partition_kernel<D, true, FP8, GT>), grid, dim3(64), lds, stream, p);
-  } else {
-    hipLaunchKernelGGL((attn_partition_kernel<D, false, FP8, GT>), grid, dim3(64), lds, stream, p);
   }
-  PTO_CHECK_HIP(hipGetLastError());
-  // "attn_skip_merge" leaves the partials unmerged: a timing aid that isolates the streaming
-  // kernel; results are not valid in that mode.
-  if (p.n_part > 1 && !pto_hip::ctx().attn_skip_merge) {
+  int rc;
+  if (bf16) rc = launch_streaming(attn_partition_kernel<D, true, FP8, GT>, grid, dim3(64), lds, stream, p);
+  else rc = launch_streaming(attn_partition_kernel<D, false, FP8, GT>, grid, dim3(64), lds, stream, p);
+  if (rc) return rc;
+  if (p.n_part > 1) {
     hipLaunchKernelGGL((attn_reduce_kernel<D>), dim3((unsigned)((batch * p.hq + 3) / 4)), dim3(256), 0,
                        stream, p);
     PTO_CHECK_HIP(hipGetLastError());
@@ -1086,7 +1100,7 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     p.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + o_bytes);
   }
   // The merge kernel writes the 16-bit copy; without a merge a cast kernel follows.
-  const bool merged = (p.n_part > 1 || p.n_wg > 0) && !cx.attn_skip_merge;
+  const bool merged = p.n_part > 1 || p.n_wg > 0;
   if (merged) {
     // the merge kernel writes the copy, blocked on request; without a merge a cast kernel writes it row-major
     p.out16 = out16;

@@ -850,8 +850,8 @@ int pto_hip_set_option(const char* name, int64_t value) {
   } else if (!std::strcmp(name, "attn_variant")) {
     PTO_CHECK_ARG(value >= -1 && value <= 1, "attn_variant must be -1, 0 or 1");
     c.attn_variant = value;
-  } else if (!std::strcmp(name, "attn_skip_merge")) {
-    c.attn_skip_merge = value != 0;
+  } else if (!std::strcmp(name, "attn_kernel_timing")) {
+    c.attn_kernel_timing = value != 0;
   } else if (!std::strcmp(name, "attn_waves_per_cu")) {
     PTO_CHECK_ARG(value >= 0 && value <= 16, "attn_waves_per_cu must be in [0, 16]");
     c.attn_waves_per_cu = value;
@@ -881,7 +881,32 @@ int pto_hip_get_option(const char* name, int64_t* value) {
   else if (!std::strcmp(name, "gemm_variant")) *value = c.gemm_variant;
   else if (!std::strcmp(name, "gemm_splits")) *value = c.gemm_splits;
   else if (!std::strcmp(name, "attn_waves_per_cu")) *value = c.attn_waves_per_cu;
-  else if (!std::strcmp(name, "attn_skip_merge")) *value = c.attn_skip_merge;
+  else if (!std::strcmp(name, "attn_kernel_timing")) *value = c.attn_kernel_timing;
+  else if (!std::strcmp(name, "attn_kernel_time_ns")) {
+    // mean interval of the event pairs recorded since the last read; waits for the last of them
+    double total_ms = 0.0;
+    int64_t n = 0;
+    hipError_t first = hipSuccess;
+    for (auto& pr : c.attn_timed) {
+      float ms = 0.f;
+      hipError_t e = hipEventSynchronize(pr.second);
+      if (e == hipSuccess) e = hipEventElapsedTime(&ms, pr.first, pr.second);
+      if (e == hipSuccess) {
+        total_ms += ms;
+        ++n;
+      } else if (first == hipSuccess) {
+        first = e;
+      }
+      (void)hipEventDestroy(pr.first);
+      (void)hipEventDestroy(pr.second);
+    }
+    c.attn_timed.clear();
+    if (first != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(PTO_HIP_ERR_RUNTIME, "attn_kernel_time_ns: %s", hipGetErrorString(first));
+    }
+    *value = n ? (int64_t)(total_ms * 1e6 / (double)n) : 0;
+  }
   else if (!std::strcmp(name, "attn_variant")) *value = c.attn_variant;
   else if (!std::strcmp(name, "attn_group_tiles")) *value = c.attn_group_tiles;
   else if (!std::strcmp(name, "w8a16_wgs_per_cu")) *value = c.w8a16_wgs_per_cu;

@@ -297,6 +297,11 @@ class ChipWorker:
     def set_option(self, name: str, value: int) -> None:
         _lib.check(self._lib.pto_hip_set_option(name.encode(), int(value)))
 
+    def get_option(self, name: str) -> int:
+        value = C.c_int64(0)
+        _lib.check(self._lib.pto_hip_get_option(name.encode(), C.byref(value)))
+        return value.value
+
     # ---- raw memory (runtime_base.py:106-118) -------------------------------------------
     def malloc(self, nbytes: int) -> int:
         self._require_ready("malloc")
@@ -501,6 +506,47 @@ class BenchmarkStats:
         return self.device_wall_us
 
 
+class PreparedBenchmark:
+    """Descriptors of one or more argument sets, built once; ``run(rounds)`` is then a single call into
+    the library's register-once loop, so a caller's own clock around it sees launches only."""
+
+    def __init__(self, handle: RegistrationHandle, arg_sets: Sequence[Sequence[Any]], stream: int = 0) -> None:
+        program = handle.compiled
+        flat: list[_lib.ChipTensor] = []
+        scalars: list[Any] = []
+        n_t = None
+        for args in arg_sets:
+            tensors, scalars = _split_args(program, args)
+            if n_t is None:
+                n_t = len(tensors)
+            elif n_t != len(tensors):
+                raise ValueError("all argument sets must have the same number of tensors")
+            for arg, direction in zip(tensors, program.signature):
+                if isinstance(arg, DeviceTensor):
+                    flat.append(_descriptor(arg.data_ptr, arg.shape, arg.dtype, arg.nbytes))
+                elif isinstance(arg, torch.Tensor) and (arg.is_cuda or direction == HOST):
+                    flat.append(_descriptor(arg.data_ptr(), tuple(arg.shape), arg.dtype,
+                                            arg.numel() * arg.element_size()))
+                else:
+                    raise ValueError("benchmark() needs device-resident tensors (DeviceTensor or CUDA torch tensors)")
+        if n_t is None:
+            raise ValueError("benchmark() needs at least one argument set")
+        self._keep = list(arg_sets)  # the descriptors hold bare addresses
+        self._handle, self._stream, self._n_sets, self._n_t = handle, stream, len(arg_sets), n_t
+        self._descs = (_lib.ChipTensor * len(flat))(*flat)
+        self._n_scalars = len(scalars)
+        self._scalars = (C.c_uint64 * max(len(scalars), 1))(*[scalar_to_uint64(x) for x in scalars])
+
+    def run(self, rounds: int, warmup: int = 0) -> "BenchmarkStats":
+        if rounds <= 0:
+            raise ValueError(f"rounds must be positive, got {rounds}")
+        avg = C.c_float(0.0)
+        _lib.check(self._handle._worker._lib.pto_hip_benchmark(
+            self._handle.cid, self._descs, self._n_sets, self._n_t, self._scalars, self._n_scalars, rounds, warmup,
+            self._stream, C.byref(avg)))
+        return BenchmarkStats(rounds=rounds, warmup=warmup, device_wall_us=float(avg.value))
+
+
 def benchmark(
     handle: RegistrationHandle,
     arg_sets: Sequence[Sequence[Any]],
@@ -517,33 +563,7 @@ def benchmark(
     """
     if rounds <= 0:
         raise ValueError(f"rounds must be positive, got {rounds}")
-    program = handle.compiled
-    worker = handle._worker
-    flat: list[_lib.ChipTensor] = []
-    scalars: list[Any] = []
-    n_t = None
-    for args in arg_sets:
-        tensors, scalars = _split_args(program, args)
-        if n_t is None:
-            n_t = len(tensors)
-        elif n_t != len(tensors):
-            raise ValueError("all argument sets must have the same number of tensors")
-        for i, (arg, direction) in enumerate(zip(tensors, program.signature)):
-            if isinstance(arg, DeviceTensor):
-                flat.append(_descriptor(arg.data_ptr, arg.shape, arg.dtype, arg.nbytes))
-            elif isinstance(arg, torch.Tensor) and (arg.is_cuda or direction == HOST):
-                flat.append(_descriptor(arg.data_ptr(), tuple(arg.shape), arg.dtype, arg.numel() * arg.element_size()))
-            else:
-                raise ValueError("benchmark() needs device-resident tensors (DeviceTensor or CUDA torch tensors)")
-    descs = (_lib.ChipTensor * len(flat))(*flat)
-    sc = (C.c_uint64 * max(len(scalars), 1))(*[scalar_to_uint64(s) for s in scalars])
-    avg = C.c_float(0.0)
-    _lib.check(
-        worker._lib.pto_hip_benchmark(
-            handle.cid, descs, len(arg_sets), n_t, sc, len(scalars), rounds, warmup, stream, C.byref(avg)
-        )
-    )
-    return BenchmarkStats(rounds=rounds, warmup=warmup, device_wall_us=float(avg.value))
+    return PreparedBenchmark(handle, arg_sets, stream).run(rounds, warmup)
 
 
 def validate_golden(

@@ -53,7 +53,7 @@ def test_calls_before_init_fail_loudly():
 def test_options_round_trip_and_ranges():
     """Every documented knob can be set and read back; out-of-range values are ValueError."""
     lib = _lib.load()
-    knobs = {"attn_tokens_per_partition": 256, "attn_waves_per_cu": 4, "attn_skip_merge": 1, "attn_variant": 1,
+    knobs = {"attn_tokens_per_partition": 256, "attn_waves_per_cu": 4, "attn_kernel_timing": 1, "attn_variant": 1,
              "attn_group_tiles": 2,
              "gemm_variant": 2, "gemm_splits": 3, "w8a16_wgs_per_cu": 3, "w8a16_min_steps": 16, "w8a16_wide": 0, "w8a16_gemm_rows": 64}
     for name, value in knobs.items():
