@@ -18,6 +18,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4s lds_v4s;
+typedef __attribute__((address_space(3))) uint16_t lds_u16;
 
 constexpr int BK = 64;        // k extent of one LDS tile
 constexpr int LDK = BK + 8;   // padded LDS row, in 16-bit elements (144 bytes)
@@ -92,8 +93,21 @@ __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
 // has a second instruction stream to draw from while one waits on memory or a barrier.
 // W8: B holds int8 codes (a 16-byte chunk is 16 columns); they are widened to the activation type,
 // exactly, on their way into LDS, and the per-column scales are applied to the accumulators.
+// DIRECT (16-bit weights, k a multiple of the tile): both operand tiles go from global memory
+// straight into LDS (global_load_lds_dwordx4: a wavefront's 64 lanes fill 1 KB of consecutive LDS
+// bytes), with no staging registers and no ds_write stream next to the MFMAs.  The hardware fixes
+// where a lane's 16 bytes land, so rows cannot be padded; bank conflicts are avoided by an XOR
+// swizzle instead, applied on the global side: the lane whose bytes land in 16-byte slot s of A row
+// r fetches logical chunk s ^ (r % 8), and for B the 64-byte group g of k-row r holds logical
+// group g ^ (r % 8).  The fragment reads apply the same XOR.
+template <bool W8, int EDGE>
+constexpr bool gemm_direct() { return !W8 && EDGE != 2; }
+
 template <int MT, int WM, int WN, bool DUAL, bool BF16, int EDGE, typename OutT, bool W8>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
+  constexpr bool DIRECT = gemm_direct<W8, EDGE>();
+  constexpr int LDK = DIRECT ? BK : gemm::LDK;  // LDS row pitch of the A tile, in elements
+  constexpr int LDN = DIRECT ? BN : gemm::LDN;  // ... of the B tile
   constexpr int NBUF = 2;
   constexpr int NT = (BN / 32) / WN;        // B fragments (32 columns each) per wavefront
   constexpr int T = 64 * WM * WN;           // threads
@@ -124,10 +138,15 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
 
   // ---- global -> register staging ---------------------------------------------------
   // A: thread owns 16-byte chunk (tid % 8) of rows tid/8 + (T/8)*i.
-  const int a_chunk = tid & 7, a_row = tid >> 3;
+  // (DIRECT: the thread's bytes land in slot tid % 8 of its row; it fetches the chunk that belongs there)
+  const int a_row = tid >> 3;
+  const int a_chunk = DIRECT ? ((tid & 7) ^ (a_row & 7)) : (tid & 7);
   // B: thread owns 16-byte chunk (tid % 32) of k rows tid/32 + (T/32)*i; in the gate/up pass chunks
   // 0..15 come from the gate weights and 16..31 from the up weights (same output columns).
-  const int b_chunk = tid % BCH, b_row = tid / BCH;
+  const int b_row = tid / BCH;
+  const int b_chunk = DIRECT ? (((((tid % BCH) >> 2) ^ (b_row & 7)) << 2) | (tid & 3)) : tid % BCH;
+  static_assert(!DIRECT || ((T / 8) % 8 == 0 && (T / BCH) % 8 == 0 && BK % 8 == 0),
+                "the swizzle key of a thread's row must not change from chunk to chunk");
   const uint16_t* bsrc;
   int b_col;  // global column of the chunk
   if (DUAL) {
@@ -195,6 +214,23 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
       *reinterpret_cast<u32x4*>(dst) = rb[i];
     }
   };
+  // DIRECT: chunk i of this thread for the tile at k0, written by the hardware to slot tid of the
+  // i-th 16 B x T run of the LDS tile (wave-uniform base + lane * 16).
+  // The instruction is written out instead of going through the compiler's builtin: told that a
+  // load writes LDS, the compiler waits for every such load in flight (vmcnt(0)) before each
+  // transposing fragment read, whatever buffer that read addresses, which puts the memory latency
+  // back into the loop.  Here the only waits are the explicit ones before the barriers.
+  auto to_lds = [&](const void* src, const uint16_t* dst) {
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const lds_u16*)dst);
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // m0 is named as clobbered on purpose
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base) : "memory", "m0");
+#pragma clang diagnostic pop
+  };
+  auto direct_a = [&](uint16_t* da, int k0, int i) { to_lds(a_ptr[i] + k0, da + (i * (T / 8) + wave * 8) * LDK); };
+  auto direct_b = [&](uint16_t* db, int k0, int i) {
+    to_lds(b_ptr + (int64_t)(k0 + (T / BCH) * i) * p.ldb * BESZ, db + (i * (T / BCH) + wave * (64 / BCH)) * LDN);
+  };
   auto load_tile = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < NA; ++i) load_a(k0, i);
@@ -225,15 +261,24 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   //     consecutive n of k-row s/4 (columns (s%4)*4..); the hardware hands lane c of the group
   //     the four k-values of column c.  Lanes 16..31 take the next 16 columns, lanes 32..63 the
   //     next 8 k-rows.
-  const int a_frag = (wm * MT * 32 + (lane & 31)) * LDK + (lane >> 5) * 8;
+  const int a_frag = (wm * MT * 32 + (lane & 31)) * LDK + (DIRECT ? 0 : (lane >> 5) * 8);
+  const int a_key = (lane >> 5) ^ (lane & 7);  // DIRECT: slot of k-chunk 2*ks + lane/32 in row lane%32 is (2*ks) ^ a_key
   const int grp = lane >> 4, sub = lane & 15;
-  int b_frag[NT];
+  int b_frag[NT][DIRECT ? 2 : 1];
 #pragma unroll
   for (int jn = 0; jn < NT; ++jn) {
     // gate/up pass: the first NT/2 fragments are gate columns, the rest the up columns of the same outputs
     const int col = DUAL ? ((jn / (NT / 2)) * (BN / 2) + wn * (16 * NT) + (jn % (NT / 2)) * 32)
                          : (wn * (32 * NT) + jn * 32);
-    b_frag[jn] = ((grp >> 1) * 8 + (sub >> 2)) * LDN + col + (grp & 1) * 16 + (sub & 3) * 4;
+    if constexpr (DIRECT) {
+      // k-row = 16*ks + 4*half + 8*(grp/2) + sub/4: its swizzle key is 4*half + sub/4
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+        b_frag[jn][half] = ((grp >> 1) * 8 + half * 4 + (sub >> 2)) * LDN +
+                           (((col >> 5) ^ (half * 4 + (sub >> 2))) << 5) + (grp & 1) * 16 + (sub & 3) * 4;
+    } else {
+      b_frag[jn][0] = ((grp >> 1) * 8 + (sub >> 2)) * LDN + col + (grp & 1) * 16 + (sub & 3) * 4;
+    }
   }
 
   // One LDS read of the fragment set for k-step `ks` of buffer `buf`: r < MT reads A fragment r,
@@ -241,10 +286,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   u32x4 fa[2][MT], fb[2][NT];
   auto read_one = [&](int buf, int ks, int set, int r) {
     if (r < MT) {
-      fa[set][r] = *reinterpret_cast<const u32x4*>(sa + buf * A_ELEMS + a_frag + ks * 16 + r * 32 * LDK);
+      const int koff = DIRECT ? (((2 * ks) ^ a_key) << 3) : ks * 16;
+      fa[set][r] = *reinterpret_cast<const u32x4*>(sa + buf * A_ELEMS + a_frag + koff + r * 32 * LDK);
     } else {
       const int jn = (r - MT) >> 1, half = (r - MT) & 1;
-      const uint16_t* src = sb + buf * B_ELEMS + (ks * 16 + half * 4) * LDN + b_frag[jn];
+      const uint16_t* src = DIRECT ? sb + buf * B_ELEMS + ks * 16 * LDN + b_frag[jn][half]
+                                   : sb + buf * B_ELEMS + (ks * 16 + half * 4) * LDN + b_frag[jn][0];
       const uint2 v = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)src));
       fb[set][jn][half * 2 + 0] = v.x;
       fb[set][jn][half * 2 + 1] = v.y;
@@ -263,16 +310,26 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   // order.  All loads are unconditional (past the end they re-read the last tile, a cache hit)
   // so the number of requests outstanding at each wait is known at compile time.
   const int nk = (klen + BK - 1) / BK;
-  load_tile(0);
-  store_tile(0);
-  load_tile(min(1, nk - 1) * BK);
+  if constexpr (DIRECT) {
+#pragma unroll
+    for (int i = 0; i < NA; ++i) direct_a(sa, 0, i);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) direct_b(sb, 0, i);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  } else {
+    load_tile(0);
+    store_tile(0);
+    load_tile(min(1, nk - 1) * BK);
+  }
   __syncthreads();
 #pragma unroll
   for (int r = 0; r < kReads; ++r) read_one(0, 0, 0, r);
 
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
-    const int k_next = min(kt + 2, nk - 1) * BK;
+    // staged form: registers hold tile kt+1, tile kt+2 is requested; DIRECT: tile kt+1 is requested
+    // into the other LDS buffer, which every wavefront finished reading before the last barrier
+    const int k_next = min(kt + (DIRECT ? 1 : 2), nk - 1) * BK;
     uint16_t* da = sa + (buf ^ 1) * A_ELEMS;
     uint16_t* db = sb + (buf ^ 1) * B_ELEMS;
 #pragma unroll
@@ -288,15 +345,22 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
         }
 #pragma unroll
         for (int e = q * kMovesPerSlot; e < (q + 1) * kMovesPerSlot; ++e) {
-          if (ks == 0 && e < NA)
-            *reinterpret_cast<u32x4*>(da + (a_row + (T / 8) * e) * LDK + a_chunk * 8) = ra[e];
-          if (ks == 1 && e < NB) store_b(db, e);
-          if (ks == 2 && e < NA) load_a(k_next, e);
-          if (ks == 3 && e < NB) load_b(k_next, e);
+          if constexpr (DIRECT) {
+            if (ks == 0 && e < NA) direct_a(da, k_next, e);
+            if (ks == 1 && e < NB) direct_b(db, k_next, e);
+          } else {
+            if (ks == 0 && e < NA)
+              *reinterpret_cast<u32x4*>(da + (a_row + (T / 8) * e) * LDK + a_chunk * 8) = ra[e];
+            if (ks == 1 && e < NB) store_b(db, e);
+            if (ks == 2 && e < NA) load_a(k_next, e);
+            if (ks == 3 && e < NB) load_b(k_next, e);
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    // DIRECT: the tile requested above must have landed in LDS before anyone reads it
+    if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < kReads; ++r) read_one(buf ^ 1, 0, 0, r);
@@ -370,7 +434,8 @@ int launch_gemm_e(GemmParams p, hipStream_t st) {
   p.tiles_m = (p.m + BM - 1) / BM;
   const int bn_out = DUAL ? BN / 2 : BN;
   p.tiles_n = (p.n + bn_out - 1) / bn_out;
-  const size_t smem = (size_t)NBUF * (BM * LDK + BK * LDN) * sizeof(uint16_t);
+  constexpr bool DIRECT = gemm_direct<W8, EDGE>();
+  const size_t smem = (size_t)NBUF * (BM * (DIRECT ? BK : LDK) + BK * (DIRECT ? BN : LDN)) * sizeof(uint16_t);
   auto kern = gemm_kernel<MT, WM, WN, DUAL, BF16, EDGE, OutT, W8>;
   static std::atomic<bool> attr_set{false};  // per instantiation; callers hold the dispatch lock
   if (!attr_set.load(std::memory_order_acquire)) {
