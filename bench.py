@@ -83,6 +83,11 @@ def main() -> int:
     ap.add_argument("--more", action="store_true",
                     help="also time shapes outside the benchmark configurations: the layer with bf16 weights, a "
                          "qwen3-14B layer, the FFN at 16 tokens, a vocabulary projection, 64-head MQA attention")
+    ap.add_argument("--no-autotune", action="store_true",
+                    help="keep the library's own choice of attention partition size and wavefronts per CU")
+    ap.add_argument("--attn-launch", default=None, metavar="TOKENS,WAVES",
+                    help="fix attn_tokens_per_partition and attn_waves_per_cu for the small configuration instead of "
+                         "measuring (for profiler runs: every traced launch then has the same shape)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy, a known-size reference for HBM byte counters")
     args = ap.parse_args()
@@ -93,8 +98,9 @@ def main() -> int:
     import torch
 
     from pypto_amd import workloads
-    from pypto_amd.runtime import (ChipWorker, PreparedBenchmark, RunConfig, benchmark, decoder_layer_decode,
-                                   decoder_layer_decode_w16, ffn_block, paged_attention, projection)
+    from pypto_amd.runtime import (ChipWorker, PreparedBenchmark, RunConfig, autotune_attention, benchmark,
+                                   decoder_layer_decode, decoder_layer_decode_w16, ffn_block, paged_attention,
+                                   projection)
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -114,6 +120,17 @@ def main() -> int:
     handle = worker.register(paged_attention)
     prepared = PreparedBenchmark(handle, [p.args() for p in pools])
 
+    # Launch shape (partition size, wavefronts per CU) chosen by measurement on this batch, as a serving
+    # engine would do once per batch composition: part of the untimed warm-up.
+    tuned = {"tokens_per_partition": 0, "waves_per_cu": 0}
+    if args.attn_launch:
+        tpp, cap = (int(v) for v in args.attn_launch.split(","))
+        worker.set_option("attn_tokens_per_partition", tpp)
+        worker.set_option("attn_waves_per_cu", cap)
+        tuned = {"tokens_per_partition": tpp, "waves_per_cu": cap}
+        args.no_autotune = True
+    elif not args.no_autotune:
+        tuned = autotune_attention(worker, handle, [p.args() for p in pools])
     prepared.run(max(args.warmup, 1))       # W untimed warm-up steps
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -150,6 +167,11 @@ def main() -> int:
             "kv_pools_rotated": KV_POOLS,
             "algorithmic_bytes_per_step": step_bytes,
             "step_us_hip_events": round(stats.device_wall_us, 2),
+            "attn_tokens_per_partition": tuned["tokens_per_partition"],
+            "attn_waves_per_cu": tuned["waves_per_cu"],
+            "autotune": ("fixed by --attn-launch" if args.attn_launch else None) if args.no_autotune else
+            f"measured in warm-up: {tuned['us']:.2f} us per step against {tuned['default_us']:.2f} us with the library's "
+            "own choice (0, 0)",
             "device": info["arch"],
             "compute_units": info["compute_units"],
         },
@@ -177,6 +199,8 @@ def main() -> int:
         del host
     handle.unregister()
     del pools, prepared
+    worker.set_option("attn_tokens_per_partition", 0)
+    worker.set_option("attn_waves_per_cu", 0)
 
     # ---- FFN block at LLaMA-7B shape (second half of the metric) ------------------------------
     if not args.no_ffn:
@@ -251,12 +275,19 @@ def main() -> int:
         torch.cuda.synchronize()
         with worker.register(decoder_layer_decode) as dh:
             dargs = [dl.args()]
+            dtuned = {"tokens_per_partition": 0, "waves_per_cu": 0}
+            if not args.no_autotune:
+                dtuned = autotune_attention(worker, dh, dargs, rounds=15)
             benchmark(dh, dargs, rounds=5, warmup=0)
             dstats = benchmark(dh, dargs, rounds=20, warmup=0)
+        worker.set_option("attn_tokens_per_partition", 0)
+        worker.set_option("attn_waves_per_cu", 0)
         dbytes = dl.algorithmic_bytes()
         result["decoder_layer"] = _hbm_block(
             "decoder-layer decode step: H4096 Hq32 Hkv8 D128 I14336 B32 ctx4096, int8 weights with per-channel "
             "scales, bf16 activations and paged KV", dbytes, dstats.device_wall_us)
+        result["decoder_layer"]["attn_tokens_per_partition"] = dtuned["tokens_per_partition"]
+        result["decoder_layer"]["attn_waves_per_cu"] = dtuned["waves_per_cu"]
         if cpu:
             # four of the 32 sequences: their blocks in a compact pool; the weights are the full ones
             seqs = [0, 9, 18, 27]

@@ -51,6 +51,7 @@ struct AttnParams {
   int pool_blocks; // physical blocks in the cache when the caller knows it, else 0 (table entries unchecked)
   int* error_flag; // set when a table entry a sequence uses addresses a block outside the cache
   int gt_rows;     // query rows one wavefront covers: 16 x its tile count; gtiles = ceil(group / gt_rows)
+  int resident_cap;  // partition grid: wavefronts allowed on a CU at once, 0 = as many as fit
   int n_wg;        // evenly split form: resident workgroups (one per CU); 0 = partition grid
   int lean_waves;  // ... and wavefronts in each
   float scale_log2e;
@@ -914,8 +915,13 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   dim3 grid((unsigned)(p.n_part * p.hkv * p.gtiles * batch));
   // Unused dynamic LDS caps the wavefronts resident per CU so that the dispatcher spreads the
   // grid over all CUs instead of filling some to their register limit.
-  const int64_t cap = pto_hip::ctx().attn_waves_per_cu;
-  const size_t lds = cap > 0 ? (size_t)(163840 / cap) / 1024 * 1024 : 0;
+  // (the kernel's own K stage counts against the same 160 KB, so the request is what is left of a
+  // wavefront's share)
+  const int64_t cap = p.resident_cap;
+  // 8 KB of the CU's LDS are left out of the division: a request of exactly 160 KB / cap lets only
+  // cap - 1 workgroups in
+  const size_t share = cap > 0 ? (size_t)((163840 - 8192) / cap) / 512 * 512 : 0;
+  const size_t lds = share > (size_t)KStage<D, FP8>::kBytes ? share - KStage<D, FP8>::kBytes : 0;
   if (p.n_wg > 0) {
     // Evenly split form: one workgroup of lean_waves wavefronts per CU.  The LDS request (K stages
     // of the wavefronts, padded past half of the CU's LDS) keeps a second workgroup off the CU.
@@ -1059,6 +1065,7 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   if (tpp > max_ctx) tpp = (max_ctx + align - 1) / align * align;
   p.tpp = (int)tpp;
   p.n_part = (int)((max_ctx + tpp - 1) / tpp);
+  p.resident_cap = (int)cx.attn_waves_per_cu;
   PTO_CHECK_ARG((int64_t)p.n_part * batch * hkv * p.gtiles < (1ll << 31),
                 "paged_attention: batch x heads x partitions exceeds the grid limit");
 

@@ -547,6 +547,36 @@ class PreparedBenchmark:
         return BenchmarkStats(rounds=rounds, warmup=warmup, device_wall_us=float(avg.value))
 
 
+def autotune_attention(worker: ChipWorker, handle: RegistrationHandle, arg_sets: Sequence[Sequence[Any]], *,
+                       rounds: int = 30,
+                       candidates: Sequence[tuple[int, int]] | None = None) -> dict:
+    """Picks the launch shape of the partition-grid attention kernel for a workload by measurement.
+
+    Two knobs decide how a launch spreads over the CUs: ``attn_tokens_per_partition`` (how finely a
+    context is cut) and ``attn_waves_per_cu`` (how many wavefronts a CU may hold at once).  Their best
+    values depend on how ragged the context lengths are, which the host launcher cannot see; a
+    serving engine that keeps its batch composition for many steps can measure instead.  Each
+    candidate ``(tokens_per_partition, waves_per_cu)`` (``0`` = the library's own choice) runs
+    ``rounds`` launches of ``handle`` over ``arg_sets``; the fastest is left set on the worker and
+    returned with the table of timings.  Works for any program that contains the attention kernel
+    (``paged_attention``, ``decoder_layer_decode``).
+    """
+    if candidates is None:
+        candidates = [(0, 0), (0, 2), (0, 3), (0, 4), (512, 3), (768, 2), (768, 3), (1024, 3), (2048, 0), (2048, 2)]
+    prepared = PreparedBenchmark(handle, arg_sets)
+    timings = {}
+    for tpp, cap in candidates:
+        worker.set_option("attn_tokens_per_partition", tpp)
+        worker.set_option("attn_waves_per_cu", cap)
+        prepared.run(max(rounds // 3, 1))
+        timings[(tpp, cap)] = prepared.run(rounds).device_wall_us
+    best = min(timings, key=timings.get)
+    worker.set_option("attn_tokens_per_partition", best[0])
+    worker.set_option("attn_waves_per_cu", best[1])
+    return {"tokens_per_partition": best[0], "waves_per_cu": best[1], "us": timings[best],
+            "default_us": timings.get((0, 0)), "timings": timings}
+
+
 def benchmark(
     handle: RegistrationHandle,
     arg_sets: Sequence[Sequence[Any]],
