@@ -64,6 +64,46 @@ def _time_cpu(fn, budget_s: float, min_runs: int = 3, max_runs: int = 400):
     return statistics.median(times), len(times)
 
 
+def _shader_clock_mhz() -> int | None:
+    """Current shader clock as rocm-smi reports it, or None when the tool is not there."""
+    import re
+    import subprocess
+
+    try:
+        out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    m = re.search(r"sclk clock level[^(]*\((\d+)Mhz\)", out)
+    return int(m.group(1)) if m else None
+
+
+def _ffn_clock_probe(worker, program, f) -> dict:
+    """The FFN block for ~1.5 s per case with the shader clock read about a second in: the benchmark's
+    random operands, then the same shapes filled with zeros (same instructions, no operand toggling)."""
+    import threading
+
+    import torch
+
+    from pypto_amd.runtime import PreparedBenchmark
+
+    out = {}
+    zeros = [torch.zeros_like(t) for t in (f.x, f.w_gate, f.w_up, f.w_down)]
+    cases = {"random_operands": (f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.out, f.eps),
+             "zero_operands": (zeros[0], f.gamma, zeros[1], zeros[2], zeros[3], f.out, f.eps)}
+    with worker.register(program) as fh:
+        for name, fargs in cases.items():
+            prepared = PreparedBenchmark(fh, [fargs])
+            prepared.run(40)
+            box = {}
+            t = threading.Thread(target=lambda: box.update(us=prepared.run(3000).device_wall_us))
+            t.start()
+            time.sleep(1.0)
+            mhz = _shader_clock_mhz()
+            t.join()
+            out[name] = {"us_per_step": round(box["us"], 1), "sclk_mhz": mhz}
+    return out
+
+
 def _hbm_block(workload: str, nbytes: int, us: float) -> dict:
     gbps = nbytes / us / 1e3
     return {"workload": workload, "algorithmic_bytes_per_step": nbytes, "us_per_step": round(us, 1),
@@ -88,6 +128,9 @@ def main() -> int:
     ap.add_argument("--attn-launch", default=None, metavar="TOKENS,WAVES",
                     help="fix attn_tokens_per_partition and attn_waves_per_cu for the small configuration instead of "
                          "measuring (for profiler runs: every traced launch then has the same shape)")
+    ap.add_argument("--ffn-clock-probe", action="store_true",
+                    help="also run the FFN for about 1.5 s on its random operands and on all-zero operands, reading the "
+                         "shader clock (rocm-smi) during each: the gap between the two is the data-dependent clock")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy, a known-size reference for HBM byte counters")
     args = ap.parse_args()
@@ -223,6 +266,8 @@ def main() -> int:
             "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
             "bound": "mfma",
         }
+        if args.ffn_clock_probe:
+            result["ffn"]["clock_probe"] = _ffn_clock_probe(worker, ffn_block, f)
         if cpu:
             rows = 256  # of the 2048 token rows; the weights are the full ones
             hx, hg = f.x[:rows].cpu(), f.gamma.cpu()

@@ -98,7 +98,9 @@ __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
 // bytes), with no staging registers and no ds_write stream next to the MFMAs.  The hardware fixes
 // where a lane's 16 bytes land, so rows cannot be padded; bank conflicts are avoided by an XOR
 // swizzle instead, applied on the global side: the lane whose bytes land in 16-byte slot s of A row
-// r fetches logical chunk s ^ (r % 8), and for B the 64-byte group g of k-row r holds logical
+// r fetches logical chunk s ^ ((r / 2) % 8) - an A row is 128 bytes and the LDS serves 256 bytes a
+// clock, so the 16 lanes of one clock of a fragment read (16 consecutive rows, one chunk each) must
+// land on 16 different slots of a row pair - and for B the 64-byte group g of k-row r holds logical
 // group g ^ (r % 8).  The fragment reads apply the same XOR.
 template <bool W8, int EDGE>
 constexpr bool gemm_direct() { return !W8 && EDGE != 2; }
@@ -140,7 +142,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   // A: thread owns 16-byte chunk (tid % 8) of rows tid/8 + (T/8)*i.
   // (DIRECT: the thread's bytes land in slot tid % 8 of its row; it fetches the chunk that belongs there)
   const int a_row = tid >> 3;
-  const int a_chunk = DIRECT ? ((tid & 7) ^ (a_row & 7)) : (tid & 7);
+  const int a_chunk = DIRECT ? ((tid & 7) ^ ((a_row >> 1) & 7)) : (tid & 7);
   // B: thread owns 16-byte chunk (tid % 32) of k rows tid/32 + (T/32)*i; in the gate/up pass chunks
   // 0..15 come from the gate weights and 16..31 from the up weights (same output columns).
   const int b_row = tid / BCH;
@@ -262,7 +264,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   //     the four k-values of column c.  Lanes 16..31 take the next 16 columns, lanes 32..63 the
   //     next 8 k-rows.
   const int a_frag = (wm * MT * 32 + (lane & 31)) * LDK + (DIRECT ? 0 : (lane >> 5) * 8);
-  const int a_key = (lane >> 5) ^ (lane & 7);  // DIRECT: slot of k-chunk 2*ks + lane/32 in row lane%32 is (2*ks) ^ a_key
+  const int a_key = (lane >> 5) ^ ((lane >> 1) & 7);  // DIRECT: slot of k-chunk 2*ks + lane/32 in row lane%32 is (2*ks) ^ a_key
   const int grp = lane >> 4, sub = lane & 15;
   int b_frag[NT][DIRECT ? 2 : 1];
 #pragma unroll

@@ -75,6 +75,9 @@ def main() -> None:
     ap.add_argument("--stats", type=Path, required=True)
     ap.add_argument("--fetch", type=Path)
     ap.add_argument("--write", type=Path)
+    ap.add_argument("--counters", type=Path, action="append", default=[],
+                    help="a *_counter_collection.csv of any other --pmc run; its counters are listed per kernel")
+    ap.add_argument("--note", action="append", default=[], help="a line of text appended under a Notes heading")
     ap.add_argument("--copy-kib", type=float, default=1048576.0, help="size of the calibration copy in KiB")
     ap.add_argument("--bench-log", type=Path, help="stdout of the traced bench.py run (its JSON line is quoted)")
     ap.add_argument("--command", action="append", default=[], help="a command line that produced the inputs")
@@ -122,6 +125,28 @@ def main() -> None:
             lines.append(f"largest {COPY_KERNEL} dispatch (the {args.copy_kib:.0f} KiB calibration copy): {cname} = "
                          f"{data['calibration'][f'{label}_kib_read_for_copy']:.0f}")
         lines += ["```", ""]
+    if args.counters:
+        lines += ["## Other counters (mean per dispatch, summed over the chip by the profiler)", "```"]
+        merged: dict[str, dict[str, dict]] = collections.defaultdict(dict)
+        for path in args.counters:
+            per = collections.defaultdict(lambda: collections.defaultdict(list))
+            with open(path, newline="") as f:
+                for r in csv.DictReader(f):
+                    per[short_name(r["Kernel_Name"])][r["Counter_Name"]].append(float(r["Counter_Value"]))
+            for k, cs in per.items():
+                for c, v in cs.items():
+                    merged[k][c] = {"mean": sum(v) / len(v), "n": len(v)}
+        for k, cs in merged.items():
+            if k.startswith("torch:") or "rocclr" in k:
+                continue
+            lines.append(k[:110])
+            for c in sorted(cs):
+                lines.append(f"    {c:34s} {cs[c]['mean']:16.0f}  n={cs[c]['n']}")
+            if k in data["kernels"]:
+                data["kernels"][k]["counters"] = {c: cs[c]["mean"] for c in cs}
+        lines += ["```", ""]
+    if args.note:
+        lines += ["## Notes", *args.note, ""]
     args.out_dir.mkdir(exist_ok=True)
     (args.out_dir / f"{args.name}.md").write_text("\n".join(lines))
     (args.out_dir / f"{args.name}.json").write_text(json.dumps(data, indent=1, sort_keys=True) + "\n")
