@@ -372,3 +372,47 @@ def test_reference_end_to_end_configs(worker, context_len):
     ref = _golden(inp)
     for tpp in (0, -4):
         _check(_run(worker, inp, tpp), ref)
+
+
+def test_autotune_attention_picks_a_launch_shape_and_results_stay_correct(worker):
+    """autotune_attention measures candidate (tokens per partition, wavefronts per CU) pairs on the batch,
+    leaves the fastest set, and whatever it picks the output still matches the golden."""
+    from pypto_amd.runtime import autotune_attention
+
+    inp = workloads.paged_attention_inputs(batch=6, num_heads=32, kv_head_num=8, block_size=128,
+                                           context_lens=[3000, 200, 1500, 64, 4096, 900], ctx_range=(1, 4096), seed=41)
+    dev = [t.cuda() if isinstance(t, torch.Tensor) and i != 6 else t for i, t in enumerate(inp.args())]
+    try:
+        with worker.register(paged_attention) as h:
+            best = autotune_attention(worker, h, [dev], rounds=5, candidates=[(0, 0), (0, 3), (512, 2), (2048, 0)])
+            assert (best["tokens_per_partition"], best["waves_per_cu"]) in best["timings"]
+            assert best["us"] == min(best["timings"].values()) and best["default_us"] == best["timings"][(0, 0)]
+            assert worker.get_option("attn_tokens_per_partition") == best["tokens_per_partition"]
+            assert worker.get_option("attn_waves_per_cu") == best["waves_per_cu"]
+            for tpp, cap in best["timings"]:
+                worker.set_option("attn_tokens_per_partition", tpp)
+                worker.set_option("attn_waves_per_cu", cap)
+                dev[5].fill_(float("nan"))
+                h(*dev)
+                worker.sync()
+                _check(dev[5].cpu(), _golden(inp))
+    finally:
+        worker.set_option("attn_tokens_per_partition", 0)
+        worker.set_option("attn_waves_per_cu", 0)
+
+
+def test_kernel_timing_option_reports_a_duration_and_leaves_results_valid(worker):
+    inp = workloads.attention_small(seed=2, pool_blocks=None)
+    dev = [t.cuda() if isinstance(t, torch.Tensor) and i != 6 else t for i, t in enumerate(inp.args())]
+    worker.set_option("attn_kernel_timing", 1)
+    try:
+        with worker.register(paged_attention) as h:
+            for _ in range(3):
+                h(*dev)
+        ns = worker.get_option("attn_kernel_time_ns")
+    finally:
+        worker.set_option("attn_kernel_timing", 0)
+    assert 1_000 < ns < 5_000_000          # a few to a few hundred microseconds
+    assert worker.get_option("attn_kernel_time_ns") == 0   # the pairs were consumed by the read
+    worker.sync()
+    _check(dev[5].cpu(), _golden(inp))
