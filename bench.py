@@ -141,7 +141,8 @@ def main() -> int:
     import torch
 
     from pypto_amd import workloads
-    from pypto_amd.runtime import (ChipWorker, PreparedBenchmark, RunConfig, autotune_attention, benchmark,
+    from pypto_amd.runtime import (ChipWorker, PreparedBenchmark, RunConfig, attention_stream_probe,
+                                   autotune_attention, benchmark,
                                    decoder_layer_decode, decoder_layer_decode_w16, ffn_block, paged_attention,
                                    projection)
 
@@ -190,6 +191,11 @@ def main() -> int:
     worker.set_option("attn_kernel_timing", 0)
     achieved = step_bytes / kernel_us / 1e3  # GB/s
     prof = _profile_figures()
+    # What the memory system gives this launch shape and access pattern: the library's load-only twin of
+    # the kernel (same grid, table walk and loads, nothing computed), over the same rotating pools.
+    probe = [attention_stream_probe(worker, p.key_cache, p.value_cache, p.block_table, p.context_lens, p.config,
+                                    rounds=1) for _ in range(12) for p in pools]
+    load_only_us = sum(probe[len(pools):]) / (len(probe) - len(pools))
 
     result = {
         "metric": "paged-attn decode HBM GB/s + FFN TFLOP/s, % of MI355X roofline, 1 GPU",
@@ -227,6 +233,9 @@ def main() -> int:
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "kernel_us": round(kernel_us, 2),
             "kernel_us_rocprof": prof["kernel_us_rocprof"],
+            "load_only_us": round(load_only_us, 2),
+            "load_only_gbps": round(step_bytes / load_only_us / 1e3, 1),
+            "frac_of_load_only": round(load_only_us / kernel_us, 4),
             "traffic": prof["traffic"],
             "traffic_source": prof["source"],
         },

@@ -200,6 +200,23 @@ PTO_HIP_API int pto_hip_paged_attention_noalloc(const void* query, const void* k
                                                 const float* k_scale, const float* v_scale,
                                                 void* stream);
 
+/* Measurement aid with no counterpart in the reference: how long the memory system takes to
+ * deliver the cache bytes of one pto_hip_paged_attention launch with these arguments.  A load-only
+ * kernel walks the same partition grid (same tokens per partition and residency cap, i.e. the
+ * current "attn_tokens_per_partition" / "attn_waves_per_cu" options), the same block table and
+ * issues the same sixteen 16-byte loads per lane and 32-token chunk, two chunks in flight,
+ * computing and writing nothing.  It is launched `rounds` times; *mean_ns receives the mean
+ * duration (dispatch begin to end) of a launch.  Warm-up, and rotating the cache tensors between
+ * calls when the last-level cache must not help, are the caller's.  The attention kernel cannot be
+ * faster than this figure; the ratio of the two separates what the kernel loses from what the
+ * memory system allows for this launch shape.  Arguments as pto_hip_paged_attention (scales are
+ * not read); launches that would take the evenly split form are PTO_HIP_ERR_UNSUPPORTED unless
+ * "attn_variant" is 0.  Blocks until the launches have finished. */
+PTO_HIP_API int pto_hip_paged_attention_stream_probe(const void* key_cache, const void* value_cache,
+                                                     const int32_t* block_table, const int32_t* context_lens,
+                                                     const int64_t* config, int q_dtype, int kv_dtype, int rounds,
+                                                     void* stream, double* mean_ns);
+
 /* out[i, :] = src[block_table[idx / bs] * bs + idx % bs, col_offset : col_offset + size]
  * (src/ir/op/tensor_ops/paged_gather.cpp:74-199), bit-exact, asynchronous on the stream.  An index
  * that addresses a block outside block_table or a row outside src is skipped and reported by

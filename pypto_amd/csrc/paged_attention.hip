@@ -910,6 +910,11 @@ int launch_streaming(Kernel kern, dim3 grid, dim3 block, size_t lds, hipStream_t
   return PTO_HIP_OK;
 }
 
+// LDS bytes one wavefront of the partition grid must hold (its own K stage included) for at most
+// `cap` of them to fit a CU; 0 = no cap.  8 KB of the CU's 160 KB are left out of the division: a
+// request of exactly 160 KB / cap lets only cap - 1 workgroups in.
+inline size_t lds_share(int cap) { return cap > 0 ? (size_t)((163840 - 8192) / cap) / 512 * 512 : 0; }
+
 template <int D, bool FP8, int GT>
 int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   dim3 grid((unsigned)(p.n_part * p.hkv * p.gtiles * batch));
@@ -917,10 +922,7 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   // grid over all CUs instead of filling some to their register limit.
   // (the kernel's own K stage counts against the same 160 KB, so the request is what is left of a
   // wavefront's share)
-  const int64_t cap = p.resident_cap;
-  // 8 KB of the CU's LDS are left out of the division: a request of exactly 160 KB / cap lets only
-  // cap - 1 workgroups in
-  const size_t share = cap > 0 ? (size_t)((163840 - 8192) / cap) / 512 * 512 : 0;
+  const size_t share = lds_share(p.resident_cap);
   const size_t lds = share > (size_t)KStage<D, FP8>::kBytes ? share - KStage<D, FP8>::kBytes : 0;
   if (p.n_wg > 0) {
     // Evenly split form: one workgroup of lean_waves wavefronts per CU.  The LDS request (K stages
@@ -960,25 +962,98 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
 
 }  // namespace
 
-namespace pto_hip {
-int paged_attention(const void* query, const void* key_cache, const void* value_cache,
-                    const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
-                    bool want_blocked, bool* wrote_blocked, const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
-                    const float* v_scale, int64_t pool_blocks, void* stream, void* fixed_scratch,
-                    size_t fixed_scratch_bytes) {
-  Context& cx = ctx();
-  if (!cx.initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
-  PTO_CHECK_ARG(config != nullptr, "paged_attention: config is null");
+namespace {
+// Load-only twin of attn_partition_kernel: the same grid, the same block-table walk and the same
+// sixteen 16-byte loads per lane and 32-token chunk (K as 1 KB-per-instruction rows, V in the
+// transposed-operand pattern), two chunks in flight, no arithmetic beyond folding the loaded words
+// into one value that is never stored.  Its duration is what the memory system gives this launch
+// shape and access pattern; the attention kernel cannot be faster than that.
+template <int D, bool FP8>
+__global__ __launch_bounds__(64) void attn_stream_probe_kernel(AttnParams p) {
+  const int lane = threadIdx.x;
+  const int c = lane & 15, j = lane >> 4;
+  const int pairs = p.batch * p.hkv * p.gtiles;
+  const int part = blockIdx.x / pairs;
+  const int pair = blockIdx.x % pairs;
+  const int b = pair / (p.hkv * p.gtiles);
+  const int h = (pair / p.gtiles) % p.hkv;
+  const int32_t* table = p.block_table + (size_t)b * p.max_blocks;
+  int win_base = part * p.tpp / p.bs;
+  int win_blk = table[min(win_base + lane, p.max_blocks - 1)];
+  int ctx = p.ctx_lens[b];
+  const int max_ctx = p.max_blocks * p.bs;
+  ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
+  const int tok_begin = part * p.tpp;
+  const int tok_end = min(ctx, tok_begin + p.tpp);
+  if (tok_begin >= tok_end) return;
+  constexpr int kEsz = FP8 ? 1 : 2;
+  const char* kc = reinterpret_cast<const char*>(p.kc);
+  const char* vc = reinterpret_cast<const char*>(p.vc);
+  const uint32_t voff = (uint32_t)(j * 4 * D * kEsz + c * 8 * kEsz);
+  auto clamp_blk = [&]() {
+    if (p.pool_blocks > 0 && (unsigned)win_blk >= (unsigned)p.pool_blocks) win_blk = 0;
+  };
+  clamp_blk();
+  auto tile_offset = [&](int tok) -> size_t {
+    if (tok >= tok_end) tok = tok_begin;
+    const int lb = tok / p.bs;
+    if (lb < win_base || lb >= win_base + 64) {
+      win_base = lb;
+      win_blk = table[min(lb + lane, p.max_blocks - 1)];
+      clamp_blk();
+    }
+    const int blk = __builtin_amdgcn_readlane(win_blk, lb - win_base);
+    return ((size_t)(blk * p.hkv + h) * p.bs + (tok % p.bs)) * (D * kEsz);
+  };
+  KFrag<D, FP8> kf[2];
+  VFrag<D, FP8> vf[2];
+  uint32_t fold = 0;
+  auto request = [&](int slot, int tok) {
+    const size_t o1 = tile_offset(tok + 16), o0 = tile_offset(tok);
+    load_k<D, FP8>(kf[slot], kc + o0, kc + o1, lane);
+    load_v<D, FP8>(vf[slot], vc + o0, vc + o1, voff);
+  };
+  auto consume = [&](int slot) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int s = 0; s < KStage<D, FP8>::kLoads; ++s)
+        fold ^= kf[slot].t[t][s][0] ^ kf[slot].t[t][s][1] ^ kf[slot].t[t][s][2] ^ kf[slot].t[t][s][3];
+#pragma unroll
+    for (int set = 0; set < D / 128; ++set)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if constexpr (FP8) fold ^= vf[slot].t[set][e].x ^ vf[slot].t[set][e].y;
+        else fold ^= vf[slot].t[set][e][0] ^ vf[slot].t[set][e][1] ^ vf[slot].t[set][e][2] ^ vf[slot].t[set][e][3];
+      }
+  };
+  request(0, tok_begin);
+  for (int tok = tok_begin; tok < tok_end; tok += 2 * kChunk) {
+    request(1, tok + kChunk);
+    consume(0);
+    request(0, tok + 2 * kChunk);
+    consume(1);
+  }
+  // never true for the launches this is used on (error_flag is 0 or 1); keeps the loads alive
+  if (fold == 0x5bd1e995u && *p.error_flag == 0x7fffffff) *p.error_flag = (int)fold;
+}
+}  // namespace
+
+namespace {
+// The launch shape for one set of arguments: checks the configuration, fills the shape fields of
+// `p` (heads, query tiles per wavefront, tokens per partition, partition count, residency cap) and
+// says whether the launch takes the evenly split form.  Shared by the attention launch and by the
+// load-only probe, so that both walk the cache in the same pieces.
+int plan_launch(const int64_t* config, int q_dtype, int kv_dtype, bool have_scales, AttnParams& p, int& gt,
+                bool& lean) {
+  pto_hip::Context& cx = pto_hip::ctx();
+  using pto_hip::dtype_name;
+  using pto_hip::fail;
   const int64_t batch = config[0], hq = config[1], hkv = config[2], d = config[3], bs = config[4],
                 max_blocks = config[5];
   uint32_t scale_bits = (uint32_t)(config[6] & 0xFFFFFFFFu);
   float scale;
   __builtin_memcpy(&scale, &scale_bits, 4);
-  PTO_CHECK_ARG(batch >= 0 && batch <= 65535, "paged_attention: batch %lld out of range [0, 65535]",
-                (long long)batch);
-  if (batch == 0) return PTO_HIP_OK;
-  PTO_CHECK_ARG(query && key_cache && value_cache && block_table && context_lens && out,
-                "paged_attention: null tensor pointer");
   PTO_CHECK_ARG(hq > 0 && hkv > 0 && hq % hkv == 0,
                 "paged_attention: num_heads %lld must be a positive multiple of kv_head_num %lld",
                 (long long)hq, (long long)hkv);
@@ -990,7 +1065,7 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
                 "paged_attention: query dtype must be BF16 or FP16, got %s", dtype_name(q_dtype));
   const bool fp8 = kv_dtype == PTO_HIP_FP8E4M3FN;
   if (fp8) {
-    PTO_CHECK_ARG(k_scale && v_scale, "paged_attention: FP8E4M3FN cache needs k_scale and v_scale");
+    PTO_CHECK_ARG(have_scales, "paged_attention: FP8E4M3FN cache needs k_scale and v_scale");
     PTO_CHECK_ARG(bs % 32 == 0, "paged_attention: FP8E4M3FN cache needs block_size %% 32 == 0, got %lld",
                   (long long)bs);
   } else {
@@ -1002,20 +1077,6 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     return fail(PTO_HIP_ERR_UNSUPPORTED, "paged_attention: head_dim %lld not built (128, 256)",
                 (long long)d);
 
-  AttnParams p{};
-  p.q = query;
-  p.kc = key_cache;
-  p.vc = value_cache;
-  p.block_table = block_table;
-  p.ctx_lens = context_lens;
-  p.out = out;
-  p.out16 = nullptr;
-  p.out16_bf16 = q_dtype == PTO_HIP_BF16;
-  p.out16_blocked = 0;
-  if (wrote_blocked) *wrote_blocked = false;
-  p.k_scale = k_scale;
-  p.v_scale = v_scale;
-  p.pool_blocks = pool_blocks > 0 && pool_blocks < (1ll << 31) ? (int)pool_blocks : 0;
   p.error_flag = cx.flags + 2;
   p.batch = (int)batch;
   p.hq = (int)hq;
@@ -1024,7 +1085,7 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   // Query tiles (16 heads each) one wavefront carries: the whole KV group when it fits, so that
   // K and V are read once per group, not once per tile.
   // "attn_group_tiles" caps the count (1 = one tile per wavefront, the KV read once per tile).
-  int gt = p.group <= 16 ? 1 : (p.group <= 32 || d == 256) ? 2 : 4;
+  gt = p.group <= 16 ? 1 : (p.group <= 32 || d == 256) ? 2 : 4;
   if (cx.attn_group_tiles > 0 && gt > cx.attn_group_tiles) gt = (int)cx.attn_group_tiles;
   p.gt_rows = 16 * gt;
   p.gtiles = (p.group + p.gt_rows - 1) / p.gt_rows;
@@ -1033,19 +1094,6 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   p.scale_log2e = scale * kLog2e;
 
   const int64_t max_ctx = max_blocks * bs;
-  const bool bf16 = q_dtype == PTO_HIP_BF16;
-  // Where the partition partials live: the caller's fixed area (never grown) or the workspace.
-  auto partials_area = [&](size_t bytes, void** ws) -> int {
-    if (!fixed_scratch) return workspace(bytes, ws);
-    if (bytes > fixed_scratch_bytes)
-      return fail(PTO_HIP_ERR_INVALID_VALUE,
-                  "paged_attention_noalloc: this launch needs %zu bytes of partition partials, the fixed scratch "
-                  "area holds %zu; use pto_hip_paged_attention for launches of this size",
-                  bytes, fixed_scratch_bytes);
-    *ws = fixed_scratch;
-    return PTO_HIP_OK;
-  };
-
   // Context partitions: about one wavefront per SIMD when every sequence is at its maximum
   // length (measured best for short launches, where the spread of finishing times matters more
   // than occupancy), but never more than 2048 tokens per partition so long contexts still
@@ -1077,7 +1125,60 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   // Many short sequences are the exception (512 sequences of 100-1000 tokens: 280 us against 239 us
   // for the grid, whose single-partition workgroups write final rows and need no merge), so the
   // table must also allow contexts of 4096 tokens.
-  const bool lean = cx.attn_variant >= 0 ? cx.attn_variant == 1 : (kv_bound >= (1ll << 30) && max_ctx >= 4096);
+  lean = cx.attn_variant >= 0 ? cx.attn_variant == 1 : (kv_bound >= (1ll << 30) && max_ctx >= 4096);
+  return PTO_HIP_OK;
+}
+}  // namespace
+
+namespace pto_hip {
+int paged_attention(const void* query, const void* key_cache, const void* value_cache,
+                    const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
+                    bool want_blocked, bool* wrote_blocked, const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
+                    const float* v_scale, int64_t pool_blocks, void* stream, void* fixed_scratch,
+                    size_t fixed_scratch_bytes) {
+  Context& cx = ctx();
+  if (!cx.initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(config != nullptr, "paged_attention: config is null");
+  const int64_t batch = config[0], hq = config[1], hkv = config[2], d = config[3];
+  PTO_CHECK_ARG(batch >= 0 && batch <= 65535, "paged_attention: batch %lld out of range [0, 65535]",
+                (long long)batch);
+  if (batch == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(query && key_cache && value_cache && block_table && context_lens && out,
+                "paged_attention: null tensor pointer");
+  AttnParams p{};
+  int gt = 1;
+  bool lean = false;
+  {
+    const int rc = plan_launch(config, q_dtype, kv_dtype, k_scale && v_scale, p, gt, lean);
+    if (rc != PTO_HIP_OK) return rc;
+  }
+  const bool fp8 = kv_dtype == PTO_HIP_FP8E4M3FN;
+  p.q = query;
+  p.kc = key_cache;
+  p.vc = value_cache;
+  p.block_table = block_table;
+  p.ctx_lens = context_lens;
+  p.out = out;
+  p.out16 = nullptr;
+  p.out16_bf16 = q_dtype == PTO_HIP_BF16;
+  p.out16_blocked = 0;
+  if (wrote_blocked) *wrote_blocked = false;
+  p.k_scale = k_scale;
+  p.v_scale = v_scale;
+  p.pool_blocks = pool_blocks > 0 && pool_blocks < (1ll << 31) ? (int)pool_blocks : 0;
+  const bool bf16 = q_dtype == PTO_HIP_BF16;
+  // Where the partition partials live: the caller's fixed area (never grown) or the workspace.
+  auto partials_area = [&](size_t bytes, void** ws) -> int {
+    if (!fixed_scratch) return workspace(bytes, ws);
+    if (bytes > fixed_scratch_bytes)
+      return fail(PTO_HIP_ERR_INVALID_VALUE,
+                  "paged_attention_noalloc: this launch needs %zu bytes of partition partials, the fixed scratch "
+                  "area holds %zu; use pto_hip_paged_attention for launches of this size",
+                  bytes, fixed_scratch_bytes);
+    *ws = fixed_scratch;
+    return PTO_HIP_OK;
+  };
+
   if (p.n_part > 1 && !lean) {
     const size_t rows = (size_t)batch * hq;
     const size_t o_bytes = rows * p.n_part * d * sizeof(float);
@@ -1183,4 +1284,58 @@ extern "C" int pto_hip_paged_attention(const void* query, const void* key_cache,
   // The size of the caches is not part of this signature: table entries are used as given.
   return pto_hip::paged_attention(query, key_cache, value_cache, block_table, context_lens, out, nullptr, false, nullptr, config,
                                   q_dtype, kv_dtype, k_scale, v_scale, 0, stream);
+}
+
+// Measurement aid: how long the memory system takes to deliver the cache bytes of one attention
+// launch (see attn_stream_probe_kernel).  Nothing is computed and no tensor is written.
+extern "C" int pto_hip_paged_attention_stream_probe(const void* key_cache, const void* value_cache,
+                                                    const int32_t* block_table, const int32_t* context_lens,
+                                                    const int64_t* config, int q_dtype, int kv_dtype, int rounds,
+                                                    void* stream, double* mean_ns) {
+  PTO_DISPATCH_LOCK();
+  pto_hip::Context& cx = pto_hip::ctx();
+  if (!cx.initialized) return pto_hip::fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(config && mean_ns, "stream_probe: config or mean_ns is null");
+  PTO_CHECK_ARG(key_cache && value_cache && block_table && context_lens, "stream_probe: null tensor pointer");
+  PTO_CHECK_ARG(rounds >= 1 && rounds <= 10000, "stream_probe: rounds %d out of range [1, 10000]", rounds);
+  PTO_CHECK_ARG(config[0] >= 1 && config[0] <= 65535, "stream_probe: batch %lld out of range [1, 65535]",
+                (long long)config[0]);
+  AttnParams p{};
+  int gt = 1;
+  bool lean = false;
+  const int rc = plan_launch(config, q_dtype, kv_dtype, true, p, gt, lean);
+  if (rc != PTO_HIP_OK) return rc;
+  if (lean)
+    return pto_hip::fail(PTO_HIP_ERR_UNSUPPORTED,
+                         "stream_probe: these arguments take the evenly split form; the probe walks the partition "
+                         "grid only (set attn_variant to 0 to probe that form)");
+  p.kc = key_cache;
+  p.vc = value_cache;
+  p.block_table = block_table;
+  p.ctx_lens = context_lens;
+  const bool fp8 = kv_dtype == PTO_HIP_FP8E4M3FN;
+  const int64_t d = config[3];
+  dim3 grid((unsigned)(p.n_part * p.hkv * p.gtiles * p.batch));
+  const size_t lds = lds_share(p.resident_cap);
+  hipStream_t hs = (hipStream_t)stream;
+  hipEvent_t e0, e1;
+  PTO_CHECK_HIP(hipEventCreate(&e0));
+  PTO_CHECK_HIP(hipEventCreate(&e1));
+  double total_ms = 0.0;
+  int status = PTO_HIP_OK;
+  for (int r = 0; r < rounds && status == PTO_HIP_OK; ++r) {
+    if (d == 128 && fp8) hipExtLaunchKernelGGL((attn_stream_probe_kernel<128, true>), grid, dim3(64), lds, hs, e0, e1, 0, p);
+    else if (d == 128) hipExtLaunchKernelGGL((attn_stream_probe_kernel<128, false>), grid, dim3(64), lds, hs, e0, e1, 0, p);
+    else if (fp8) hipExtLaunchKernelGGL((attn_stream_probe_kernel<256, true>), grid, dim3(64), lds, hs, e0, e1, 0, p);
+    else hipExtLaunchKernelGGL((attn_stream_probe_kernel<256, false>), grid, dim3(64), lds, hs, e0, e1, 0, p);
+    float ms = 0.f;
+    if (hipGetLastError() != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+        hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
+      status = pto_hip::fail(PTO_HIP_ERR_RUNTIME, "stream_probe: launch %d failed", r);
+    total_ms += ms;
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (status == PTO_HIP_OK) *mean_ns = total_ms * 1e6 / rounds;
+  return status;
 }

@@ -577,6 +577,31 @@ def autotune_attention(worker: ChipWorker, handle: RegistrationHandle, arg_sets:
             "default_us": timings.get((0, 0)), "timings": timings}
 
 
+def attention_stream_probe(worker: ChipWorker, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                           block_table: torch.Tensor, context_lens: torch.Tensor, config: torch.Tensor, *,
+                           q_dtype: torch.dtype = torch.bfloat16, rounds: int = 50, stream: int = 0) -> float:
+    """Microseconds the memory system needs to deliver the cache bytes of one ``paged_attention`` launch.
+
+    Runs the library's load-only twin of the partition-grid attention kernel (same grid, block-table
+    walk and loads under the worker's current ``attn_tokens_per_partition`` / ``attn_waves_per_cu``;
+    nothing computed, nothing written) ``rounds`` times on device-resident tensors and returns the
+    mean duration of one launch.  The attention kernel's time over this figure is what the kernel
+    itself loses; this figure over bytes / 8 TB/s is what the launch shape and access pattern lose.
+    """
+    worker._require_ready("attention_stream_probe")
+    for name, t in (("key_cache", key_cache), ("value_cache", value_cache), ("block_table", block_table),
+                    ("context_lens", context_lens)):
+        if not t.is_cuda or not t.is_contiguous():
+            raise ValueError(f"attention_stream_probe: {name} must be a contiguous device tensor")
+    cfg = config.to("cpu", torch.int64).contiguous()
+    mean_ns = C.c_double(0.0)
+    _lib.check(worker._lib.pto_hip_paged_attention_stream_probe(
+        key_cache.data_ptr(), value_cache.data_ptr(), block_table.data_ptr(), context_lens.data_ptr(),
+        C.cast(cfg.data_ptr(), C.POINTER(C.c_int64)), _dtype_code(q_dtype), _dtype_code(key_cache.dtype), int(rounds),
+        stream, C.byref(mean_ns)))
+    return mean_ns.value / 1e3
+
+
 def benchmark(
     handle: RegistrationHandle,
     arg_sets: Sequence[Sequence[Any]],

@@ -416,3 +416,43 @@ def test_kernel_timing_option_reports_a_duration_and_leaves_results_valid(worker
     assert worker.get_option("attn_kernel_time_ns") == 0   # the pairs were consumed by the read
     worker.sync()
     _check(dev[5].cpu(), _golden(inp))
+
+
+def test_stream_probe_bounds_the_kernel_and_touches_nothing(worker):
+    """The load-only twin of the attention kernel (same grid, table walk and loads) returns a duration,
+    writes no tensor, is not slower than the kernel it bounds, and refuses what it does not cover."""
+    from pypto_amd.runtime import attention_stream_probe
+
+    inp = workloads.attention_small(seed=3, pool_blocks=None)
+    dev = [t.cuda() if isinstance(t, torch.Tensor) and i != 6 else t for i, t in enumerate(inp.args())]
+    query, kc, vc, table, lens, out, cfg = dev
+    before = [t.clone() for t in (kc, vc, table, lens)]
+    attention_stream_probe(worker, kc, vc, table, lens, cfg, rounds=3)          # warm-up
+    probe_us = attention_stream_probe(worker, kc, vc, table, lens, cfg, rounds=20)
+    assert 1.0 < probe_us < 5_000.0
+    for a, b in zip(before, (kc, vc, table, lens)):
+        assert torch.equal(a, b)
+    worker.set_option("attn_kernel_timing", 1)
+    try:
+        with worker.register(paged_attention) as h:
+            for _ in range(23):
+                h(*dev)
+        kernel_us = worker.get_option("attn_kernel_time_ns") / 1e3
+    finally:
+        worker.set_option("attn_kernel_timing", 0)
+    worker.sync()
+    _check(out.cpu(), _golden(inp))
+    assert probe_us < 1.1 * kernel_us, (probe_us, kernel_us)    # the bound may not sit above what it bounds
+    # an e4m3 cache and head_dim 256 have their own instantiations
+    f8 = workloads.paged_attention_inputs(batch=3, num_heads=8, kv_head_num=2, head_dim=256, block_size=64,
+                                          context_lens=[700, 64, 2000], ctx_range=(1, 2048), seed=5, fp8_kv=True)
+    assert attention_stream_probe(worker, f8.key_cache.cuda(), f8.value_cache.cuda(), f8.block_table.cuda(),
+                                  f8.context_lens.cuda(), f8.config, rounds=2) > 0
+    worker.set_option("attn_variant", 1)
+    try:
+        with pytest.raises(RuntimeError, match="evenly split form"):
+            attention_stream_probe(worker, kc, vc, table, lens, cfg, rounds=1)
+    finally:
+        worker.set_option("attn_variant", -1)
+    with pytest.raises(ValueError, match="rounds"):
+        attention_stream_probe(worker, kc, vc, table, lens, cfg, rounds=0)
