@@ -30,6 +30,7 @@ from pathlib import Path
 
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+MFMA_FP8_PEAK_TFLOPS = 5000.0   # MI355X dense fp8
 KV_POOLS = 4                   # 4 x 537 MB of K+V, cycled
 ROOT = Path(__file__).resolve().parent
 PROFILE = ROOT / "profiles" / "bench_attention_small_ffn_llama7b.json"
@@ -77,9 +78,10 @@ def _shader_clock_mhz() -> int | None:
     return int(m.group(1)) if m else None
 
 
-def _ffn_clock_probe(worker, program, f) -> dict:
+def _ffn_clock_probe(worker, program, fargs, zero_idx) -> dict:
     """The FFN block for ~1.5 s per case with the shader clock read about a second in: the benchmark's
-    random operands, then the same shapes filled with zeros (same instructions, no operand toggling)."""
+    random operands, then the same shapes with the tensors at `zero_idx` filled with zeros (same
+    instructions, no operand toggling)."""
     import threading
 
     import torch
@@ -87,9 +89,8 @@ def _ffn_clock_probe(worker, program, f) -> dict:
     from pypto_amd.runtime import PreparedBenchmark
 
     out = {}
-    zeros = [torch.zeros_like(t) for t in (f.x, f.w_gate, f.w_up, f.w_down)]
-    cases = {"random_operands": (f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.out, f.eps),
-             "zero_operands": (zeros[0], f.gamma, zeros[1], zeros[2], zeros[3], f.out, f.eps)}
+    zargs = tuple(torch.zeros_like(a) if i in zero_idx else a for i, a in enumerate(fargs))
+    cases = {"random_operands": tuple(fargs), "zero_operands": zargs}
     with worker.register(program) as fh:
         for name, fargs in cases.items():
             prepared = PreparedBenchmark(fh, [fargs])
@@ -143,7 +144,8 @@ def main() -> int:
     from pypto_amd import workloads
     from pypto_amd.runtime import (ChipWorker, PreparedBenchmark, RunConfig, attention_stream_probe,
                                    autotune_attention, benchmark,
-                                   decoder_layer_decode, decoder_layer_decode_w16, ffn_block, paged_attention,
+                                   decoder_layer_decode, decoder_layer_decode_w16, ffn_block, ffn_block_fp8,
+                                   paged_attention,
                                    projection)
 
     if not torch.cuda.is_available():
@@ -276,7 +278,7 @@ def main() -> int:
             "bound": "mfma",
         }
         if args.ffn_clock_probe:
-            result["ffn"]["clock_probe"] = _ffn_clock_probe(worker, ffn_block, f)
+            result["ffn"]["clock_probe"] = _ffn_clock_probe(worker, ffn_block, fargs[0], (0, 2, 3, 4))
         if cpu:
             rows = 256  # of the 2048 token rows; the weights are the full ones
             hx, hg = f.x[:rows].cpu(), f.gamma.cpu()
@@ -288,7 +290,39 @@ def main() -> int:
                 "sample": f"{rows} of the {f.x.shape[0]} token rows through the oracle's ffn_block with the full weights: "
                           f"median of {n} runs, {med * 1e3:.0f} ms per run"}
             del hx, hw
-        del f, fargs
+        del fargs
+
+        # the same block on e4m3 operands (8-bit MFMA path; the weights quantised per output channel)
+        q, _ = workloads.ffn_fp8_inputs(tokens=2048, hidden=4096, intermediate=11008, seed=0, device="cuda")
+        torch.cuda.synchronize()
+        with worker.register(ffn_block_fp8) as qh:
+            qargs = [q.args()]
+            benchmark(qh, qargs, rounds=20, warmup=0)
+            qstats = benchmark(qh, qargs, rounds=max(20, args.steps // 2), warmup=0)
+        q_tflops = q.flops() / qstats.device_wall_us / 1e6
+        rel = float(((q.out - f.out).norm() / f.out.norm()).item())
+        result["ffn_fp8"] = {
+            "workload": "the same FFN on e4m3 operands: weights e4m3 + one fp32 scale per output channel, activations "
+                        "quantised per token after RMSNorm and after SwiGLU, v_mfma_f32_32x32x64_f8f6f4, fp32 accumulate",
+            "flops_per_step": q.flops(), "us_per_step": round(qstats.device_wall_us, 1),
+            "achieved": round(q_tflops, 1), "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(q_tflops / MFMA_FP8_PEAK_TFLOPS, 4), "bound": "mfma", "dtype": "fp8 e4m3",
+            "rel_distance_to_bf16_block": round(rel, 5),
+        }
+        if args.ffn_clock_probe:
+            result["ffn_fp8"]["clock_probe"] = _ffn_clock_probe(worker, ffn_block_fp8, qargs[0], (0, 2, 4, 6))
+        if cpu:
+            rows = 256
+            hq_args = [t.cpu() for t in q.args()[1:8]]
+            hx = q.x[:rows].cpu()
+            med, n = _time_cpu(lambda: oracle.ffn_block_fp8(hx, *hq_args, q.eps), 6.0)
+            result["ffn_fp8"]["cpu_baseline"] = {
+                "value": round(q.flops() * rows // q.x.shape[0] / med / 1e12, 4), "unit": "TFLOP/s", "cores": cores,
+                "kind": "port",
+                "sample": f"{rows} of the {q.x.shape[0]} token rows through the oracle's ffn_block_fp8 with the full weights: "
+                          f"median of {n} runs, {med * 1e3:.0f} ms per run"}
+            del hq_args, hx
+        del f, q, qargs
         torch.cuda.empty_cache()
 
     # ---- the path's other configurations --------------------------------------------------------

@@ -121,6 +121,10 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *  "ffn_block"         tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:155-187
  *      tensors: x[T,H], gamma[1,H] fp32, w_gate[H,I], w_up[H,I], w_down[I,H], out[T,H]
  *      scalars: eps (f32 bits)
+ *  "ffn_block_fp8"     the same block on FP8E4M3FN operands (no counterpart in the reference)
+ *      tensors: x[T,H], gamma[1,H] fp32, w_gate8[I,H] e4m3, w_gate_scale[I] fp32, w_up8[I,H], w_up_scale[I],
+ *               w_down8[H,I], w_down_scale[H], out[T,H] (fp32 or dtype of x);  codes are one row per OUTPUT
+ *               channel with k contiguous;  scalars: eps (f32 bits)
  *  "w8a16_matmul"      examples/models/qwen3_jit/kernels/projection.py:145-177 with int8 weights
  *      tensors: x[M,K], w_q[K,N] i8, w_scale[N] fp32, [residual[M,N],] out[M,N]
  *  "w8a16_swiglu"      examples/models/qwen3_jit/kernels/mlp.py:22-61 with int8 weights
@@ -239,6 +243,42 @@ PTO_HIP_API int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void
                                    const void* w_up, const void* w_down, void* out,
                                    int64_t tokens, int64_t hidden, int64_t intermediate,
                                    float eps, int dtype, int out_dtype, void* stream);
+
+/* The FFN block on e4m3 operands (program "ffn_block_fp8").  No counterpart in the reference,
+ * whose FFN is 16-bit (examples/models/01_ffn.py:111-131, qwen3_jit/kernels/mlp.py:22-61): this is
+ * the same block with the matrix products on the 8-bit MFMA path (v_mfma_f32_32x32x64_f8f6f4, twice
+ * the 16-bit rate).  x is BF16/FP16 [T, H]; the weights are FP8E4M3FN codes stored one row per
+ * OUTPUT channel with k contiguous - w_gate8, w_up8 [I, H], w_down8 [H, I], i.e. the transpose of the
+ * 16-bit layout - with one fp32 scale per output channel (w = code * scale; pto_hip_quantize_rows_fp8
+ * applied to W^T makes them).  Steps: RMSNorm rounded to the activation type (gamma NULL skips it);
+ * per-token quantisation x8 = e4m3(xn / sx), sx = amax/448; g, u = (x8 . w8) * sx[t] * sw[n] with fp32
+ * accumulation; h = SiLU(g) * u rounded to the activation type; per-token quantisation of h; down
+ * product rescaled the same way.  out is FP32 or the activation type.  H and I must be multiples
+ * of 128 (PTO_HIP_ERR_UNSUPPORTED otherwise) and at most 16384. */
+PTO_HIP_API int pto_hip_ffn_swiglu_fp8(const void* x, const float* gamma, const void* w_gate8,
+                                       const float* w_gate_scale, const void* w_up8, const float* w_up_scale,
+                                       const void* w_down8, const float* w_down_scale, void* out, int64_t tokens,
+                                       int64_t hidden, int64_t intermediate, float eps, int x_dtype, int out_dtype,
+                                       void* stream);
+
+/* The stages of pto_hip_ffn_swiglu_fp8, callable on their own (none has a counterpart in the
+ * reference).  rms_norm_quantize_fp8: RMSNorm rounded to x_dtype, then the row quantiser below.
+ * gate_up_swiglu_fp8: h[M, N] = x_dtype(SiLU(g) * u), g = (x8 . w_gate8[n]) * x_scale[m] * w_gate_scale[n]
+ * (u likewise), codes [M, K] and [N, K], fp32 accumulation.  projection_fp8: out[M, N] =
+ * (a8 . w8[n]) * a_scale[m] * w_scale[n].  K a multiple of 128 (PTO_HIP_ERR_UNSUPPORTED otherwise). */
+PTO_HIP_API int pto_hip_rms_norm_quantize_fp8(const void* x, const float* gamma, void* codes, float* scale,
+                                              int64_t rows, int64_t cols, float eps, int x_dtype, void* stream);
+PTO_HIP_API int pto_hip_gate_up_swiglu_fp8(const void* x8, const float* x_scale, const void* w_gate8,
+                                           const float* w_gate_scale, const void* w_up8, const float* w_up_scale,
+                                           void* h, int64_t m, int64_t k, int64_t n, int h_dtype, void* stream);
+PTO_HIP_API int pto_hip_projection_fp8(const void* a8, const float* a_scale, const void* w8, const float* w_scale,
+                                       void* out, int64_t m, int64_t k, int64_t n, int out_dtype, void* stream);
+
+/* Per-row symmetric e4m3 quantisation of a BF16/FP16 [rows, cols] tensor: scale[r] = amax|row| / 448
+ * (1 for an all-zero row), codes = e4m3(clamp(row / scale, +-448)), round to nearest even.  cols a
+ * multiple of 8, at most 16384.  No counterpart in the reference. */
+PTO_HIP_API int pto_hip_quantize_rows_fp8(const void* x, void* codes, float* scale, int64_t rows, int64_t cols,
+                                          int x_dtype, void* stream);
 
 /* out[M, N] = x[M, K] @ w[K, N] (+ residual[M, N]), 16-bit x and w of the same type, fp32
  * accumulation, out FP32 or that type: the reference's projection kernels

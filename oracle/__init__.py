@@ -45,7 +45,8 @@ from .attention import (  # noqa: F401
     quantize_kv_fp8,
 )
 from . import stages  # noqa: F401
-from .ffn import ffn_block, ffn_swiglu, projection, rms_norm, swiglu  # noqa: F401
+from .ffn import (ffn_block, ffn_block_fp8, ffn_swiglu, projection, quantize_rows_fp8, rms_norm,  # noqa: F401
+                  swiglu)
 from .layer import (  # noqa: F401
     decoder_layer_decode,
     kv_append_fp8,

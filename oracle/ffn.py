@@ -15,6 +15,11 @@ programs:
 
 Weights are ``[in, out]`` row-major and used as ``x @ W`` (01_ffn.py:165).
 All matmuls upcast to fp32 first, i.e. fp32 accumulation of exact products.
+
+``quantize_rows_fp8`` / ``ffn_block_fp8`` describe the e4m3 form of the block.  The reference has no
+8-bit FFN, so nothing of the reference pins them: PARITY UNPINNED against the reference; they are
+pinned by mathematics only (tests/test_oracle_ffn.py: the e4m3 rounding bound, the row maximum
+mapping to +-448, idempotence, all-zero rows, and the distance to the 16-bit block).
 """
 
 from __future__ import annotations
@@ -82,3 +87,41 @@ def ffn_block(x, gamma, w_gate, w_up, w_down, eps: float = 1e-6,
     if residual is not None:
         y = y + residual.float()
     return y
+
+
+FP8_E4M3_MAX = 448.0
+
+
+def quantize_rows_fp8(x: torch.Tensor):
+    """Per-row symmetric e4m3: ``(codes float8_e4m3fn [R, C], scale fp32 [R])``.
+
+    ``scale = amax(|row|) / 448`` (1 for an all-zero row), ``codes = e4m3(clamp(row / scale, +-448))``
+    with round-to-nearest-even - the recipe of the per-(block, head) KV quantiser
+    (``oracle.attention.quantize_kv_fp8``) applied to rows.  Activations are quantised per token,
+    weights per output channel (a weight is handed over as ``W^T``, one row per output channel).
+    """
+    xf = x.float()
+    amax = xf.abs().amax(dim=-1)
+    scale = torch.where(amax > 0, amax / FP8_E4M3_MAX, torch.ones_like(amax))
+    codes = (xf / scale.unsqueeze(-1)).clamp(-FP8_E4M3_MAX, FP8_E4M3_MAX).to(torch.float8_e4m3fn)
+    return codes.contiguous(), scale.contiguous()
+
+
+def ffn_block_fp8(x, gamma, wg8, wg_scale, wu8, wu_scale, wd8, wd_scale, eps: float = 1e-6) -> torch.Tensor:
+    """The FFN block on e4m3 operands -> fp32.
+
+    ``x`` is 16-bit; ``wg8, wu8`` are codes ``[I, H]`` and ``wd8`` codes ``[H, I]`` (one row per output
+    channel, k contiguous) with fp32 scales per output channel.  Steps: RMSNorm rounded to the
+    activation dtype (as ``ffn_block``), per-token quantisation, gate/up products accumulated in
+    fp32 and rescaled ``acc * sx[t] * sw[n]``, ``h = SiLU(g) * u`` rounded to the activation dtype,
+    per-token quantisation of ``h``, down product rescaled the same way.
+    """
+    act = x.dtype
+    normed = rms_norm(x, gamma, eps, out_dtype=act) if gamma is not None else x
+    x8, sx = quantize_rows_fp8(normed)
+    xf = x8.float()
+    gate = torch.matmul(xf, wg8.float().t()) * sx[:, None] * wg_scale.float()[None, :]
+    up = torch.matmul(xf, wu8.float().t()) * sx[:, None] * wu_scale.float()[None, :]
+    h = swiglu(gate, up).to(act)
+    h8, sh = quantize_rows_fp8(h)
+    return torch.matmul(h8.float(), wd8.float().t()) * sh[:, None] * wd_scale.float()[None, :]

@@ -1,0 +1,584 @@
+// FFN block on e4m3 operands (no counterpart in the reference, whose FFN is 16-bit: this is the
+// "fp8 MFMA" form of examples/models/01_ffn.py:111-131 / qwen3_jit/kernels/mlp.py:22-61).
+//
+//   xn  = bf16(RMSNorm(x) * gamma)                 one row kernel, which also quantises:
+//   x8  = e4m3(xn / sx),  sx[t] = amax_row(xn) / 448
+//   g,u = (x8 @ Wg8^T) * sx[t] * sg[n],  (x8 @ Wu8^T) * sx[t] * su[n]      fp32 accumulation
+//   h   = bf16(SiLU(g) * u)                        epilogue of the gate/up GEMM
+//   h8  = e4m3(h / sh),   sh[t] = amax_row(h) / 448                        row kernel
+//   out = (h8 @ Wd8^T) * sh[t] * sd[n]
+//
+// Weights are e4m3 codes stored one row per OUTPUT channel with k contiguous ([out, in], i.e. the
+// transpose of the 16-bit layout) plus one fp32 scale per output channel, so both GEMM operands
+// are k-major and go global -> LDS -> registers without any transpose.  The GEMM uses
+// v_mfma_f32_32x32x64_f8f6f4: lane l holds row/column l % 32 and the 32 codes k = 32 * (l / 32) .. +32.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+
+#include "common.h"
+
+namespace pto_hip {
+namespace gemm8 {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+typedef __attribute__((address_space(3))) uint8_t lds_u8;
+
+constexpr int BK = 128;   // k extent of one LDS tile row, in codes (= bytes)
+constexpr int BN = 256;   // B rows (output channels) per tile
+constexpr int kXcds = 8;
+constexpr float kE4m3Max = 448.f;
+
+struct Params {
+  const uint8_t* a;    // [M, K] codes, k contiguous
+  const uint8_t* b0;   // [N, K] codes, one row per output channel
+  const uint8_t* b1;   // gate/up pass: the up weights
+  const float* sa;     // [M] row scales of a
+  const float* sb0;    // [N] channel scales of b0
+  const float* sb1;
+  void* c;             // [M, N]
+  int64_t lda, ldb, ldc;
+  int m, n, k;
+  int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ float silu(float g) { return g * __frcp_rn(1.f + __expf(-g)); }
+
+__device__ __forceinline__ int xcd_remap(int pid, int nwg) {
+  const int x = pid % kXcds, local = pid / kXcds;
+  const int full = nwg / kXcds, rem = nwg % kXcds;
+  const int base = x < rem ? x * (full + 1) : rem * (full + 1) + (x - rem) * full;
+  return base + local;
+}
+
+// Tile (32*MT*WM) x 256 x 128 with WM x WN wavefronts; wavefront (wm, wn) owns (32*MT) x (32*NT) as
+// MT x NT accumulators of 32x32, NT = 8 / WN.  In the gate/up pass the 256 B rows of a tile are 128
+// gate channels followed by the 128 up channels of the same outputs, and accumulator columns
+// jn / jn + NT/2 of a wavefront are gate / up of the same 32 outputs, so SiLU(g) * u is applied on
+// the accumulators.
+// Both tiles have 128-byte rows and go global -> LDS directly (1 KB per wavefront instruction =
+// 8 rows); the hardware fixes where a lane's 16 bytes land, so instead of padding, the lane whose
+// bytes land in slot s of row r fetches logical chunk s ^ ((r / 2) % 8) and the fragment reads apply
+// the same XOR: the 16 lanes the LDS serves per clock (16 consecutive rows, one logical chunk) then
+// hit 16 different slots of 8 row pairs.
+// A wavefront reads (32*MT + 32*NT) x 128 bytes of fragments per k-tile: eight wavefronts of 128 x 64
+// read 192 KB per k-tile next to 64 KB of tile writes, which at the LDS's ~128 bytes a clock is as
+// many LDS clocks as the k-tile has MFMA clocks (2048 per SIMD).
+template <int MT, int NT, int WM, int WN, bool DUAL, typename OutT>
+__global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
+  constexpr int T = 64 * WM * WN;
+  constexpr int BM = 32 * MT * WM;
+  static_assert(32 * NT * WN == BN && (!DUAL || NT % 2 == 0), "wavefront grid must cover 256 B rows");
+  constexpr int RPR = T / 8;       // tile rows one round of 16-byte requests covers
+  constexpr int NA = BM / RPR;     // rounds (= requests per thread) for the A tile
+  constexpr int NB = BN / RPR;
+  static_assert(RPR % 16 == 0, "the swizzle key of a thread's row must not change from round to round");
+  constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem8[];
+  uint8_t* sa = smem8;                 // [2][BM][128]
+  uint8_t* sb = smem8 + 2 * A_BYTES;   // [2][256][128]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % WM, wn = wave / WM;
+  const int ntiles = p.tiles_m * p.tiles_n;
+  const int tile = xcd_remap(blockIdx.x, ntiles);
+  const int tm = tile % p.tiles_m, tn = tile / p.tiles_m;
+  const int m0 = tm * BM;
+  const int n0 = tn * (DUAL ? BN / 2 : BN);
+
+  // ---- global -> LDS requests ----------------------------------------------------------------
+  const int row_in_round = tid >> 3;
+  const int chunk = (tid & 7) ^ ((row_in_round >> 1) & 7);  // logical chunk whose slot this thread fills
+  const uint8_t* a_ptr[NA];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    const int r = min(m0 + i * RPR + row_in_round, p.m - 1);
+    a_ptr[i] = p.a + (int64_t)r * p.lda + chunk * 16;
+  }
+  const uint8_t* b_ptr[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const int tr = i * RPR + row_in_round;  // row of the B tile
+    const uint8_t* src = (DUAL && tr >= BN / 2) ? p.b1 : p.b0;
+    const int ch = min(n0 + (DUAL ? tr % (BN / 2) : tr), p.n - 1);
+    b_ptr[i] = src + (int64_t)ch * p.ldb + chunk * 16;
+  }
+  // The instruction is written out: told that a load writes LDS, the compiler waits for every such
+  // load in flight before each later LDS read, whatever buffer that read addresses.
+  auto to_lds = [&](const void* src, const uint8_t* dst) {
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const lds_u8*)dst);
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // m0 is named as clobbered on purpose
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base) : "memory", "m0");
+#pragma clang diagnostic pop
+  };
+  auto request = [&](int buf, int k0, int e) {  // e < NA: A round e, else B round e - NA
+    if (e < NA) to_lds(a_ptr[e] + k0, sa + buf * A_BYTES + (e * RPR + wave * 8) * BK);
+    else to_lds(b_ptr[e - NA] + k0, sb + buf * B_BYTES + ((e - NA) * RPR + wave * 8) * BK);
+  };
+
+  // ---- fragments -------------------------------------------------------------------------------
+  // lane l: row/column l % 32, logical chunks 4*ks + 2*(l/32) and the next; every fragment starts at
+  // a row that is a multiple of 32, so the swizzle key is (l / 2) % 8 for all of them.
+  const int key = (lane >> 1) & 7;
+  const int frag_row = (lane & 31) * BK;
+  const int c_lane = (lane >> 5) * 2;
+  v8i fa[MT], fb[NT];
+  auto read16 = [&](const uint8_t* tile_base, int row_off, int c) -> u32x4 {
+    return *reinterpret_cast<const u32x4*>(tile_base + row_off + frag_row + ((c ^ key) << 4));
+  };
+  auto read_a = [&](int buf, int ks, int i) {
+    const uint8_t* base = sa + buf * A_BYTES;
+    const int row_off = (wm * MT * 32 + i * 32) * BK;
+    const u32x4 lo = read16(base, row_off, 4 * ks + c_lane), hi = read16(base, row_off, 4 * ks + c_lane + 1);
+    fa[i] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+  };
+  auto read_b = [&](int buf, int ks, int jn) {
+    const uint8_t* base = sb + buf * B_BYTES;
+    const int row = DUAL ? (jn / (NT / 2)) * (BN / 2) + wn * (16 * NT) + (jn % (NT / 2)) * 32 : wn * (32 * NT) + jn * 32;
+    const u32x4 lo = read16(base, row * BK, 4 * ks + c_lane), hi = read16(base, row * BK, 4 * ks + c_lane + 1);
+    fb[jn] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+  };
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int jn = 0; jn < NT; ++jn)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][jn][r] = 0.f;
+
+  // One k-step (64 codes): MT x NT MFMAs, column by column.  A fragment register is reloaded for the
+  // next k-step right after its last use - fb[jn] after column jn, fa[i] after MFMA (i, NT-1) - so one
+  // set of fragment registers serves as its own double buffer and every fragment is requested at
+  // least MT - 1 MFMAs (200 cycles and more) ahead of its first use.
+  // `mid` runs once after column 0, before the first reload; per_slot(q) after MFMA number q.
+  auto k_step = [&](int next_buf, int next_ks, auto&& mid, auto&& per_slot) {
+#pragma unroll
+    for (int jn = 0; jn < NT; ++jn) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        acc[i][jn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[jn], acc[i][jn], 0, 0, 0, 0, 0, 0);
+        if (jn == NT - 1) read_a(next_buf, next_ks, i);
+        per_slot(jn * MT + i);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (jn == 0) mid();
+      read_b(next_buf, next_ks, jn);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // Tiles kt (being multiplied), kt+1 (landed in the other buffer) and kt+2 (in flight into the
+  // buffer of kt) are live at once.  The one barrier of a k-tile sits in its second k-step, after
+  // column 0: by then this wavefront has read the last fragment of tile kt (the wait for it is
+  // covered by those MFMAs) and waits for its own requests of tile kt+1; past the barrier every
+  // wavefront has done both, so tile kt+1 may be read and the buffer of tile kt refilled.
+  const int nk = p.k / BK;
+  {
+    const int k1 = min(1, nk - 1) * BK;
+#pragma unroll
+    for (int e = 0; e < NA + NB; ++e) request(0, 0, e);
+#pragma unroll
+    for (int e = 0; e < NA + NB; ++e) request(1, k1, e);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < MT; ++i) read_a(0, 0, i);
+#pragma unroll
+  for (int jn = 0; jn < NT; ++jn) read_b(0, 0, jn);
+
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    const int k2 = min(kt + 2, nk - 1) * BK;
+    // first k-step: reloads fetch the second k-step of the same tile
+    k_step(buf, 1, [] {}, [](int) {});
+    // second k-step: barrier after column 0, then reloads from tile kt+1 and the requests of tile kt+2
+    k_step(
+        buf ^ 1, 0,
+        [&] {
+          asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_sched_barrier(0);
+        },
+        [&](int slot) {
+          // the slots of columns 1 .. NT-1 come after the barrier: NA + NB requests spread over them
+          if (slot >= MT) {
+            constexpr int kAfter = MT * (NT - 1);
+            constexpr int per = (NA + NB + kAfter - 1) / kAfter;
+#pragma unroll
+            for (int e = (slot - MT) * per; e < (slot - MT + 1) * per; ++e)
+              if (e < NA + NB) request(buf, k2, e);
+          }
+        });
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land in LDS after the workgroup has gone
+
+  // ---- epilogue ----------------------------------------------------------------------------------
+  // acc[i][jn][r]: row m0 + wm*MT*32 + i*32 + (r/4)*8 + (lane/32)*4 + r%4, column lane % 32 of fragment jn
+  OutT* c = reinterpret_cast<OutT*>(p.c);
+  const int row_base = m0 + wm * MT * 32 + (lane >> 5) * 4;
+  int col[NT];
+  float sc[NT];
+#pragma unroll
+  for (int jn = 0; jn < NT; ++jn) {
+    col[jn] = DUAL ? n0 + wn * (16 * NT) + (jn % (NT / 2)) * 32 + (lane & 31) : n0 + wn * (32 * NT) + jn * 32 + (lane & 31);
+    const float* s = (DUAL && jn >= NT / 2) ? p.sb1 : p.sb0;
+    sc[jn] = col[jn] < p.n ? s[col[jn]] : 0.f;
+  }
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = row_base + i * 32 + (r >> 2) * 8 + (r & 3);
+      if (row >= p.m) continue;
+      const float sr = p.sa[row];
+      if constexpr (DUAL) {
+#pragma unroll
+        for (int jn = 0; jn < NT / 2; ++jn)
+          if (col[jn] < p.n) {
+            const float g = acc[i][jn][r] * sr * sc[jn], u = acc[i][jn + NT / 2][r] * sr * sc[jn + NT / 2];
+            c[(int64_t)row * p.ldc + col[jn]] = (OutT)(silu(g) * u);
+          }
+      } else {
+#pragma unroll
+        for (int jn = 0; jn < NT; ++jn)
+          if (col[jn] < p.n) c[(int64_t)row * p.ldc + col[jn]] = (OutT)(acc[i][jn][r] * sr * sc[jn]);
+      }
+    }
+}
+
+template <int MT, int NT, int WM, int WN, bool DUAL, typename OutT>
+int launch(Params p, hipStream_t st) {
+  constexpr int BM = 32 * MT * WM;
+  p.tiles_m = (p.m + BM - 1) / BM;
+  const int bn_out = DUAL ? BN / 2 : BN;
+  p.tiles_n = (p.n + bn_out - 1) / bn_out;
+  const size_t smem = 2 * (size_t)(BM * BK + BN * BK);
+  auto kern = gemm8_kernel<MT, NT, WM, WN, DUAL, OutT>;
+  static std::atomic<bool> attr_set{false};  // per instantiation; callers hold the dispatch lock
+  if (!attr_set.load(std::memory_order_acquire)) {
+    PTO_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)smem));
+    attr_set.store(true, std::memory_order_release);
+  }
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(64 * WM * WN), smem, st, p);
+  PTO_CHECK_HIP(hipGetLastError());
+  return PTO_HIP_OK;
+}
+
+// Tile height: 256 rows unless that leaves CUs idle and 128 rows do not.  Eight wavefronts (two per
+// SIMD) by default; "gemm_variant" 1 selects four wavefronts of 128 x 128 on the tall tile, which
+// read a third less from LDS per MFMA but leave a SIMD nothing to issue while its one wavefront
+// waits (LLaMA-7B block: 361 us against 334 us).
+template <bool DUAL, typename OutT>
+int launch_any(const Params& p, hipStream_t st) {
+  const int64_t tiles_n = (p.n + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256);
+  const int64_t tall = (int64_t)((p.m + 255) / 256) * tiles_n;
+  if (tall < pto_hip::ctx().num_cu && p.m > 128) return launch<2, 2, 2, 4, DUAL, OutT>(p, st);
+  if (pto_hip::ctx().gemm_variant == 1) return launch<4, 4, 2, 2, DUAL, OutT>(p, st);
+  return launch<4, 2, 2, 4, DUAL, OutT>(p, st);
+}
+
+// ---- row kernels: (RMSNorm +) per-row e4m3 quantisation -----------------------------------------
+constexpr int kRowThreads = 256;
+constexpr int kRowVecs = 8;  // 8-element groups a thread keeps in registers: rows of up to 16384 columns
+
+__device__ __forceinline__ float clamp_e4m3(float v) { return fminf(fmaxf(v, -kE4m3Max), kE4m3Max); }
+
+__device__ __forceinline__ float block_reduce(float v, bool take_max, float* shared) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float o = __shfl_xor(v, off);
+    v = take_max ? fmaxf(v, o) : v + o;
+  }
+  __syncthreads();  // the previous use of `shared` is over
+  if ((threadIdx.x & 63) == 0) shared[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float tot = shared[0];
+#pragma unroll
+  for (int w = 1; w < kRowThreads / 64; ++w) tot = take_max ? fmaxf(tot, shared[w]) : tot + shared[w];
+  return tot;
+}
+
+// One workgroup per row, the row held in registers.  NORM: y = T(x * rsqrt(mean x^2 + eps) * gamma)
+// first (rounded to the 16-bit activation type, as the 16-bit block's RMSNorm output is); then
+// scale = amax|y| / 448 (1 for an all-zero row) and codes = e4m3(clamp(y / scale)).
+template <typename TI, bool NORM>
+__global__ __launch_bounds__(kRowThreads) void row_quant_kernel(const TI* __restrict__ x, const float* __restrict__ gamma,
+                                                                uint8_t* __restrict__ codes, float* __restrict__ scale,
+                                                                int64_t cols, float eps) {
+  typedef __attribute__((__vector_size__(8 * sizeof(TI)))) TI vec8;
+  __shared__ float red[kRowThreads / 64];
+  const int64_t row = blockIdx.x;
+  const vec8* xr = reinterpret_cast<const vec8*>(x + row * cols);
+  const int nvec = (int)(cols / 8);
+  float y[kRowVecs][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < kRowVecs; ++u) {
+    const int i = threadIdx.x + u * kRowThreads;
+    if (i < nvec) {
+      const vec8 v = xr[i];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        y[u][e] = (float)v[e];
+        ss += y[u][e] * y[u][e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[u][e] = 0.f;
+    }
+  }
+  if constexpr (NORM) {
+    const float inv = rsqrtf(block_reduce(ss, false, red) / (float)cols + eps);
+#pragma unroll
+    for (int u = 0; u < kRowVecs; ++u) {
+      const int i = threadIdx.x + u * kRowThreads;
+      if (i < nvec) {
+        const float4 g0 = gamma ? reinterpret_cast<const float4*>(gamma)[2 * i] : float4{1.f, 1.f, 1.f, 1.f};
+        const float4 g1 = gamma ? reinterpret_cast<const float4*>(gamma)[2 * i + 1] : float4{1.f, 1.f, 1.f, 1.f};
+        const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[u][e] = (float)(TI)(y[u][e] * inv * g[e]);
+      }
+    }
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int u = 0; u < kRowVecs; ++u)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(y[u][e]));
+  amax = block_reduce(amax, true, red);
+  const float s = amax > 0.f ? amax / kE4m3Max : 1.f;
+  if (threadIdx.x == 0) scale[row] = s;
+  uint2* crow = reinterpret_cast<uint2*>(codes + row * cols);
+#pragma unroll
+  for (int u = 0; u < kRowVecs; ++u) {
+    const int i = threadIdx.x + u * kRowThreads;
+    if (i < nvec) {
+      float q[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) q[e] = clamp_e4m3(y[u][e] / s);
+      int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
+      w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], w0, true);
+      int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], 0, false);
+      w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], w1, true);
+      crow[i] = uint2{(uint32_t)w0, (uint32_t)w1};
+    }
+  }
+}
+
+int row_quant(const void* x, const float* gamma, bool norm, void* codes, float* scale, int64_t rows, int64_t cols,
+              float eps, int x_dtype, hipStream_t st) {
+  PTO_CHECK_ARG(cols % 8 == 0 && cols <= 8 * kRowThreads * kRowVecs,
+                "quantize_rows_fp8: %lld columns; rows must be a multiple of 8 and at most %d long", (long long)cols,
+                8 * kRowThreads * kRowVecs);
+  PTO_CHECK_ARG(rows < (1ll << 31), "quantize_rows_fp8: too many rows");
+  PTO_CHECK_ARG(((uintptr_t)x | (uintptr_t)gamma) % 16 == 0 && (uintptr_t)codes % 8 == 0,
+                "quantize_rows_fp8: misaligned operand");
+  if (rows == 0) return PTO_HIP_OK;
+  dim3 grid((unsigned)rows), block(kRowThreads);
+  auto go = [&](auto kern, auto* typed) {
+    hipLaunchKernelGGL(kern, grid, block, 0, st, typed, gamma, reinterpret_cast<uint8_t*>(codes), scale, cols, eps);
+  };
+  if (x_dtype == PTO_HIP_BF16) {
+    if (norm) go(row_quant_kernel<__bf16, true>, reinterpret_cast<const __bf16*>(x));
+    else go(row_quant_kernel<__bf16, false>, reinterpret_cast<const __bf16*>(x));
+  } else if (x_dtype == PTO_HIP_FP16) {
+    if (norm) go(row_quant_kernel<_Float16, true>, reinterpret_cast<const _Float16*>(x));
+    else go(row_quant_kernel<_Float16, false>, reinterpret_cast<const _Float16*>(x));
+  } else {
+    return pto_hip::fail(PTO_HIP_ERR_INVALID_VALUE, "quantize_rows_fp8: dtype %s not in {BF16, FP16}",
+                         pto_hip::dtype_name(x_dtype));
+  }
+  PTO_CHECK_HIP(hipGetLastError());
+  return PTO_HIP_OK;
+}
+
+}  // namespace gemm8
+}  // namespace pto_hip
+
+extern "C" int pto_hip_quantize_rows_fp8(const void* x, void* codes, float* scale, int64_t rows, int64_t cols,
+                                         int x_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
+  using namespace pto_hip;
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(rows >= 0 && cols > 0, "quantize_rows_fp8: bad shape [%lld, %lld]", (long long)rows, (long long)cols);
+  if (rows == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(x && codes && scale, "quantize_rows_fp8: null tensor pointer");
+  return gemm8::row_quant(x, nullptr, false, codes, scale, rows, cols, 0.f, x_dtype, (hipStream_t)stream);
+}
+
+extern "C" int pto_hip_rms_norm_quantize_fp8(const void* x, const float* gamma, void* codes, float* scale,
+                                             int64_t rows, int64_t cols, float eps, int x_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
+  using namespace pto_hip;
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(rows >= 0 && cols > 0, "rms_norm_quantize_fp8: bad shape [%lld, %lld]", (long long)rows,
+                (long long)cols);
+  if (rows == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(x && codes && scale, "rms_norm_quantize_fp8: null tensor pointer");
+  return gemm8::row_quant(x, gamma, true, codes, scale, rows, cols, eps, x_dtype, (hipStream_t)stream);
+}
+
+namespace {
+int check_gemm8(const char* what, int64_t m, int64_t k, int64_t n, const void* a, const void* b, const void* c) {
+  using namespace pto_hip;
+  PTO_CHECK_ARG(m >= 0 && k > 0 && n > 0 && m < (1 << 30) && k < (1 << 30) && n < (1 << 30),
+                "%s: bad shape M=%lld K=%lld N=%lld", what, (long long)m, (long long)k, (long long)n);
+  if (k % gemm8::BK != 0)
+    return fail(PTO_HIP_ERR_UNSUPPORTED, "%s: k %lld must be a multiple of %d", what, (long long)k, gemm8::BK);
+  PTO_CHECK_ARG(((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) % 16 == 0, "%s: operand pointers must be 16-byte aligned",
+                what);
+  return PTO_HIP_OK;
+}
+}  // namespace
+
+extern "C" int pto_hip_gate_up_swiglu_fp8(const void* x8, const float* x_scale, const void* w_gate8,
+                                          const float* w_gate_scale, const void* w_up8, const float* w_up_scale,
+                                          void* h, int64_t m, int64_t k, int64_t n, int h_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
+  using namespace pto_hip;
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  int rc = check_gemm8("gate_up_swiglu_fp8", m, k, n, x8, w_gate8, h);
+  if (rc) return rc;
+  if (m == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(x8 && x_scale && w_gate8 && w_gate_scale && w_up8 && w_up_scale && h,
+                "gate_up_swiglu_fp8: null tensor pointer");
+  PTO_CHECK_ARG((uintptr_t)w_up8 % 16 == 0, "gate_up_swiglu_fp8: operand pointers must be 16-byte aligned");
+  PTO_CHECK_ARG(h_dtype == PTO_HIP_BF16 || h_dtype == PTO_HIP_FP16, "gate_up_swiglu_fp8: h dtype %s not in {BF16, FP16}",
+                dtype_name(h_dtype));
+  gemm8::Params p{};
+  p.a = reinterpret_cast<const uint8_t*>(x8);
+  p.b0 = reinterpret_cast<const uint8_t*>(w_gate8);
+  p.b1 = reinterpret_cast<const uint8_t*>(w_up8);
+  p.sa = x_scale;
+  p.sb0 = w_gate_scale;
+  p.sb1 = w_up_scale;
+  p.c = h;
+  p.lda = k;
+  p.ldb = k;
+  p.ldc = n;
+  p.m = (int)m;
+  p.n = (int)n;
+  p.k = (int)k;
+  hipStream_t st = (hipStream_t)stream;
+  return h_dtype == PTO_HIP_BF16 ? gemm8::launch_any<true, __bf16>(p, st) : gemm8::launch_any<true, _Float16>(p, st);
+}
+
+extern "C" int pto_hip_projection_fp8(const void* a8, const float* a_scale, const void* w8, const float* w_scale,
+                                      void* out, int64_t m, int64_t k, int64_t n, int out_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
+  using namespace pto_hip;
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  int rc = check_gemm8("projection_fp8", m, k, n, a8, w8, out);
+  if (rc) return rc;
+  if (m == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(a8 && a_scale && w8 && w_scale && out, "projection_fp8: null tensor pointer");
+  gemm8::Params p{};
+  p.a = reinterpret_cast<const uint8_t*>(a8);
+  p.b0 = reinterpret_cast<const uint8_t*>(w8);
+  p.sa = a_scale;
+  p.sb0 = w_scale;
+  p.c = out;
+  p.lda = k;
+  p.ldb = k;
+  p.ldc = n;
+  p.m = (int)m;
+  p.n = (int)n;
+  p.k = (int)k;
+  hipStream_t st = (hipStream_t)stream;
+  switch (out_dtype) {
+    case PTO_HIP_FP32: return gemm8::launch_any<false, float>(p, st);
+    case PTO_HIP_BF16: return gemm8::launch_any<false, __bf16>(p, st);
+    case PTO_HIP_FP16: return gemm8::launch_any<false, _Float16>(p, st);
+    default:
+      return fail(PTO_HIP_ERR_INVALID_VALUE, "projection_fp8: output dtype %s not in {FP32, BF16, FP16}",
+                  dtype_name(out_dtype));
+  }
+}
+
+extern "C" int pto_hip_ffn_swiglu_fp8(const void* x, const float* gamma, const void* w_gate8, const float* w_gate_scale,
+                                      const void* w_up8, const float* w_up_scale, const void* w_down8,
+                                      const float* w_down_scale, void* out, int64_t tokens, int64_t hidden,
+                                      int64_t intermediate, float eps, int x_dtype, int out_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
+  using namespace pto_hip;
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(tokens >= 0 && hidden > 0 && intermediate > 0, "ffn_fp8: bad shape T=%lld H=%lld I=%lld",
+                (long long)tokens, (long long)hidden, (long long)intermediate);
+  PTO_CHECK_ARG(tokens < (1 << 30) && hidden < (1 << 30) && intermediate < (1 << 30), "ffn_fp8: shape too large");
+  if (tokens == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(x && w_gate8 && w_gate_scale && w_up8 && w_up_scale && w_down8 && w_down_scale && out,
+                "ffn_fp8: null tensor pointer");
+  PTO_CHECK_ARG(x_dtype == PTO_HIP_BF16 || x_dtype == PTO_HIP_FP16, "ffn_fp8: activation dtype %s not in {BF16, FP16}",
+                dtype_name(x_dtype));
+  PTO_CHECK_ARG(out_dtype == PTO_HIP_FP32 || out_dtype == x_dtype,
+                "ffn_fp8: output dtype %s must be FP32 or the activation dtype %s", dtype_name(out_dtype),
+                dtype_name(x_dtype));
+  if (hidden % gemm8::BK != 0 || intermediate % gemm8::BK != 0)
+    return fail(PTO_HIP_ERR_UNSUPPORTED, "ffn_fp8: hidden %lld and intermediate %lld must be multiples of %d",
+                (long long)hidden, (long long)intermediate, gemm8::BK);
+  PTO_CHECK_ARG(((uintptr_t)x | (uintptr_t)gamma | (uintptr_t)w_gate8 | (uintptr_t)w_up8 | (uintptr_t)w_down8 |
+                 (uintptr_t)out) % 16 == 0,
+                "ffn_fp8: operand pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+
+  auto pad = [](size_t b) { return (b + 255) / 256 * 256; };
+  const size_t x8_bytes = pad((size_t)tokens * hidden), h8_bytes = pad((size_t)tokens * intermediate);
+  const size_t h_bytes = pad((size_t)tokens * intermediate * 2), s_bytes = pad((size_t)tokens * sizeof(float));
+  void* ws = nullptr;
+  int rc = workspace(x8_bytes + h8_bytes + h_bytes + 2 * s_bytes, &ws);
+  if (rc) return rc;
+  char* base = reinterpret_cast<char*>(ws);
+  uint8_t* x8 = reinterpret_cast<uint8_t*>(base);
+  uint8_t* h8 = reinterpret_cast<uint8_t*>(base + x8_bytes);
+  void* h = base + x8_bytes + h8_bytes;
+  float* sx = reinterpret_cast<float*>(base + x8_bytes + h8_bytes + h_bytes);
+  float* sh = reinterpret_cast<float*>(base + x8_bytes + h8_bytes + h_bytes + s_bytes);
+
+  // RMSNorm prologue and the activation quantiser are one row kernel
+  rc = gemm8::row_quant(x, gamma, gamma != nullptr, x8, sx, tokens, hidden, eps, x_dtype, st);
+  if (rc) return rc;
+
+  gemm8::Params p1{};
+  p1.a = x8;
+  p1.b0 = reinterpret_cast<const uint8_t*>(w_gate8);
+  p1.b1 = reinterpret_cast<const uint8_t*>(w_up8);
+  p1.sa = sx;
+  p1.sb0 = w_gate_scale;
+  p1.sb1 = w_up_scale;
+  p1.c = h;
+  p1.lda = hidden;
+  p1.ldb = hidden;
+  p1.ldc = intermediate;
+  p1.m = (int)tokens;
+  p1.n = (int)intermediate;
+  p1.k = (int)hidden;
+  rc = x_dtype == PTO_HIP_BF16 ? gemm8::launch_any<true, __bf16>(p1, st) : gemm8::launch_any<true, _Float16>(p1, st);
+  if (rc) return rc;
+
+  rc = gemm8::row_quant(h, nullptr, false, h8, sh, tokens, intermediate, 0.f, x_dtype, st);
+  if (rc) return rc;
+
+  gemm8::Params p2{};
+  p2.a = h8;
+  p2.b0 = reinterpret_cast<const uint8_t*>(w_down8);
+  p2.sa = sh;
+  p2.sb0 = w_down_scale;
+  p2.c = out;
+  p2.lda = intermediate;
+  p2.ldb = intermediate;
+  p2.ldc = hidden;
+  p2.m = (int)tokens;
+  p2.n = (int)hidden;
+  p2.k = (int)intermediate;
+  if (out_dtype == PTO_HIP_FP32) return gemm8::launch_any<false, float>(p2, st);
+  return x_dtype == PTO_HIP_BF16 ? gemm8::launch_any<false, __bf16>(p2, st)
+                                 : gemm8::launch_any<false, _Float16>(p2, st);
+}

@@ -94,13 +94,14 @@ enum ProgramKind {
   kDecoderLayerDecode,
   kProjection,
   kGateUpSwiglu,
+  kFfnBlockFp8,
   kNumPrograms
 };
 
 const char* const kProgramNames[kNumPrograms] = {
     "paged_attention", "paged_gather",  "rms_norm",           "ffn_swiglu",          "ffn_block",
     "w8a16_matmul",    "w8a16_swiglu",  "rope_kv_cache_update", "rope_kv_cache_update_fp8",
-    "decoder_layer_decode", "projection", "gate_up_swiglu"};
+    "decoder_layer_decode", "projection", "gate_up_swiglu", "ffn_block_fp8"};
 
 std::mutex g_mu;
 std::vector<int> g_callables;  // callable id -> ProgramKind, -1 once unregistered
@@ -301,6 +302,38 @@ int run_ffn(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStr
   }
   return pto_hip_ffn_swiglu(tptr(x), gamma, tptr(wg), tptr(wu), tptr(wd), tptr_mut(out), tokens,
                             hidden, inter, eps, (int)x.dtype, (int)out.dtype, stream);
+}
+
+// x, gamma, w_gate8, w_gate_scale, w_up8, w_up_scale, w_down8, w_down_scale, out + eps
+int run_ffn_fp8(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStream_t stream) {
+  const char* prog = "ffn_block_fp8";
+  PTO_CHECK_ARG(nt == 9 && ns == 1, "%s: expected 9 tensors + 1 scalar, got %d + %d", prog, nt, ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor(prog, "operand", t[i], 1, 2);
+    if (rc) return rc;
+  }
+  const PtoHipChipTensor &x = t[0], &gamma = t[1], &wg = t[2], &sg = t[3], &wu = t[4], &su = t[5], &wd = t[6],
+                         &sd = t[7], &out = t[8];
+  PTO_CHECK_ARG(x.ndims == 2 && wg.ndims == 2 && wu.ndims == 2 && wd.ndims == 2 && out.ndims == 2,
+                "%s: x, the weights and out must be 2-D", prog);
+  const int64_t tokens = x.shapes[0], hidden = x.shapes[1], inter = wg.shapes[0];
+  PTO_CHECK_ARG(wg.shapes[1] == hidden && wu.shapes[0] == inter && wu.shapes[1] == hidden &&
+                    wd.shapes[0] == hidden && wd.shapes[1] == inter,
+                "%s: weight codes must be gate/up [I,H] and down [H,I] (one row per output channel) with H=%lld",
+                prog, (long long)hidden);
+  PTO_CHECK_ARG(wg.dtype == PTO_HIP_FP8E4M3FN && wu.dtype == PTO_HIP_FP8E4M3FN && wd.dtype == PTO_HIP_FP8E4M3FN,
+                "%s: weight codes must be FP8E4M3FN", prog);
+  PTO_CHECK_ARG(sg.dtype == PTO_HIP_FP32 && su.dtype == PTO_HIP_FP32 && sd.dtype == PTO_HIP_FP32 &&
+                    numel(sg) == inter && numel(su) == inter && numel(sd) == hidden,
+                "%s: scales must be FP32 with one entry per output channel", prog);
+  PTO_CHECK_ARG(gamma.dtype == PTO_HIP_FP32 && numel(gamma) == hidden, "%s: gamma must be FP32 with %lld elements",
+                prog, (long long)hidden);
+  PTO_CHECK_ARG(out.shapes[0] == tokens && out.shapes[1] == hidden, "%s: out must be [T,H]", prog);
+  return pto_hip_ffn_swiglu_fp8(tptr(x), reinterpret_cast<const float*>(tptr(gamma)), tptr(wg),
+                                reinterpret_cast<const float*>(tptr(sg)), tptr(wu),
+                                reinterpret_cast<const float*>(tptr(su)), tptr(wd),
+                                reinterpret_cast<const float*>(tptr(sd)), tptr_mut(out), tokens, hidden, inter,
+                                scalar_f32(s[0]), (int)x.dtype, (int)out.dtype, stream);
 }
 
 int run_w8a16_matmul(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
@@ -574,6 +607,7 @@ int dispatch(int kind, const PtoHipChipTensor* t, int nt, const uint64_t* s, int
     case kRmsNorm: return run_rms_norm(t, nt, s, ns, stream);
     case kFfnSwiglu: return run_ffn(t, nt, s, ns, stream, false);
     case kFfnBlock: return run_ffn(t, nt, s, ns, stream, true);
+    case kFfnBlockFp8: return run_ffn_fp8(t, nt, s, ns, stream);
     case kW8a16Matmul: return run_w8a16_matmul(t, nt, s, ns, stream);
     case kProjection: return run_projection(t, nt, s, ns, stream);
     case kGateUpSwiglu: return run_gate_up_swiglu(t, nt, s, ns, stream);

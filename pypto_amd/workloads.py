@@ -201,6 +201,52 @@ def ffn_inputs(*, tokens: int, hidden: int, intermediate: int, dtype=torch.bfloa
     return FfnInputs(x, gamma, w_gate, w_up, w_down, out)
 
 
+def quantize_rows_fp8(x: torch.Tensor):
+    """Per-row symmetric e4m3 of a 2-D tensor: (codes float8_e4m3fn, scale fp32 [rows]);
+    scale = amax/448 (1 for an all-zero row), RNE cast."""
+    xf = x.float()
+    amax = xf.abs().amax(dim=-1)
+    scale = torch.where(amax > 0, amax / FP8_E4M3_MAX, torch.ones_like(amax))
+    codes = (xf / scale.unsqueeze(-1)).clamp(-FP8_E4M3_MAX, FP8_E4M3_MAX).to(torch.float8_e4m3fn)
+    return codes.contiguous(), scale.contiguous()
+
+
+@dataclass
+class FfnFp8Inputs:
+    """The FFN block with e4m3 weights: codes one row per output channel ([out, in]) + fp32 scale [out]."""
+    x: torch.Tensor
+    gamma: torch.Tensor | None
+    w_gate8: torch.Tensor
+    w_gate_scale: torch.Tensor
+    w_up8: torch.Tensor
+    w_up_scale: torch.Tensor
+    w_down8: torch.Tensor
+    w_down_scale: torch.Tensor
+    out: torch.Tensor
+    eps: float = 1e-6
+
+    def flops(self) -> int:
+        t, h = self.x.shape
+        return 6 * t * h * self.w_gate8.shape[0]
+
+    def args(self):
+        return (self.x, self.gamma, self.w_gate8, self.w_gate_scale, self.w_up8, self.w_up_scale, self.w_down8,
+                self.w_down_scale, self.out, self.eps)
+
+
+def ffn_fp8_inputs(*, tokens: int, hidden: int, intermediate: int, dtype=torch.bfloat16, out_dtype=torch.float32,
+                   seed: int = 0, device="cpu") -> tuple[FfnFp8Inputs, FfnInputs]:
+    """The tensors of ``ffn_inputs`` (same seed, same draws) with the three weights quantised per output
+    channel; returns the e4m3 problem and the 16-bit one it came from."""
+    f = ffn_inputs(tokens=tokens, hidden=hidden, intermediate=intermediate, dtype=dtype, with_norm=True,
+                   out_dtype=out_dtype, seed=seed, device=device)
+    wg8, sg = quantize_rows_fp8(f.w_gate.t())
+    wu8, su = quantize_rows_fp8(f.w_up.t())
+    wd8, sd = quantize_rows_fp8(f.w_down.t())
+    q = FfnFp8Inputs(f.x, f.gamma, wg8, sg, wu8, su, wd8, sd, torch.zeros_like(f.out), f.eps)
+    return q, f
+
+
 def ffn_tiny(seed: int = 0, device="cpu") -> FfnInputs:
     """FFN tile program of the reference's example at x[128,512] fp16, I=1024, no norm."""
     return ffn_inputs(tokens=128, hidden=512, intermediate=1024, dtype=torch.float16, with_norm=False,

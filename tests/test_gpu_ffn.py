@@ -311,3 +311,268 @@ def test_reference_scope3_from_the_public_programs(worker):
     mlp_bf16 = (gate * torch.sigmoid(gate) * up).bfloat16()
     want = (mlp_bf16.float() @ w_down.float() + r1).bfloat16()
     validate_golden({"out": out.float().cpu()}, {"out": want.float().cpu()}, rtol=2e-2, atol=1e-3)
+
+
+# ---- the block on e4m3 operands (8-bit MFMA path) ---------------------------------------------
+def _lib_ptr(t):
+    return t.data_ptr()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols", [(1, 128), (37, 4096), (5, 11008), (3, 16384), (2, 1000)])
+def test_quantize_rows_fp8_matches_oracle(worker, dtype, rows, cols):
+    """Codes and scales of the device quantiser equal the oracle's (same fp32 arithmetic, RNE)."""
+    from pypto_amd import _lib
+    from pypto_amd.runtime import _dtype_code
+
+    g = torch.Generator().manual_seed(rows * 131 + cols)
+    x = (torch.randn((rows, cols), generator=g) * torch.logspace(-3, 2, rows)[:, None]).to(dtype)
+    if rows > 2:
+        x[2] = 0
+    xd = x.cuda()
+    codes = torch.zeros((rows, cols), dtype=torch.uint8, device="cuda")
+    scale = torch.zeros(rows, dtype=torch.float32, device="cuda")
+    _lib.check(_lib.load().pto_hip_quantize_rows_fp8(xd.data_ptr(), codes.data_ptr(), scale.data_ptr(), rows, cols,
+                                                     _dtype_code(dtype), 0))
+    worker.sync()
+    want_codes, want_scale = oracle.quantize_rows_fp8(x)
+    assert torch.equal(scale.cpu(), want_scale)
+    assert torch.equal(codes.cpu(), want_codes.view(torch.uint8))
+
+
+def test_quantize_rows_fp8_argument_rules(worker):
+    from pypto_amd import _lib
+    from pypto_amd.runtime import _dtype_code
+
+    x = torch.zeros((2, 16392), dtype=torch.bfloat16, device="cuda")
+    c = torch.zeros((2, 16392), dtype=torch.uint8, device="cuda")
+    s = torch.zeros(2, device="cuda")
+    lib = _lib.load()
+    with pytest.raises(ValueError, match="at most 16384"):
+        _lib.check(lib.pto_hip_quantize_rows_fp8(x.data_ptr(), c.data_ptr(), s.data_ptr(), 2, 16392, _dtype_code(torch.bfloat16), 0))
+    with pytest.raises(ValueError, match="multiple of 8"):
+        _lib.check(lib.pto_hip_quantize_rows_fp8(x.data_ptr(), c.data_ptr(), s.data_ptr(), 2, 12, _dtype_code(torch.bfloat16), 0))
+    with pytest.raises(ValueError, match="BF16, FP16"):
+        _lib.check(lib.pto_hip_quantize_rows_fp8(x.data_ptr(), c.data_ptr(), s.data_ptr(), 2, 16, _dtype_code(torch.float32), 0))
+
+
+def _fp8_stage_lib():
+    from pypto_amd import _lib
+    from pypto_amd.runtime import _dtype_code
+
+    return _lib, _lib.load(), _dtype_code
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols", [(3, 128), (64, 4096), (7, 11008)])
+def test_rms_norm_quantize_fp8_matches_oracle(worker, dtype, rows, cols):
+    """RMSNorm rounded to the activation type, then the row quantiser: codes and scales of the oracle.
+    The device rsqrt and torch's may differ in the last fp32 bit, which can move a normed value across a
+    rounding boundary: at most 1 code in 10^4 may differ, and then by one step."""
+    _lib, lib, code = _fp8_stage_lib()
+    g = torch.Generator().manual_seed(rows + cols)
+    x = (torch.randn((rows, cols), generator=g) * 2).to(dtype)
+    gamma = 1 + 0.02 * torch.randn((1, cols), generator=g)
+    codes = torch.zeros((rows, cols), dtype=torch.uint8, device="cuda")
+    scale = torch.zeros(rows, device="cuda")
+    xd, gd = x.cuda(), gamma.cuda()
+    _lib.check(lib.pto_hip_rms_norm_quantize_fp8(xd.data_ptr(), gd.data_ptr(), codes.data_ptr(), scale.data_ptr(), rows,
+                                                 cols, 1e-6, code(dtype), 0))
+    worker.sync()
+    want_c, want_s = oracle.quantize_rows_fp8(oracle.rms_norm(x, gamma, 1e-6, out_dtype=dtype))
+    assert torch.allclose(scale.cpu(), want_s, rtol=1e-2, atol=0)
+    got = codes.cpu().view(torch.float8_e4m3fn).float()
+    diff = got != want_c.float()
+    assert diff.sum().item() <= max(1, rows * cols // 10000), diff.sum().item()
+    assert torch.all((got - want_c.float()).abs() <= want_c.float().abs() / 8 + 2.0 ** -9)
+
+
+def _codes_and_scales(rows, cols, seed, spread=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return oracle.quantize_rows_fp8((torch.randn((rows, cols), generator=g) * spread).to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("h_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,n", [(1, 128, 128), (130, 256, 96), (300, 512, 1408), (700, 1024, 640), (48, 4096, 200)])
+def test_gate_up_swiglu_fp8_stage_matches_oracle(worker, h_dtype, m, k, n):
+    """The gate/up product on given codes: row counts below, at and across both tile heights, column
+    counts that are not multiples of the 128-output tile (96, 200), k from one tile to 32."""
+    _lib, lib, code = _fp8_stage_lib()
+    x8, sx = _codes_and_scales(m, k, 1, 2.0)
+    wg8, sg = _codes_and_scales(n, k, 2, 0.02)
+    wu8, su = _codes_and_scales(n, k, 3, 0.02)
+    dev = [t.cuda() for t in (x8, sx, wg8, sg, wu8, su)]
+    h = torch.full((m, n), float("nan"), dtype=h_dtype, device="cuda")
+    _lib.check(lib.pto_hip_gate_up_swiglu_fp8(*(t.data_ptr() for t in dev), h.data_ptr(), m, k, n, code(h_dtype), 0))
+    worker.sync()
+    gate = (x8.float() @ wg8.float().t()) * sx[:, None] * sg[None, :]
+    up = (x8.float() @ wu8.float().t()) * sx[:, None] * su[None, :]
+    ref = oracle.swiglu(gate, up).to(h_dtype).float()
+    # one ulp of the 16-bit type (the device's exp/recip SiLU against torch.sigmoid); sums that cancel to
+    # nearly zero differ with the accumulation order, hence the absolute floor (h is of order 1)
+    tol = 8e-3 if h_dtype == torch.bfloat16 else 2e-3
+    validate_golden({"h": h.cpu().float()}, {"h": ref}, rtol=tol, atol=1e-3)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,k,n", [(1, 128, 256), (130, 384, 200), (300, 1408, 512), (2048, 256, 4096), (64, 11008, 320)])
+def test_projection_fp8_stage_matches_oracle(worker, out_dtype, m, k, n):
+    _lib, lib, code = _fp8_stage_lib()
+    a8, sa = _codes_and_scales(m, k, 4, 1.0)
+    w8, sw = _codes_and_scales(n, k, 5, 0.02)
+    dev = [t.cuda() for t in (a8, sa, w8, sw)]
+    out = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+    _lib.check(lib.pto_hip_projection_fp8(*(t.data_ptr() for t in dev), out.data_ptr(), m, k, n, code(out_dtype), 0))
+    worker.sync()
+    ref = (a8.float() @ w8.float().t()) * sa[:, None] * sw[None, :]
+    # exact products, fp32 sums in another order
+    tol = 1e-4 if out_dtype == torch.float32 else 8e-3
+    validate_golden({"out": out.cpu().float()}, {"out": ref}, rtol=tol, atol=1e-4 * ref.abs().max().item())
+
+
+def test_projection_fp8_is_linear_and_exact_on_small_integers(worker):
+    """Operands e4m3 holds exactly with power-of-two scales: the product is exact in fp32, whatever the
+    accumulation order; and out(a, 2 s) = 2 out(a, s)."""
+    _lib, lib, code = _fp8_stage_lib()
+    g = torch.Generator().manual_seed(9)
+    m, k, n = 257, 640, 384
+    a = torch.randint(-4, 5, (m, k), generator=g).float()
+    w = torch.randint(-4, 5, (n, k), generator=g).float()
+    a8, w8 = a.to(torch.float8_e4m3fn).cuda(), w.to(torch.float8_e4m3fn).cuda()
+    sa = torch.full((m,), 0.5, device="cuda")
+    sw = torch.full((n,), 0.25, device="cuda")
+    out = torch.zeros((m, n), device="cuda")
+    out2 = torch.zeros((m, n), device="cuda")
+    f32 = code(torch.float32)
+    _lib.check(lib.pto_hip_projection_fp8(a8.data_ptr(), sa.data_ptr(), w8.data_ptr(), sw.data_ptr(), out.data_ptr(), m, k, n, f32, 0))
+    sw2 = sw * 2
+    _lib.check(lib.pto_hip_projection_fp8(a8.data_ptr(), sa.data_ptr(), w8.data_ptr(), sw2.data_ptr(), out2.data_ptr(), m, k, n, f32, 0))
+    worker.sync()
+    assert torch.equal(out.cpu(), (a @ w.t()) * 0.125)
+    assert torch.equal(out2, out * 2)
+
+
+@pytest.mark.parametrize("dtype,out_dtype", [(torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                             (torch.float16, torch.float32)])
+@pytest.mark.parametrize("t,h,i", [(1, 128, 128), (48, 256, 512), (300, 512, 1408), (2048, 1024, 2816), (130, 4096, 1280)])
+def test_ffn_block_fp8_is_the_chain_of_its_stages_and_matches_oracle(worker, dtype, out_dtype, t, h, i):
+    """The block is bit-identical to its four stages run one by one (each of which is held to the oracle
+    above).  Against the oracle's whole block the bound is looser on purpose: a value of h that differs in
+    its last 16-bit ulp (device SiLU vs torch.sigmoid, ~2 % of the elements) can take another e4m3 code,
+    and when it is the row's maximum it moves the row's scale and with it a few per cent of the row's
+    codes - equally valid quantisations of the same row.  So: nearly all rows within 0.5 %, none beyond
+    5 % (the distance of the 8-bit block from the 16-bit one)."""
+    from pypto_amd.runtime import ffn_block_fp8
+
+    _lib, lib, code = _fp8_stage_lib()
+    q, _ = workloads.ffn_fp8_inputs(tokens=t, hidden=h, intermediate=i, dtype=dtype, out_dtype=out_dtype, seed=t + h,
+                                    device="cuda")
+    with worker.register(ffn_block_fp8) as hd:
+        hd(*q.args())
+    worker.sync()
+    x8 = torch.zeros((t, h), dtype=torch.uint8, device="cuda")
+    sx = torch.zeros(t, device="cuda")
+    hbuf = torch.zeros((t, i), dtype=dtype, device="cuda")
+    h8 = torch.zeros((t, i), dtype=torch.uint8, device="cuda")
+    sh = torch.zeros(t, device="cuda")
+    out = torch.zeros_like(q.out)
+    _lib.check(lib.pto_hip_rms_norm_quantize_fp8(q.x.data_ptr(), q.gamma.data_ptr(), x8.data_ptr(), sx.data_ptr(), t, h,
+                                                 q.eps, code(dtype), 0))
+    _lib.check(lib.pto_hip_gate_up_swiglu_fp8(x8.data_ptr(), sx.data_ptr(), q.w_gate8.data_ptr(), q.w_gate_scale.data_ptr(),
+                                              q.w_up8.data_ptr(), q.w_up_scale.data_ptr(), hbuf.data_ptr(), t, h, i,
+                                              code(dtype), 0))
+    _lib.check(lib.pto_hip_quantize_rows_fp8(hbuf.data_ptr(), h8.data_ptr(), sh.data_ptr(), t, i, code(dtype), 0))
+    _lib.check(lib.pto_hip_projection_fp8(h8.data_ptr(), sh.data_ptr(), q.w_down8.data_ptr(), q.w_down_scale.data_ptr(),
+                                          out.data_ptr(), t, i, h, code(out_dtype), 0))
+    worker.sync()
+    assert torch.equal(q.out, out)
+    ref = oracle.ffn_block_fp8(*(a.cpu() for a in q.args()[:8]), q.eps)
+    got = q.out.cpu().float()
+    row_err = (got - ref).norm(dim=1) / ref.norm(dim=1).clamp_min(1e-6)
+    slack = 4e-3 if out_dtype == torch.float32 else 8e-3   # a 16-bit output adds its own rounding
+    assert row_err.max().item() < 0.05, row_err.max().item()
+    assert (row_err > 5e-3 + slack).float().mean().item() <= 0.05, (row_err > 5e-3 + slack).sum().item()
+    assert ((got - ref).norm() / ref.norm()).item() < 5e-3 + slack
+
+
+def test_ffn_block_fp8_llama7b_shape_rows_and_distance_to_16_bit(worker):
+    """Full LLaMA-7B shape: the gate/up stage on every 16th row and the down stage on every 16th row,
+    each against the oracle on the device's own codes, and the whole output against the 16-bit block of
+    the unquantised weights (what the quantisation costs)."""
+    from pypto_amd.runtime import ffn_block_fp8
+
+    _lib, lib, code = _fp8_stage_lib()
+    t, h, i = 2048, 4096, 11008
+    q, f = workloads.ffn_fp8_inputs(tokens=t, hidden=h, intermediate=i, seed=0, device="cuda")
+    with worker.register(ffn_block_fp8) as hd:
+        hd(*q.args())
+    worker.sync()
+    bf = code(torch.bfloat16)
+    x8 = torch.zeros((t, h), dtype=torch.uint8, device="cuda")
+    sx = torch.zeros(t, device="cuda")
+    hbuf = torch.zeros((t, i), dtype=torch.bfloat16, device="cuda")
+    h8 = torch.zeros((t, i), dtype=torch.uint8, device="cuda")
+    sh = torch.zeros(t, device="cuda")
+    _lib.check(lib.pto_hip_rms_norm_quantize_fp8(q.x.data_ptr(), q.gamma.data_ptr(), x8.data_ptr(), sx.data_ptr(), t, h,
+                                                 q.eps, bf, 0))
+    _lib.check(lib.pto_hip_gate_up_swiglu_fp8(x8.data_ptr(), sx.data_ptr(), q.w_gate8.data_ptr(), q.w_gate_scale.data_ptr(),
+                                              q.w_up8.data_ptr(), q.w_up_scale.data_ptr(), hbuf.data_ptr(), t, h, i, bf, 0))
+    _lib.check(lib.pto_hip_quantize_rows_fp8(hbuf.data_ptr(), h8.data_ptr(), sh.data_ptr(), t, i, bf, 0))
+    worker.sync()
+    rows = torch.arange(0, t, 16)
+    xf = x8.cpu()[rows].view(torch.float8_e4m3fn).float()
+    sxr = sx.cpu()[rows]
+    gate = (xf @ q.w_gate8.cpu().float().t()) * sxr[:, None] * q.w_gate_scale.cpu()[None, :]
+    up = (xf @ q.w_up8.cpu().float().t()) * sxr[:, None] * q.w_up_scale.cpu()[None, :]
+    validate_golden({"h": hbuf.cpu()[rows].float()}, {"h": oracle.swiglu(gate, up).to(torch.bfloat16).float()},
+                    rtol=8e-3, atol=1e-3)
+    hf = h8.cpu()[rows].view(torch.float8_e4m3fn).float()
+    ref = (hf @ q.w_down8.cpu().float().t()) * sh.cpu()[rows][:, None] * q.w_down_scale.cpu()[None, :]
+    validate_golden({"out": q.out.cpu()[rows]}, {"out": ref}, rtol=1e-4, atol=1e-4 * ref.abs().max().item())
+    with worker.register(ffn_block) as hd:
+        hd(f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.out, f.eps)
+    worker.sync()
+    rel = ((q.out - f.out).norm() / f.out.norm()).item()
+    assert 1e-3 < rel < 0.08, rel
+
+
+def test_ffn_block_fp8_four_wavefront_form_is_bit_identical(worker):
+    """"gemm_variant" 1 runs the tall tile with four wavefronts of 128 x 128 instead of eight of 128 x 64:
+    every accumulator still sums its k-steps in the same order, so the results are the same bits."""
+    from pypto_amd.runtime import ffn_block_fp8
+
+    q, _ = workloads.ffn_fp8_inputs(tokens=2048, hidden=512, intermediate=4096, seed=6, device="cuda")
+    with worker.register(ffn_block_fp8) as hd:
+        hd(*q.args())
+        worker.sync()
+        first = q.out.clone()
+        q.out.zero_()
+        worker.set_option("gemm_variant", 1)
+        try:
+            hd(*q.args())
+            worker.sync()
+        finally:
+            worker.set_option("gemm_variant", 0)
+    assert first.abs().max().item() > 0 and torch.equal(first, q.out)
+
+
+def test_ffn_block_fp8_argument_rules(worker):
+    from pypto_amd.runtime import ffn_block_fp8
+
+    q, _ = workloads.ffn_fp8_inputs(tokens=4, hidden=192, intermediate=256, seed=1)
+    with worker.register(ffn_block_fp8) as hd:
+        with pytest.raises(RuntimeError, match="multiples of 128"):
+            hd(*q.args())
+        q, _ = workloads.ffn_fp8_inputs(tokens=4, hidden=128, intermediate=256, seed=1)
+        bad = list(q.args())
+        bad[2] = q.w_gate8.t().contiguous()          # [H, I]: the 16-bit layout, not one row per output channel
+        with pytest.raises(ValueError, match="one row per output channel"):
+            hd(*bad)
+        bad = list(q.args())
+        bad[3] = q.w_gate_scale[:-1].contiguous()
+        with pytest.raises(ValueError, match="one entry per output channel"):
+            hd(*bad)
+        bad = list(q.args())
+        bad[6] = q.w_down8.view(torch.uint8).to(torch.int8)
+        with pytest.raises(ValueError, match="FP8E4M3FN"):
+            hd(*bad)

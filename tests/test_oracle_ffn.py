@@ -164,3 +164,76 @@ def test_layer_with_16bit_weights_follows_reference_scope3_golden():
         for h in range(hkv):
             row = (int(table[b, 0]) * hkv + h) * 16
             assert torch.equal(kc[row], k[b, h]) and torch.equal(vc[row], v[b, h])
+
+
+def test_quantize_rows_fp8_properties():
+    """The e4m3 row quantiser has nothing in the reference to be checked against; what the format
+    fixes is checked instead: the rounding bound of a 3-bit mantissa, the row maximum landing on
+    +-448, the decoded codes being a fixed point, all-zero rows, and the code table itself."""
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn((7, 512), generator=g) * torch.tensor([1e-3, 0.02, 1.0, 30.0, 1e4, 1.0, 1.0])[:, None])
+    x[5] = 0.0
+    x[6, 17] = -9.0   # a negative row maximum
+    x = x.to(torch.bfloat16)
+    codes, scale = oracle.quantize_rows_fp8(x)
+    assert codes.dtype == torch.float8_e4m3fn and scale.dtype == torch.float32
+    xf = x.float()
+    amax = xf.abs().amax(dim=1)
+    assert torch.equal(scale[5], torch.tensor(1.0)) and torch.all(codes[5].float() == 0)
+    live = [0, 1, 2, 3, 4, 6]
+    assert torch.allclose(scale[live], amax[live] / 448.0, rtol=1e-7)
+    deq = codes.float() * scale[:, None]
+    # |x - q s| <= 2^-4 |x| for normal codes, <= 2^-10 s for subnormal ones; nothing overflows to NaN
+    assert not torch.isnan(codes.float()).any()
+    bound = torch.maximum(xf.abs() * 2.0 ** -4, scale[:, None] * 2.0 ** -10) * (1 + 1e-6)
+    assert torch.all((xf - deq).abs() <= bound)
+    # the row maximum is code +-448 exactly and keeps its sign
+    idx = xf.abs().argmax(dim=1)
+    top = codes.float()[torch.arange(7), idx]
+    assert torch.all(top[live].abs() == 448.0) and top[6] == -448.0
+    # decoded values quantise to themselves
+    codes2, scale2 = oracle.quantize_rows_fp8(deq)
+    assert torch.equal(codes2.view(torch.uint8), codes.view(torch.uint8)) and torch.allclose(scale2, scale, rtol=1e-6)
+    # the code table: sign, 4 exponent bits (bias 7), 3 mantissa bits, no infinities, 0x7f/0xff NaN
+    table = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float()
+    for c in (0x00, 0x01, 0x08, 0x38, 0x7e, 0xb8, 0xfe):
+        s, e, m = c >> 7, (c >> 3) & 15, c & 7
+        v = (m / 8.0) * 2.0 ** -6 if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7)
+        assert table[c].item() == (-v if s else v)
+    assert table[0x7e].item() == 448.0 and torch.isnan(table[0x7f]) and torch.isnan(table[0xff])
+
+
+def test_ffn_block_fp8_is_the_16_bit_block_up_to_quantisation_noise():
+    """With scales of 1 and operands that e4m3 holds exactly the 8-bit block IS the 16-bit block; on
+    random data it stays within the noise three per-row e4m3 roundings allow (a dropped scale, a
+    transposed weight or a missing SiLU would be off by far more)."""
+    from pypto_amd import workloads
+
+    # exact case: small integers, power-of-two scales folded into the codes
+    g = torch.Generator().manual_seed(5)
+    t, h, i = 6, 128, 256
+    x = torch.randint(-3, 4, (t, h), generator=g).to(torch.bfloat16)
+    wg = torch.randint(-2, 3, (h, i), generator=g).float() / 8
+    wu = torch.randint(-2, 3, (h, i), generator=g).float() / 8
+    wd = torch.randint(-2, 3, (i, h), generator=g).float() / 8
+    one_i, one_h = torch.ones(i), torch.ones(h)
+    # no norm; x codes are exact only if the row scale is a power of two: make every row's amax 3.5 -> use 448/128
+    x[:, 0] = 3.5
+    out8 = oracle.ffn_block_fp8(x, None, wg.t().contiguous().to(torch.float8_e4m3fn), one_i,
+                                wu.t().contiguous().to(torch.float8_e4m3fn), one_i,
+                                wd.t().contiguous().to(torch.float8_e4m3fn), one_h)
+    gate, up = x.float() @ wg, x.float() @ wu
+    hh = oracle.swiglu(gate, up).to(torch.bfloat16)
+    h8, sh = oracle.quantize_rows_fp8(hh)
+    want = (h8.float() * sh[:, None]) @ wd
+    assert torch.allclose(out8, want, rtol=1e-5, atol=1e-5)
+
+    # random case against the 16-bit block
+    q, f = workloads.ffn_fp8_inputs(tokens=48, hidden=256, intermediate=512, seed=2)
+    ref16 = oracle.ffn_block(f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.eps)
+    out = oracle.ffn_block_fp8(q.x, q.gamma, q.w_gate8, q.w_gate_scale, q.w_up8, q.w_up_scale, q.w_down8,
+                               q.w_down_scale, q.eps)
+    rel = (out - ref16).norm() / ref16.norm()
+    assert 1e-3 < rel < 0.08, rel   # measurably quantised, and no worse than three e4m3 roundings give
+    # the weights really are one row per output channel: swapping the layout must not go unnoticed
+    assert q.w_gate8.shape == (512, 256) and q.w_down8.shape == (256, 512)
