@@ -61,8 +61,8 @@ __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
 // Both tiles have 128-byte rows and go global -> LDS directly (1 KB per wavefront instruction =
 // 8 rows); the hardware fixes where a lane's 16 bytes land, so instead of padding, the lane whose
 // bytes land in slot s of row r fetches logical chunk s ^ ((r / 2) % 8) and the fragment reads apply
-// the same XOR: the 16 lanes the LDS serves per clock (16 consecutive rows, one logical chunk) then
-// hit 16 different slots of 8 row pairs.
+// the same XOR: the 16 lanes the LDS checks together for bank conflicts (16 consecutive rows, one
+// logical chunk, 256 bytes = all 64 banks) then hit 16 different slots of 8 row pairs.
 // A wavefront reads (32*MT + 32*NT) x 128 bytes of fragments per k-tile: eight wavefronts of 128 x 64
 // read 192 KB per k-tile next to 64 KB of tile writes, which at the LDS's ~128 bytes a clock is as
 // many LDS clocks as the k-tile has MFMA clocks (2048 per SIMD).

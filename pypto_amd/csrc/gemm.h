@@ -98,10 +98,10 @@ __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
 // bytes), with no staging registers and no ds_write stream next to the MFMAs.  The hardware fixes
 // where a lane's 16 bytes land, so rows cannot be padded; bank conflicts are avoided by an XOR
 // swizzle instead, applied on the global side: the lane whose bytes land in 16-byte slot s of A row
-// r fetches logical chunk s ^ ((r / 2) % 8) - an A row is 128 bytes and the LDS serves 256 bytes a
-// clock, so the 16 lanes of one clock of a fragment read (16 consecutive rows, one chunk each) must
-// land on 16 different slots of a row pair - and for B the 64-byte group g of k-row r holds logical
-// group g ^ (r % 8).  The fragment reads apply the same XOR.
+// r fetches logical chunk s ^ ((r / 2) % 8) - an A row is 128 bytes and the LDS checks 16 lanes of
+// a 16-byte read (256 bytes, all 64 banks) together for conflicts, so those 16 lanes (16 consecutive
+// rows, one chunk each) must land on the 16 different slots of a row pair - and for B the 64-byte
+// group g of k-row r holds logical group g ^ (r % 8).  The fragment reads apply the same XOR.
 template <bool W8, int EDGE>
 constexpr bool gemm_direct() { return !W8 && EDGE != 2; }
 
