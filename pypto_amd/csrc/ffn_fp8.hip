@@ -44,7 +44,10 @@ struct Params {
   int tiles_m, tiles_n;
 };
 
-__device__ __forceinline__ float silu(float g) { return g * __frcp_rn(1.f + __expf(-g)); }
+// SiLU in the device form of the reference, g * recip(1 + exp(-g)) (01_ffn.py:70-74), with the hardware's
+// 1-ulp reciprocal: the correctly rounded one is a ten-instruction division, and an epilogue computes
+// 64 of them per lane while the matrix pipes idle.
+__device__ __forceinline__ float silu(float g) { return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)); }
 
 __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
   const int x = pid % kXcds, local = pid / kXcds;
@@ -79,6 +82,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem8[];
   uint8_t* sa = smem8;                 // [2][BM][128]
   uint8_t* sb = smem8 + 2 * A_BYTES;   // [2][256][128]
+  float* s_rows = reinterpret_cast<float*>(smem8 + 2 * A_BYTES + 2 * B_BYTES);  // [BM] row scales of this tile
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -88,6 +92,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
   const int tm = tile % p.tiles_m, tn = tile / p.tiles_m;
   const int m0 = tm * BM;
   const int n0 = tn * (DUAL ? BN / 2 : BN);
+
+  // the tile's row scales go to LDS once (rows past m clamped): the epilogue reads them four at a time
+  for (int r = tid; r < BM; r += T) s_rows[r] = p.sa[min(m0 + r, p.m - 1)];
 
   // ---- global -> LDS requests ----------------------------------------------------------------
   const int row_in_round = tid >> 3;
@@ -143,6 +150,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
     fb[jn] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
   };
 
+  // this lane's output columns and their channel scales (fetched now, used in the epilogue)
+  int col[NT];
+  float sc[NT];
+#pragma unroll
+  for (int jn = 0; jn < NT; ++jn) {
+    col[jn] = DUAL ? n0 + wn * (16 * NT) + (jn % (NT / 2)) * 32 + (lane & 31) : n0 + wn * (32 * NT) + jn * 32 + (lane & 31);
+    const float* s = (DUAL && jn >= NT / 2) ? p.sb1 : p.sb0;
+    sc[jn] = col[jn] < p.n ? s[col[jn]] : 0.f;
+  }
+
   f32x16 acc[MT][NT];
 #pragma unroll
   for (int i = 0; i < MT; ++i)
@@ -172,18 +189,19 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
     }
   };
 
+  const int nk = p.k / BK;
   // Tiles kt (being multiplied), kt+1 (landed in the other buffer) and kt+2 (in flight into the
   // buffer of kt) are live at once.  The one barrier of a k-tile sits in its second k-step, after
   // column 0: by then this wavefront has read the last fragment of tile kt (the wait for it is
   // covered by those MFMAs) and waits for its own requests of tile kt+1; past the barrier every
   // wavefront has done both, so tile kt+1 may be read and the buffer of tile kt refilled.
-  const int nk = p.k / BK;
   {
-    const int k1 = min(1, nk - 1) * BK;
 #pragma unroll
     for (int e = 0; e < NA + NB; ++e) request(0, 0, e);
+    if (nk > 1) {
 #pragma unroll
-    for (int e = 0; e < NA + NB; ++e) request(1, k1, e);
+      for (int e = 0; e < NA + NB; ++e) request(1, BK, e);
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
@@ -194,7 +212,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
 
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
-    const int k2 = min(kt + 2, nk - 1) * BK;
+    const int k2 = (kt + 2) * BK;
+    const bool more = kt + 2 < nk;  // requests past the last tile are skipped (the waits are explicit)
     // first k-step: reloads fetch the second k-step of the same tile
     k_step(buf, 1, [] {}, [](int) {});
     // second k-step: barrier after column 0, then reloads from tile kt+1 and the requests of tile kt+2
@@ -212,42 +231,47 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
             constexpr int per = (NA + NB + kAfter - 1) / kAfter;
 #pragma unroll
             for (int e = (slot - MT) * per; e < (slot - MT + 1) * per; ++e)
-              if (e < NA + NB) request(buf, k2, e);
+              if (e < NA + NB && more) request(buf, k2, e);
           }
         });
   }
+
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land in LDS after the workgroup has gone
 
   // ---- epilogue ----------------------------------------------------------------------------------
   // acc[i][jn][r]: row m0 + wm*MT*32 + i*32 + (r/4)*8 + (lane/32)*4 + r%4, column lane % 32 of fragment jn
   OutT* c = reinterpret_cast<OutT*>(p.c);
   const int row_base = m0 + wm * MT * 32 + (lane >> 5) * 4;
-  int col[NT];
-  float sc[NT];
+  // Row scales from the LDS copy made at the start (visible since the loop's barriers): four
+  // consecutive rows per read.  One global load per row here would put 16 * MT loads per lane
+  // through the CU's address unit while the matrix pipes idle.
+  float sr[MT][16];
 #pragma unroll
-  for (int jn = 0; jn < NT; ++jn) {
-    col[jn] = DUAL ? n0 + wn * (16 * NT) + (jn % (NT / 2)) * 32 + (lane & 31) : n0 + wn * (32 * NT) + jn * 32 + (lane & 31);
-    const float* s = (DUAL && jn >= NT / 2) ? p.sb1 : p.sb0;
-    sc[jn] = col[jn] < p.n ? s[col[jn]] : 0.f;
-  }
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 v = *reinterpret_cast<const float4*>(s_rows + wm * MT * 32 + (lane >> 5) * 4 + i * 32 + q * 8);
+      sr[i][q * 4 + 0] = v.x;
+      sr[i][q * 4 + 1] = v.y;
+      sr[i][q * 4 + 2] = v.z;
+      sr[i][q * 4 + 3] = v.w;
+    }
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int row = row_base + i * 32 + (r >> 2) * 8 + (r & 3);
-      if (row >= p.m) continue;
-      const float sr = p.sa[row];
+      const bool row_ok = row < p.m;
       if constexpr (DUAL) {
 #pragma unroll
-        for (int jn = 0; jn < NT / 2; ++jn)
-          if (col[jn] < p.n) {
-            const float g = acc[i][jn][r] * sr * sc[jn], u = acc[i][jn + NT / 2][r] * sr * sc[jn + NT / 2];
-            c[(int64_t)row * p.ldc + col[jn]] = (OutT)(silu(g) * u);
-          }
+        for (int jn = 0; jn < NT / 2; ++jn) {
+          const float g = acc[i][jn][r] * sr[i][r] * sc[jn], u = acc[i][jn + NT / 2][r] * sr[i][r] * sc[jn + NT / 2];
+          if (row_ok && col[jn] < p.n) c[(int64_t)row * p.ldc + col[jn]] = (OutT)(silu(g) * u);
+        }
       } else {
 #pragma unroll
         for (int jn = 0; jn < NT; ++jn)
-          if (col[jn] < p.n) c[(int64_t)row * p.ldc + col[jn]] = (OutT)(acc[i][jn][r] * sr * sc[jn]);
+          if (row_ok && col[jn] < p.n) c[(int64_t)row * p.ldc + col[jn]] = (OutT)(acc[i][jn][r] * sr[i][r] * sc[jn]);
       }
     }
 }
@@ -258,7 +282,7 @@ int launch(Params p, hipStream_t st) {
   p.tiles_m = (p.m + BM - 1) / BM;
   const int bn_out = DUAL ? BN / 2 : BN;
   p.tiles_n = (p.n + bn_out - 1) / bn_out;
-  const size_t smem = 2 * (size_t)(BM * BK + BN * BK);
+  const size_t smem = 2 * (size_t)(BM * BK + BN * BK) + BM * sizeof(float);
   auto kern = gemm8_kernel<MT, NT, WM, WN, DUAL, OutT>;
   static std::atomic<bool> attr_set{false};  // per instantiation; callers hold the dispatch lock
   if (!attr_set.load(std::memory_order_acquire)) {
