@@ -63,8 +63,10 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 template <typename OutT>
 __device__ __forceinline__ void store_out(OutT* p, float v) { *p = (OutT)v; }
 
-// Sigmoid in the device form of the reference, recip(1 + exp(-g)) (01_ffn.py:70-74).
-__device__ __forceinline__ float silu(float g) { return g * __frcp_rn(1.f + __expf(-g)); }
+// Sigmoid in the device form of the reference, recip(1 + exp(-g)) (01_ffn.py:70-74), with the
+// hardware's 1-ulp reciprocal: the correctly rounded one is a ten-instruction division, and the
+// epilogue of a gate/up tile computes 64 of them per lane while the matrix pipes idle.
+__device__ __forceinline__ float silu(float g) { return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)); }
 
 // Two small integers held as fp32 -> packed pair of 16-bit floats, exact (|value| <= 128 has at most
 // 8 significant bits: the upper half of the fp32 pattern is its bf16).
