@@ -47,8 +47,19 @@ def ffn_block_case():
     return {"x": f.x, "gamma": f.gamma, "w_gate": f.w_gate, "w_up": f.w_up, "w_down": f.w_down, "out": out}
 
 
+def ffn_block_fp8_case():
+    """The e4m3 form of the block: codes are stored as their bytes (uint8 views)."""
+    q, _ = workloads.ffn_fp8_inputs(tokens=24, hidden=128, intermediate=256, seed=4)
+    out = oracle.ffn_block_fp8(q.x, q.gamma, q.w_gate8, q.w_gate_scale, q.w_up8, q.w_up_scale, q.w_down8, q.w_down_scale,
+                               q.eps)
+    u8 = lambda t: t.view(torch.uint8)
+    return {"x": q.x, "gamma": q.gamma, "w_gate8": u8(q.w_gate8), "w_gate_scale": q.w_gate_scale, "w_up8": u8(q.w_up8),
+            "w_up_scale": q.w_up_scale, "w_down8": u8(q.w_down8), "w_down_scale": q.w_down_scale, "out": out}
+
+
 if __name__ == "__main__":
-    for name, fn in (("attention_b3", attention_case), ("ffn_64x64_seed0", ffn_case), ("ffn_block_32x128", ffn_block_case)):
+    for name, fn in (("attention_b3", attention_case), ("ffn_64x64_seed0", ffn_case), ("ffn_block_32x128", ffn_block_case),
+                     ("ffn_block_fp8_24x128", ffn_block_fp8_case)):
         tensors = {k: v.contiguous() for k, v in fn().items()}
         save_file(tensors, str(HERE / f"{name}.safetensors"))
         print(name, {k: tuple(v.shape) for k, v in tensors.items()})

@@ -37,6 +37,36 @@ def test_ffn_fixtures_cpu():
     assert torch.allclose(out, b["out"], atol=1e-6)
 
 
+def _fp8_fixture():
+    t = _load("ffn_block_fp8_24x128")
+    f8 = lambda k: t[k].view(torch.float8_e4m3fn)
+    return t, (t["x"], t["gamma"], f8("w_gate8"), t["w_gate_scale"], f8("w_up8"), t["w_up_scale"], f8("w_down8"),
+               t["w_down_scale"])
+
+
+def test_ffn_fp8_fixture_cpu():
+    t, args = _fp8_fixture()
+    assert torch.allclose(oracle.ffn_block_fp8(*args, 1e-6), t["out"], atol=1e-6)
+    # the stored codes are what the input builder's quantiser makes of the 16-bit weights of the same seed
+    from pypto_amd import workloads
+
+    q, _ = workloads.ffn_fp8_inputs(tokens=24, hidden=128, intermediate=256, seed=4)
+    assert torch.equal(q.w_down8.view(torch.uint8), t["w_down8"]) and torch.equal(q.w_gate_scale, t["w_gate_scale"])
+
+
+@pytest.mark.gpu
+def test_ffn_fp8_fixture_gpu(worker):
+    from pypto_amd.runtime import ffn_block_fp8
+
+    t, args = _fp8_fixture()
+    out = torch.zeros_like(t["out"])
+    with worker.register(ffn_block_fp8) as h:
+        h(*args, out, 1e-6)
+    ref = t["out"]
+    row_err = (out - ref).norm(dim=1) / ref.norm(dim=1)
+    assert row_err.max().item() < 0.05 and row_err.median().item() < 5e-3
+
+
 @pytest.mark.gpu
 def test_attention_fixture_gpu(worker):
     from pypto_amd.runtime import paged_attention, validate_golden
