@@ -30,9 +30,21 @@ Pinning status (what fixes each function independently of its own formula):
 * ``rope_rotate_half``        — pinned: complex-rotation closed form, position-0
                                  identity, norm preservation, relative-position
                                  property.
+* ``tile_ops.*``              — pinned: one meaning per op name of the hot
+                                 programs (torch_codegen.py:954-1128), known
+                                 answers for load padding, pad values, RNE casts,
+                                 keepdim reductions and the 16-bit-rounded
+                                 tile.matmul; the reference's kernels written op
+                                 by op equal ``stages.*`` to the bit
+                                 (tests/test_oracle_tile_ops.py).
 * fp8-e4m3 KV and W8A16       — the reference has no such path; pinned by
                                  closed forms only (exhaustive 256-code table,
                                  integer matmul identity).
+* ``quantize_rows_fp8`` / ``ffn_block_fp8`` — the reference has no 8-bit FFN:
+                                 PARITY UNPINNED against it; pinned by the format
+                                 only (rounding bound, row maximum on +-448,
+                                 idempotence, exact small-integer case, distance
+                                 to the 16-bit block; tests/test_oracle_ffn.py).
 """
 
 from .attention import (  # noqa: F401
@@ -44,7 +56,7 @@ from .attention import (  # noqa: F401
     paged_gather,
     quantize_kv_fp8,
 )
-from . import stages  # noqa: F401
+from . import stages, tile_ops  # noqa: F401
 from .ffn import (ffn_block, ffn_block_fp8, ffn_swiglu, projection, quantize_rows_fp8, rms_norm,  # noqa: F401
                   swiglu)
 from .layer import (  # noqa: F401
