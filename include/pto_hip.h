@@ -125,6 +125,9 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *      tensors: x[T,H], gamma[1,H] fp32, w_gate8[I,H] e4m3, w_gate_scale[I] fp32, w_up8[I,H], w_up_scale[I],
  *               w_down8[H,I], w_down_scale[H], out[T,H] (fp32 or dtype of x);  codes are one row per OUTPUT
  *               channel with k contiguous;  scalars: eps (f32 bits)
+ *  "llama_mini"        examples/models/08_llama_mini.py:384-483
+ *      tensors: hidden[S,D], causal_mask[S,S], cos_emb[S,D/2], sin_emb[S,D/2], wq, wk, wv, w_dense, w_gate, w_up,
+ *               w_down [D,D], w_lm[D,V], logits[S,V], all fp32
  *  "w8a16_matmul"      examples/models/qwen3_jit/kernels/projection.py:145-177 with int8 weights
  *      tensors: x[M,K], w_q[K,N] i8, w_scale[N] fp32, [residual[M,N],] out[M,N]
  *  "w8a16_swiglu"      examples/models/qwen3_jit/kernels/mlp.py:22-61 with int8 weights
@@ -243,6 +246,19 @@ PTO_HIP_API int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void
                                    const void* w_up, const void* w_down, void* out,
                                    int64_t tokens, int64_t hidden, int64_t intermediate,
                                    float eps, int dtype, int out_dtype, void* stream);
+
+/* The reference's minimal single-head LLaMA forward (program "llama_mini"; examples/models/08_llama_mini.py:
+ * 384-483, golden tests/st/examples/03_llm_models/test_llama_7b_mini_1h.py:119-198): RMSNorm (no weight, eps as
+ * given; the reference uses 1e-6) -> Q/K/V = normed @ w -> rotate-half RoPE with the [S, D/2] tables -> softmax(q k^T
+ * / sqrt(D) + causal_mask) v -> @ w_dense + hidden -> RMSNorm -> SiLU(x w_gate) * (x w_up) @ w_down + residual ->
+ * RMSNorm -> @ w_lm.  All tensors FP32: hidden [S, D], causal_mask [S, S], cos/sin [S, D/2], seven [D, D] weights,
+ * w_lm [D, V], logits [S, V].  One launch: a single workgroup keeps every intermediate in LDS, which bounds the
+ * shape to 5*S*D + S*S + S floats <= 150 KB (PTO_HIP_ERR_UNSUPPORTED beyond; the reference's example is S 16, D 64). */
+PTO_HIP_API int pto_hip_llama_mini(const float* hidden, const float* causal_mask, const float* cos_emb,
+                                   const float* sin_emb, const float* wq, const float* wk, const float* wv,
+                                   const float* w_dense, const float* w_gate, const float* w_up, const float* w_down,
+                                   const float* w_lm, float* logits, int64_t seq_len, int64_t head_dim,
+                                   int64_t vocab_size, float eps, void* stream);
 
 /* The FFN block on e4m3 operands (program "ffn_block_fp8").  No counterpart in the reference,
  * whose FFN is 16-bit (examples/models/01_ffn.py:111-131, qwen3_jit/kernels/mlp.py:22-61): this is

@@ -30,6 +30,10 @@ Pinning status (what fixes each function independently of its own formula):
 * ``rope_rotate_half``        — pinned: complex-rotation closed form, position-0
                                  identity, norm preservation, relative-position
                                  property.
+* ``llama_mini_forward``      — pinned: dense causal attention against
+                                 ``scaled_dot_product_attention(is_causal=True)``,
+                                 first-token and zero-weight closed forms
+                                 (tests/test_oracle_ffn.py).
 * ``tile_ops.*``              — pinned: one meaning per op name of the hot
                                  programs (torch_codegen.py:954-1128), known
                                  answers for load padding, pad values, RNE casts,
@@ -62,6 +66,7 @@ from .ffn import (ffn_block, ffn_block_fp8, ffn_swiglu, projection, quantize_row
 from .layer import (  # noqa: F401
     decoder_layer_decode,
     kv_append_fp8,
+    llama_mini_forward,
     quantize_w8,
     rope_cos_sin,
     rope_rotate_half,

@@ -177,3 +177,35 @@ def decoder_layer_decode(
     if fp8:
         return out, key_cache, value_cache, k_scale, v_scale
     return out, key_cache, value_cache
+
+
+def llama_mini_forward(hidden, causal_mask, cos_emb, sin_emb, wq, wk, wv, w_dense, w_gate, w_up, w_down, w_lm,
+                       eps: float = 1e-6) -> torch.Tensor:
+    """The reference's minimal single-head LLaMA forward, fp32 -> logits ``[S, V]``.
+
+    Follows ``compute_expected`` of tests/st/examples/03_llm_models/test_llama_7b_mini_1h.py:119-198 (the
+    program is examples/models/08_llama_mini.py:384-483): RMSNorm without a weight, ``x / sqrt(sum(x^2) / D +
+    eps)`` (:137-141); Q, K, V = normed @ w (:158-160); rotate-half RoPE with shared ``[S, D/2]`` tables,
+    ``lo' = lo cos - hi sin, hi' = hi cos + lo sin`` (:143-155); ``softmax(q k^T / sqrt(D) + mask) v``
+    (:167-170); dense projection and first residual (:173-174); RMSNorm, ``SiLU(gate) * up @ w_down`` and the
+    second residual (:177-184); final RMSNorm and the LM head (:187-190).
+    """
+    hidden = hidden.float()
+    d = hidden.shape[1]
+    half = d // 2
+
+    def norm(h):
+        return h / torch.sqrt((h ** 2).sum(dim=-1, keepdim=True) / d + eps)
+
+    def rope(x):
+        lo, hi = x[:, :half], x[:, half:]
+        return torch.cat([lo * cos_emb - hi * sin_emb, hi * cos_emb + lo * sin_emb], dim=-1)
+
+    normed = norm(hidden)
+    q, k, v = rope(normed @ wq), rope(normed @ wk), normed @ wv
+    probs = torch.softmax(q @ k.T * (1.0 / d ** 0.5) + causal_mask, dim=-1)
+    attn_res = hidden + (probs @ v) @ w_dense
+    normed2 = norm(attn_res)
+    gate, up = normed2 @ w_gate, normed2 @ w_up
+    h1 = attn_res + (gate * torch.sigmoid(gate) * up) @ w_down
+    return norm(h1) @ w_lm

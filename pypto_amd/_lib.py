@@ -27,7 +27,7 @@ EXPORTS = (
     "pto_hip_decoder_layer_decode", "pto_hip_select_program", "pto_hip_projection",
     "pto_hip_gate_up_swiglu", "pto_hip_paged_attention_noalloc", "pto_hip_paged_attention_stream_probe",
     "pto_hip_ffn_swiglu_fp8", "pto_hip_quantize_rows_fp8", "pto_hip_rms_norm_quantize_fp8",
-    "pto_hip_gate_up_swiglu_fp8", "pto_hip_projection_fp8",
+    "pto_hip_gate_up_swiglu_fp8", "pto_hip_projection_fp8", "pto_hip_llama_mini",
     "pto_hip_write_manifest", "pto_hip_backend_info", "pto_hip_backend_op_name", "pto_hip_backend_op_info",
     "pto_hip_backend_codegen", "pto_hip_backend_check_ops", "pto_hip_backend_program_ops",
     "pto_hip_backend_mem_path", "pto_hip_backend_handler_query",
@@ -126,6 +126,7 @@ def load() -> C.CDLL:
         "pto_hip_rms_norm_quantize_fp8": [vp, vp, vp, vp, i64, i64, C.c_float, C.c_int, vp],
         "pto_hip_gate_up_swiglu_fp8": [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, C.c_int, vp],
         "pto_hip_projection_fp8": [vp, vp, vp, vp, vp, i64, i64, i64, C.c_int, vp],
+        "pto_hip_llama_mini": [vp] * 13 + [i64, i64, i64, C.c_float, vp],
         "pto_hip_w8a16_matmul": [vp, vp, vp, vp, vp, i64, i64, i64, C.c_int, C.c_int, C.c_int, vp],
         "pto_hip_w8a16_swiglu": [vp, vp, vp, vp, vp, vp, i64, i64, i64, C.c_int, C.c_int, vp],
         "pto_hip_projection": [vp, vp, vp, vp, i64, i64, i64, C.c_int, C.c_int, C.c_int, vp],

@@ -309,7 +309,15 @@ BackendHIP::BackendHIP() : Backend(CreateGfx950SoC()) {
   const std::vector<std::string> attn_norm = Join({&kAttn, &kNorm});
   const std::vector<std::string> vec_all = Join({&kAttn, &kGemm, &kNorm});
   const std::vector<std::string> rope = {"rope_kv_cache_update", "rope_kv_cache_update_fp8", "decoder_layer_decode"};
-  auto op = [&](const char* name, PipeType pipe, const std::vector<std::string>& progs, const char* how) {
+  // the ops the single-workgroup fp32 model (examples/models/08_llama_mini.py) is written in: that program
+  // realises each of them as plain fp32 arithmetic on LDS-resident tiles, next to whatever else realises it
+  static const char* const kMiniOps[] = {
+      "tile.load", "tile.store", "tile.move", "tile.transpose_view", "tile.create", "tile.reshape", "tile.matmul",
+      "tile.matmul_acc", "tile.mul", "tile.muls", "tile.add", "tile.adds", "tile.sub", "tile.exp", "tile.recip",
+      "tile.sqrt", "tile.row_max", "tile.row_sum", "tile.row_expand_sub", "tile.row_expand_div", "tensor.create"};
+  auto op = [&](const char* name, PipeType pipe, std::vector<std::string> progs, const char* how) {
+    for (const char* m : kMiniOps)
+      if (std::string(m) == name) progs.push_back("llama_mini");
     RegisterOp(name).f_codegen(cg).f_infer_pipe(Pipe(pipe)).realised_by(progs, how);
   };
   // The ops the hot programs are written in (semantics: python/pypto/debug/torch_codegen.py:954-1128;
@@ -400,6 +408,24 @@ BackendHIP::BackendHIP() : Backend(CreateGfx950SoC()) {
                   with({"tile.mul", "tile.create", "tile.row_sum", "tile.muls", "tile.reshape", "tile.adds",
                         "tile.sqrt", "tile.row_expand_div", "tile.col_expand_mul"}),
                   "examples/intermediate/03_normalization.py:33-65"},
+      ProgramSpec{"llama_mini", {"llama_mini_orch"},
+                  {kIn, kIn, kIn, kIn, kIn, kIn, kIn, kIn, kIn, kIn, kIn, kIn, kOut},
+                  {KernelRole{{"kernel_rms_norm"}, CoreType::VECTOR, 1, 1, {kIn, kOut}},
+                   KernelRole{{"kernel_matmul"}, CoreType::CUBE, 1, 1, {kIn, kIn, kOut}},
+                   KernelRole{{"kernel_lm_head"}, CoreType::CUBE, 1, 1, {kIn, kIn, kOut}},
+                   KernelRole{{"kernel_matmul_trans_b"}, CoreType::CUBE, 1, 1, {kIn, kIn, kOut}},
+                   KernelRole{{"kernel_matmul_attn"}, CoreType::CUBE, 1, 1, {kIn, kIn, kOut}},
+                   KernelRole{{"kernel_softmax"}, CoreType::VECTOR, 1, 1, {kIn, kOut}},
+                   KernelRole{{"kernel_scale_scores"}, CoreType::VECTOR, 1, 1, {kIn, kOut}},
+                   KernelRole{{"kernel_add_scores"}, CoreType::VECTOR, 1, 1, {kIn, kIn, kOut}},
+                   KernelRole{{"kernel_add"}, CoreType::VECTOR, 1, 1, {kIn, kIn, kOut}},
+                   KernelRole{{"kernel_rope"}, CoreType::VECTOR, 1, 1, {kIn, kIn, kIn, kOut}},
+                   KernelRole{{"kernel_swiglu"}, CoreType::VECTOR, 1, 1, {kIn, kIn, kOut}}},
+                  with({"tile.move", "tile.transpose_view", "tile.create", "tile.reshape", "tile.matmul",
+                        "tile.matmul_acc", "tile.mul", "tile.muls", "tile.add", "tile.adds", "tile.sub", "tile.exp",
+                        "tile.recip", "tile.sqrt", "tile.row_max", "tile.row_sum", "tile.row_expand_sub",
+                        "tile.row_expand_div", "tensor.create"}),
+                  "examples/models/08_llama_mini.py:74-483"},
       ProgramSpec{"paged_gather", {"paged_gather", "paged_gather_orch"}, {kIn, kIn, kIn, kOut},
                   {KernelRole{{"paged_gather", "paged_gather_kernel", "kernel_paged_gather"}, CoreType::VECTOR, 1, 1,
                               {kIn, kIn, kIn, kOut}}},

@@ -95,13 +95,14 @@ enum ProgramKind {
   kProjection,
   kGateUpSwiglu,
   kFfnBlockFp8,
+  kLlamaMini,
   kNumPrograms
 };
 
 const char* const kProgramNames[kNumPrograms] = {
     "paged_attention", "paged_gather",  "rms_norm",           "ffn_swiglu",          "ffn_block",
     "w8a16_matmul",    "w8a16_swiglu",  "rope_kv_cache_update", "rope_kv_cache_update_fp8",
-    "decoder_layer_decode", "projection", "gate_up_swiglu", "ffn_block_fp8"};
+    "decoder_layer_decode", "projection", "gate_up_swiglu", "ffn_block_fp8", "llama_mini"};
 
 std::mutex g_mu;
 std::vector<int> g_callables;  // callable id -> ProgramKind, -1 once unregistered
@@ -334,6 +335,32 @@ int run_ffn_fp8(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hi
                                 reinterpret_cast<const float*>(tptr(su)), tptr(wd),
                                 reinterpret_cast<const float*>(tptr(sd)), tptr_mut(out), tokens, hidden, inter,
                                 scalar_f32(s[0]), (int)x.dtype, (int)out.dtype, stream);
+}
+
+// hidden, causal_mask, cos_emb, sin_emb, wq, wk, wv, w_dense, w_gate, w_up, w_down, w_lm, logits
+// (the orchestration signature of examples/models/08_llama_mini.py:385-407), all fp32
+int run_llama_mini(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
+  const char* prog = "llama_mini";
+  PTO_CHECK_ARG(nt == 13 && ns == 0, "%s: expected 13 tensors and no scalars, got %d + %d", prog, nt, ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor(prog, "operand", t[i], 2, 2, 4);
+    if (rc) return rc;
+    PTO_CHECK_ARG(t[i].dtype == PTO_HIP_FP32, "%s: tensor %d must be FP32, got %s", prog, i, dtype_name(t[i].dtype));
+  }
+  const int64_t s = t[0].shapes[0], d = t[0].shapes[1], v = t[11].shapes[1];
+  PTO_CHECK_ARG(t[1].shapes[0] == s && t[1].shapes[1] == s, "%s: causal_mask must be [S,S] with S=%lld", prog, (long long)s);
+  PTO_CHECK_ARG(d % 2 == 0 && t[2].shapes[0] == s && t[2].shapes[1] == d / 2 && t[3].shapes[0] == s &&
+                    t[3].shapes[1] == d / 2,
+                "%s: cos_emb and sin_emb must be [S, D/2] with S=%lld, D=%lld", prog, (long long)s, (long long)d);
+  for (int i = 4; i <= 10; ++i)
+    PTO_CHECK_ARG(t[i].shapes[0] == d && t[i].shapes[1] == d, "%s: weight %d must be [D,D] with D=%lld", prog, i,
+                  (long long)d);
+  PTO_CHECK_ARG(t[11].shapes[0] == d, "%s: w_lm must be [D,V] with D=%lld", prog, (long long)d);
+  PTO_CHECK_ARG(t[12].shapes[0] == s && t[12].shapes[1] == v, "%s: logits must be [S,V]", prog);
+  auto f = [&](int i) { return reinterpret_cast<const float*>(tptr(t[i])); };
+  // eps is the constant of the reference's kernel_rms_norm (examples/models/08_llama_mini.py:111)
+  return pto_hip_llama_mini(f(0), f(1), f(2), f(3), f(4), f(5), f(6), f(7), f(8), f(9), f(10), f(11),
+                            reinterpret_cast<float*>(tptr_mut(t[12])), s, d, v, 1e-6f, stream);
 }
 
 int run_w8a16_matmul(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
@@ -608,6 +635,7 @@ int dispatch(int kind, const PtoHipChipTensor* t, int nt, const uint64_t* s, int
     case kFfnSwiglu: return run_ffn(t, nt, s, ns, stream, false);
     case kFfnBlock: return run_ffn(t, nt, s, ns, stream, true);
     case kFfnBlockFp8: return run_ffn_fp8(t, nt, s, ns, stream);
+    case kLlamaMini: return run_llama_mini(t, nt, s, ns, stream);
     case kW8a16Matmul: return run_w8a16_matmul(t, nt, s, ns, stream);
     case kProjection: return run_projection(t, nt, s, ns, stream);
     case kGateUpSwiglu: return run_gate_up_swiglu(t, nt, s, ns, stream);

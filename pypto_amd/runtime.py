@@ -73,6 +73,9 @@ ffn_block = HipProgram("ffn_block", (IN, IN, IN, IN, IN, OUT), scalars=("eps",))
 # the block on e4m3 operands: x, gamma, then (codes [out, in], scale [out]) for gate, up and down
 ffn_block_fp8 = HipProgram("ffn_block_fp8", (IN,) * 8 + (OUT,), scalars=("eps",))
 
+# the reference's minimal single-head LLaMA forward: hidden, causal_mask, cos, sin, 7 x [D,D], w_lm, logits
+llama_mini = HipProgram("llama_mini", (IN,) * 12 + (OUT,))
+
 projection = HipProgram("projection", (IN, IN, OUT))
 projection_residual = HipProgram("projection", (IN, IN, IN, OUT))
 gate_up_swiglu = HipProgram("gate_up_swiglu", (IN, IN, IN, OUT))
@@ -102,8 +105,8 @@ decoder_layer_decode_w16_fp8kv = HipProgram(
     "decoder_layer_decode", (IN, IN, IN, INOUT, INOUT, INOUT, INOUT) + (IN,) * 9 + (OUT,),
     scalars=("num_heads", "kv_head_num", "head_dim", "block_size", "eps"))
 
-PROGRAMS = {p.name: p for p in (paged_attention, paged_gather, rms_norm, ffn_swiglu, ffn_block, ffn_block_fp8, projection,
-                                gate_up_swiglu,
+PROGRAMS = {p.name: p for p in (paged_attention, paged_gather, rms_norm, ffn_swiglu, ffn_block, ffn_block_fp8, llama_mini,
+                                projection, gate_up_swiglu,
                                 w8a16_matmul,
                                 w8a16_swiglu, rope_kv_cache_update, rope_kv_cache_update_fp8,
                                 decoder_layer_decode)}

@@ -259,6 +259,21 @@ def ffn_llama7b(seed: int = 0, device="cpu") -> FfnInputs:
                       seed=seed, device=device)
 
 
+def llama_mini_inputs(*, seq_len: int = 16, head_dim: int = 64, vocab_size: int = 64, seed: int = 0, device="cpu"):
+    """The tensors of the reference's minimal LLaMA test, in orchestration order (tests/st/examples/03_llm_models/
+    test_llama_7b_mini_1h.py:69-113): hidden ~ N(0,1); causal mask 0 / -1e9; RoPE tables with theta_i =
+    10000^(-2i/D); eight weights ~ U(-0.02, 0.02); logits zeroed."""
+    g = torch.Generator().manual_seed(seed)
+    half = head_dim // 2
+    angles = torch.arange(seq_len).float()[:, None] * (1.0 / 10000.0 ** (2 * torch.arange(half).float() / head_dim))[None, :]
+    mask = torch.zeros(seq_len, seq_len).masked_fill(torch.triu(torch.ones(seq_len, seq_len), diagonal=1).bool(), -1e9)
+    small = lambda *shape: torch.rand(shape, generator=g) * 0.04 - 0.02
+    tensors = [torch.randn((seq_len, head_dim), generator=g), mask, torch.cos(angles), torch.sin(angles)]
+    tensors += [small(head_dim, head_dim) for _ in range(7)] + [small(head_dim, vocab_size)]
+    tensors.append(torch.zeros(seq_len, vocab_size))
+    return [t.to(device) for t in tensors]
+
+
 def quantize_w8(w: torch.Tensor):
     """Per-output-channel symmetric int8 of a [in, out] weight: (codes int8, scale fp32 [out])."""
     wf = w.float()

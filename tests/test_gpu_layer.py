@@ -550,3 +550,38 @@ def test_decoder_layer_decode_fp8_kv(worker, dtype):
     got = oracle.dequant_kv_fp8(vc_d, vs_d, 128)
     want = oracle.dequant_kv_fp8(ref_v, ref_vs, 128)
     assert ((got - want).abs() <= ref_vs.max() * 32.0 + 1e-6).all()
+
+
+@pytest.mark.parametrize("s,d,v", [(16, 64, 64), (1, 16, 8), (33, 128, 1000), (64, 64, 50), (7, 30, 3)])
+def test_llama_mini_forward_matches_oracle(worker, s, d, v):
+    """The one-launch minimal LLaMA forward at the reference's shape and at shapes around it (one token, odd
+    sequence lengths, a head_dim that is no multiple of 16, a vocabulary wider than the workgroup)."""
+    from pypto_amd.runtime import llama_mini
+
+    t = workloads.llama_mini_inputs(seq_len=s, head_dim=d, vocab_size=v, seed=s + d)
+    t[12].fill_(float("nan"))
+    with worker.register(llama_mini) as h:
+        h(*t)
+    validate_golden({"logits": t[12]}, {"logits": oracle.llama_mini_forward(*t[:12])}, rtol=1e-4, atol=1e-5)
+
+
+def test_llama_mini_argument_rules(worker):
+    from pypto_amd.runtime import llama_mini
+
+    with worker.register(llama_mini) as h:
+        t = workloads.llama_mini_inputs(seq_len=128, head_dim=128, vocab_size=8)
+        with pytest.raises(RuntimeError, match="150 KB"):
+            h(*t)
+        t = workloads.llama_mini_inputs(seq_len=8, head_dim=32, vocab_size=8)
+        bad = list(t)
+        bad[1] = t[1][:, :4].contiguous()
+        with pytest.raises(ValueError, match="causal_mask"):
+            h(*bad)
+        bad = list(t)
+        bad[5] = t[5].to(torch.bfloat16)
+        with pytest.raises(ValueError, match="FP32"):
+            h(*bad)
+        bad = list(t)
+        bad[2] = torch.zeros(8, 32)
+        with pytest.raises(ValueError, match="cos_emb"):
+            h(*bad)

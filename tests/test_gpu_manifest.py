@@ -33,3 +33,15 @@ def test_manifest_to_ffn_run(worker, tmp_path):
         h(x, wg, wu, wd, out)
     ref = oracle.ffn_swiglu(x, wg, wu, wd)
     validate_golden({"out": out}, {"out": ref}, rtol=3e-3, atol=3e-3)
+
+
+def test_manifest_to_llama_mini_run(worker, tmp_path):
+    """The reference's minimal LLaMA test case (tests/st/examples/03_llm_models/test_llama_7b_mini_1h.py: S 16,
+    D 64, V 64, fp32) from its artifact directory to logits, against the oracle's restatement of its golden."""
+    from test_manifest import MINI_KERNELS, MINI_SIG
+
+    program, _, _ = mf.compile_and_assemble(_write(tmp_path, "llama_mini_orch", MINI_SIG, MINI_KERNELS))
+    t = workloads.llama_mini_inputs(seed=0)
+    with worker.register(program) as h:
+        h(*t)
+    validate_golden({"logits": t[12]}, {"logits": oracle.llama_mini_forward(*t[:12])}, rtol=1e-4, atol=1e-5)

@@ -110,3 +110,22 @@ def test_missing_manifest_and_platform(tmp_path):
     (tmp_path / "kernel_config.py").write_text("KERNELS = []\n")
     with pytest.raises(ValueError, match="KERNELS and ORCHESTRATION"):
         mf.read_kernel_config(tmp_path)
+
+
+MINI_KERNELS = [("kernel_rms_norm", "aiv", ["IN", "OUT"]), ("kernel_matmul", "aic", ["IN", "IN", "OUT"]),
+                ("kernel_lm_head", "aic", ["IN", "IN", "OUT"]), ("kernel_matmul_trans_b", "aic", ["IN", "IN", "OUT"]),
+                ("kernel_matmul_attn", "aic", ["IN", "IN", "OUT"]), ("kernel_softmax", "aiv", ["IN", "OUT"]),
+                ("kernel_scale_scores", "aiv", ["IN", "OUT"]), ("kernel_add_scores", "aiv", ["IN", "IN", "OUT"]),
+                ("kernel_add", "aiv", ["IN", "IN", "OUT"]), ("kernel_rope", "aiv", ["IN", "IN", "IN", "OUT"]),
+                ("kernel_swiglu", "aiv", ["IN", "IN", "OUT"])]
+MINI_SIG = ["IN"] * 12 + ["OUT"]
+
+
+def test_llama_mini_manifest_selects_the_single_launch_program(tmp_path):
+    """The eleven kernels and the orchestration of examples/models/08_llama_mini.py:74-483 map to the one-launch
+    program; the same set without its softmax kernel is not that program."""
+    prog, _, _ = mf.compile_and_assemble(_write(tmp_path, "llama_mini_orch", MINI_SIG, MINI_KERNELS))
+    assert prog.name == "llama_mini" and prog.signature == (IN,) * 12 + (OUT,)
+    with pytest.raises(ValueError):
+        mf.compile_and_assemble(_write(tmp_path, "llama_mini_orch", MINI_SIG,
+                                       [k for k in MINI_KERNELS if k[0] != "kernel_softmax"]))

@@ -237,3 +237,42 @@ def test_ffn_block_fp8_is_the_16_bit_block_up_to_quantisation_noise():
     assert 1e-3 < rel < 0.08, rel   # measurably quantised, and no worse than three e4m3 roundings give
     # the weights really are one row per output channel: swapping the layout must not go unnoticed
     assert q.w_gate8.shape == (512, 256) and q.w_down8.shape == (256, 512)
+
+
+def test_llama_mini_forward_closed_forms():
+    """The minimal LLaMA forward: its attention is a library routine on the same q, k, v; the first token can
+    only attend to itself; with the dense and down weights zero the residual stream is untouched."""
+    import torch.nn.functional as F
+
+    from pypto_amd import workloads
+
+    t = workloads.llama_mini_inputs(seq_len=16, head_dim=64, vocab_size=48, seed=5)
+    hidden, mask, cos, sin, wq, wk, wv, wde, wg, wu, wdn, wlm, _ = t
+    out = oracle.llama_mini_forward(*t[:12])
+    assert out.shape == (16, 48)
+
+    def norm(h):
+        return h / torch.sqrt((h ** 2).mean(dim=-1, keepdim=True) + 1e-6)
+
+    def rope(x):   # complex rotation of the pairs (lo_j, hi_j) by the position's angle
+        z = torch.complex(x[:, :32], x[:, 32:]) * torch.complex(cos, sin)
+        return torch.cat([z.real, z.imag], dim=-1)
+
+    n = norm(hidden)
+    attn = F.scaled_dot_product_attention(rope(n @ wq)[None], rope(n @ wk)[None], (n @ wv)[None], is_causal=True)[0]
+    res = hidden + attn @ wde
+    n2 = norm(res)
+    h1 = res + (F.silu(n2 @ wg) * (n2 @ wu)) @ wdn
+    assert torch.allclose(out, norm(h1) @ wlm, rtol=1e-5, atol=1e-6)
+    # token 0 sees only itself: its attention output is its own v row
+    probe = list(t[:12])
+    probe[7] = torch.eye(64)            # w_dense = I
+    probe[10] = torch.zeros(64, 64)     # w_down = 0: the MLP adds nothing
+    probe[11] = torch.eye(64)           # the "logits" are the final normed stream
+    got = oracle.llama_mini_forward(*probe)
+    assert torch.allclose(got[0], norm((hidden + n @ wv)[0:1])[0], rtol=1e-5, atol=1e-6)
+    # zero dense and down weights: logits = norm(hidden) @ w_lm
+    probe = list(t[:12])
+    probe[7] = torch.zeros(64, 64)
+    probe[10] = torch.zeros(64, 64)
+    assert torch.allclose(oracle.llama_mini_forward(*probe), norm(hidden) @ wlm, rtol=1e-6, atol=1e-7)
