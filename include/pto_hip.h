@@ -109,6 +109,17 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *               config[7] i64 = {B,Hq,Hkv,D,bs,max_blocks,scale_bits}  (HOST or device memory)
  *               [, k_scale[pool,Hkv] fp32, v_scale[pool,Hkv] fp32]  when the caches are FP8E4M3FN
  *      cache row of (block p, kv head h, token t) = (p*Hkv + h)*bs + t
+ *  "paged_attention_batch"    examples/models/05_paged_attention_batch.py:373-386
+ *      tensors: the seven of "paged_attention", then size_query, size_key_cache, size_value_cache (i64[1] each;
+ *               the orchestration never reads them and neither does this library)
+ *  "paged_attention_dynamic"  examples/models/06_paged_attention_dynamic.py:262-300
+ *      tensors: query[B*Hq,D], key_cache[rows,D], value_cache[rows,D], block_table[B*max_blocks] i32,
+ *               context_lens[B] i32, out[B*Hq,D] fp32 - no config: B = context_lens.dim(0), Hq = query.dim(0)/B,
+ *               max_blocks = block_table.dim(0)/B, bs = value_cache.dim(0)/block_table.dim(0), one KV head, scale 1
+ *  "paged_attention_spmd"     examples/models/09_paged_attention_spmd.py:445-482
+ *      tensors: query, key_cache, value_cache, block_table, context_lens, scale[1] fp32 (HOST or device), out,
+ *               config[7] i64 = {B,Hq,Hkv,D,bs,block_num_capacity,active_block_num}: no sequence attends beyond
+ *               its first active_block_num blocks; a sequence with nothing to attend to gives zeros (:647-651)
  *  "paged_gather"      src/ir/op/tensor_ops/paged_gather.cpp:74-199
  *      tensors: src[rows,hidden], indices[n] i32, block_table[nblk] i32, out[n,size]
  *      scalars: block_size, col_offset

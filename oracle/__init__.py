@@ -17,6 +17,12 @@ Pinning status (what fixes each function independently of its own formula):
                                  on gathered dense K/V, softmax invariants
                                  (uniform scores -> mean of V, dominant score ->
                                  that V row), partition independence.
+* ``paged_attention_dynamic_golden`` / ``paged_attention_spmd_golden`` — the same
+                                 block loop behind the reference's other two
+                                 signatures; pinned: shape-derived config equals
+                                 the explicit one, and an ``active_block_num`` of
+                                 N equals contexts clipped to N blocks under the
+                                 dense routine (tests/test_oracle_attention.py).
 * ``stages.*``                — pinned: the reference's kernel-level known answers
                                  (all-ones scores -> m = scale, P = 1, l = block
                                  size; the four is_first / is_last cases on its
@@ -55,7 +61,9 @@ from .attention import (  # noqa: F401
     decode_config,
     dequant_kv_fp8,
     paged_attention_dense,
+    paged_attention_dynamic_golden,
     paged_attention_golden,
+    paged_attention_spmd_golden,
     paged_attention_grouped_golden,
     paged_gather,
     quantize_kv_fp8,

@@ -132,6 +132,7 @@ def paged_attention_golden(
     config: torch.Tensor,
     k_scale: torch.Tensor | None = None,
     v_scale: torch.Tensor | None = None,
+    active_num_blocks: int | None = None,
 ) -> torch.Tensor:
     """Block-loop online-softmax paged attention; returns out [B*Hq, D] fp32.
 
@@ -144,6 +145,10 @@ def paged_attention_golden(
     (:527-536) and ``out = o / l`` (:539).  Sequences whose ``l`` stays 0
     (context length 0) produce zeros, the guard of
     examples/models/09_paged_attention_spmd.py:647-651.
+
+    ``active_num_blocks`` bounds the block loop for every sequence,
+    ``max_bn = min(active_num_blocks, ceil(max ctx / bs))`` - the SPMD form's config slot
+    (examples/models/09_paged_attention_spmd.py:600-603): tokens beyond it are not attended to.
 
     The reference walks query heads in tiles of 16 rows; rows are independent,
     so all heads of a KV group are processed at once here.
@@ -164,6 +169,8 @@ def paged_attention_golden(
     li = torch.zeros((b, kv, group, 1), dtype=torch.float32)
     mi = torch.zeros((b, kv, group, 1), dtype=torch.float32)
     max_bn = int((int(ctx.max().item()) + bs - 1) // bs) if b > 0 else 0
+    if active_num_blocks is not None:
+        max_bn = min(int(active_num_blocks), max_bn)
     pos = torch.arange(bs).reshape(1, 1, 1, bs)
 
     for bn in range(max_bn):
@@ -193,6 +200,32 @@ def paged_attention_golden(
 
     out = torch.where(li > 0, oi / li, torch.zeros_like(oi))
     return out.reshape(b * hq, d)
+
+
+def paged_attention_dynamic_golden(query, key_cache, value_cache, block_table, context_lens) -> torch.Tensor:
+    """The form without a config tensor (examples/models/06_paged_attention_dynamic.py:395-411): every
+    dimension is read off the tensors - batch = context_lens rows, num_heads = query rows / batch,
+    block_size = value_cache rows / block_table entries, max blocks = block_table entries / batch - with
+    one KV head and scale 1.0; then the same block loop."""
+    batch = context_lens.shape[0]
+    num_heads = query.shape[0] // batch
+    block_size = value_cache.shape[0] // block_table.shape[0]
+    max_blocks = block_table.shape[0] // batch
+    config = torch.tensor([batch, num_heads, 1, query.shape[1], block_size, max_blocks, encode_scale(1.0)],
+                          dtype=torch.int64)
+    return paged_attention_golden(query, key_cache, value_cache, block_table, context_lens, config)
+
+
+def paged_attention_spmd_golden(query, key_cache, value_cache, block_table, context_lens, scale, config) -> torch.Tensor:
+    """The SPMD form (examples/models/09_paged_attention_spmd.py:579-654): the scale is an FP32[1] tensor
+    (:588) and config = [batch, num_heads, kv_head_num, head_dim, block_size, block_num_capacity,
+    active_block_num] (:581-587), whose last slot bounds the block loop (:600-603); rows with nothing
+    attended to are zero (:647-651)."""
+    cfg = config.clone()
+    active = int(cfg[6].item())
+    cfg[6] = encode_scale(float(scale.reshape(-1)[0].item()))
+    return paged_attention_golden(query, key_cache, value_cache, block_table, context_lens, cfg,
+                                  active_num_blocks=active)
 
 
 def paged_attention_grouped_golden(

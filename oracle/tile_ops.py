@@ -4,7 +4,7 @@ TEST INFRASTRUCTURE ONLY - see ``oracle/__init__.py``.
 
 The reference gives every op a torch meaning in ``python/pypto/debug/torch_codegen.py:954-1128``
 (the table) and ``:489-610`` (the helpers behind load / store / fillpad / assemble).  This module
-restates those meanings for the 36 ops that the paged-attention, FFN, RMSNorm, projection and
+restates those meanings for the 38 ops that the paged-attention, FFN, RMSNorm, projection and
 paged-gather programs use - exactly the names the HIP target's op registry knows
 (``pypto_amd.backend.registered_ops()``; the test holds the two sets equal) - so that
 
@@ -194,13 +194,26 @@ def paged_gather(src, indices, block_table, block_size: int, col_offset: int = 0
                          col_offset)
 
 
+def get_block_idx() -> int:
+    """The block a kernel instance runs as under SPMD dispatch: 0 on the CPU (``:1068``), where one instance
+    does all the work."""
+    return 0
+
+
+def get_block_num() -> int:
+    """The number of SPMD instances.  The table gives this op no meaning; with the index fixed at 0 the
+    only count under which ``for b in range(idx, batch, num)`` (09_paged_attention_spmd.py:129) still
+    visits every sequence is 1."""
+    return 1
+
+
 # op name -> meaning.  The keys are the op registry's names.
 TILE_OPS: dict[str, Callable] = {
     "tensor.create": create, "tensor.dim": dim, "tensor.paged_gather": paged_gather, "tensor.read": read,
     "tensor.slice": slice_,
     "tile.add": add, "tile.adds": adds, "tile.assemble": assemble, "tile.cast": cast,
     "tile.col_expand_mul": col_expand_mul, "tile.create": create, "tile.exp": exp, "tile.fillpad": fillpad,
-    "tile.full": full, "tile.load": load, "tile.matmul": matmul, "tile.matmul_acc": matmul_acc,
+    "tile.full": full, "tile.get_block_idx": get_block_idx, "tile.get_block_num": get_block_num, "tile.load": load, "tile.matmul": matmul, "tile.matmul_acc": matmul_acc,
     "tile.maximum": maximum, "tile.move": move, "tile.mul": mul, "tile.muls": muls, "tile.neg": neg,
     "tile.read": read, "tile.recip": recip, "tile.reshape": reshape, "tile.row_expand_div": row_expand_div,
     "tile.row_expand_mul": row_expand_mul, "tile.row_expand_sub": row_expand_sub, "tile.row_max": row_max,

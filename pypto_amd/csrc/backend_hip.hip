@@ -265,11 +265,15 @@ BackendPipeInferFunc Pipe(PipeType p) {
   return [p](const CallPtr&) { return p; };
 }
 
-const std::vector<std::string> kAttn = {"paged_attention", "decoder_layer_decode"};
+// the plain orchestration and its three other call forms (batched kernels, shapes from tensor dims, SPMD
+// dispatch) are one fused launch; what realises an op in one realises it in all of them
+const std::vector<std::string> kAttn = {"paged_attention", "paged_attention_batch", "paged_attention_dynamic",
+                                        "paged_attention_spmd", "decoder_layer_decode"};
 const std::vector<std::string> kGemm = {"ffn_swiglu", "ffn_block", "projection", "gate_up_swiglu", "w8a16_matmul",
                                         "w8a16_swiglu", "decoder_layer_decode"};
 const std::vector<std::string> kNorm = {"rms_norm", "ffn_block", "decoder_layer_decode"};
-const std::vector<std::string> kAll = {"paged_attention", "paged_gather", "rms_norm", "ffn_swiglu", "ffn_block",
+const std::vector<std::string> kAll = {"paged_attention", "paged_attention_batch", "paged_attention_dynamic",
+                                       "paged_attention_spmd", "paged_gather", "rms_norm", "ffn_swiglu", "ffn_block",
                                        "projection", "gate_up_swiglu", "w8a16_matmul", "w8a16_swiglu",
                                        "rope_kv_cache_update", "rope_kv_cache_update_fp8", "decoder_layer_decode"};
 
@@ -370,6 +374,11 @@ BackendHIP::BackendHIP() : Backend(CreateGfx950SoC()) {
   op("tensor.read", PipeType::S, kAll, "host read of config; context_lens and block_table are read inside the kernel");
   op("tensor.slice", PipeType::S, kAll, "ChipTensor view: start_offset + shape");
   op("tensor.dim", PipeType::S, kAll, "shapes[] of the tensor descriptor");
+  // -- SPMD dispatch (09_paged_attention_spmd.py:127-129: b starts at the block index and steps by the block count)
+  op("tile.get_block_idx", PipeType::S, {"paged_attention_spmd"},
+     "blockIdx.x of the fused launch; which (sequence, head group, context partition) a workgroup takes is the "
+     "launcher's choice, not the program's core_num");
+  op("tile.get_block_num", PipeType::S, {"paged_attention_spmd"}, "gridDim.x of the fused launch");
   op("tensor.paged_gather", PipeType::MTE2, {"paged_gather"},
      "one lane group per row: index -> table -> row, 16-byte copies, bit-exact");
 
@@ -392,6 +401,42 @@ BackendHIP::BackendHIP() : Backend(CreateGfx950SoC()) {
                         "tile.maximum", "tile.sub", "tile.mul", "tile.add", "tile.row_expand_mul",
                         "tile.row_expand_div", "tile.full", "tensor.create", "tensor.read", "tensor.slice"}),
                   "examples/models/04_paged_attention.py:48-367"},
+      ProgramSpec{"paged_attention_batch", {"BatchPagedAttention"}, {kIn, kIn, kIn, kIn, kIn, kOut, kIn, kIn, kIn, kIn},
+                  {KernelRole{{"KernelQkMatmul"}, CoreType::CUBE, 1, 1, {kIn, kIn, kOut, kIn}},
+                   KernelRole{{"KernelSoftmaxPrepare"}, CoreType::VECTOR, 1, 1, {kIn, kOut, kOut, kOut, kIn}},
+                   KernelRole{{"KernelPvMatmul"}, CoreType::CUBE, 1, 1, {kIn, kIn, kOut, kIn}},
+                   KernelRole{{"KernelOnlineUpdate"}, CoreType::VECTOR, 1, 1,
+                              {kIn, kIn, kIn, kInOut, kInOut, kInOut, kOut}}},
+                  with({"tile.move", "tile.transpose_view", "tile.matmul", "tile.mul", "tile.muls", "tile.create",
+                        "tile.row_max", "tile.row_expand_sub", "tile.exp", "tile.cast", "tile.row_sum", "tile.fillpad",
+                        "tile.reshape", "tile.maximum", "tile.sub", "tile.add", "tile.row_expand_mul",
+                        "tile.row_expand_div", "tile.read", "tensor.create", "tensor.read"}),
+                  "examples/models/05_paged_attention_batch.py:88-491"},
+      ProgramSpec{"paged_attention_dynamic", {"paged_attention"}, {kIn, kIn, kIn, kIn, kIn, kOut},
+                  {KernelRole{{"dyn_kernel_qk_matmul"}, CoreType::CUBE, 1, 1, {kIn, kIn, kOut}},
+                   KernelRole{{"dyn_kernel_softmax_prepare"}, CoreType::VECTOR, 1, 1, {kIn, kOut, kOut, kOut}},
+                   KernelRole{{"dyn_kernel_pv_matmul"}, CoreType::CUBE, 1, 1, {kIn, kIn, kOut}},
+                   KernelRole{{"dyn_kernel_online_update"}, CoreType::VECTOR, 1, 1,
+                              {kIn, kIn, kIn, kInOut, kInOut, kInOut, kOut}},
+                   KernelRole{{"dyn_kernel_init_inplace"}, CoreType::VECTOR, 0, 1, {kOut, kOut, kOut}}},
+                  with({"tile.move", "tile.transpose_view", "tile.matmul", "tile.mul", "tile.muls", "tile.create",
+                        "tile.row_max", "tile.row_expand_sub", "tile.exp", "tile.cast", "tile.row_sum", "tile.fillpad",
+                        "tile.reshape", "tile.maximum", "tile.sub", "tile.add", "tile.row_expand_mul",
+                        "tile.row_expand_div", "tile.full", "tensor.create", "tensor.read", "tensor.slice",
+                        "tensor.dim"}),
+                  "examples/models/06_paged_attention_dynamic.py:77-392"},
+      ProgramSpec{"paged_attention_spmd", {"paged_attention_spmd"}, {kIn, kIn, kIn, kIn, kIn, kIn, kOut, kIn},
+                  {KernelRole{{"SpmdQkMatmul"}, CoreType::CUBE, 1, 1, {kIn, kIn, kOut, kIn, kIn}},
+                   KernelRole{{"SpmdSoftmaxPrepare"}, CoreType::VECTOR, 1, 1, {kIn, kOut, kOut, kOut, kIn}},
+                   KernelRole{{"SpmdPvMatmul"}, CoreType::CUBE, 1, 1, {kIn, kIn, kOut, kIn, kIn}},
+                   KernelRole{{"SpmdOnlineUpdate"}, CoreType::VECTOR, 1, 1, {kIn, kIn, kIn, kInOut, kInOut, kInOut}},
+                   KernelRole{{"SpmdNormalize"}, CoreType::VECTOR, 1, 1, {kIn, kIn, kOut}}},
+                  with({"tile.move", "tile.transpose_view", "tile.matmul", "tile.mul", "tile.create", "tile.row_max",
+                        "tile.row_expand_sub", "tile.exp", "tile.cast", "tile.row_sum", "tile.fillpad", "tile.reshape",
+                        "tile.maximum", "tile.sub", "tile.add", "tile.row_expand_mul", "tile.row_expand_div",
+                        "tile.full", "tile.read", "tile.get_block_idx", "tile.get_block_num", "tensor.create",
+                        "tensor.read"}),
+                  "examples/models/09_paged_attention_spmd.py:111-577"},
       ProgramSpec{"ffn_swiglu", {"ffn_swiglu"}, {kIn, kIn, kIn, kIn, kOut},
                   {KernelRole{{"matmul_kernel"}, CoreType::CUBE, 1, 3, {kIn, kIn, kOut}},
                    KernelRole{{"swiglu_kernel"}, CoreType::VECTOR, 1, 1, {kIn, kIn, kOut}}},

@@ -158,12 +158,14 @@ int cast_from_f32(const float* in, void* out, size_t n, int out_dtype, hipStream
 // *wrote_blocked says whether that is how it was written (only a launch with a merge kernel can).
 // pool_blocks > 0: the number of physical blocks in the caches; a table entry beyond it that a
 // sequence uses reads block 0 instead and is reported by the next pto_hip_sync.
+// active_blocks >= 0: no sequence attends beyond its first active_blocks blocks (the bound the SPMD
+// form of the orchestration carries in its config, 09_paged_attention_spmd.py:468,482); < 0: no bound.
 int paged_attention(const void* query, const void* key_cache, const void* value_cache,
                     const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
                     bool want_blocked, bool* wrote_blocked,
                     const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
                     const float* v_scale, int64_t pool_blocks, void* stream, void* fixed_scratch = nullptr,
-                    size_t fixed_scratch_bytes = 0);
+                    size_t fixed_scratch_bytes = 0, int64_t active_blocks = -1);
 // fixed_scratch != null: the partition partials go there instead of the grow-only workspace, and a
 // launch that needs more than fixed_scratch_bytes is refused (nothing is allocated either way).
 //

@@ -48,6 +48,7 @@ struct AttnParams {
   const float* k_scale;  // [pool_blocks, Hkv] for an e4m3 cache, else null
   const float* v_scale;
   int batch, hq, hkv, group, gtiles, bs, max_blocks, tpp, n_part;
+  int ctx_cap;     // tokens a sequence may attend to: max_blocks * bs, or fewer when the caller limits the KV loop
   int pool_blocks; // physical blocks in the cache when the caller knows it, else 0 (table entries unchecked)
   int* error_flag; // set when a table entry a sequence uses addresses a block outside the cache
   int gt_rows;     // query rows one wavefront covers: 16 x its tile count; gtiles = ceil(group / gt_rows)
@@ -495,7 +496,7 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   const int first_window =
       p.block_table[(size_t)b * p.max_blocks + min(part * p.tpp / p.bs + lane, p.max_blocks - 1)];
   int ctx = p.ctx_lens[b];
-  const int max_ctx = p.max_blocks * p.bs;
+  const int max_ctx = p.ctx_cap;
   ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
   const int tok_begin = part * p.tpp;
   const int tok_end = min(ctx, tok_begin + p.tpp);
@@ -550,7 +551,7 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
   if (row >= p.batch * p.hq) return;
   const int b = row / p.hq;
   int ctx = p.ctx_lens[b];
-  const int max_ctx = p.max_blocks * p.bs;
+  const int max_ctx = p.ctx_cap;
   ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
   const int np = (ctx + p.tpp - 1) / p.tpp;
   const float* ml = p.part_ml + (size_t)row * p.n_part * 2;
@@ -669,7 +670,7 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
 constexpr int kLeanMaxWaves = 8;
 
 __device__ __forceinline__ int seq_chunks(const AttnParams& p, int ctx) {
-  const int max_ctx = p.max_blocks * p.bs;
+  const int max_ctx = p.ctx_cap;
   ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
   return (ctx + kChunk - 1) / kChunk;
 }
@@ -727,7 +728,7 @@ __global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(A
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, j = lane >> 4;
   const int hg_count = p.hkv * p.gtiles;
-  const int max_ctx = p.max_blocks * p.bs;
+  const int max_ctx = p.ctx_cap;
   char* kbuf = lean_lds + wave * KStage<D, FP8>::kBytes;
 
   // Wavefronts are numbered CU-fastest, so that a short item list still spreads over the CUs;
@@ -981,7 +982,7 @@ __global__ __launch_bounds__(64) void attn_stream_probe_kernel(AttnParams p) {
   int win_base = part * p.tpp / p.bs;
   int win_blk = table[min(win_base + lane, p.max_blocks - 1)];
   int ctx = p.ctx_lens[b];
-  const int max_ctx = p.max_blocks * p.bs;
+  const int max_ctx = p.ctx_cap;
   ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
   const int tok_begin = part * p.tpp;
   const int tok_end = min(ctx, tok_begin + p.tpp);
@@ -1044,8 +1045,10 @@ namespace {
 // `p` (heads, query tiles per wavefront, tokens per partition, partition count, residency cap) and
 // says whether the launch takes the evenly split form.  Shared by the attention launch and by the
 // load-only probe, so that both walk the cache in the same pieces.
-int plan_launch(const int64_t* config, int q_dtype, int kv_dtype, bool have_scales, AttnParams& p, int& gt,
-                bool& lean) {
+// active_blocks >= 0 bounds the KV loop of every sequence to that many blocks, as the SPMD form's
+// config slot does (09_paged_attention_spmd.py:482: max_bn = min(max_bn, active_block_num)); < 0: no bound.
+int plan_launch(const int64_t* config, int q_dtype, int kv_dtype, bool have_scales, int64_t active_blocks,
+                AttnParams& p, int& gt, bool& lean) {
   pto_hip::Context& cx = pto_hip::ctx();
   using pto_hip::dtype_name;
   using pto_hip::fail;
@@ -1092,8 +1095,12 @@ int plan_launch(const int64_t* config, int q_dtype, int kv_dtype, bool have_scal
   p.bs = (int)bs;
   p.max_blocks = (int)max_blocks;
   p.scale_log2e = scale * kLog2e;
+  const int64_t cap_blocks = active_blocks >= 0 && active_blocks < max_blocks ? active_blocks : max_blocks;
+  p.ctx_cap = (int)(cap_blocks * bs);
 
-  const int64_t max_ctx = max_blocks * bs;
+  // the launch is shaped for the longest context a sequence can have (one block at least, so that a
+  // bound of zero blocks still plans a grid: every sequence then has nothing to attend to)
+  const int64_t max_ctx = (cap_blocks > 0 ? cap_blocks : 1) * bs;
   // Context partitions: about one wavefront per SIMD when every sequence is at its maximum
   // length (measured best for short launches, where the spread of finishing times matters more
   // than occupancy), but never more than 2048 tokens per partition so long contexts still
@@ -1135,7 +1142,7 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
                     const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
                     bool want_blocked, bool* wrote_blocked, const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
                     const float* v_scale, int64_t pool_blocks, void* stream, void* fixed_scratch,
-                    size_t fixed_scratch_bytes) {
+                    size_t fixed_scratch_bytes, int64_t active_blocks) {
   Context& cx = ctx();
   if (!cx.initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(config != nullptr, "paged_attention: config is null");
@@ -1149,7 +1156,7 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   int gt = 1;
   bool lean = false;
   {
-    const int rc = plan_launch(config, q_dtype, kv_dtype, k_scale && v_scale, p, gt, lean);
+    const int rc = plan_launch(config, q_dtype, kv_dtype, k_scale && v_scale, active_blocks, p, gt, lean);
     if (rc != PTO_HIP_OK) return rc;
   }
   const bool fp8 = kv_dtype == PTO_HIP_FP8E4M3FN;
@@ -1303,7 +1310,7 @@ extern "C" int pto_hip_paged_attention_stream_probe(const void* key_cache, const
   AttnParams p{};
   int gt = 1;
   bool lean = false;
-  const int rc = plan_launch(config, q_dtype, kv_dtype, true, p, gt, lean);
+  const int rc = plan_launch(config, q_dtype, kv_dtype, true, -1, p, gt, lean);
   if (rc != PTO_HIP_OK) return rc;
   if (lean)
     return pto_hip::fail(PTO_HIP_ERR_UNSUPPORTED,

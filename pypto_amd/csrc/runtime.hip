@@ -96,13 +96,17 @@ enum ProgramKind {
   kGateUpSwiglu,
   kFfnBlockFp8,
   kLlamaMini,
+  kPagedAttentionBatch,
+  kPagedAttentionDynamic,
+  kPagedAttentionSpmd,
   kNumPrograms
 };
 
 const char* const kProgramNames[kNumPrograms] = {
     "paged_attention", "paged_gather",  "rms_norm",           "ffn_swiglu",          "ffn_block",
     "w8a16_matmul",    "w8a16_swiglu",  "rope_kv_cache_update", "rope_kv_cache_update_fp8",
-    "decoder_layer_decode", "projection", "gate_up_swiglu", "ffn_block_fp8", "llama_mini"};
+    "decoder_layer_decode", "projection", "gate_up_swiglu", "ffn_block_fp8", "llama_mini",
+    "paged_attention_batch", "paged_attention_dynamic", "paged_attention_spmd"};
 
 std::mutex g_mu;
 std::vector<int> g_callables;  // callable id -> ProgramKind, -1 once unregistered
@@ -151,76 +155,183 @@ int check_tensor(const char* prog, const char* name, const PtoHipChipTensor& t, 
   return PTO_HIP_OK;
 }
 
-// Reads the 7-slot int64 config wherever it lives.  The reference's orchestration reads it
-// with tensor.read on a host-visible buffer; a device-resident config costs one blocking copy.
-int read_config(const PtoHipChipTensor& t, hipStream_t stream, int64_t out[7]) {
-  PTO_CHECK_ARG(t.dtype == PTO_HIP_INT64 && numel(t) == 7,
-                "paged_attention: config must be INT64[7], got %s[%lld]", dtype_name(t.dtype),
-                (long long)numel(t));
+// Reads a small tensor the orchestration would read with tensor.read wherever it lives.  The
+// reference's orchestration reads it on a host-visible buffer; a device-resident one costs one
+// blocking copy.
+int read_small(const PtoHipChipTensor& t, hipStream_t stream, void* out, size_t bytes) {
   const void* src = tptr(t);
   hipPointerAttribute_t attr;
   hipError_t e = hipPointerGetAttributes(&attr, src);
   if (e != hipSuccess) {
     (void)hipGetLastError();  // plain host memory: not an error for us
-    std::memcpy(out, src, 7 * sizeof(int64_t));
+    std::memcpy(out, src, bytes);
     return PTO_HIP_OK;
   }
   if (attr.type == hipMemoryTypeDevice) {
-    PTO_CHECK_HIP(hipMemcpyAsync(out, src, 7 * sizeof(int64_t), hipMemcpyDeviceToHost, stream));
+    PTO_CHECK_HIP(hipMemcpyAsync(out, src, bytes, hipMemcpyDeviceToHost, stream));
     PTO_CHECK_HIP(hipStreamSynchronize(stream));
   } else {
-    std::memcpy(out, src, 7 * sizeof(int64_t));
+    std::memcpy(out, src, bytes);
   }
   return PTO_HIP_OK;
 }
 
+int read_config(const char* prog, const PtoHipChipTensor& t, hipStream_t stream, int64_t out[7]) {
+  PTO_CHECK_ARG(t.dtype == PTO_HIP_INT64 && numel(t) == 7, "%s: config must be INT64[7], got %s[%lld]", prog,
+                dtype_name(t.dtype), (long long)numel(t));
+  return read_small(t, stream, out, 7 * sizeof(int64_t));
+}
+
+// One paged-attention call as any of the orchestration forms hands it over: the six tensors all forms
+// share, the decoded 7-slot config {B, Hq, Hkv, D, bs, max_blocks, scale bits}, the optional scales of
+// an FP8E4M3FN cache and the optional bound on the KV loop.
+struct AttnCall {
+  const char* prog;
+  const PtoHipChipTensor *query, *key_cache, *value_cache, *block_table, *context_lens, *out;
+  const PtoHipChipTensor *k_scale = nullptr, *v_scale = nullptr;
+  int64_t cfg[7];
+  int64_t active_blocks = -1;
+};
+
+int launch_attention(const AttnCall& a, hipStream_t stream) {
+  const PtoHipChipTensor* six[6] = {a.query, a.key_cache, a.value_cache, a.block_table, a.context_lens, a.out};
+  static const char* names[6] = {"query", "key_cache", "value_cache", "block_table", "context_lens", "out"};
+  for (int i = 0; i < 6; ++i) {
+    int rc = check_tensor(a.prog, names[i], *six[i], 1, 2);
+    if (rc) return rc;
+  }
+  const PtoHipChipTensor &q = *a.query, &kc = *a.key_cache, &vc = *a.value_cache, &out = *a.out;
+  const int64_t batch = a.cfg[0], hq = a.cfg[1], hkv = a.cfg[2], d = a.cfg[3], bs = a.cfg[4], mb = a.cfg[5];
+  PTO_CHECK_ARG(batch >= 0 && hq > 0 && hkv > 0 && d > 0 && bs > 0 && mb > 0,
+                "%s: config holds a non-positive dimension", a.prog);
+  PTO_CHECK_ARG(a.block_table->dtype == PTO_HIP_INT32 && a.context_lens->dtype == PTO_HIP_INT32,
+                "%s: block_table and context_lens must be INT32", a.prog);
+  PTO_CHECK_ARG(out.dtype == PTO_HIP_FP32, "%s: out must be FP32, got %s", a.prog, dtype_name(out.dtype));
+  PTO_CHECK_ARG(numel(q) == batch * hq * d, "%s: query has %lld elements, config says %lld", a.prog,
+                (long long)numel(q), (long long)(batch * hq * d));
+  PTO_CHECK_ARG(numel(out) == batch * hq * d, "%s: out has %lld elements, config says %lld", a.prog,
+                (long long)numel(out), (long long)(batch * hq * d));
+  PTO_CHECK_ARG(numel(*a.block_table) >= batch * mb, "%s: block_table has %lld entries, needs %lld", a.prog,
+                (long long)numel(*a.block_table), (long long)(batch * mb));
+  PTO_CHECK_ARG(numel(*a.context_lens) >= batch, "%s: context_lens has %lld entries, needs %lld", a.prog,
+                (long long)numel(*a.context_lens), (long long)batch);
+  PTO_CHECK_ARG(numel(kc) % (hkv * bs * d) == 0 && numel(kc) == numel(vc) && kc.dtype == vc.dtype,
+                "%s: key/value cache must be equal-shaped [pool*Hkv*bs, D]", a.prog);
+  const float* ks = nullptr;
+  const float* vs = nullptr;
+  if (kc.dtype == PTO_HIP_FP8E4M3FN) {
+    PTO_CHECK_ARG(a.k_scale && a.v_scale, "%s: FP8E4M3FN cache needs k_scale and v_scale tensors", a.prog);
+    int rc = check_tensor(a.prog, "k_scale", *a.k_scale, 1, 2);
+    if (!rc) rc = check_tensor(a.prog, "v_scale", *a.v_scale, 1, 2);
+    if (rc) return rc;
+    const int64_t pool = numel(kc) / (hkv * bs * d);
+    PTO_CHECK_ARG(a.k_scale->dtype == PTO_HIP_FP32 && a.v_scale->dtype == PTO_HIP_FP32 &&
+                      numel(*a.k_scale) == pool * hkv && numel(*a.v_scale) == pool * hkv,
+                  "%s: k_scale/v_scale must be FP32[pool_blocks, Hkv]", a.prog);
+    ks = reinterpret_cast<const float*>(tptr(*a.k_scale));
+    vs = reinterpret_cast<const float*>(tptr(*a.v_scale));
+  }
+  // The tensor view says how many blocks the caches hold: table entries beyond that are caught.
+  return paged_attention(tptr(q), tptr(kc), tptr(vc), reinterpret_cast<const int32_t*>(tptr(*a.block_table)),
+                         reinterpret_cast<const int32_t*>(tptr(*a.context_lens)), reinterpret_cast<float*>(tptr_mut(out)),
+                         nullptr, false, nullptr, a.cfg, (int)q.dtype, (int)kc.dtype, ks, vs,
+                         numel(kc) / (hkv * bs * d), stream, nullptr, 0, a.active_blocks);
+}
+
+// examples/models/04_paged_attention.py:272-288 (and 07_paged_attention_multi_config.py:498): query,
+// key_cache, value_cache, block_table, context_lens, out, config [, k_scale, v_scale].
 int run_paged_attention(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns,
                         hipStream_t stream) {
   PTO_CHECK_ARG(nt == 7 || nt == 9, "paged_attention: expected 7 tensors (9 with FP8 scales), got %d", nt);
   PTO_CHECK_ARG(ns == 0, "paged_attention: expected no scalars, got %d", ns);
-  static const char* names[9] = {"query", "key_cache", "value_cache", "block_table", "context_lens",
-                                 "out", "config", "k_scale", "v_scale"};
-  for (int i = 0; i < nt; ++i) {
-    int rc = check_tensor("paged_attention", names[i], t[i], 1, 2);
-    if (rc) return rc;
+  AttnCall a{"paged_attention", &t[0], &t[1], &t[2], &t[3], &t[4], &t[5]};
+  if (nt == 9) {
+    a.k_scale = &t[7];
+    a.v_scale = &t[8];
   }
-  int64_t cfg[7];
-  int rc = read_config(t[6], stream, cfg);
+  int rc = check_tensor(a.prog, "config", t[6], 1, 2);
+  if (!rc) rc = read_config(a.prog, t[6], stream, a.cfg);
   if (rc) return rc;
-  const int64_t batch = cfg[0], hq = cfg[1], hkv = cfg[2], d = cfg[3], bs = cfg[4], mb = cfg[5];
-  PTO_CHECK_ARG(batch >= 0 && hq > 0 && hkv > 0 && d > 0 && bs > 0 && mb > 0,
-                "paged_attention: config holds a non-positive dimension");
-  PTO_CHECK_ARG(t[3].dtype == PTO_HIP_INT32 && t[4].dtype == PTO_HIP_INT32,
-                "paged_attention: block_table and context_lens must be INT32");
-  PTO_CHECK_ARG(t[5].dtype == PTO_HIP_FP32, "paged_attention: out must be FP32, got %s",
-                dtype_name(t[5].dtype));
-  PTO_CHECK_ARG(numel(t[0]) == batch * hq * d, "paged_attention: query has %lld elements, config says %lld",
-                (long long)numel(t[0]), (long long)(batch * hq * d));
-  PTO_CHECK_ARG(numel(t[5]) == batch * hq * d, "paged_attention: out has %lld elements, config says %lld",
-                (long long)numel(t[5]), (long long)(batch * hq * d));
-  PTO_CHECK_ARG(numel(t[3]) >= batch * mb, "paged_attention: block_table has %lld entries, needs %lld",
-                (long long)numel(t[3]), (long long)(batch * mb));
-  PTO_CHECK_ARG(numel(t[4]) >= batch, "paged_attention: context_lens has %lld entries, needs %lld",
-                (long long)numel(t[4]), (long long)batch);
-  PTO_CHECK_ARG(numel(t[1]) % (hkv * bs * d) == 0 && numel(t[1]) == numel(t[2]) &&
-                    t[1].dtype == t[2].dtype,
-                "paged_attention: key/value cache must be equal-shaped [pool*Hkv*bs, D]");
-  const float* ks = nullptr;
-  const float* vs = nullptr;
-  if (t[1].dtype == PTO_HIP_FP8E4M3FN) {
-    PTO_CHECK_ARG(nt == 9, "paged_attention: FP8E4M3FN cache needs k_scale and v_scale tensors");
-    const int64_t pool = numel(t[1]) / (hkv * bs * d);
-    PTO_CHECK_ARG(t[7].dtype == PTO_HIP_FP32 && t[8].dtype == PTO_HIP_FP32 &&
-                      numel(t[7]) == pool * hkv && numel(t[8]) == pool * hkv,
-                  "paged_attention: k_scale/v_scale must be FP32[pool_blocks, Hkv]");
-    ks = reinterpret_cast<const float*>(tptr(t[7]));
-    vs = reinterpret_cast<const float*>(tptr(t[8]));
+  return launch_attention(a, stream);
+}
+
+// examples/models/05_paged_attention_batch.py:373-386: the seven tensors of the plain form followed by
+// size_query, size_key_cache, size_value_cache (INT64[1] each: byte sizes the orchestration's body
+// never reads; accepted and left alone).
+int run_paged_attention_batch(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
+  const char* prog = "paged_attention_batch";
+  PTO_CHECK_ARG(nt == 10, "%s: expected 10 tensors (query, key_cache, value_cache, block_table, context_lens, out, "
+                "config, size_query, size_key_cache, size_value_cache), got %d", prog, nt);
+  PTO_CHECK_ARG(ns == 0, "%s: expected no scalars, got %d", prog, ns);
+  static const char* sizes[3] = {"size_query", "size_key_cache", "size_value_cache"};
+  for (int i = 0; i < 3; ++i)
+    PTO_CHECK_ARG(t[7 + i].dtype == PTO_HIP_INT64 && numel(t[7 + i]) == 1, "%s: %s must be INT64[1], got %s[%lld]", prog,
+                  sizes[i], dtype_name(t[7 + i].dtype), (long long)numel(t[7 + i]));
+  AttnCall a{prog, &t[0], &t[1], &t[2], &t[3], &t[4], &t[5]};
+  int rc = check_tensor(prog, "config", t[6], 1, 2);
+  if (!rc) rc = read_config(prog, t[6], stream, a.cfg);
+  if (rc) return rc;
+  return launch_attention(a, stream);
+}
+
+// examples/models/06_paged_attention_dynamic.py:262-300: no config tensor; every dimension comes from
+// the tensors' shapes (batch = context_lens.dim(0), head_dim = query.dim(1), num_heads = query.dim(0) /
+// batch, block_num = block_table.dim(0) / batch, block_size = value_cache.dim(0) / block_table.dim(0)),
+// one KV head, scale 1.0 (:411).
+int run_paged_attention_dynamic(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
+  const char* prog = "paged_attention_dynamic";
+  PTO_CHECK_ARG(nt == 6, "%s: expected 6 tensors (query, key_cache, value_cache, block_table, context_lens, out), got %d",
+                prog, nt);
+  PTO_CHECK_ARG(ns == 0, "%s: expected no scalars, got %d", prog, ns);
+  PTO_CHECK_ARG(t[0].ndims == 2 && t[1].ndims == 2 && t[2].ndims == 2 && t[3].ndims == 1 && t[4].ndims == 1,
+                "%s: query and the caches must be 2-D, block_table and context_lens 1-D (their shapes are the "
+                "configuration)", prog);
+  const int64_t batch = t[4].shapes[0], rows = t[0].shapes[0], d = t[0].shapes[1], table = t[3].shapes[0],
+                cache_rows = t[2].shapes[0];
+  AttnCall a{prog, &t[0], &t[1], &t[2], &t[3], &t[4], &t[5]};
+  if (batch == 0) {
+    PTO_CHECK_ARG(rows == 0 && numel(t[5]) == 0, "%s: an empty batch with %lld query rows", prog, (long long)rows);
+    return PTO_HIP_OK;
   }
-  // The tensor view says how many blocks the caches hold: table entries beyond that are caught.
-  return paged_attention(tptr(t[0]), tptr(t[1]), tptr(t[2]), reinterpret_cast<const int32_t*>(tptr(t[3])),
-                         reinterpret_cast<const int32_t*>(tptr(t[4])), reinterpret_cast<float*>(tptr_mut(t[5])),
-                         nullptr, false, nullptr, cfg, (int)t[0].dtype, (int)t[1].dtype, ks, vs,
-                         numel(t[1]) / (hkv * bs * d), stream);
+  PTO_CHECK_ARG(rows % batch == 0 && rows > 0, "%s: %lld query rows do not divide into %lld sequences", prog,
+                (long long)rows, (long long)batch);
+  PTO_CHECK_ARG(table % batch == 0 && table > 0, "%s: %lld block_table entries do not divide into %lld sequences", prog,
+                (long long)table, (long long)batch);
+  PTO_CHECK_ARG(cache_rows % table == 0 && cache_rows > 0,
+                "%s: %lld cache rows are not a whole number of rows for each of the %lld block_table entries", prog,
+                (long long)cache_rows, (long long)table);
+  const float one = 1.0f;
+  uint32_t one_bits;
+  std::memcpy(&one_bits, &one, 4);
+  const int64_t cfg[7] = {batch, rows / batch, 1, d, cache_rows / table, table / batch, (int64_t)one_bits};
+  std::memcpy(a.cfg, cfg, sizeof(cfg));
+  return launch_attention(a, stream);
+}
+
+// examples/models/09_paged_attention_spmd.py:445-482: query, key_cache, value_cache, block_table,
+// context_lens, scale (FP32[1]), out, config, where config = {B, Hq, Hkv, D, bs, block_num_capacity,
+// active_block_num}: the last slot bounds the KV loop of every sequence instead of carrying the scale.
+int run_paged_attention_spmd(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream) {
+  const char* prog = "paged_attention_spmd";
+  PTO_CHECK_ARG(nt == 8, "%s: expected 8 tensors (query, key_cache, value_cache, block_table, context_lens, scale, out, "
+                "config), got %d", prog, nt);
+  PTO_CHECK_ARG(ns == 0, "%s: expected no scalars, got %d", prog, ns);
+  PTO_CHECK_ARG(t[5].dtype == PTO_HIP_FP32 && numel(t[5]) == 1, "%s: scale must be FP32[1], got %s[%lld]", prog,
+                dtype_name(t[5].dtype), (long long)numel(t[5]));
+  AttnCall a{prog, &t[0], &t[1], &t[2], &t[3], &t[4], &t[6]};
+  int rc = check_tensor(prog, "config", t[7], 1, 2);
+  if (!rc) rc = check_tensor(prog, "scale", t[5], 1, 2, 4);
+  if (!rc) rc = read_config(prog, t[7], stream, a.cfg);
+  if (rc) return rc;
+  PTO_CHECK_ARG(a.cfg[6] >= 0 && a.cfg[6] <= a.cfg[5],
+                "%s: active_block_num %lld outside [0, block_num_capacity %lld]", prog, (long long)a.cfg[6],
+                (long long)a.cfg[5]);
+  a.active_blocks = a.cfg[6];
+  uint32_t scale_bits = 0;
+  rc = read_small(t[5], stream, &scale_bits, 4);
+  if (rc) return rc;
+  a.cfg[6] = (int64_t)scale_bits;
+  return launch_attention(a, stream);
 }
 
 int run_paged_gather(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns,
@@ -630,6 +741,9 @@ int dispatch(int kind, const PtoHipChipTensor* t, int nt, const uint64_t* s, int
              hipStream_t stream) {
   switch (kind) {
     case kPagedAttention: return run_paged_attention(t, nt, s, ns, stream);
+    case kPagedAttentionBatch: return run_paged_attention_batch(t, nt, s, ns, stream);
+    case kPagedAttentionDynamic: return run_paged_attention_dynamic(t, nt, s, ns, stream);
+    case kPagedAttentionSpmd: return run_paged_attention_spmd(t, nt, s, ns, stream);
     case kPagedGather: return run_paged_gather(t, nt, s, ns, stream);
     case kRmsNorm: return run_rms_norm(t, nt, s, ns, stream);
     case kFfnSwiglu: return run_ffn(t, nt, s, ns, stream, false);

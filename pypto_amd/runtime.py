@@ -65,6 +65,13 @@ class HipProgram:
 
 
 paged_attention = HipProgram("paged_attention", (IN, IN, IN, IN, IN, OUT, HOST, IN, IN), optional=2)
+# the same attention through the reference's other orchestration signatures
+# 05_paged_attention_batch.py:373-386: ... config, size_query, size_key_cache, size_value_cache (never read)
+paged_attention_batch = HipProgram("paged_attention_batch", (IN, IN, IN, IN, IN, OUT, HOST, HOST, HOST, HOST))
+# 06_paged_attention_dynamic.py:262-270: no config, the tensors' shapes are the configuration
+paged_attention_dynamic = HipProgram("paged_attention_dynamic", (IN, IN, IN, IN, IN, OUT))
+# 09_paged_attention_spmd.py:445-456: scale as an FP32[1] tensor before out; config[6] = active_block_num
+paged_attention_spmd = HipProgram("paged_attention_spmd", (IN, IN, IN, IN, IN, HOST, OUT, HOST))
 paged_gather = HipProgram("paged_gather", (IN, IN, IN, OUT), scalars=("block_size", "col_offset"))
 rms_norm = HipProgram("rms_norm", (IN, IN, OUT), scalars=("eps",))
 rms_norm_unweighted = HipProgram("rms_norm", (IN, OUT), scalars=("eps",))  # 08_llama_mini.py:93-118
@@ -105,7 +112,8 @@ decoder_layer_decode_w16_fp8kv = HipProgram(
     "decoder_layer_decode", (IN, IN, IN, INOUT, INOUT, INOUT, INOUT) + (IN,) * 9 + (OUT,),
     scalars=("num_heads", "kv_head_num", "head_dim", "block_size", "eps"))
 
-PROGRAMS = {p.name: p for p in (paged_attention, paged_gather, rms_norm, ffn_swiglu, ffn_block, ffn_block_fp8, llama_mini,
+PROGRAMS = {p.name: p for p in (paged_attention, paged_attention_batch, paged_attention_dynamic, paged_attention_spmd,
+                                paged_gather, rms_norm, ffn_swiglu, ffn_block, ffn_block_fp8, llama_mini,
                                 projection, gate_up_swiglu,
                                 w8a16_matmul,
                                 w8a16_swiglu, rope_kv_cache_update, rope_kv_cache_update_fp8,

@@ -45,6 +45,30 @@ class AttentionInputs:
             return base + (self.k_scale, self.v_scale)
         return base
 
+    # -- the same problem through the reference's other orchestration signatures --------------------
+    def args_batch(self) -> tuple:
+        """05_paged_attention_batch.py:373-386: the plain arguments + three INT64[1] byte sizes."""
+        sizes = [torch.tensor([t.numel() * t.element_size()], dtype=torch.int64)
+                 for t in (self.query, self.key_cache, self.value_cache)]
+        return self.args()[:7] + tuple(sizes)
+
+    def args_dynamic(self) -> tuple:
+        """06_paged_attention_dynamic.py:262-270: no config; the shapes must say everything (one KV head,
+        scale 1.0, exactly one cache block per block-table entry)."""
+        return self.args()[:6]
+
+    def args_spmd(self, active_num_blocks: int | None = None) -> tuple:
+        """09_paged_attention_spmd.py:445-456: scale tensor before out, config[6] = active_block_num
+        (default: the blocks of the longest context, as build_tensor_specs :687-691 sets it)."""
+        cfg = self.config.clone()
+        bs, cap = int(cfg[4]), int(cfg[5])
+        if active_num_blocks is None:
+            top = int(self.context_lens.max().item()) if self.context_lens.numel() else 0
+            active_num_blocks = min(cap, (top + bs - 1) // bs)
+        scale = torch.tensor([struct.unpack("f", struct.pack("I", int(cfg[6]) & 0xFFFFFFFF))[0]], dtype=torch.float32)
+        cfg[6] = active_num_blocks
+        return (self.query, self.key_cache, self.value_cache, self.block_table, self.context_lens, scale, self.out, cfg)
+
     def kv_bytes(self) -> int:
         """Algorithmic K+V bytes one decode pass must read: sum(ctx) * Hkv * D * 2 * elem."""
         cfg = self.config.tolist()
@@ -148,6 +172,30 @@ def paged_attention_inputs(
         k_scale=k_scale,
         v_scale=v_scale,
     )
+
+
+def reference_example_inputs(*, batch: int, num_heads: int, head_dim: int, block_size: int, context_len,
+                             max_model_len: int, scale: float = 1.0, seed: int = 0, device="cpu") -> AttentionInputs:
+    """The inputs the reference's own attention examples and system tests draw
+    (09_paged_attention_spmd.py:655-730, tests/st/runtime/framework_and_models/test_dynamic_paged_attention.py):
+    one KV head, a pool of exactly batch * max_blocks blocks, a block table of random entries WITH
+    replacement, q/K/V ~ N(0,1) in bf16, ``context_len`` one number or one per sequence."""
+    dev = torch.device(device)
+    max_blocks = max_model_len // block_size
+    pool = batch * max_blocks
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    ctx = (torch.full((batch,), int(context_len)) if isinstance(context_len, int)
+           else torch.tensor(list(context_len))).to(torch.int32)
+    assert ctx.numel() == batch
+    table = torch.randint(0, max(pool, 1), (batch * max_blocks,), generator=g, dtype=torch.int32)
+    gd = torch.Generator(device=dev).manual_seed(seed + 1)
+    rows = pool * block_size
+    mk = lambda r: torch.randn((r, head_dim), generator=gd, device=dev, dtype=torch.bfloat16)
+    config = torch.tensor([batch, num_heads, 1, head_dim, block_size, max_blocks, scale_bits(scale)], dtype=torch.int64)
+    return AttentionInputs(query=mk(batch * num_heads), key_cache=mk(rows), value_cache=mk(rows),
+                           block_table=table.to(dev), context_lens=ctx.to(dev),
+                           out=torch.zeros((batch * num_heads, head_dim), dtype=torch.float32, device=dev),
+                           config=config)
 
 
 def attention_small(seed: int = 0, device="cpu", **over) -> AttentionInputs:

@@ -129,3 +129,53 @@ def test_llama_mini_manifest_selects_the_single_launch_program(tmp_path):
     with pytest.raises(ValueError):
         mf.compile_and_assemble(_write(tmp_path, "llama_mini_orch", MINI_SIG,
                                        [k for k in MINI_KERNELS if k[0] != "kernel_softmax"]))
+
+
+# the reference's other three paged-attention programs: kernel names, core types and directions as in
+# examples/models/05_paged_attention_batch.py:88-386, 06_paged_attention_dynamic.py:77-270,
+# 09_paged_attention_spmd.py:111-456
+_UPD = ["IN", "IN", "IN", "INOUT", "INOUT", "INOUT"]
+ATTN_FORMS = {
+    "paged_attention_batch": ("BatchPagedAttention", ["IN"] * 5 + ["OUT"] + ["IN"] * 4, [
+        ("KernelQkMatmul", "aic", ["IN", "IN", "OUT", "IN"]),
+        ("KernelSoftmaxPrepare", "aiv", ["IN", "OUT", "OUT", "OUT", "IN"]),
+        ("KernelPvMatmul", "aic", ["IN", "IN", "OUT", "IN"]),
+        ("KernelOnlineUpdate", "aiv", _UPD + ["OUT"])]),
+    "paged_attention_dynamic": ("paged_attention", ["IN"] * 5 + ["OUT"], [
+        ("dyn_kernel_init_inplace", "aiv", ["OUT"] * 3), ("dyn_kernel_qk_matmul", "aic", ["IN", "IN", "OUT"]),
+        ("dyn_kernel_softmax_prepare", "aiv", ["IN", "OUT", "OUT", "OUT"]),
+        ("dyn_kernel_pv_matmul", "aic", ["IN", "IN", "OUT"]),
+        ("dyn_kernel_online_update", "aiv", _UPD + ["OUT"])]),
+    "paged_attention_spmd": ("paged_attention_spmd", ["IN"] * 6 + ["OUT", "IN"], [
+        ("SpmdQkMatmul", "aic", ["IN", "IN", "OUT", "IN", "IN"]),
+        ("SpmdSoftmaxPrepare", "aiv", ["IN", "OUT", "OUT", "OUT", "IN"]),
+        ("SpmdPvMatmul", "aic", ["IN", "IN", "OUT", "IN", "IN"]),
+        ("SpmdOnlineUpdate", "aiv", _UPD), ("SpmdNormalize", "aiv", ["IN", "IN", "OUT"])]),
+}
+
+
+@pytest.mark.parametrize("name", sorted(ATTN_FORMS))
+def test_the_other_attention_programs_select_their_call_form(tmp_path, name):
+    orch, sig, kernels = ATTN_FORMS[name]
+    prog, _, _ = mf.compile_and_assemble(_write(tmp_path, orch, sig, kernels))
+    assert prog.name == name and len(prog.signature) == len(sig)
+    # tensors the launcher reads on the host stay host-read operands, whatever the manifest calls them
+    from pypto_amd.runtime import PROGRAMS
+    assert [i for i, d in enumerate(prog.signature) if d == HOST] == \
+        [i for i, d in enumerate(PROGRAMS[name].signature) if d == HOST]
+    # and the written manifest of that program reads back to the same selection
+    out = tmp_path / "written"
+    out.mkdir()
+    mf.write_kernel_config(out, name)
+    again, _, _ = mf.compile_and_assemble(out)
+    assert again.name == name
+
+
+def test_same_orchestration_name_different_kernels_are_told_apart(tmp_path):
+    """04's and 06's orchestration functions are both called paged_attention; the kernel names and the
+    number of orchestration tensors decide."""
+    _, sig6, k6 = ATTN_FORMS["paged_attention_dynamic"]
+    assert mf.compile_and_assemble(_write(tmp_path, "paged_attention", ATTN_SIG, ATTN_KERNELS))[0].name == "paged_attention"
+    assert mf.compile_and_assemble(_write(tmp_path, "paged_attention", sig6, k6))[0].name == "paged_attention_dynamic"
+    with pytest.raises(ValueError, match="no fused HIP program"):   # 04's kernels under 06's six tensors
+        mf.compile_and_assemble(_write(tmp_path, "paged_attention", sig6, ATTN_KERNELS))

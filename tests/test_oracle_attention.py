@@ -195,3 +195,53 @@ def test_fp8_golden_close_to_bf16_golden():
     out = oracle.paged_attention_golden(inp.query, kq, vq, inp.block_table, inp.context_lens, inp.config, ks, vs)
     assert (out - ref).abs().max() < 0.15  # e4m3 quantisation noise on N(0,1) data
     assert (out - ref).abs().mean() < 0.03
+
+
+# ---- the reference's other orchestration signatures (05 batch, 06 dynamic, 09 SPMD) --------------------
+def test_reference_example_inputs_have_the_example_layout():
+    """09_paged_attention_spmd.py:666-730 / 06's test: one KV head, a pool of batch * max_blocks blocks,
+    table entries drawn with replacement from the whole pool."""
+    inp = workloads.reference_example_inputs(batch=4, num_heads=16, head_dim=32, block_size=16,
+                                             context_len=[20, 64, 1, 33], max_model_len=128, seed=3)
+    assert inp.config.tolist()[:6] == [4, 16, 1, 32, 16, 8]
+    assert inp.key_cache.shape == (4 * 8 * 16, 32) and inp.block_table.shape == (32,)
+    assert inp.block_table.min() >= 0 and inp.block_table.max() < 32
+    assert inp.context_lens.tolist() == [20, 64, 1, 33] and inp.query.dtype == torch.bfloat16
+
+
+def test_dynamic_form_reads_its_configuration_off_the_shapes():
+    inp = workloads.reference_example_inputs(batch=3, num_heads=16, head_dim=32, block_size=16,
+                                             context_len=[40, 7, 96], max_model_len=96, seed=5)
+    explicit = oracle.paged_attention_golden(*inp.args()[:5], inp.config)
+    assert torch.equal(oracle.paged_attention_dynamic_golden(*inp.args_dynamic()[:5]), explicit)
+    # and what it computes is the definition (fp64 loops), scale 1
+    assert torch.allclose(explicit, _brute_force(inp), atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("active", [0, 1, 2, 3, 6])
+def test_spmd_active_block_num_clips_every_context(active):
+    """config[6] = N means no sequence attends beyond its first N blocks (09:600-603): the result is the
+    textbook attention over contexts clipped to N * bs tokens; a row with nothing left is zero (:647-651)."""
+    ctx = [40, 7, 96, 0]
+    inp = workloads.reference_example_inputs(batch=4, num_heads=16, head_dim=32, block_size=16, context_len=ctx,
+                                             max_model_len=96, scale=0.3, seed=6)
+    q, kc, vc, table, lens, scale, _, cfg = inp.args_spmd(active)
+    assert cfg[6] == active and abs(float(scale) - 0.3) < 1e-7
+    out = oracle.paged_attention_spmd_golden(q, kc, vc, table, lens, scale, cfg)
+    clipped = torch.tensor([min(c, active * 16) for c in ctx], dtype=torch.int32)
+    dense = oracle.paged_attention_dense(q, kc, vc, table, clipped, inp.config)
+    assert torch.allclose(out, dense, atol=1e-2, rtol=1e-2)
+    assert torch.equal(out.reshape(4, 16, 32)[3], torch.zeros(16, 32))
+    if active == 0:
+        assert not out.any()
+    if active >= 6:   # a bound that reaches every context changes nothing
+        assert torch.equal(out, oracle.paged_attention_golden(q, kc, vc, table, lens, inp.config))
+
+
+def test_spmd_default_active_blocks_follow_the_longest_context():
+    inp = workloads.reference_example_inputs(batch=2, num_heads=16, head_dim=32, block_size=16, context_len=[33, 5],
+                                             max_model_len=256, seed=1)
+    assert int(inp.args_spmd()[7][6]) == 3          # ceil(33 / 16), build_tensor_specs :687-691
+    assert int(inp.args_spmd(100)[7][6]) == 100
+    sizes = inp.args_batch()[7:]
+    assert [int(s) for s in sizes] == [2 * 16 * 32 * 2, 2 * 16 * 16 * 32 * 2, 2 * 16 * 16 * 32 * 2]
