@@ -109,6 +109,8 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *               config[7] i64 = {B,Hq,Hkv,D,bs,max_blocks,scale_bits}  (HOST or device memory)
  *               [, k_scale[pool,Hkv] fp32, v_scale[pool,Hkv] fp32]  when the caches are FP8E4M3FN
  *      cache row of (block p, kv head h, token t) = (p*Hkv + h)*bs + t
+ *      head_dim 128 / 256 with bs a multiple of 16 (32 for FP8E4M3FN) run on the tiled MFMA kernels; any other
+ *      head_dim up to 256 and any bs up to 4096 on a plain one-wavefront-per-head kernel; beyond: UNSUPPORTED
  *  "paged_attention_batch"    examples/models/05_paged_attention_batch.py:373-386
  *      tensors: the seven of "paged_attention", then size_query, size_key_cache, size_value_cache (i64[1] each;
  *               the orchestration never reads them and neither does this library)

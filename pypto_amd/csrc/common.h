@@ -166,6 +166,13 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
                     const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
                     const float* v_scale, int64_t pool_blocks, void* stream, void* fixed_scratch = nullptr,
                     size_t fixed_scratch_bytes = 0, int64_t active_blocks = -1);
+// The same contract for the shapes the tiled kernels are not built for (head_dim other than 128 / 256
+// up to 256, block sizes off the 16-token grid); attention_needs_generic says which launches take it.
+bool attention_needs_generic(const int64_t* config, int kv_dtype);
+int paged_attention_generic(const void* query, const void* key_cache, const void* value_cache,
+                            const int32_t* block_table, const int32_t* context_lens, float* out,
+                            const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
+                            const float* v_scale, int64_t pool_blocks, int64_t active_blocks, hipStream_t stream);
 // fixed_scratch != null: the partition partials go there instead of the grow-only workspace, and a
 // launch that needs more than fixed_scratch_bytes is refused (nothing is allocated either way).
 //

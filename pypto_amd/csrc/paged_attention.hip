@@ -1152,6 +1152,15 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   if (batch == 0) return PTO_HIP_OK;
   PTO_CHECK_ARG(query && key_cache && value_cache && block_table && context_lens && out,
                 "paged_attention: null tensor pointer");
+  if (attention_needs_generic(config, kv_dtype)) {
+    // shapes the tiled kernels are not built for: one wavefront per (sequence, head), no workspace
+    if (wrote_blocked) *wrote_blocked = false;
+    const int rc = paged_attention_generic(query, key_cache, value_cache, block_table, context_lens, out, config,
+                                           q_dtype, kv_dtype, k_scale, v_scale, pool_blocks, active_blocks,
+                                           (hipStream_t)stream);
+    if (rc || !out16) return rc;
+    return cast_from_f32(out, out16, (size_t)batch * hq * d, q_dtype, (hipStream_t)stream);
+  }
   AttnParams p{};
   int gt = 1;
   bool lean = false;
