@@ -131,6 +131,8 @@ PTO_HIP_API int pto_hip_sync(void* stream);
  *  "ffn_swiglu"        examples/models/01_ffn.py:111-131
  *      tensors: hidden_states[T,H], gate_proj_weight[H,I], up_proj_weight[H,I],
  *               down_proj_weight[I,H], output[T,H] (fp32 or dtype of x)
+ *  "ffn_gelu", "ffn_relu"   examples/models/01_ffn.py:90-108, :133-151
+ *      tensors: hidden_states[T,H], gate_proj_weight[H,I], down_proj_weight[I,H], output[T,H] (fp32 or dtype of x)
  *  "ffn_block"         tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:155-187
  *      tensors: x[T,H], gamma[1,H] fp32, w_gate[H,I], w_up[H,I], w_down[I,H], out[T,H]
  *      scalars: eps (f32 bits)
@@ -250,6 +252,16 @@ PTO_HIP_API int pto_hip_paged_gather(const void* src, const int32_t* indices,
 PTO_HIP_API int pto_hip_rms_norm(const void* x, const float* gamma, void* out, int64_t rows,
                                  int64_t hidden, float eps, int x_dtype, int out_dtype,
                                  void* stream);
+
+/* out = act(x Wg) Wd: the reference example's FFNs with one-operand activations
+ * (examples/models/01_ffn.py:90-108 ffn_gelu with GELU as x * sigmoid(1.702 x), :133-151 ffn_relu).
+ * dtype FP32 (out FP32), or BF16 / FP16 with fp32 accumulation, h rounded to dtype once and out in
+ * FP32 or dtype (hidden and intermediate multiples of 8). */
+#define PTO_HIP_ACT_GELU 1
+#define PTO_HIP_ACT_RELU 2
+PTO_HIP_API int pto_hip_ffn_activation(const void* x, const void* w_gate, const void* w_down, void* out,
+                                       int64_t tokens, int64_t hidden, int64_t intermediate, int activation,
+                                       int dtype, int out_dtype, void* stream);
 
 /* out = (silu(x Wg) * (x Wu)) Wd ; gamma != NULL adds the RMSNorm prologue (ffn_block).
  * Up to 32 tokens run as weight-streaming skinny projections (HBM-bound), more as MFMA-tiled

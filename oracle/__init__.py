@@ -32,6 +32,12 @@ Pinning status (what fixes each function independently of its own formula):
                                  (tests/test_oracle_stages.py).
 * ``ffn_swiglu`` / ``ffn_block`` — pinned: ``torch.nn.functional.silu`` form in
                                  fp64, committed seeded fixture.
+* ``ffn_gelu`` / ``ffn_relu``  — pinned: the kernel's ``recip(1 + exp(-1.702 g))``
+                                 form in fp64, the distance of that form to
+                                 the erf GELU, ``clamp(min=0)``, and the two
+                                 identities relu FFN(x) + relu FFN(-x) and
+                                 gelu(g) - gelu(-g) = g
+                                 (tests/test_oracle_ffn.py).
 * ``rms_norm``                — pinned: ``torch.nn.functional.rms_norm``.
 * ``rope_rotate_half``        — pinned: complex-rotation closed form, position-0
                                  identity, norm preservation, relative-position
@@ -69,7 +75,7 @@ from .attention import (  # noqa: F401
     quantize_kv_fp8,
 )
 from . import stages, tile_ops  # noqa: F401
-from .ffn import (ffn_block, ffn_block_fp8, ffn_swiglu, projection, quantize_rows_fp8, rms_norm,  # noqa: F401
+from .ffn import (ffn_block, ffn_block_fp8, ffn_gelu, ffn_relu, ffn_swiglu, projection, quantize_rows_fp8, rms_norm,  # noqa: F401
                   swiglu)
 from .layer import (  # noqa: F401
     decoder_layer_decode,

@@ -6,6 +6,7 @@ Restates the expected-value formulas the reference keeps next to its FFN tile
 programs:
 
 * SwiGLU FFN, fp32 64x64            examples/models/01_ffn.py:174-176
+* GELU / ReLU FFN, fp32 64x64       examples/models/01_ffn.py:165-167, :183-185
 * bf16 model form (h rounded)       tests/st/runtime/framework_and_models/
                                     test_qwen3_decode_scope3_mixed.py:278-287
                                     examples/models/qwen3_jit/kernels/mlp.py:58-60
@@ -68,6 +69,25 @@ def ffn_swiglu(x, w_gate, w_up, w_down, h_dtype: torch.dtype | None = None) -> t
     gate = torch.matmul(xf, w_gate.float())
     up = torch.matmul(xf, w_up.float())
     h = swiglu(gate, up)
+    if h_dtype is not None:
+        h = h.to(h_dtype).float()
+    return torch.matmul(h, w_down.float())
+
+
+def ffn_gelu(x, w_gate, w_down, h_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """``(g * sigmoid(1.702 g)) Wd`` with ``g = x Wg`` -> fp32 (01_ffn.py:165-167; the kernel's own form is
+    ``g * recip(1 + exp(-1.702 g))``, :51-62).  ``h_dtype`` rounds the activated intermediate before the
+    down projection, as in ``ffn_swiglu``."""
+    gate = torch.matmul(x.float(), w_gate.float())
+    h = gate * torch.sigmoid(1.702 * gate)
+    if h_dtype is not None:
+        h = h.to(h_dtype).float()
+    return torch.matmul(h, w_down.float())
+
+
+def ffn_relu(x, w_gate, w_down, h_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """``relu(x Wg) Wd`` -> fp32 (01_ffn.py:183-185)."""
+    h = torch.relu(torch.matmul(x.float(), w_gate.float()))
     if h_dtype is not None:
         h = h.to(h_dtype).float()
     return torch.matmul(h, w_down.float())

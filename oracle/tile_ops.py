@@ -4,7 +4,7 @@ TEST INFRASTRUCTURE ONLY - see ``oracle/__init__.py``.
 
 The reference gives every op a torch meaning in ``python/pypto/debug/torch_codegen.py:954-1128``
 (the table) and ``:489-610`` (the helpers behind load / store / fillpad / assemble).  This module
-restates those meanings for the 38 ops that the paged-attention, FFN, RMSNorm, projection and
+restates those meanings for the 39 ops that the paged-attention, FFN, RMSNorm, projection and
 paged-gather programs use - exactly the names the HIP target's op registry knows
 (``pypto_amd.backend.registered_ops()``; the test holds the two sets equal) - so that
 
@@ -156,6 +156,7 @@ exp = _unary(torch.exp)
 sqrt = _unary(torch.sqrt)
 rsqrt = _unary(torch.rsqrt)          # the tile form may carry a scratch tile, ignored (:1004)
 recip = _unary(torch.reciprocal)
+relu = _unary(torch.relu)           # :1071
 # broadcasting forms: a [rows, cols] tile with a [rows, 1] column or a [1, cols] row
 row_expand_sub = _binary(torch.sub)
 row_expand_mul = _binary(torch.mul)
@@ -215,7 +216,7 @@ TILE_OPS: dict[str, Callable] = {
     "tile.col_expand_mul": col_expand_mul, "tile.create": create, "tile.exp": exp, "tile.fillpad": fillpad,
     "tile.full": full, "tile.get_block_idx": get_block_idx, "tile.get_block_num": get_block_num, "tile.load": load, "tile.matmul": matmul, "tile.matmul_acc": matmul_acc,
     "tile.maximum": maximum, "tile.move": move, "tile.mul": mul, "tile.muls": muls, "tile.neg": neg,
-    "tile.read": read, "tile.recip": recip, "tile.reshape": reshape, "tile.row_expand_div": row_expand_div,
+    "tile.read": read, "tile.recip": recip, "tile.relu": relu, "tile.reshape": reshape, "tile.row_expand_div": row_expand_div,
     "tile.row_expand_mul": row_expand_mul, "tile.row_expand_sub": row_expand_sub, "tile.row_max": row_max,
     "tile.row_sum": row_sum, "tile.rsqrt": rsqrt, "tile.slice": slice_, "tile.sqrt": sqrt, "tile.store": store,
     "tile.sub": sub, "tile.transpose_view": transpose_view,

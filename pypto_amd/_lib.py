@@ -21,7 +21,7 @@ EXPORTS = (
     "pto_hip_malloc", "pto_hip_free", "pto_hip_copy_to", "pto_hip_copy_from", "pto_hip_sync",
     "pto_hip_register", "pto_hip_unregister", "pto_hip_run", "pto_hip_kernel_entry",
     "pto_hip_benchmark", "pto_hip_paged_attention", "pto_hip_paged_gather", "pto_hip_rms_norm",
-    "pto_hip_ffn_swiglu", "pto_hip_set_option", "pto_hip_get_option",
+    "pto_hip_ffn_swiglu", "pto_hip_ffn_activation", "pto_hip_set_option", "pto_hip_get_option",
     "pto_hip_w8a16_matmul", "pto_hip_w8a16_swiglu", "pto_hip_rope_kv_cache_update",
     "pto_hip_rope_kv_cache_update_fp8",
     "pto_hip_decoder_layer_decode", "pto_hip_select_program", "pto_hip_projection",
@@ -121,6 +121,7 @@ def load() -> C.CDLL:
         "pto_hip_paged_gather": [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, C.c_int, vp],
         "pto_hip_rms_norm": [vp, vp, vp, i64, i64, C.c_float, C.c_int, C.c_int, vp],
         "pto_hip_ffn_swiglu": [vp, vp, vp, vp, vp, vp, i64, i64, i64, C.c_float, C.c_int, C.c_int, vp],
+        "pto_hip_ffn_activation": [vp, vp, vp, vp, i64, i64, i64, C.c_int, C.c_int, C.c_int, vp],
         "pto_hip_ffn_swiglu_fp8": [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, C.c_float, C.c_int, C.c_int, vp],
         "pto_hip_quantize_rows_fp8": [vp, vp, vp, i64, i64, C.c_int, vp],
         "pto_hip_rms_norm_quantize_fp8": [vp, vp, vp, vp, i64, i64, C.c_float, C.c_int, vp],

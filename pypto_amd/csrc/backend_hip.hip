@@ -269,11 +269,11 @@ BackendPipeInferFunc Pipe(PipeType p) {
 // dispatch) are one fused launch; what realises an op in one realises it in all of them
 const std::vector<std::string> kAttn = {"paged_attention", "paged_attention_batch", "paged_attention_dynamic",
                                         "paged_attention_spmd", "decoder_layer_decode"};
-const std::vector<std::string> kGemm = {"ffn_swiglu", "ffn_block", "projection", "gate_up_swiglu", "w8a16_matmul",
+const std::vector<std::string> kGemm = {"ffn_swiglu", "ffn_gelu", "ffn_relu", "ffn_block", "projection", "gate_up_swiglu", "w8a16_matmul",
                                         "w8a16_swiglu", "decoder_layer_decode"};
 const std::vector<std::string> kNorm = {"rms_norm", "ffn_block", "decoder_layer_decode"};
 const std::vector<std::string> kAll = {"paged_attention", "paged_attention_batch", "paged_attention_dynamic",
-                                       "paged_attention_spmd", "paged_gather", "rms_norm", "ffn_swiglu", "ffn_block",
+                                       "paged_attention_spmd", "paged_gather", "rms_norm", "ffn_swiglu", "ffn_gelu", "ffn_relu", "ffn_block",
                                        "projection", "gate_up_swiglu", "w8a16_matmul", "w8a16_swiglu",
                                        "rope_kv_cache_update", "rope_kv_cache_update_fp8", "decoder_layer_decode"};
 
@@ -374,6 +374,7 @@ BackendHIP::BackendHIP() : Backend(CreateGfx950SoC()) {
   op("tensor.read", PipeType::S, kAll, "host read of config; context_lens and block_table are read inside the kernel");
   op("tensor.slice", PipeType::S, kAll, "ChipTensor view: start_offset + shape");
   op("tensor.dim", PipeType::S, kAll, "shapes[] of the tensor descriptor");
+  op("tile.relu", PipeType::V, {"ffn_relu"}, "v_max_f32 with 0 on the first product's fp32 values");
   // -- SPMD dispatch (09_paged_attention_spmd.py:127-129: b starts at the block index and steps by the block count)
   op("tile.get_block_idx", PipeType::S, {"paged_attention_spmd"},
      "blockIdx.x of the fused launch; which (sequence, head group, context partition) a workgroup takes is the "
@@ -443,6 +444,17 @@ BackendHIP::BackendHIP() : Backend(CreateGfx950SoC()) {
                   with({"tile.move", "tile.matmul", "tile.muls", "tile.exp", "tile.adds", "tile.recip", "tile.mul",
                         "tensor.create"}),
                   "examples/models/01_ffn.py:36-45,65-77,111-131"},
+      ProgramSpec{"ffn_gelu", {"ffn_gelu"}, {kIn, kIn, kIn, kOut},
+                  {KernelRole{{"matmul_kernel"}, CoreType::CUBE, 1, 2, {kIn, kIn, kOut}},
+                   KernelRole{{"gelu_kernel"}, CoreType::VECTOR, 1, 1, {kIn, kOut}}},
+                  with({"tile.move", "tile.matmul", "tile.muls", "tile.exp", "tile.adds", "tile.recip", "tile.mul",
+                        "tensor.create"}),
+                  "examples/models/01_ffn.py:36-62,90-108"},
+      ProgramSpec{"ffn_relu", {"ffn_relu"}, {kIn, kIn, kIn, kOut},
+                  {KernelRole{{"matmul_kernel"}, CoreType::CUBE, 1, 2, {kIn, kIn, kOut}},
+                   KernelRole{{"relu_kernel"}, CoreType::VECTOR, 1, 1, {kIn, kOut}}},
+                  with({"tile.move", "tile.matmul", "tile.relu", "tensor.create"}),
+                  "examples/models/01_ffn.py:36-45,80-86,133-151"},
       ProgramSpec{"projection", {"matmul_orch", "orchestrator", "matmul"}, {kIn, kIn, kOut},
                   {KernelRole{{"matmul_kernel", "matmul"}, CoreType::CUBE, 1, 1, {kIn, kIn, kOut}}},
                   with({"tile.move", "tile.matmul", "tile.matmul_acc", "tile.assemble", "tensor.create"}),

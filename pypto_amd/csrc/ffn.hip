@@ -46,8 +46,16 @@ int launch_typed(const GemmParams& p, int dtype, int out_dtype, hipStream_t st) 
 
 // ---- fp32 operands: the reference's 64x64 teaching example (01_ffn.py:155-160) ---------------
 // Plain tiled SIMT kernels; small shapes only, not tuned.
+// The single-operand activations of the reference's FFN example (01_ffn.py:51-62 GELU in its
+// x * sigmoid(1.702 x) form, written recip(1 + exp(-1.702 x)); :80-86 ReLU).
+__device__ __forceinline__ float activate(int act, float g) {
+  if (act == PTO_HIP_ACT_GELU) return g * __builtin_amdgcn_rcpf(1.f + __expf(-1.702f * g));
+  if (act == PTO_HIP_ACT_RELU) return fmaxf(g, 0.f);
+  return g;
+}
+
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* a, const float* b0, const float* b1,
-                                                       float* c, int m, int n, int k) {
+                                                       float* c, int m, int n, int k, int act) {
   __shared__ float ta[16][17], tb0[16][17], tb1[16][17];
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
   const int row = blockIdx.y * 16 + ty, col = blockIdx.x * 16 + tx;
@@ -64,7 +72,15 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* a, const flo
     }
     __syncthreads();
   }
-  if (row < m && col < n) c[(int64_t)row * n + col] = b1 ? silu(g) * u : g;
+  if (row < m && col < n) c[(int64_t)row * n + col] = b1 ? silu(g) * u : activate(act, g);
+}
+
+// h = act(gate) rounded to the activation type once, as the SwiGLU product is (mlp.py:60)
+template <typename TO>
+__global__ __launch_bounds__(256) void activation_kernel(const float* __restrict__ gate, TO* __restrict__ h, size_t n,
+                                                         int act) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+    h[i] = (TO)activate(act, gate[i]);
 }
 
 constexpr int64_t kSkinnyMaxTokens = 32;
@@ -205,11 +221,11 @@ extern "C" int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void*
     PTO_CHECK_ARG(out_dtype == PTO_HIP_FP32, "ffn: FP32 operands need an FP32 output");
     dim3 g1((unsigned)((intermediate + 15) / 16), (unsigned)((tokens + 15) / 16));
     hipLaunchKernelGGL(gemm_f32_kernel, g1, dim3(256), 0, st, (const float*)a1, (const float*)w_gate,
-                       (const float*)w_up, (float*)hbuf, (int)tokens, (int)intermediate, (int)hidden);
+                       (const float*)w_up, (float*)hbuf, (int)tokens, (int)intermediate, (int)hidden, 0);
     PTO_CHECK_HIP(hipGetLastError());
     dim3 g2((unsigned)((hidden + 15) / 16), (unsigned)((tokens + 15) / 16));
     hipLaunchKernelGGL(gemm_f32_kernel, g2, dim3(256), 0, st, (const float*)hbuf, (const float*)w_down,
-                       (const float*)nullptr, (float*)out, (int)tokens, (int)hidden, (int)intermediate);
+                       (const float*)nullptr, (float*)out, (int)tokens, (int)hidden, (int)intermediate, 0);
     PTO_CHECK_HIP(hipGetLastError());
     return PTO_HIP_OK;
   }
@@ -246,6 +262,61 @@ extern "C" int pto_hip_ffn_swiglu(const void* x, const float* gamma, const void*
   p2.n = (int)hidden;
   p2.k = (int)intermediate;
   return launch_typed<false>(p2, dtype, out_dtype, st);
+}
+
+// out = act(x Wg) Wd with act = GELU (x * sigmoid(1.702 x)) or ReLU: the other two FFNs of the
+// reference's example (01_ffn.py:90-108 ffn_gelu, :133-151 ffn_relu; expected values :165-167,
+// :183-185).  fp32 operands run the small SIMT kernels with the activation in the first product's
+// epilogue; 16-bit operands run gate = x Wg in fp32 through the projection path, one pass that applies
+// the activation and rounds h to the operand type, and the down projection.
+extern "C" int pto_hip_ffn_activation(const void* x, const void* w_gate, const void* w_down, void* out,
+                                      int64_t tokens, int64_t hidden, int64_t intermediate, int activation, int dtype,
+                                      int out_dtype, void* stream) {
+  PTO_DISPATCH_LOCK();
+  using namespace pto_hip;
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  PTO_CHECK_ARG(activation == PTO_HIP_ACT_GELU || activation == PTO_HIP_ACT_RELU,
+                "ffn_activation: activation %d is neither PTO_HIP_ACT_GELU nor PTO_HIP_ACT_RELU", activation);
+  PTO_CHECK_ARG(tokens >= 0 && hidden > 0 && intermediate > 0 && tokens < (1 << 30) && hidden < (1 << 30) &&
+                    intermediate < (1 << 30),
+                "ffn_activation: bad shape T=%lld H=%lld I=%lld", (long long)tokens, (long long)hidden,
+                (long long)intermediate);
+  if (tokens == 0) return PTO_HIP_OK;
+  PTO_CHECK_ARG(x && w_gate && w_down && out, "ffn_activation: null tensor pointer");
+  PTO_CHECK_ARG(dtype == PTO_HIP_BF16 || dtype == PTO_HIP_FP16 || dtype == PTO_HIP_FP32,
+                "ffn_activation: dtype %s not in {BF16, FP16, FP32}", dtype_name(dtype));
+  hipStream_t st = (hipStream_t)stream;
+  const size_t n_h = (size_t)tokens * intermediate;
+  if (dtype == PTO_HIP_FP32) {
+    PTO_CHECK_ARG(out_dtype == PTO_HIP_FP32, "ffn_activation: FP32 operands need an FP32 output");
+    void* hbuf = nullptr;
+    int rc = workspace(n_h * sizeof(float), &hbuf);
+    if (rc) return rc;
+    dim3 g1((unsigned)((intermediate + 15) / 16), (unsigned)((tokens + 15) / 16));
+    hipLaunchKernelGGL(gemm_f32_kernel, g1, dim3(256), 0, st, (const float*)x, (const float*)w_gate,
+                       (const float*)nullptr, (float*)hbuf, (int)tokens, (int)intermediate, (int)hidden, activation);
+    PTO_CHECK_HIP(hipGetLastError());
+    dim3 g2((unsigned)((hidden + 15) / 16), (unsigned)((tokens + 15) / 16));
+    hipLaunchKernelGGL(gemm_f32_kernel, g2, dim3(256), 0, st, (const float*)hbuf, (const float*)w_down,
+                       (const float*)nullptr, (float*)out, (int)tokens, (int)hidden, (int)intermediate, 0);
+    PTO_CHECK_HIP(hipGetLastError());
+    return PTO_HIP_OK;
+  }
+  const size_t gate_bytes = (n_h * sizeof(float) + 255) / 256 * 256;
+  void* ws = nullptr;
+  int rc = workspace(gate_bytes + n_h * 2, &ws);
+  if (rc) return rc;
+  float* gate = reinterpret_cast<float*>(ws);
+  void* h = reinterpret_cast<char*>(ws) + gate_bytes;
+  rc = pto_hip_projection(x, w_gate, nullptr, gate, tokens, hidden, intermediate, dtype, 0, PTO_HIP_FP32, stream);
+  if (rc) return rc;
+  const unsigned blocks = (unsigned)std::min<size_t>((n_h + 255) / 256, (size_t)ctx().num_cu * 16);
+  if (dtype == PTO_HIP_BF16)
+    hipLaunchKernelGGL((activation_kernel<__bf16>), dim3(blocks), dim3(256), 0, st, gate, (__bf16*)h, n_h, activation);
+  else
+    hipLaunchKernelGGL((activation_kernel<_Float16>), dim3(blocks), dim3(256), 0, st, gate, (_Float16*)h, n_h, activation);
+  PTO_CHECK_HIP(hipGetLastError());
+  return pto_hip_projection(h, w_down, nullptr, out, tokens, intermediate, hidden, dtype, 0, out_dtype, stream);
 }
 
 // out[M, N] = x[M, K] @ w[K, N] (+ residual[M, N]): the reference's projection kernels

@@ -99,6 +99,8 @@ enum ProgramKind {
   kPagedAttentionBatch,
   kPagedAttentionDynamic,
   kPagedAttentionSpmd,
+  kFfnGelu,
+  kFfnRelu,
   kNumPrograms
 };
 
@@ -106,7 +108,7 @@ const char* const kProgramNames[kNumPrograms] = {
     "paged_attention", "paged_gather",  "rms_norm",           "ffn_swiglu",          "ffn_block",
     "w8a16_matmul",    "w8a16_swiglu",  "rope_kv_cache_update", "rope_kv_cache_update_fp8",
     "decoder_layer_decode", "projection", "gate_up_swiglu", "ffn_block_fp8", "llama_mini",
-    "paged_attention_batch", "paged_attention_dynamic", "paged_attention_spmd"};
+    "paged_attention_batch", "paged_attention_dynamic", "paged_attention_spmd", "ffn_gelu", "ffn_relu"};
 
 std::mutex g_mu;
 std::vector<int> g_callables;  // callable id -> ProgramKind, -1 once unregistered
@@ -414,6 +416,25 @@ int run_ffn(const PtoHipChipTensor* t, int nt, const uint64_t* s, int ns, hipStr
   }
   return pto_hip_ffn_swiglu(tptr(x), gamma, tptr(wg), tptr(wu), tptr(wd), tptr_mut(out), tokens,
                             hidden, inter, eps, (int)x.dtype, (int)out.dtype, stream);
+}
+
+// hidden_states, gate_proj_weight, down_proj_weight, output (01_ffn.py:90-108, :133-151)
+int run_ffn_activation(const PtoHipChipTensor* t, int nt, const uint64_t*, int ns, hipStream_t stream, int act) {
+  const char* prog = act == PTO_HIP_ACT_GELU ? "ffn_gelu" : "ffn_relu";
+  PTO_CHECK_ARG(nt == 4 && ns == 0, "%s: expected 4 tensors + 0 scalars, got %d + %d", prog, nt, ns);
+  for (int i = 0; i < nt; ++i) {
+    int rc = check_tensor(prog, "operand", t[i], 2, 2);
+    if (rc) return rc;
+  }
+  const PtoHipChipTensor &x = t[0], &wg = t[1], &wd = t[2], &out = t[3];
+  const int64_t tokens = x.shapes[0], hidden = x.shapes[1], inter = wg.shapes[1];
+  PTO_CHECK_ARG(wg.shapes[0] == hidden && wd.shapes[0] == inter && wd.shapes[1] == hidden,
+                "%s: weight shapes must be gate [H,I] and down [I,H] with H=%lld", prog, (long long)hidden);
+  PTO_CHECK_ARG(wg.dtype == x.dtype && wd.dtype == x.dtype, "%s: weights must have the dtype of x (%s)", prog,
+                dtype_name(x.dtype));
+  PTO_CHECK_ARG(out.shapes[0] == tokens && out.shapes[1] == hidden, "%s: out must be [T,H]", prog);
+  return pto_hip_ffn_activation(tptr(x), tptr(wg), tptr(wd), tptr_mut(out), tokens, hidden, inter, act, (int)x.dtype,
+                                (int)out.dtype, stream);
 }
 
 // x, gamma, w_gate8, w_gate_scale, w_up8, w_up_scale, w_down8, w_down_scale, out + eps
@@ -749,6 +770,8 @@ int dispatch(int kind, const PtoHipChipTensor* t, int nt, const uint64_t* s, int
     case kFfnSwiglu: return run_ffn(t, nt, s, ns, stream, false);
     case kFfnBlock: return run_ffn(t, nt, s, ns, stream, true);
     case kFfnBlockFp8: return run_ffn_fp8(t, nt, s, ns, stream);
+    case kFfnGelu: return run_ffn_activation(t, nt, s, ns, stream, PTO_HIP_ACT_GELU);
+    case kFfnRelu: return run_ffn_activation(t, nt, s, ns, stream, PTO_HIP_ACT_RELU);
     case kLlamaMini: return run_llama_mini(t, nt, s, ns, stream);
     case kW8a16Matmul: return run_w8a16_matmul(t, nt, s, ns, stream);
     case kProjection: return run_projection(t, nt, s, ns, stream);

@@ -76,6 +76,9 @@ paged_gather = HipProgram("paged_gather", (IN, IN, IN, OUT), scalars=("block_siz
 rms_norm = HipProgram("rms_norm", (IN, IN, OUT), scalars=("eps",))
 rms_norm_unweighted = HipProgram("rms_norm", (IN, OUT), scalars=("eps",))  # 08_llama_mini.py:93-118
 ffn_swiglu = HipProgram("ffn_swiglu", (IN, IN, IN, IN, OUT))
+# the example's two other FFNs: act(x Wg) Wd with GELU (x * sigmoid(1.702 x)) or ReLU (01_ffn.py:90-108, :133-151)
+ffn_gelu = HipProgram("ffn_gelu", (IN, IN, IN, OUT))
+ffn_relu = HipProgram("ffn_relu", (IN, IN, IN, OUT))
 ffn_block = HipProgram("ffn_block", (IN, IN, IN, IN, IN, OUT), scalars=("eps",))
 # the block on e4m3 operands: x, gamma, then (codes [out, in], scale [out]) for gate, up and down
 ffn_block_fp8 = HipProgram("ffn_block_fp8", (IN,) * 8 + (OUT,), scalars=("eps",))
@@ -113,7 +116,7 @@ decoder_layer_decode_w16_fp8kv = HipProgram(
     scalars=("num_heads", "kv_head_num", "head_dim", "block_size", "eps"))
 
 PROGRAMS = {p.name: p for p in (paged_attention, paged_attention_batch, paged_attention_dynamic, paged_attention_spmd,
-                                paged_gather, rms_norm, ffn_swiglu, ffn_block, ffn_block_fp8, llama_mini,
+                                paged_gather, rms_norm, ffn_swiglu, ffn_gelu, ffn_relu, ffn_block, ffn_block_fp8, llama_mini,
                                 projection, gate_up_swiglu,
                                 w8a16_matmul,
                                 w8a16_swiglu, rope_kv_cache_update, rope_kv_cache_update_fp8,

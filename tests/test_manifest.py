@@ -79,10 +79,10 @@ def test_matmul_only_manifest_is_a_projection(tmp_path):
 
 
 def test_unknown_kernel_sets_are_rejected(tmp_path):
-    # gelu FFN of the same example file: no fused program here
-    kernels = [("matmul_kernel", "aic", None), ("gelu_kernel", "aiv", None)]
-    with pytest.raises(ValueError, match="no fused HIP program.*gelu_kernel:aiv"):
-        mf.compile_and_assemble(_write(tmp_path, "ffn_gelu", None, kernels))
+    # an FFN with an activation kernel this target has no program for
+    kernels = [("matmul_kernel", "aic", None), ("tanh_kernel", "aiv", None)]
+    with pytest.raises(ValueError, match="no fused HIP program.*tanh_kernel:aiv"):
+        mf.compile_and_assemble(_write(tmp_path, "ffn_tanh", None, kernels))
     # attention kernels outlined for the wrong core type
     bad = [(n, "aiv", s) for n, _, s in ATTN_KERNELS]
     with pytest.raises(ValueError, match="no fused HIP program"):
@@ -179,3 +179,14 @@ def test_same_orchestration_name_different_kernels_are_told_apart(tmp_path):
     assert mf.compile_and_assemble(_write(tmp_path, "paged_attention", sig6, k6))[0].name == "paged_attention_dynamic"
     with pytest.raises(ValueError, match="no fused HIP program"):   # 04's kernels under 06's six tensors
         mf.compile_and_assemble(_write(tmp_path, "paged_attention", sig6, ATTN_KERNELS))
+
+
+@pytest.mark.parametrize("name,act", [("ffn_gelu", "gelu_kernel"), ("ffn_relu", "relu_kernel")])
+def test_the_examples_other_two_ffns(tmp_path, name, act):
+    """01_ffn.py:90-108 / :133-151: matmul_kernel (used twice, listed once or twice) + one activation kernel."""
+    kernels = [("matmul_kernel", "aic", ["IN", "IN", "OUT"]), (act, "aiv", ["IN", "OUT"])]
+    prog, _, _ = mf.compile_and_assemble(_write(tmp_path, name, ["IN"] * 3 + ["OUT"], kernels))
+    assert prog.name == name and prog.signature == (IN, IN, IN, OUT)
+    with pytest.raises(ValueError, match="no fused HIP program"):   # the activation kernel of the other program
+        other = "relu_kernel" if act == "gelu_kernel" else "gelu_kernel"
+        mf.compile_and_assemble(_write(tmp_path, name, None, [kernels[0], (other, "aiv", None)]))

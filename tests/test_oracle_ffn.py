@@ -276,3 +276,27 @@ def test_llama_mini_forward_closed_forms():
     probe[7] = torch.zeros(64, 64)
     probe[10] = torch.zeros(64, 64)
     assert torch.allclose(oracle.llama_mini_forward(*probe), norm(hidden) @ wlm, rtol=1e-6, atol=1e-7)
+
+
+# ---- the example's one-operand activations (01_ffn.py: ffn_gelu, ffn_relu) ----------------------------
+def test_gelu_and_relu_ffn_forms():
+    torch.manual_seed(0)   # the seed and shapes of tests/st/examples/02_intermediate/test_ffn_activations.py:30-34
+    x, wg, wd = (torch.randn(64, 64) for _ in range(3))
+    g = x.double() @ wg.double()
+    # the kernel's device form (01_ffn.py:55-60) in fp64
+    kernel_form = (g * (1.0 / (1.0 + torch.exp(-1.702 * g)))) @ wd.double()
+    assert torch.allclose(oracle.ffn_gelu(x, wg, wd).double(), kernel_form, rtol=1e-4, atol=1e-3)
+    # x * sigmoid(1.702 x) is the "quick" approximation of the erf GELU: within 0.021 of it everywhere
+    t = torch.linspace(-8, 8, 4001, dtype=torch.float64)
+    assert (t * torch.sigmoid(1.702 * t) - torch.nn.functional.gelu(t)).abs().max() < 0.021
+    assert torch.allclose(oracle.ffn_relu(x, wg, wd).double(), g.clamp(min=0) @ wd.double(), rtol=1e-4, atol=1e-3)
+    # identities a wrong sign or a dropped factor breaks:
+    #   relu(g) - relu(-g) = g   and   g*sigmoid(cg) - (-g)*sigmoid(-cg) = g   =>   F(x) - F(-x) = (x Wg) Wd
+    lin = (g @ wd.double()).float()
+    for f in (oracle.ffn_relu, oracle.ffn_gelu):
+        assert torch.allclose(f(x, wg, wd) - f(-x, wg, wd), lin, rtol=1e-4, atol=2e-3)
+    # zero input -> zero output; h rounding is applied when asked for
+    assert not oracle.ffn_gelu(torch.zeros(4, 64), wg, wd).any()
+    xb, wgb, wdb = x.bfloat16(), wg.bfloat16(), wd.bfloat16()
+    full, rounded = oracle.ffn_gelu(xb, wgb, wdb), oracle.ffn_gelu(xb, wgb, wdb, h_dtype=torch.bfloat16)
+    assert not torch.equal(full, rounded) and torch.allclose(full, rounded, rtol=2e-2, atol=0.5)
