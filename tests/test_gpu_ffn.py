@@ -25,6 +25,21 @@ def test_rms_norm(worker, dtype, rows, hidden):
     validate_golden({"out": out.float()}, {"out": ref.float()}, rtol=tol, atol=tol)
 
 
+def test_rms_norm_reference_example_fp32(worker):
+    """The reference's own case (tests/st/examples/02_intermediate/test_rms_norm.py:23-41): 32x64 fp32,
+    seed 0, gamma ~ N(0,1) of shape [1, 64], eps 1e-5, sqrt then divide, rtol = atol = 1e-5."""
+    torch.manual_seed(0)
+    x = torch.randn(32, 64, dtype=torch.float32)
+    gamma = torch.randn(1, 64, dtype=torch.float32)
+    output = torch.zeros_like(x)
+    with worker.register(rms_norm) as h:
+        h(x, gamma, output, 1e-5)
+    rms = torch.sqrt((x ** 2).sum(dim=-1, keepdim=True) / 64 + 1e-5)
+    expected = (x / rms) * gamma
+    assert torch.allclose(output, expected, rtol=1e-5, atol=1e-5)
+    assert torch.allclose(oracle.rms_norm(x, gamma, 1e-5), expected, rtol=1e-5, atol=1e-5)
+
+
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,hidden", [(64, 4096), (3, 8192), (5, 1000), (2, 8200)])
 def test_rms_norm_of_fp32_rows_to_16_bit(worker, out_dtype, rows, hidden):
