@@ -302,9 +302,11 @@ extern "C" int pto_hip_ffn_activation(const void* x, const void* w_gate, const v
     PTO_CHECK_HIP(hipGetLastError());
     return PTO_HIP_OK;
   }
+  // The intermediates outlive two projection calls, and a projection of up to 32 rows keeps its split
+  // partial sums in workspace(): they live in the arena those calls leave alone.
   const size_t gate_bytes = (n_h * sizeof(float) + 255) / 256 * 256;
   void* ws = nullptr;
-  int rc = workspace(gate_bytes + n_h * 2, &ws);
+  int rc = layer_workspace(gate_bytes + n_h * 2, &ws);
   if (rc) return rc;
   float* gate = reinterpret_cast<float*>(ws);
   void* h = reinterpret_cast<char*>(ws) + gate_bytes;

@@ -45,6 +45,7 @@ def test_fp32_ragged_shapes(worker, program, golden, t, h, i):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("t,h,i", [(128, 512, 1024),      # the tiny FFN configuration's shape
                                    (16, 1024, 2816),      # decode-size rows: the weight-streaming projections
+                                   (32, 4096, 256),       # ... whose split partial sums outsize the intermediates
                                    (300, 512, 1536)])     # ragged tile edges
 def test_16bit_operands(worker, program, golden, dtype, t, h, i):
     g = torch.Generator().manual_seed(i)
