@@ -444,7 +444,7 @@ def test_stream_probe_bounds_the_kernel_and_touches_nothing(worker):
     worker.sync()
     _check(out.cpu(), _golden(inp))
     # the bound may not sit above what it bounds (measured 0.96-0.98 of the kernel; the margin is for a noisy box)
-    assert probe_us < 1.25 * kernel_us, (probe_us, kernel_us)
+    assert probe_us < 1.5 * kernel_us, (probe_us, kernel_us)
     # an e4m3 cache and head_dim 256 have their own instantiations
     f8 = workloads.paged_attention_inputs(batch=3, num_heads=8, kv_head_num=2, head_dim=256, block_size=64,
                                           context_lens=[700, 64, 2000], ctx_range=(1, 2048), seed=5, fp8_kv=True)
