@@ -49,6 +49,51 @@ struct Params {
 // 64 of them per lane while the matrix pipes idle.
 __device__ __forceinline__ float silu(float g) { return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)); }
 
+// 4 x 4 transpose across the four lanes of a quad.  In: v[k] = the value of row R + k at this lane's
+// column.  Out: v[k] = the value of row R + (lane % 4) at column 4 * (this lane's column / 4) + k.
+// An MFMA accumulator holds four consecutive rows of ONE column per lane; after the transpose a lane
+// holds four consecutive columns of one row, which is a single 8- or 16-byte store instead of four
+// 2- or 4-byte ones - the epilogue is bound by the number of store instructions, not by bytes.
+__device__ __forceinline__ float quad_xor1(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));  // quad_perm 1,0,3,2
+}
+__device__ __forceinline__ float quad_xor2(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));  // quad_perm 2,3,0,1
+}
+__device__ __forceinline__ void quad_transpose(float (&v)[4], int lane) {
+  const bool b0 = (lane & 1) != 0, b1 = (lane & 2) != 0;
+  const float r01 = quad_xor1(b0 ? v[0] : v[1]), r23 = quad_xor1(b0 ? v[2] : v[3]);
+  if (b0) {
+    v[0] = r01;
+    v[2] = r23;
+  } else {
+    v[1] = r01;
+    v[3] = r23;
+  }
+  const float r02 = quad_xor2(b1 ? v[0] : v[2]), r13 = quad_xor2(b1 ? v[1] : v[3]);
+  if (b1) {
+    v[0] = r02;
+    v[1] = r13;
+  } else {
+    v[2] = r02;
+    v[3] = r13;
+  }
+}
+
+// four consecutive outputs of one row as one store
+template <typename OutT>
+__device__ __forceinline__ void store4(OutT* dst, const float (&v)[4]) {
+  if constexpr (sizeof(OutT) == 4) {
+    *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
+  } else {
+    const OutT a = (OutT)v[0], b = (OutT)v[1], c = (OutT)v[2], d = (OutT)v[3];
+    uint2 w;
+    w.x = (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+    w.y = (uint32_t)__builtin_bit_cast(uint16_t, c) | ((uint32_t)__builtin_bit_cast(uint16_t, d) << 16);
+    *reinterpret_cast<uint2*>(dst) = w;
+  }
+}
+
 __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
   const int x = pid % kXcds, local = pid / kXcds;
   const int full = nwg / kXcds, rem = nwg % kXcds;
@@ -256,6 +301,36 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
       sr[i][q * 4 + 2] = v.z;
       sr[i][q * 4 + 3] = v.w;
     }
+  if (p.n % 4 == 0 && p.ldc % 4 == 0) {
+    // rows of four: quad-transposed so that every lane writes four consecutive columns of one row
+    const int my_row = row_base + (lane & 3);            // + i * 32 + q * 8
+    const int col_shift = ((lane & 31) & ~3) - (lane & 31);  // this lane's first column after the transpose
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = my_row + i * 32 + q * 8;
+        const bool row_ok = row < p.m;
+#pragma unroll
+        for (int jn = 0; jn < (DUAL ? NT / 2 : NT); ++jn) {
+          float v[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const int r = q * 4 + k;
+            if constexpr (DUAL) {
+              const float g = acc[i][jn][r] * sr[i][r] * sc[jn], u = acc[i][jn + NT / 2][r] * sr[i][r] * sc[jn + NT / 2];
+              v[k] = silu(g) * u;
+            } else {
+              v[k] = acc[i][jn][r] * sr[i][r] * sc[jn];
+            }
+          }
+          quad_transpose(v, lane);
+          const int c0 = col[jn] + col_shift;
+          if (row_ok && c0 < p.n) store4<OutT>(c + (int64_t)row * p.ldc + c0, v);
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
