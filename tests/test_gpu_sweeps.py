@@ -248,3 +248,45 @@ def test_decoder_layer_and_gather_sweep(worker):
         gout = gout.cpu()
         assert torch.equal(gout[:idx.numel()], oracle.paged_gather(src, idx, table, bs, size, off))
         assert (gout[idx.numel():] == 7).all()
+
+
+def test_attention_sweep_off_the_mfma_tiles(worker):
+    """Head sizes other than 128 / 256 and block sizes off the 16-token grid (the one-wavefront-per-head
+    kernel), through the plain signature and, every third case, the SPMD one with a random block bound."""
+    from pypto_amd.runtime import paged_attention_spmd
+    rng = random.Random(77)
+    for case in range(45):
+        d = rng.choice([1, 2, 8, 16, 24, 32, 48, 64, 72, 96, 100, 128, 160, 200, 256])
+        bs = rng.choice([1, 3, 7, 8, 17, 24, 31, 100, 200] if d in (128, 256) else [1, 3, 7, 8, 16, 17, 24, 32, 64, 100, 128])
+        hkv = rng.choice([1, 2, 3, 4])
+        group = rng.choice([1, 2, 4, 5, 8, 16])
+        batch = rng.randint(1, 5)
+        fp8 = rng.random() < 0.3
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        ctxs = [rng.choice([0, 1, max(bs - 1, 0), bs, bs + 1, rng.randint(1, 6 * bs)]) for _ in range(batch)]
+        inp = workloads.paged_attention_inputs(batch=batch, num_heads=hkv * group, kv_head_num=hkv, head_dim=d,
+                                               block_size=bs, context_lens=ctxs, ctx_range=(1, max(max(ctxs), 1)),
+                                               dtype=dtype, fp8_kv=fp8, scale=rng.choice([1.0, 0.5, 0.1]), seed=case)
+        spmd = case % 3 == 2 and not fp8
+        cap = int(inp.config[5])
+        active = rng.randint(0, cap) if spmd else None
+        print(f"off-tile attention case {case}: D{d} bs{bs} hkv{hkv} group{group} ctx{ctxs} fp8={fp8} {dtype} "
+              f"active={active}", flush=True)
+        if spmd:
+            args = inp.args_spmd(active)
+            ref = oracle.paged_attention_spmd_golden(*args[:6], args[7])
+            dev = [t.cuda() if i not in (5, 7) else t for i, t in enumerate(args)]
+            dev[6].fill_(float("nan"))
+            with worker.register(paged_attention_spmd) as h:
+                h(*dev)
+            out = dev[6]
+        else:
+            ref = oracle.paged_attention_golden(inp.query, inp.key_cache, inp.value_cache, inp.block_table,
+                                                inp.context_lens, inp.config, inp.k_scale, inp.v_scale)
+            dev = [t.cuda() if i != 6 else t for i, t in enumerate(inp.args())]
+            dev[5].fill_(float("nan"))
+            with worker.register(paged_attention) as h:
+                h(*dev)
+            out = dev[5]
+        worker.sync()
+        _close(f"off-tile attention case {case}", out.cpu(), ref, 2e-2, 1e-2)
