@@ -427,6 +427,19 @@ def main() -> int:
             st.device_wall_us)
         del dq
         torch.cuda.empty_cache()
+        # the reference's own decode model (examples/models/qwen3_jit/config.py:16-29) in its own cache layout:
+        # one block of MAX_SEQ tokens per sequence
+        dj = workloads.decoder_layer_inputs(batch=16, hidden=8192, num_heads=64, kv_head_num=8, head_dim=128,
+                                            intermediate=25600, context=4096, block_size=4096, theta=1e6, device="cuda",
+                                            int8_weights=False, weight_std=None)
+        with worker.register(decoder_layer_decode_w16) as dh:
+            benchmark(dh, [dj.args()], rounds=5, warmup=0)
+            st = benchmark(dh, [dj.args()], rounds=20, warmup=0)
+        more["decoder_layer_qwen3_jit"] = _hbm_block(
+            "the reference's qwen3_jit decode model, one layer step, bf16 weights: H8192 Hq64 Hkv8 D128 I25600 B16 "
+            "ctx4096, one 4096-token block per sequence", dj.algorithmic_bytes(), st.device_wall_us)
+        del dj
+        torch.cuda.empty_cache()
         fd = [workloads.ffn_inputs(tokens=16, hidden=4096, intermediate=11008, seed=s, device="cuda") for s in (0, 1)]
         with worker.register(ffn_block) as fh:
             fdargs = [(f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.out, f.eps) for f in fd]

@@ -1106,7 +1106,16 @@ int plan_launch(const int64_t* config, int q_dtype, int kv_dtype, bool have_scal
   // than occupancy), but never more than 2048 tokens per partition so long contexts still
   // bring several wavefronts per SIMD.  Each partition is a whole number of 32-token chunks (and
   // of KV blocks when blocks are at least that big).
-  const int64_t align = bs >= kChunk ? bs : kChunk;
+  // Blocks of more than 512 tokens are cut inside (the chunk loop finds every chunk's block and offset on its
+  // own): the reference's decode model keeps ONE block of MAX_SEQ tokens per sequence
+  // (examples/models/qwen3_jit/kernels/attention.py:64-80), and whole-block partitions would leave
+  // one wavefront per (sequence, KV head).
+  int64_t align = bs >= kChunk ? bs : kChunk;
+  if (align > 512) {
+    int64_t pow2 = 512;
+    while (pow2 >= kChunk && bs % pow2 != 0) pow2 /= 2;
+    if (pow2 >= kChunk) align = pow2;
+  }
   int64_t tpp = cx.attn_tokens_per_partition;
   if (tpp <= 0) {
     const int64_t units = batch * hkv * p.gtiles;

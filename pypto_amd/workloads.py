@@ -377,9 +377,11 @@ class DecoderLayerInputs:
 def decoder_layer_inputs(*, batch=32, hidden=4096, num_heads=32, kv_head_num=8, head_dim=128,
                          intermediate=14336, context=4096, block_size=128, theta=5e5,
                          dtype=torch.bfloat16, seed=0, device="cpu", context_lens=None,
-                         int8_weights=True) -> DecoderLayerInputs:
-    """One decode step of a LLaMA-style layer: weights from N(0,0.02) as int8 codes + scales or, with
-    ``int8_weights=False``, in the activation dtype; 16-bit activations and KV."""
+                         int8_weights=True, weight_std: float | None = 0.02) -> DecoderLayerInputs:
+    """One decode step of a LLaMA-style layer: weights from N(0, weight_std) as int8 codes + scales or, with
+    ``int8_weights=False``, in the activation dtype; 16-bit activations and KV.  ``weight_std=None`` scales
+    every weight by 1/sqrt(its input width), the reference system test's way of keeping activations O(1) at any
+    model size (tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:296-326)."""
     dev = torch.device(device)
     g = torch.Generator(device=dev).manual_seed(seed)
 
@@ -403,12 +405,13 @@ def decoder_layer_inputs(*, batch=32, hidden=4096, num_heads=32, kv_head_num=8, 
     rows = total * kv_head_num * block_size
     qkv_n = (num_heads + 2 * kv_head_num) * head_dim
     pack = quantize_w8 if int8_weights else (lambda w: (w.to(dtype), None))
+    std = (lambda fan_in: weight_std) if weight_std is not None else (lambda fan_in: fan_in ** -0.5)
     weights = {
-        "qkv": pack(rn((hidden, qkv_n), 0.02)),
-        "o": pack(rn((num_heads * head_dim, hidden), 0.02)),
-        "gate": pack(rn((hidden, intermediate), 0.02)),
-        "up": pack(rn((hidden, intermediate), 0.02)),
-        "down": pack(rn((intermediate, hidden), 0.02)),
+        "qkv": pack(rn((hidden, qkv_n), std(hidden))),
+        "o": pack(rn((num_heads * head_dim, hidden), std(num_heads * head_dim))),
+        "gate": pack(rn((hidden, intermediate), std(hidden))),
+        "up": pack(rn((hidden, intermediate), std(hidden))),
+        "down": pack(rn((intermediate, hidden), std(intermediate))),
     }
     cos, sin = rope_tables(max_blocks * block_size, head_dim, theta, device=dev)
     return DecoderLayerInputs(

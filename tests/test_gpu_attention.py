@@ -458,3 +458,22 @@ def test_stream_probe_bounds_the_kernel_and_touches_nothing(worker):
         worker.set_option("attn_variant", -1)
     with pytest.raises(ValueError, match="rounds"):
         attention_stream_probe(worker, kc, vc, table, lens, cfg, rounds=0)
+
+
+@pytest.mark.parametrize("bs,ctxs,fp8", [
+    (4096, [4096, 1, 2500, 4095, 33], False),     # the reference decode model's layout: one block of MAX_SEQ per sequence
+    (4096, [4096, 700], True),
+    (2048, [5000, 2048, 2049, 100], False),
+    (1024, [3000, 1024, 1], True),
+    (528, [1500, 528, 529], False),               # 16 x 33 tokens: no power-of-two cut of 32 or more divides it
+    (1536, [4000, 1537], False),                  # cut at 512
+])
+def test_blocks_longer_than_a_partition(worker, bs, ctxs, fp8):
+    """Blocks of more than 512 tokens are cut inside by the context partitions (otherwise a sequence kept in
+    one MAX_SEQ-long block, as examples/models/qwen3_jit/kernels/attention.py:64-80 keeps it, would be one
+    wavefront per KV head).  Every launch form, against the golden."""
+    inp = workloads.paged_attention_inputs(batch=len(ctxs), num_heads=16, kv_head_num=2, head_dim=128, block_size=bs,
+                                           context_lens=ctxs, ctx_range=(1, max(ctxs)), fp8_kv=fp8, seed=bs)
+    ref = _golden(inp)
+    for tpp in (0, 512, 1024, -4):
+        _check(_run(worker, inp, tpp), ref)

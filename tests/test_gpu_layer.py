@@ -419,6 +419,60 @@ def test_decoder_layer_full_configuration(worker):
     assert torch.equal(torch.nonzero(k_changed).flatten().sort().values, want_rows.sort().values)
 
 
+def test_decoder_layer_reference_decode_model_shape(worker):
+    """The reference's own decode model at its full size (examples/models/qwen3_jit/config.py:16-29: batch 16,
+    hidden 8192, 64 query / 8 KV heads of 128, intermediate 25600, MAX_SEQ 4096, bf16 weights - 1.56 GB of them)
+    with its cache layout: one block of MAX_SEQ tokens per sequence, block_table[b] = b, so the row of
+    (sequence, KV head, position) is (b * Hkv + h) * MAX_SEQ + pos as in kernels/attention.py:64-80.  Ragged
+    sequence lengths; weights scaled by 1/sqrt(fan-in) as the reference's system test scales them, so that
+    activations stay O(1) at this width; four whole sequences against the oracle, the K/V rows they appended,
+    nothing else touched."""
+    g = torch.Generator().manual_seed(3)
+    ctxs = torch.randint(1, 4097, (16,), generator=g).tolist()
+    ctxs[0], ctxs[15] = 4096, 1
+    inp = workloads.decoder_layer_inputs(batch=16, hidden=8192, num_heads=64, kv_head_num=8, head_dim=128,
+                                         intermediate=25600, block_size=4096, context_lens=ctxs, theta=1e6, seed=2,
+                                         device="cuda", int8_weights=False, weight_std=None)
+    batch, hkv, d, bs, mb = 16, 8, 128, 4096, inp.max_num_blocks_per_req
+    assert mb == 1 and inp.weights["down"][0].shape == (25600, 8192) and inp.weights["down"][1] is None
+    seqs = [0, 6, 11, 15]
+    table = inp.block_table.reshape(batch, mb)
+
+    def sub_pool(cache):
+        blocks = table[seqs].reshape(-1).long()
+        rows = (blocks[:, None] * (hkv * bs) + torch.arange(hkv * bs, device="cuda")[None, :]).reshape(-1)
+        return cache[rows].cpu()
+
+    k0, v0 = sub_pool(inp.key_cache), sub_pool(inp.value_cache)
+    kc_before, vc_before = inp.key_cache.clone(), inp.value_cache.clone()
+    with worker.register(decoder_layer_decode_w16) as h:
+        h(*inp.args())
+    worker.sync()
+    w = {name: c.cpu() for name, (c, _) in inp.weights.items()}
+    ref_out, ref_k, ref_v = oracle.decoder_layer_decode(
+        inp.hidden[seqs].cpu(), inp.seq_lens[seqs].cpu(), torch.arange(len(seqs) * mb, dtype=torch.int32), k0, v0,
+        inp.rope_cos.cpu(), inp.rope_sin.cpu(), inp.gamma_in.cpu(), inp.gamma_post.cpu(),
+        w["qkv"], None, w["o"], None, w["gate"], None, w["up"], None, w["down"], None,
+        num_heads=inp.num_heads, kv_head_num=hkv, head_dim=d, block_size=bs, max_num_blocks_per_req=mb, eps=inp.eps)
+    got = inp.out[seqs].float().cpu()
+    print("max_abs_err", (got - ref_out.float()).abs().max().item(), "ref_max", ref_out.float().abs().max().item(),
+          flush=True)
+    assert torch.isfinite(inp.out.float()).all()
+    validate_golden({"out": got}, {"out": ref_out.float()}, rtol=2e-2, atol=2e-2)
+    k1, v1 = sub_pool(inp.key_cache), sub_pool(inp.value_cache)
+    assert torch.allclose(k1.float(), ref_k.float(), atol=2e-2, rtol=2e-2)
+    assert torch.allclose(v1.float(), ref_v.float(), atol=2e-2, rtol=2e-2)
+    assert torch.equal((k1 != k0).any(dim=1), (ref_k != k0).any(dim=1))
+    # over the whole cache: one row per (sequence, KV head), at position seq_len - 1 of the sequence's block
+    k_changed = (inp.key_cache != kc_before).any(dim=1)
+    v_changed = (inp.value_cache != vc_before).any(dim=1)
+    pos = (inp.seq_lens.long() - 1)
+    want_rows = ((table[:, 0].long()[:, None] * hkv + torch.arange(hkv, device="cuda")[None, :]) * bs
+                 + pos[:, None]).reshape(-1)
+    assert torch.equal(torch.nonzero(k_changed).flatten().sort().values, want_rows.sort().values)
+    assert torch.equal(torch.nonzero(v_changed).flatten().sort().values, want_rows.sort().values)
+
+
 @pytest.mark.parametrize("batch,gemm_rows", [(45, 0), (100, 0), (100, 33), (300, 33)])
 def test_decoder_layer_decode_int8_weights_many_sequences(worker, batch, gemm_rows):
     """More than 32 sequences with int8 weights: as groups of 32 through the skinny projections
