@@ -45,7 +45,7 @@ def test_attention_sweep(worker):
                 group = 32
             hq = hkv * group
             fp8 = rng.random() < 0.35
-            bs = rng.choice([32, 64, 128, 256] if fp8 else [16, 32, 48, 64, 128, 256])
+            bs = rng.choice([32, 64, 128, 256, 1024] if fp8 else [16, 32, 48, 64, 128, 256, 1024, 1536])
             batch = rng.randint(1, 5)
             top = rng.choice([40, 300, 1200, 2500])
             ctxs = [rng.choice([0, 1, bs - 1, bs, bs + 1, rng.randint(1, top), rng.randint(1, top)]) for _ in range(batch)]
