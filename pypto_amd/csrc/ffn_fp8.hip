@@ -14,6 +14,7 @@
 // v_mfma_f32_32x32x64_f8f6f4: lane l holds row/column l % 32 and the 32 codes k = 32 * (l / 32) .. +32.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 
 #include "common.h"
@@ -42,6 +43,11 @@ struct Params {
   int64_t lda, ldb, ldc;
   int m, n, k;
   int tiles_m, tiles_n;
+  // k split over `splits` workgroups per output tile (single-operand pass only): each writes its raw
+  // fp32 accumulators to its own slab [split][m][n]; gemm8_finish_kernel sums the slabs in split
+  // order and applies the scales.  splits == 1: the epilogue finishes the tile.
+  int splits, k_per_split;
+  float* slabs;
 };
 
 // SiLU in the device form of the reference, g * recip(1 + exp(-g)) (01_ffn.py:70-74), with the hardware's
@@ -133,8 +139,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % WM, wn = wave / WM;
   const int ntiles = p.tiles_m * p.tiles_n;
-  const int tile = xcd_remap(blockIdx.x, ntiles);
+  const int logical = xcd_remap(blockIdx.x, ntiles * p.splits);
+  const int split = logical / ntiles, tile = logical % ntiles;
   const int tm = tile % p.tiles_m, tn = tile / p.tiles_m;
+  const int k_begin = split * p.k_per_split;  // this workgroup's k range: [k_begin, k_begin + nk * BK)
   const int m0 = tm * BM;
   const int n0 = tn * (DUAL ? BN / 2 : BN);
 
@@ -148,7 +156,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
     const int r = min(m0 + i * RPR + row_in_round, p.m - 1);
-    a_ptr[i] = p.a + (int64_t)r * p.lda + chunk * 16;
+    a_ptr[i] = p.a + (int64_t)r * p.lda + k_begin + chunk * 16;
   }
   const uint8_t* b_ptr[NB];
 #pragma unroll
@@ -156,7 +164,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
     const int tr = i * RPR + row_in_round;  // row of the B tile
     const uint8_t* src = (DUAL && tr >= BN / 2) ? p.b1 : p.b0;
     const int ch = min(n0 + (DUAL ? tr % (BN / 2) : tr), p.n - 1);
-    b_ptr[i] = src + (int64_t)ch * p.ldb + chunk * 16;
+    b_ptr[i] = src + (int64_t)ch * p.ldb + k_begin + chunk * 16;
   }
   // The instruction is written out: told that a load writes LDS, the compiler waits for every such
   // load in flight before each later LDS read, whatever buffer that read addresses.
@@ -234,7 +242,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
     }
   };
 
-  const int nk = p.k / BK;
+  const int nk = (min(p.k, k_begin + p.k_per_split) - k_begin) / BK;
   // Tiles kt (being multiplied), kt+1 (landed in the other buffer) and kt+2 (in flight into the
   // buffer of kt) are live at once.  The one barrier of a k-tile sits in its second k-step, after
   // column 0: by then this wavefront has read the last fragment of tile kt (the wait for it is
@@ -287,6 +295,30 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
   // acc[i][jn][r]: row m0 + wm*MT*32 + i*32 + (r/4)*8 + (lane/32)*4 + r%4, column lane % 32 of fragment jn
   OutT* c = reinterpret_cast<OutT*>(p.c);
   const int row_base = m0 + wm * MT * 32 + (lane >> 5) * 4;
+  if constexpr (!DUAL) {
+    if (p.splits > 1) {
+      // raw accumulators to this split's slab, four consecutive columns of a row per store (n % 4 == 0)
+      float* mine = p.slabs + (int64_t)split * p.m * p.n;
+      const int my_row = row_base + (lane & 3);
+      const int col_shift = ((lane & 31) & ~3) - (lane & 31);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int row = my_row + i * 32 + q * 8;
+#pragma unroll
+          for (int jn = 0; jn < NT; ++jn) {
+            float v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v[k] = acc[i][jn][q * 4 + k];
+            quad_transpose(v, lane);
+            const int c0 = col[jn] + col_shift;
+            if (row < p.m && c0 < p.n) *reinterpret_cast<float4*>(mine + (int64_t)row * p.n + c0) = float4{v[0], v[1], v[2], v[3]};
+          }
+        }
+      return;
+    }
+  }
   // Row scales from the LDS copy made at the start (visible since the loop's barriers): four
   // consecutive rows per read.  One global load per row here would put 16 * MT loads per lane
   // through the CU's address unit while the matrix pipes idle.
@@ -365,7 +397,7 @@ int launch(Params p, hipStream_t st) {
                                       (int)smem));
     attr_set.store(true, std::memory_order_release);
   }
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(64 * WM * WN), smem, st, p);
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(64 * WM * WN), smem, st, p);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
 }
@@ -374,11 +406,67 @@ int launch(Params p, hipStream_t st) {
 // SIMD) by default; "gemm_variant" 1 selects four wavefronts of 128 x 128 on the tall tile, which
 // read a third less from LDS per MFMA but leave a SIMD nothing to issue while its one wavefront
 // waits (LLaMA-7B block: 361 us against 334 us).
+// Sum of the k splits' slabs in split order, times the row and column scales, cast and store.
+template <typename OutT>
+__global__ __launch_bounds__(256) void gemm8_finish_kernel(const float* __restrict__ slabs, int splits,
+                                                           const float* __restrict__ sa, const float* __restrict__ sb,
+                                                           OutT* __restrict__ c, int64_t ldc, int m, int n) {
+  const int nq = n / 4;
+  const int64_t quads = (int64_t)m * nq, mn = (int64_t)m * n;
+  for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < quads; q += (int64_t)gridDim.x * 256) {
+    const int64_t row = q / nq;
+    const int col = (int)(q % nq) * 4;
+    const float* src = slabs + row * n + col;
+    float4 t = *reinterpret_cast<const float4*>(src);
+    for (int s = 1; s < splits; ++s) {
+      const float4 v = *reinterpret_cast<const float4*>(src + s * mn);
+      t = float4{t.x + v.x, t.y + v.y, t.z + v.z, t.w + v.w};
+    }
+    const float r = sa[row];
+    const float4 w = *reinterpret_cast<const float4*>(sb + col);
+    const float out[4] = {t.x * r * w.x, t.y * r * w.y, t.z * r * w.z, t.w * r * w.w};
+    store4<OutT>(c + row * ldc + col, out);
+  }
+}
+
+// Tile height: 256 rows unless that leaves CUs idle and 128 rows do not.  Eight wavefronts (two per
+// SIMD) by default; "gemm_variant" 1 selects four wavefronts of 128 x 128 on the tall tile, which
+// read a third less from LDS per MFMA but leave a SIMD nothing to issue while its one wavefront
+// waits (LLaMA-7B block: 361 us against 334 us).
+// A single-operand pass whose tall tiles fill at most half the CUs splits k instead of halving the
+// tile: a k-tile takes a workgroup the same ~1.4 us with 128 rows as with 256 (the tile's arrival,
+// not the MFMAs, sets it), so two workgroups per 256 x 256 tile do the same work in half the k-tiles.
 template <bool DUAL, typename OutT>
-int launch_any(const Params& p, hipStream_t st) {
+int launch_any(const Params& p0, hipStream_t st) {
+  Params p = p0;
+  p.splits = 1;
+  p.k_per_split = p.k;
+  p.slabs = nullptr;
+  const int64_t num_cu = pto_hip::ctx().num_cu;
   const int64_t tiles_n = (p.n + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256);
   const int64_t tall = (int64_t)((p.m + 255) / 256) * tiles_n;
-  if (tall < pto_hip::ctx().num_cu && p.m > 128) return launch<2, 2, 2, 4, DUAL, OutT>(p, st);
+  if constexpr (!DUAL) {
+    const int nk = p.k / BK;
+    int64_t want = pto_hip::ctx().gemm_splits > 0 ? pto_hip::ctx().gemm_splits : std::min<int64_t>(num_cu / tall, 4);
+    if (pto_hip::ctx().gemm_variant == 0 && p.m > 128 && want >= 2 && nk >= 8 * want && p.n % 4 == 0 && p.ldc % 4 == 0) {
+      const int per = (int)((nk + want - 1) / want);
+      p.k_per_split = per * BK;
+      p.splits = (nk + per - 1) / per;
+      void* ws = nullptr;
+      const int rc = pto_hip::gemm_workspace((size_t)p.splits * p.m * p.n * sizeof(float), &ws);
+      if (rc) return rc;
+      p.slabs = reinterpret_cast<float*>(ws);
+      const int rc2 = launch<4, 2, 2, 4, DUAL, OutT>(p, st);
+      if (rc2) return rc2;
+      const int64_t quads = (int64_t)p.m * (p.n / 4);
+      const unsigned blocks = (unsigned)std::min<int64_t>((quads + 255) / 256, 4096);
+      hipLaunchKernelGGL((gemm8_finish_kernel<OutT>), dim3(blocks), dim3(256), 0, st, p.slabs, p.splits, p.sa, p.sb0,
+                         reinterpret_cast<OutT*>(p.c), p.ldc, p.m, p.n);
+      PTO_CHECK_HIP(hipGetLastError());
+      return PTO_HIP_OK;
+    }
+  }
+  if (tall < num_cu && p.m > 128) return launch<2, 2, 2, 4, DUAL, OutT>(p, st);
   if (pto_hip::ctx().gemm_variant == 1) return launch<4, 4, 2, 2, DUAL, OutT>(p, st);
   return launch<4, 2, 2, 4, DUAL, OutT>(p, st);
 }

@@ -43,37 +43,6 @@ struct GemmParams {
   pto_hip::W8Partials* partials_out;  // non-null: leave the k-split slabs unsummed and describe them here
 };
 
-// 4 x 4 transpose across the four lanes of a quad.  In: v[k] = the value of row R + k at this lane's
-// column.  Out: v[k] = the value of row R + (lane % 4) at column 4 * (this lane's column / 4) + k.
-// An MFMA accumulator holds four consecutive rows of ONE column per lane; after the transpose a lane
-// holds four consecutive columns of one row, which is a single 8- or 16-byte store instead of four
-// 2- or 4-byte ones - the epilogue is bound by the number of store instructions, not by bytes.
-__device__ __forceinline__ float quad_xor1(float x) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));  // quad_perm 1,0,3,2
-}
-__device__ __forceinline__ float quad_xor2(float x) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));  // quad_perm 2,3,0,1
-}
-__device__ __forceinline__ void quad_transpose(float (&v)[4], int lane) {
-  const bool b0 = (lane & 1) != 0, b1 = (lane & 2) != 0;
-  const float r01 = quad_xor1(b0 ? v[0] : v[1]), r23 = quad_xor1(b0 ? v[2] : v[3]);
-  if (b0) {
-    v[0] = r01;
-    v[2] = r23;
-  } else {
-    v[1] = r01;
-    v[3] = r23;
-  }
-  const float r02 = quad_xor2(b1 ? v[0] : v[2]), r13 = quad_xor2(b1 ? v[1] : v[3]);
-  if (b1) {
-    v[0] = r02;
-    v[1] = r13;
-  } else {
-    v[2] = r02;
-    v[3] = r13;
-  }
-}
-
 __device__ __forceinline__ float load_residual(const void* r, int dt, int64_t i) {
   if (dt == PTO_HIP_FP32) return reinterpret_cast<const float*>(r)[i];
   if (dt == PTO_HIP_BF16) return (float)reinterpret_cast<const __bf16*>(r)[i];
@@ -93,19 +62,6 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 
 template <typename OutT>
 __device__ __forceinline__ void store_out(OutT* p, float v) { *p = (OutT)v; }
-// four consecutive outputs of one row as one store (dst aligned to four elements)
-template <typename OutT>
-__device__ __forceinline__ void store_out4(OutT* dst, const float (&v)[4]) {
-  if constexpr (sizeof(OutT) == 4) {
-    *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
-  } else {
-    const OutT a = (OutT)v[0], b = (OutT)v[1], c = (OutT)v[2], d = (OutT)v[3];
-    uint2 w;
-    w.x = (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
-    w.y = (uint32_t)__builtin_bit_cast(uint16_t, c) | ((uint32_t)__builtin_bit_cast(uint16_t, d) << 16);
-    *reinterpret_cast<uint2*>(dst) = w;
-  }
-}
 
 // Sigmoid in the device form of the reference, recip(1 + exp(-g)) (01_ffn.py:70-74), with the
 // hardware's 1-ulp reciprocal: the correctly rounded one is a ten-instruction division, and the
@@ -427,66 +383,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
       const float* s = (DUAL && jn >= NT / 2) ? p.scale1 : p.scale0;
       sc[jn] = col < p.n ? s[col] : 0.f;
     }
-  }
-  // Rows of four, quad-transposed so that every lane writes four consecutive columns of one row.
-  // Needs rows of the output (and of the slabs, whose rows are n long) to start on four elements.
-  if (p.n % 4 == 0 && p.ldc % 4 == 0 && ((uintptr_t)p.c % 16 == 0)) {
-    const int64_t mn = (int64_t)p.m * p.n;
-    const int my_row = row_base + (lane & 3);                 // + i * 32 + q * 8
-    const int col_shift = ((lane & 31) & ~3) - (lane & 31);   // this lane's first column after the transpose
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int row = my_row + i * 32 + q * 8;
-        const bool row_ok = row < p.m;
-#pragma unroll
-        for (int jn = 0; jn < (DUAL ? NT / 2 : NT); ++jn) {
-          const int c0 = (DUAL ? n0 + wn * (16 * NT) + jn * 32 : n0 + wn * (32 * NT) + jn * 32) + (lane & 31) + col_shift;
-          const bool ok = row_ok && c0 < p.n;
-          float v[4];
-          if (p.splits > 1) {
-#pragma unroll
-            for (int k = 0; k < 4; ++k) v[k] = acc[i][jn][q * 4 + k];
-            quad_transpose(v, lane);
-            float* s = p.slabs + (int64_t)split * (DUAL ? 2 : 1) * mn + (int64_t)row * p.n + c0;
-            if (ok) *reinterpret_cast<float4*>(s) = float4{v[0], v[1], v[2], v[3]};
-            if constexpr (DUAL) {
-#pragma unroll
-              for (int k = 0; k < 4; ++k) v[k] = acc[i][jn + NT / 2][q * 4 + k];
-              quad_transpose(v, lane);
-              if (ok) *reinterpret_cast<float4*>(s + mn) = float4{v[0], v[1], v[2], v[3]};
-            }
-            continue;
-          }
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const int r = q * 4 + k;
-            if constexpr (DUAL) {
-              float g = acc[i][jn][r], u = acc[i][jn + NT / 2][r];
-              if constexpr (W8) {
-                g *= sc[jn];
-                u *= sc[jn + NT / 2];
-              }
-              v[k] = silu(g) * u;
-            } else {
-              v[k] = acc[i][jn][r];
-              if constexpr (W8) v[k] *= sc[jn];
-            }
-          }
-          quad_transpose(v, lane);
-          if (!ok) continue;
-          if constexpr (!DUAL) {
-            if (p.residual) {
-#pragma unroll
-              for (int k = 0; k < 4; ++k) v[k] += load_residual(p.residual, p.res_dtype, (int64_t)row * p.n + c0 + k);
-            }
-          }
-          store_out4<OutT>(c + (int64_t)row * p.ldc + c0, v);
-        }
-      }
-    }
-    return;
   }
 #pragma unroll
   for (int i = 0; i < MT; ++i) {

@@ -557,18 +557,63 @@ def test_ffn_block_fp8_four_wavefront_form_is_bit_identical(worker):
     from pypto_amd.runtime import ffn_block_fp8
 
     q, _ = workloads.ffn_fp8_inputs(tokens=2048, hidden=512, intermediate=4096, seed=6, device="cuda")
-    with worker.register(ffn_block_fp8) as hd:
-        hd(*q.args())
-        worker.sync()
-        first = q.out.clone()
-        q.out.zero_()
-        worker.set_option("gemm_variant", 1)
-        try:
+    worker.set_option("gemm_splits", 1)   # the eight-wavefront form would split the down pass's k, the other does not
+    try:
+        with worker.register(ffn_block_fp8) as hd:
             hd(*q.args())
             worker.sync()
-        finally:
-            worker.set_option("gemm_variant", 0)
+            first = q.out.clone()
+            q.out.zero_()
+            worker.set_option("gemm_variant", 1)
+            hd(*q.args())
+            worker.sync()
+    finally:
+        worker.set_option("gemm_variant", 0)
+        worker.set_option("gemm_splits", 0)
     assert first.abs().max().item() > 0 and torch.equal(first, q.out)
+
+
+@pytest.mark.parametrize("m,k,n,splits", [(2048, 11008, 4096, 0),    # the LLaMA-7B down pass: the library's own choice (2)
+                                          (300, 4096, 520, 3), (257, 4096, 256, 4), (1000, 2048, 1024, 2)])
+def test_projection_fp8_k_split_sums_the_same_products(worker, m, k, n, splits):
+    """A single-operand pass whose 256-row tiles fill at most half the CUs splits k over 2-4 workgroups per
+    tile; a finish kernel sums their fp32 slabs and applies the scales.  Small-integer operands with
+    power-of-two scales make every sum exact: identical to the unsplit pass and to the product itself."""
+    _lib, lib, code = _fp8_stage_lib()
+    g = torch.Generator().manual_seed(m + splits)
+    a = torch.randint(-3, 4, (m, k), generator=g).float()
+    w = torch.randint(-3, 4, (n, k), generator=g).float()
+    a8, w8 = a.to(torch.float8_e4m3fn).cuda(), w.to(torch.float8_e4m3fn).cuda()
+    sa = torch.full((m,), 0.5, device="cuda")
+    sw = torch.full((n,), 0.125, device="cuda")
+    outs = []
+    f32 = code(torch.float32)
+    for s in (1, splits):
+        worker.set_option("gemm_splits", s)
+        try:
+            out = torch.full((m, n), float("nan"), device="cuda")
+            _lib.check(lib.pto_hip_projection_fp8(a8.data_ptr(), sa.data_ptr(), w8.data_ptr(), sw.data_ptr(),
+                                                  out.data_ptr(), m, k, n, f32, 0))
+            worker.sync()
+        finally:
+            worker.set_option("gemm_splits", 0)
+        outs.append(out.cpu())
+    assert torch.equal(outs[0], outs[1])
+    assert torch.equal(outs[1], (a @ w.t()) * 0.5 * 0.125)
+    # and random codes in 16-bit output against the oracle's product
+    a8r, sar = _codes_and_scales(m, k, 14, 1.0)
+    w8r, swr = _codes_and_scales(n, k, 15, 0.02)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    dev = [t.cuda() for t in (a8r, sar, w8r, swr)]   # kept alive across the call: the entry takes bare addresses
+    worker.set_option("gemm_splits", splits)
+    try:
+        _lib.check(lib.pto_hip_projection_fp8(*(t.data_ptr() for t in dev), out.data_ptr(), m, k, n,
+                                              code(torch.bfloat16), 0))
+        worker.sync()
+    finally:
+        worker.set_option("gemm_splits", 0)
+    ref = (a8r.float() @ w8r.float().t()) * sar[:, None] * swr[None, :]
+    validate_golden({"out": out.cpu().float()}, {"out": ref}, rtol=8e-3, atol=1e-4 * ref.abs().max().item())
 
 
 def test_ffn_block_fp8_argument_rules(worker):
