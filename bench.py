@@ -130,8 +130,10 @@ def main() -> int:
                     help="fix attn_tokens_per_partition and attn_waves_per_cu for the small configuration instead of "
                          "measuring (for profiler runs: every traced launch then has the same shape)")
     ap.add_argument("--ffn-clock-probe", action="store_true",
-                    help="also run the FFN for about 1.5 s on its random operands and on all-zero operands, reading the "
-                         "shader clock (rocm-smi) during each: the gap between the two is the data-dependent clock")
+                    help="run the FFN for about 1.5 s on its random operands and on all-zero operands, reading the "
+                         "shader clock (rocm-smi) during each: the gap between the two is the data-dependent clock. "
+                         "On by default for the 16-bit block; with this flag also for the e4m3 block")
+    ap.add_argument("--no-ffn-clock-probe", action="store_true", help="skip the clock probe (saves about 3 s)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy, a known-size reference for HBM byte counters")
     args = ap.parse_args()
@@ -278,7 +280,7 @@ def main() -> int:
             "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
             "bound": "mfma",
         }
-        if args.ffn_clock_probe:
+        if not args.no_ffn_clock_probe:
             result["ffn"]["clock_probe"] = _ffn_clock_probe(worker, ffn_block, fargs[0], (0, 2, 3, 4))
         if cpu:
             rows = 256  # of the 2048 token rows; the weights are the full ones
