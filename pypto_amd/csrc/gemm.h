@@ -384,46 +384,57 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
       sc[jn] = col < p.n ? s[col] : 0.f;
     }
   }
+  // Addresses: the lane's part (its first row and column) is computed once; every row of the tile is a
+  // compile-time number of rows further on, so the rest of an address is scalar arithmetic.  Computing
+  // row * ld per output instead costs two quarter-rate integer multiplies and a 64-bit multiply-add for
+  // each of a lane's 64-128 outputs - more than the SiLU.  Bounds are only checked where the launch
+  // can have edges (EDGE 1: rows, EDGE 2: rows and columns).
+  const int col0 = (DUAL ? n0 + wn * (16 * NT) : n0 + wn * (32 * NT)) + (lane & 31);
+  const int64_t mn = (int64_t)p.m * p.n;
+  constexpr int JN = DUAL ? NT / 2 : NT;
+  if (p.splits > 1) {
+    float* lane_s = p.slabs + (int64_t)split * (DUAL ? 2 : 1) * mn + (int64_t)row_base * p.n + col0;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int rr = i * 32 + (r >> 2) * 8 + (r & 3);
+        if (EDGE != 0 && row_base + rr >= p.m) continue;
+        float* s = lane_s + (int64_t)rr * p.n;
+#pragma unroll
+        for (int jn = 0; jn < JN; ++jn) {
+          if (EDGE == 2 && col0 + jn * 32 >= p.n) continue;
+          s[jn * 32] = acc[i][jn][r];
+          if constexpr (DUAL) s[mn + jn * 32] = acc[i][jn + NT / 2][r];
+        }
+      }
+    }
+    return;
+  }
+  OutT* lane_c = c + (int64_t)row_base * p.ldc + col0;
+  const int64_t lane_res = (int64_t)row_base * p.n + col0;
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int row = row_base + i * 32 + (r >> 2) * 8 + (r & 3);
-      if (row >= p.m) continue;
-      const int64_t mn = (int64_t)p.m * p.n;
-      if constexpr (DUAL) {
+      const int rr = i * 32 + (r >> 2) * 8 + (r & 3);
+      if (EDGE != 0 && row_base + rr >= p.m) continue;
+      OutT* dst = lane_c + (int64_t)rr * p.ldc;
 #pragma unroll
-        for (int jn = 0; jn < NT / 2; ++jn) {
-          const int col = n0 + wn * (16 * NT) + jn * 32 + (lane & 31);
-          if (col < p.n) {
-            if (p.splits > 1) {
-              float* s = p.slabs + (int64_t)split * 2 * mn + (int64_t)row * p.n + col;
-              s[0] = acc[i][jn][r];
-              s[mn] = acc[i][jn + NT / 2][r];
-            } else {
-              float g = acc[i][jn][r], u = acc[i][jn + NT / 2][r];
-              if constexpr (W8) {
-                g *= sc[jn];
-                u *= sc[jn + NT / 2];
-              }
-              store_out<OutT>(c + (int64_t)row * p.ldc + col, silu(g) * u);
-            }
+      for (int jn = 0; jn < JN; ++jn) {
+        if (EDGE == 2 && col0 + jn * 32 >= p.n) continue;
+        if constexpr (DUAL) {
+          float g = acc[i][jn][r], u = acc[i][jn + NT / 2][r];
+          if constexpr (W8) {
+            g *= sc[jn];
+            u *= sc[jn + NT / 2];
           }
-        }
-      } else {
-#pragma unroll
-        for (int jn = 0; jn < NT; ++jn) {
-          const int col = n0 + wn * (32 * NT) + jn * 32 + (lane & 31);
-          if (col < p.n) {
-            if (p.splits > 1) {
-              p.slabs[(int64_t)split * mn + (int64_t)row * p.n + col] = acc[i][jn][r];
-            } else {
-              float v = acc[i][jn][r];
-              if constexpr (W8) v *= sc[jn];
-              if (p.residual) v += load_residual(p.residual, p.res_dtype, (int64_t)row * p.n + col);
-              store_out<OutT>(c + (int64_t)row * p.ldc + col, v);
-            }
-          }
+          store_out<OutT>(dst + jn * 32, silu(g) * u);
+        } else {
+          float v = acc[i][jn][r];
+          if constexpr (W8) v *= sc[jn];
+          if (p.residual) v += load_residual(p.residual, p.res_dtype, lane_res + (int64_t)rr * p.n + jn * 32);
+          store_out<OutT>(dst + jn * 32, v);
         }
       }
     }
