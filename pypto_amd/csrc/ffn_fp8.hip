@@ -542,6 +542,19 @@ __global__ __launch_bounds__(kRowThreads) void row_quant_kernel(const TI* __rest
     for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(y[u][e]));
   amax = block_reduce(amax, true, red);
   const float s = amax > 0.f ? amax / kE4m3Max : 1.f;
+  // y / s, correctly rounded, without the compiler's ten-instruction division per element: the
+  // reciprocal of s is refined once per row to within half an ulp (one Newton step on v_rcp_f32), and
+  // each quotient is q0 = y * r corrected twice by its exact remainder, q + (y - q * s) * r (two
+  // fused multiply-adds each; one correction alone leaves a few quotients in ten million an ulp off).  |y| <= amax = 448 * s, so no quotient leaves [-448, 448]: nothing over- or
+  // underflows, which is all the full sequence adds.
+  float r = __builtin_amdgcn_rcpf(s);
+  r = fmaf(fmaf(-s, r, 1.f), r, r);
+  auto quot = [&](float v) {
+    const float q0 = v * r;
+    const float q1 = fmaf(fmaf(-q0, s, v), r, q0);  // within an ulp of v / s
+    const float q2 = fmaf(fmaf(-q1, s, v), r, q1);  // its exact remainder settles the last bit
+    return v == 0.f ? v : q2;                       // a zero keeps its sign (the corrections add +0 to -0)
+  };
   if (threadIdx.x == 0) scale[row] = s;
   uint2* crow = reinterpret_cast<uint2*>(codes + row * cols);
 #pragma unroll
@@ -550,7 +563,7 @@ __global__ __launch_bounds__(kRowThreads) void row_quant_kernel(const TI* __rest
     if (i < nvec) {
       float q[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) q[e] = clamp_e4m3(y[u][e] / s);
+      for (int e = 0; e < 8; ++e) q[e] = clamp_e4m3(quot(y[u][e]));
       int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
       w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], w0, true);
       int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], 0, false);

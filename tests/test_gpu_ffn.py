@@ -355,6 +355,36 @@ def test_quantize_rows_fp8_matches_oracle(worker, dtype, rows, cols):
     assert torch.equal(codes.cpu(), want_codes.view(torch.uint8))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_quantize_rows_fp8_quotients_are_the_divisions(worker, dtype):
+    """The quantiser forms y / scale from a refined reciprocal and two remainder corrections instead of a
+    division per element.  Every code must still be the one the division gives: rows spanning 16-bit
+    denormals to the type's large values, negative zeros (a zero keeps its sign: code 0x80), and rows whose
+    maximum makes 1 / scale a power of two or the mantissa of scale all ones."""
+    from pypto_amd import _lib
+    from pypto_amd.runtime import _dtype_code
+
+    rows, cols = 512, 4096
+    g = torch.Generator().manual_seed(41)
+    spread = torch.logspace(-7, 4 if dtype == torch.float16 else 30, rows)[:, None]
+    x = (torch.randn((rows, cols), generator=g) * spread).to(dtype)
+    x[torch.rand((rows, cols), generator=g) < 0.01] = -0.0
+    x[7, 0] = 448.0          # scale exactly 1
+    x[8] = x[8].clamp(-3.5, 3.5)
+    x[8, 0] = 3.5            # scale 2^-7
+    x[9] = (x[9].float().clamp(-1, 1) * 0.999).to(dtype)
+    xd = x.cuda()
+    codes = torch.zeros((rows, cols), dtype=torch.uint8, device="cuda")
+    scale = torch.zeros(rows, dtype=torch.float32, device="cuda")
+    _lib.check(_lib.load().pto_hip_quantize_rows_fp8(xd.data_ptr(), codes.data_ptr(), scale.data_ptr(), rows, cols,
+                                                     _dtype_code(dtype), 0))
+    worker.sync()
+    want_codes, want_scale = oracle.quantize_rows_fp8(x)
+    assert torch.equal(scale.cpu(), want_scale)
+    assert torch.equal(codes.cpu(), want_codes.view(torch.uint8))
+    assert int((want_codes.view(torch.uint8) == 0x80).sum()) > 1000   # the negative zeros are in there
+
+
 def test_quantize_rows_fp8_argument_rules(worker):
     from pypto_amd import _lib
     from pypto_amd.runtime import _dtype_code
