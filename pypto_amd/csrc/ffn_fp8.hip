@@ -411,11 +411,12 @@ template <typename OutT>
 __global__ __launch_bounds__(256) void gemm8_finish_kernel(const float* __restrict__ slabs, int splits,
                                                            const float* __restrict__ sa, const float* __restrict__ sb,
                                                            OutT* __restrict__ c, int64_t ldc, int m, int n) {
-  const int nq = n / 4;
-  const int64_t quads = (int64_t)m * nq, mn = (int64_t)m * n;
-  for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < quads; q += (int64_t)gridDim.x * 256) {
-    const int64_t row = q / nq;
-    const int col = (int)(q % nq) * 4;
+  // blockIdx.x, threadIdx.x: four columns; blockIdx.y: rows, strided (no division per element)
+  const int col = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (col >= n) return;
+  const int64_t mn = (int64_t)m * n;
+  const float4 w = *reinterpret_cast<const float4*>(sb + col);
+  for (int64_t row = blockIdx.y; row < m; row += gridDim.y) {
     const float* src = slabs + row * n + col;
     float4 t = *reinterpret_cast<const float4*>(src);
     for (int s = 1; s < splits; ++s) {
@@ -423,7 +424,6 @@ __global__ __launch_bounds__(256) void gemm8_finish_kernel(const float* __restri
       t = float4{t.x + v.x, t.y + v.y, t.z + v.z, t.w + v.w};
     }
     const float r = sa[row];
-    const float4 w = *reinterpret_cast<const float4*>(sb + col);
     const float out[4] = {t.x * r * w.x, t.y * r * w.y, t.z * r * w.z, t.w * r * w.w};
     store4<OutT>(c + row * ldc + col, out);
   }
@@ -458,9 +458,9 @@ int launch_any(const Params& p0, hipStream_t st) {
       p.slabs = reinterpret_cast<float*>(ws);
       const int rc2 = launch<4, 2, 2, 4, DUAL, OutT>(p, st);
       if (rc2) return rc2;
-      const int64_t quads = (int64_t)p.m * (p.n / 4);
-      const unsigned blocks = (unsigned)std::min<int64_t>((quads + 255) / 256, 4096);
-      hipLaunchKernelGGL((gemm8_finish_kernel<OutT>), dim3(blocks), dim3(256), 0, st, p.slabs, p.splits, p.sa, p.sb0,
+      const unsigned bx = (unsigned)((p.n / 4 + 255) / 256);
+      const unsigned by = (unsigned)std::min<int64_t>(p.m, std::max<int64_t>(1, 4096 / bx));
+      hipLaunchKernelGGL((gemm8_finish_kernel<OutT>), dim3(bx, by), dim3(256), 0, st, p.slabs, p.splits, p.sa, p.sb0,
                          reinterpret_cast<OutT*>(p.c), p.ldc, p.m, p.n);
       PTO_CHECK_HIP(hipGetLastError());
       return PTO_HIP_OK;

@@ -480,12 +480,13 @@ template <bool DUAL, typename OutT>
 __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* slabs, OutT* c, int64_t ldc, int m, int n,
                                                           int splits, const void* residual, int res_dtype,
                                                           const float* scale0, const float* scale1) {
-  const int nq = n / 4;
-  const int64_t quads = (int64_t)m * nq, mn = (int64_t)m * n;
+  // blockIdx.x, threadIdx.x: four columns; blockIdx.y: rows, strided.  No division per element: a 64-bit
+  // quotient and remainder cost more instructions than the sums they would index.
+  const int col = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (col >= n) return;
+  const int64_t mn = (int64_t)m * n;
   constexpr int kMats = DUAL ? 2 : 1;
-  for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < quads; q += (int64_t)gridDim.x * 256) {
-    const int64_t row = q / nq;
-    const int col = (int)(q % nq) * 4;
+  for (int64_t row = blockIdx.y; row < m; row += gridDim.y) {
     const float* src = slabs + row * n + col;
     float4 t[kMats];
 #pragma unroll
@@ -535,9 +536,9 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const float* slabs, Ou
 
 template <bool DUAL, typename OutT>
 int launch_finish(const GemmParams& p, hipStream_t st) {
-  const int64_t quads = (int64_t)p.m * (p.n / 4);
-  const unsigned blocks = (unsigned)std::min<int64_t>((quads + 255) / 256, 4096);
-  hipLaunchKernelGGL((gemm_finish_kernel<DUAL, OutT>), dim3(blocks), dim3(256), 0, st, p.slabs,
+  const unsigned bx = (unsigned)((p.n / 4 + 255) / 256);
+  const unsigned by = (unsigned)std::min<int64_t>(p.m, std::max<int64_t>(1, 4096 / bx));
+  hipLaunchKernelGGL((gemm_finish_kernel<DUAL, OutT>), dim3(bx, by), dim3(256), 0, st, p.slabs,
                      reinterpret_cast<OutT*>(p.c), p.ldc, p.m, p.n, p.splits, p.residual, p.res_dtype, p.scale0,
                      p.scale1);
   PTO_CHECK_HIP(hipGetLastError());
