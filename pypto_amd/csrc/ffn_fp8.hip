@@ -504,21 +504,22 @@ __global__ __launch_bounds__(kRowThreads) void row_quant_kernel(const TI* __rest
   const int64_t row = blockIdx.x;
   const vec8* xr = reinterpret_cast<const vec8*>(x + row * cols);
   const int nvec = (int)(cols / 8);
-  float y[kRowVecs][8];
+  // The row stays in registers in its 16-bit form (four registers per group of eight, not eight):
+  // with the whole row's workgroups resident at once the kernel is one round of loads, not two.
+  vec8 y[kRowVecs];
   float ss = 0.f;
 #pragma unroll
   for (int u = 0; u < kRowVecs; ++u) {
     const int i = threadIdx.x + u * kRowThreads;
     if (i < nvec) {
-      const vec8 v = xr[i];
+      y[u] = xr[i];
+      if constexpr (NORM) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        y[u][e] = (float)v[e];
-        ss += y[u][e] * y[u][e];
+        for (int e = 0; e < 8; ++e) ss += (float)y[u][e] * (float)y[u][e];
       }
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) y[u][e] = 0.f;
+      for (int e = 0; e < 8; ++e) y[u][e] = (TI)0.f;
     }
   }
   if constexpr (NORM) {
@@ -531,7 +532,7 @@ __global__ __launch_bounds__(kRowThreads) void row_quant_kernel(const TI* __rest
         const float4 g1 = gamma ? reinterpret_cast<const float4*>(gamma)[2 * i + 1] : float4{1.f, 1.f, 1.f, 1.f};
         const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) y[u][e] = (float)(TI)(y[u][e] * inv * g[e]);
+        for (int e = 0; e < 8; ++e) y[u][e] = (TI)((float)y[u][e] * inv * g[e]);
       }
     }
   }
@@ -539,7 +540,7 @@ __global__ __launch_bounds__(kRowThreads) void row_quant_kernel(const TI* __rest
 #pragma unroll
   for (int u = 0; u < kRowVecs; ++u)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(y[u][e]));
+    for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf((float)y[u][e]));
   amax = block_reduce(amax, true, red);
   const float s = amax > 0.f ? amax / kE4m3Max : 1.f;
   // y / s, correctly rounded, without the compiler's ten-instruction division per element: the
@@ -563,7 +564,7 @@ __global__ __launch_bounds__(kRowThreads) void row_quant_kernel(const TI* __rest
     if (i < nvec) {
       float q[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) q[e] = clamp_e4m3(quot(y[u][e]));
+      for (int e = 0; e < 8; ++e) q[e] = clamp_e4m3(quot((float)y[u][e]));
       int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
       w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], w0, true);
       int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], 0, false);
