@@ -1,10 +1,10 @@
 """Turns rocprofv3 output of ``bench.py`` into the short summaries kept under ``profiles/``.
 
     python -m pypto_amd.profile_summary --name bench_attention_small_ffn_llama7b \\
-        --stats gpurun_out/prof_bench/bench_kernel_stats.csv \\
-        --fetch gpurun_out/pmc_fetch/bench_counter_collection.csv \\
-        --write gpurun_out/pmc_write/bench_counter_collection.csv \\
-        --bench-log gpurun_out/prof_bench.log --command "rocprofv3 ... -- python3 bench.py ..." [--command ...]
+        --stats out/prof_bench/bench_kernel_stats.csv \\
+        --fetch out/pmc_fetch/bench_counter_collection.csv \\
+        --write out/pmc_write/bench_counter_collection.csv \\
+        --bench-log out/prof_bench.log --command "rocprofv3 ... -- python3 bench.py ..." [--command ...]
 
 writes ``profiles/<name>.md`` (the figures a reader wants, with the commands that made them) and
 ``profiles/<name>.json`` (the same figures as data).  ``bench.py`` reads the JSON for the HBM traffic of
