@@ -121,6 +121,8 @@ def main() -> int:
     ap.add_argument("--no-ffn", action="store_true", help="skip the FFN measurement")
     ap.add_argument("--no-extra", action="store_true",
                     help="skip the long-context e4m3 attention configuration and the decoder layer")
+    ap.add_argument("--no-long", action="store_true", help="skip the long-context e4m3 attention configuration")
+    ap.add_argument("--no-layer", action="store_true", help="skip the decoder layer")
     ap.add_argument("--more", action="store_true",
                     help="also time shapes outside the benchmark configurations: the layer with bf16 weights, a "
                          "qwen3-14B layer, the FFN at 16 tokens, a vocabulary projection, 64-head MQA attention")
@@ -329,7 +331,7 @@ def main() -> int:
         torch.cuda.empty_cache()
 
     # ---- the path's other configurations --------------------------------------------------------
-    if not args.no_extra:
+    if not args.no_extra and not args.no_long:
         lf = workloads.attention_long_fp8(seed=0, device="cuda")
         torch.cuda.synchronize()
         with worker.register(paged_attention) as lh:
@@ -362,6 +364,7 @@ def main() -> int:
         del lf, largs
         torch.cuda.empty_cache()
 
+    if not args.no_extra and not args.no_layer:
         dl = workloads.decoder_layer_inputs(device="cuda")
         torch.cuda.synchronize()
         with worker.register(decoder_layer_decode) as dh:

@@ -58,7 +58,7 @@ struct Context {
   // options
   int64_t attn_tokens_per_partition = 0;
   int64_t attn_waves_per_cu = 0;
-  int64_t attn_variant = -1;  // -1 by launch size, 0 partition grid, 1 evenly split form
+  int64_t attn_variant = -1;  // -1 by launch size, 0 partition grid, 1 evenly split form, 2 workgroup form (merge in LDS)
   // "attn_kernel_timing": the streaming attention kernel of every launch is bracketed by a pair of
   // HIP events on its stream; "attn_kernel_time_ns" reads the mean interval and drops the pairs.
   int64_t attn_kernel_timing = 0;

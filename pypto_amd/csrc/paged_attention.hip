@@ -18,6 +18,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
@@ -53,6 +54,7 @@ struct AttnParams {
   int* error_flag; // set when a table entry a sequence uses addresses a block outside the cache
   int gt_rows;     // query rows one wavefront covers: 16 x its tile count; gtiles = ceil(group / gt_rows)
   int resident_cap;  // partition grid: wavefronts allowed on a CU at once, 0 = as many as fit
+  int wg_merge;    // one workgroup per (sequence, KV head, query tile), merged through LDS: 1, else 0
   int n_wg;        // evenly split form: resident workgroups (one per CU); 0 = partition grid
   int lean_waves;  // ... and wavefronts in each
   float scale_log2e;
@@ -655,6 +657,112 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(AttnParams p) {
 
 
 // ---------------------------------------------------------------------------------------------
+// Workgroup form.  One workgroup per (sequence, KV head, query tile); wavefront w takes context
+// partition w and the workgroup merges its own partials through LDS - the arithmetic of
+// attn_reduce_kernel's short path in the same order, so the result is the same bit for bit - and
+// writes the final rows (and their 16-bit copy).  No partials in memory and no merge launch: worth
+// it when there are enough (sequence, head) pairs to give every CU a workgroup.  A wavefront's LDS
+// region first holds its K stage and, once its partition is done, its partial (rows padded by four
+// floats against bank conflicts; the last two hold the row's maximum and sum).
+// ---------------------------------------------------------------------------------------------
+template <int D, bool FP8, int GT>
+constexpr int wg_region_bytes() {
+  constexpr int part = GT * 16 * (D + 4) * 4;
+  return part > KStage<D, FP8>::kBytes ? part : KStage<D, FP8>::kBytes;
+}
+// as many wavefronts as the register file allows at the tile count (see lean_max_waves)
+constexpr int wg_max_parts(int d, int gt) { return d == 128 && gt == 1 ? 8 : 4; }
+
+template <int D, bool BF16, bool FP8, int GT>
+__global__ __launch_bounds__(wg_max_parts(D, GT) * 64) void attn_wg_kernel(AttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) char wg_lds[];
+  constexpr int kRegion = wg_region_bytes<D, FP8, GT>();
+  constexpr int kPitch = D + 4;  // floats per partial row
+  const int lane = threadIdx.x & 63;
+  const int part = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 15, j = lane >> 4;
+  const int pair = blockIdx.x;
+  const int b = pair / (p.hkv * p.gtiles);
+  const int h = (pair / p.gtiles) % p.hkv;
+  const int gt = pair % p.gtiles;
+  const int first_window =
+      p.block_table[(size_t)b * p.max_blocks + min(part * p.tpp / p.bs + lane, p.max_blocks - 1)];
+  int ctx = p.ctx_lens[b];
+  const int max_ctx = p.ctx_cap;
+  ctx = ctx < 0 ? 0 : (ctx > max_ctx ? max_ctx : ctx);
+  const int np = (ctx + p.tpp - 1) / p.tpp;  // partitions with tokens: 0 .. blockDim.x / 64
+  const int tok_begin = part * p.tpp;
+  const int tok_end = min(ctx, tok_begin + p.tpp);
+  const int g0 = gt * (16 * GT);
+  const int hq_row0 = b * p.hq + h * p.group + g0;
+  float* region = reinterpret_cast<float*>(wg_lds + part * kRegion);
+
+  if (tok_begin < tok_end) {
+    f32x4 acc[GT][D / 128][8];
+    float m_run[GT], l_run[GT], v_unit;
+    attend_range<D, BF16, FP8, GT>(p, b, h, hq_row0, g0, tok_begin, tok_end, kChunk, c, j,
+                                   reinterpret_cast<char*>(region), first_window, acc, m_run, l_run, v_unit);
+    // the K stage is dead (LDS operations of one wavefront complete in order): the partial takes its place
+#pragma unroll
+    for (int t = 0; t < GT; ++t) {
+      float* row = region + (t * 16 + c) * kPitch;
+      store_rows<D>(row, acc[t], j, v_unit);
+      if (j == 0) {
+        row[D] = m_run[t];
+        row[D + 1] = l_run[t];
+      }
+    }
+  }
+  __syncthreads();
+
+  const int n_threads = blockDim.x;
+  for (int item = threadIdx.x; item < GT * 16 * (D / 4); item += n_threads) {
+    const int r = item / (D / 4), e = (item % (D / 4)) * 4;
+    if (g0 + r >= p.group) continue;  // padding rows of the last query tile
+    const float* src = reinterpret_cast<const float*>(wg_lds) + r * kPitch;
+    constexpr int kStride = kRegion / 4;  // floats between the regions of consecutive partitions
+    float m = kMinMax;
+#pragma unroll
+    for (int u = 0; u < wg_max_parts(D, GT); ++u) m = u < np ? fmaxf(m, src[u * kStride + D]) : m;
+    float l = 0.f;
+    float o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < wg_max_parts(D, GT); ++u) {
+      if (u < np) {
+        const float wgt = __builtin_amdgcn_exp2f(src[u * kStride + D] - m);
+        l += wgt * src[u * kStride + D + 1];
+        const float4 v = *reinterpret_cast<const float4*>(src + u * kStride + e);
+        o[0] += wgt * v.x;
+        o[1] += wgt * v.y;
+        o[2] += wgt * v.z;
+        o[3] += wgt * v.w;
+      }
+    }
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    const float4 y = {o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
+    const int row = hq_row0 + r;
+    const size_t idx = (size_t)row * D + e;
+    *reinterpret_cast<float4*>(p.out + idx) = y;
+    if (p.out16) {
+      size_t i16 = idx;
+      if (p.out16_blocked) {
+        const int bb = row / p.hq, kk = (row % p.hq) * D + e;  // elements kk .. kk+3 of batch row bb
+        i16 = ((size_t)(kk >> 3) * 32 + bb) * 8 + (kk & 7);
+      }
+      if (p.out16_bf16) {
+        typedef __bf16 b4 __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<b4*>(reinterpret_cast<__bf16*>(p.out16) + i16) = b4{(__bf16)y.x, (__bf16)y.y, (__bf16)y.z, (__bf16)y.w};
+      } else {
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<h4*>(reinterpret_cast<_Float16*>(p.out16) + i16) =
+            h4{(_Float16)y.x, (_Float16)y.y, (_Float16)y.z, (_Float16)y.w};
+      }
+    }
+  }
+}
+
+
+// ---------------------------------------------------------------------------------------------
 // Evenly split form.  A launch of the partition grid lasts as long as its slowest wavefront: one
 // wavefront streams its partition with one or two chunks in flight, i.e. at a rate set by the
 // memory latency, partitions differ in length, and the hardware dispatcher parks between 2 and
@@ -949,6 +1057,26 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
     PTO_CHECK_HIP(hipGetLastError());
     return PTO_HIP_OK;
   }
+  if (p.wg_merge) {
+    // One workgroup of n_part wavefronts per (sequence, KV head, query tile).  The LDS request is at
+    // least the wavefronts' regions and is padded so that a CU takes no more workgroups than its share.
+    const int pairs = batch * p.hkv * p.gtiles;
+    const int num_cu = pto_hip::ctx().num_cu;
+    int per_cu = p.resident_cap > 0 ? std::max(1, p.resident_cap / p.n_part) : (pairs + num_cu - 1) / num_cu;
+    const size_t need = (size_t)p.n_part * wg_region_bytes<D, FP8, GT>();
+    const size_t wg_lds_bytes = std::max(need, lds_share(per_cu));
+    auto go = [&](auto kern) -> int {
+      static std::atomic<bool> attr_set{false};
+      if (!attr_set.load(std::memory_order_acquire)) {
+        PTO_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_set.store(true, std::memory_order_release);
+      }
+      return launch_streaming(kern, dim3((unsigned)pairs), dim3((unsigned)p.n_part * 64), wg_lds_bytes, stream, p);
+    };
+    if (bf16) return go(attn_wg_kernel<D, true, FP8, GT>);
+    return go(attn_wg_kernel<D, false, FP8, GT>);
+  }
   int rc;
   if (bf16) rc = launch_streaming(attn_partition_kernel<D, true, FP8, GT>, grid, dim3(64), lds, stream, p);
   else rc = launch_streaming(attn_partition_kernel<D, false, FP8, GT>, grid, dim3(64), lds, stream, p);
@@ -1119,7 +1247,11 @@ int plan_launch(const int64_t* config, int q_dtype, int kv_dtype, bool have_scal
   int64_t tpp = cx.attn_tokens_per_partition;
   if (tpp <= 0) {
     const int64_t units = batch * hkv * p.gtiles;
-    const int64_t slots = (int64_t)cx.num_cu * 4;
+    // With a (sequence, head) pair or more per CU the launch takes the workgroup form (see
+    // paged_attention below), where two wavefronts per CU measured best (decoder layer, 32 sequences
+    // of 4096 tokens: 182.5 us a step against 184.0 with four).
+    const bool wg_form = cx.attn_variant == 2 || (cx.attn_variant < 0 && units >= cx.num_cu);
+    const int64_t slots = (int64_t)cx.num_cu * (wg_form ? 2 : 4);
     int64_t want = (slots + units - 1) / units;
     if (want < 1) want = 1;
     tpp = (max_ctx + want - 1) / want;
@@ -1204,7 +1336,13 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     return PTO_HIP_OK;
   };
 
-  if (p.n_part > 1 && !lean) {
+  // Workgroup form (merge through LDS, no partials in memory): by default when every CU gets a
+  // workgroup from the (sequence, KV head, query tile) pairs alone; "attn_variant" 2 asks for it
+  // whenever the partition count allows.
+  const int64_t pairs = batch * hkv * p.gtiles;
+  p.wg_merge = !lean && p.n_part > 1 && p.n_part <= wg_max_parts((int)d, gt) &&
+               (cx.attn_variant == 2 || (cx.attn_variant < 0 && pairs >= cx.num_cu));
+  if (p.n_part > 1 && !lean && !p.wg_merge) {
     const size_t rows = (size_t)batch * hq;
     const size_t o_bytes = rows * p.n_part * d * sizeof(float);
     const size_t ml_bytes = rows * p.n_part * 2 * sizeof(float);
@@ -1233,7 +1371,7 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     p.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + o_bytes);
   }
   // The merge kernel writes the 16-bit copy; without a merge a cast kernel follows.
-  const bool merged = p.n_part > 1 || p.n_wg > 0;
+  const bool merged = p.n_part > 1 || p.n_wg > 0;  // (the workgroup form merges too: n_part > 1)
   if (merged) {
     // the merge kernel writes the copy, blocked on request; without a merge a cast kernel writes it row-major
     p.out16 = out16;
@@ -1317,7 +1455,8 @@ extern "C" int pto_hip_paged_attention_stream_probe(const void* key_cache, const
                                                     const int32_t* block_table, const int32_t* context_lens,
                                                     const int64_t* config, int q_dtype, int kv_dtype, int rounds,
                                                     void* stream, double* mean_ns) {
-  PTO_DISPATCH_LOCK();
+  // The dispatch lock covers planning and each launch, not the waits for the launches.
+  std::unique_lock<std::recursive_mutex> lock(pto_hip::dispatch_mutex());
   pto_hip::Context& cx = pto_hip::ctx();
   if (!cx.initialized) return pto_hip::fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(config && mean_ns, "stream_probe: config or mean_ns is null");
@@ -1349,12 +1488,15 @@ extern "C" int pto_hip_paged_attention_stream_probe(const void* key_cache, const
   double total_ms = 0.0;
   int status = PTO_HIP_OK;
   for (int r = 0; r < rounds && status == PTO_HIP_OK; ++r) {
+    if (!lock.owns_lock()) lock.lock();
     if (d == 128 && fp8) hipExtLaunchKernelGGL((attn_stream_probe_kernel<128, true>), grid, dim3(64), lds, hs, e0, e1, 0, p);
     else if (d == 128) hipExtLaunchKernelGGL((attn_stream_probe_kernel<128, false>), grid, dim3(64), lds, hs, e0, e1, 0, p);
     else if (fp8) hipExtLaunchKernelGGL((attn_stream_probe_kernel<256, true>), grid, dim3(64), lds, hs, e0, e1, 0, p);
     else hipExtLaunchKernelGGL((attn_stream_probe_kernel<256, false>), grid, dim3(64), lds, hs, e0, e1, 0, p);
     float ms = 0.f;
-    if (hipGetLastError() != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+    const bool launched = hipGetLastError() == hipSuccess;
+    lock.unlock();
+    if (!launched || hipEventSynchronize(e1) != hipSuccess ||
         hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
       status = pto_hip::fail(PTO_HIP_ERR_RUNTIME, "stream_probe: launch %d failed", r);
     total_ms += ms;

@@ -863,6 +863,13 @@ int pto_hip_close(void) {
   c.gemm_ws_bytes = 0;
   for (void* old : c.retired) release(old, "hipFree(retired workspace)");
   c.retired.clear();
+  // event pairs of "attn_kernel_timing" that were never read
+  for (auto& pr : c.attn_timed) {
+    (void)hipEventDestroy(pr.first);
+    (void)hipEventDestroy(pr.second);
+  }
+  c.attn_timed.clear();
+  c.attn_kernel_timing = 0;
   c.initialized = false;
   {
     std::lock_guard<std::mutex> lk(g_mu);
@@ -926,9 +933,12 @@ int pto_hip_copy_from(void* dst_host_ptr, uint64_t src_dev_ptr, size_t nbytes) {
 }
 
 int pto_hip_sync(void* stream) {
-  PTO_DISPATCH_LOCK();
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
+  // The wait runs without the dispatch lock: a thread blocked on its stream must not keep the
+  // others from launching.  The lock is taken for the flags only.
   PTO_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
+  PTO_DISPATCH_LOCK();
+  if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "the library was closed during the wait");
   // Device-side argument errors of launches that do not block are reported here.
   int flags[3] = {0, 0, 0};
   PTO_CHECK_HIP(hipMemcpy(flags, ctx().flags, sizeof(flags), hipMemcpyDeviceToHost));
@@ -1000,7 +1010,8 @@ int pto_hip_kernel_entry(int callable_id, int64_t* args, int n_tensors, int n_sc
 int pto_hip_benchmark(int callable_id, const PtoHipChipTensor* tensors, int n_sets, int n_tensors,
                       const uint64_t* scalars, int n_scalars, int rounds, int warmup, void* stream,
                       float* avg_us) {
-  PTO_DISPATCH_LOCK();
+  // No dispatch lock here: every pto_hip_run below takes it for its own launch, and the waits on
+  // the stream and on the closing event run without it.
   if (!ctx().initialized) return fail(PTO_HIP_ERR_NOT_INITIALIZED, "pto_hip_init has not been called");
   PTO_CHECK_ARG(n_sets >= 1 && rounds >= 1 && warmup >= 0 && avg_us, "benchmark: bad arguments");
   hipStream_t st = (hipStream_t)stream;
@@ -1047,7 +1058,7 @@ int pto_hip_set_option(const char* name, int64_t value) {
     PTO_CHECK_ARG(value == 0 || value == 1 || value == 2 || value == 4, "attn_group_tiles must be 0, 1, 2 or 4");
     c.attn_group_tiles = value;
   } else if (!std::strcmp(name, "attn_variant")) {
-    PTO_CHECK_ARG(value >= -1 && value <= 1, "attn_variant must be -1, 0 or 1");
+    PTO_CHECK_ARG(value >= -1 && value <= 2, "attn_variant must be -1, 0, 1 or 2");
     c.attn_variant = value;
   } else if (!std::strcmp(name, "attn_kernel_timing")) {
     c.attn_kernel_timing = value != 0;
@@ -1066,6 +1077,7 @@ int pto_hip_set_option(const char* name, int64_t value) {
   } else if (!std::strcmp(name, "w8a16_gemm_rows")) {
     PTO_CHECK_ARG(value >= 0 && value <= (1 << 20), "w8a16_gemm_rows must be in [0, 2^20]");
     c.w8a16_gemm_rows = value;
+
   } else {
     return fail(PTO_HIP_ERR_NOT_FOUND, "unknown option '%s'", name);
   }
