@@ -509,9 +509,12 @@ PTO_HIP_API int pto_hip_backend_handler_query(const char* hook, int32_t arg, cha
  *                               not for launches under graph capture)
  *  "attn_kernel_time_ns"        read only: mean interval of the pairs recorded since the last read, in
  *                               nanoseconds (0 when there are none); waits for the last recorded launch
- *  "attn_variant"               0 = one wavefront per (sequence, KV head, partition), 1 = one pinned
- *                               workgroup per CU and the chunk list cut evenly over their wavefronts,
- *                               -1 = by launch size and table capacity (default)
+ *  "attn_variant"               0 = one wavefront per (sequence, KV head, partition) and a merge launch,
+ *                               1 = one pinned workgroup per CU and the chunk list cut evenly over
+ *                               their wavefronts, 2 = one workgroup per (sequence, KV head, query
+ *                               tile) whose wavefronts take the partitions and merge through LDS (up
+ *                               to 8 partitions; bit-identical to 0), -1 = by launch size, table
+ *                               capacity and the number of (sequence, KV head) pairs (default)
  *  "attn_group_tiles"           cap on the 16-head query tiles one wavefront carries: 0 = the whole KV
  *                               group up to 64 heads (32 at head_dim 256), the cache read once per
  *                               group (default); 1, 2, 4 = at most that many, read once per wavefront
