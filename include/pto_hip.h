@@ -504,6 +504,15 @@ PTO_HIP_API int pto_hip_backend_handler_query(const char* hook, int32_t arg, cha
  *  "attn_tokens_per_partition"  0 = choose from the device's CU count (default)
  *  "attn_waves_per_cu"          cap on resident attention wavefronts per CU, 0 = none (default); for
  *                               the evenly split form the wavefronts per CU (0 = 4, at most 8)
+ *  "attn_autotune"              1 = while "attn_waves_per_cu" is 0 and "attn_variant" is -1, the first calls of
+ *                               every launch signature (shape, types, partition size) time a short list
+ *                               of launch shapes that give bit-identical results (residency caps 0, 2,
+ *                               3, 4 of the partition grid and, with up to 8 partitions, the workgroup
+ *                               form) with events read back on later calls - nothing blocks - and the
+ *                               fastest is used from then on (default); 0 = the fixed rule only.  Calls
+ *                               under stream capture and pto_hip_paged_attention_noalloc never measure.
+ *  "attn_tuned_waves_per_cu"    read only: the cap the last launch's signature settled on (-1 = not yet)
+ *  "attn_tuned_workgroup_form"  read only: 1 when it settled on the workgroup form, 0 the grid, -1 = not yet
  *  "attn_kernel_timing"         1 = every paged-attention launch gives its streaming kernel a start and a stop
  *                               HIP event that take the dispatch's own timestamps (results are unaffected;
  *                               not for launches under graph capture)

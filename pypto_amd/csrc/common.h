@@ -64,6 +64,7 @@ struct Context {
   int64_t attn_kernel_timing = 0;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> attn_timed;
   int64_t attn_group_tiles = 0;  // cap on the query tiles one wavefront carries (0 = by group size)
+  int64_t attn_autotune = 1;     // first calls of a launch signature time bit-identical launch shapes and keep the fastest
   int64_t gemm_variant = 0;
   int64_t gemm_splits = 0;       // k splits of the tiled GEMM: 0 = by shape, 1..16 = as given (when k allows)
   int64_t w8a16_wgs_per_cu = 1;  // workgroups of the W8A16 partial kernel aimed at per compute unit
@@ -166,6 +167,10 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
                     const int64_t* config, int q_dtype, int kv_dtype, const float* k_scale,
                     const float* v_scale, int64_t pool_blocks, void* stream, void* fixed_scratch = nullptr,
                     size_t fixed_scratch_bytes = 0, int64_t active_blocks = -1);
+// Forgets every measured launch shape (and releases the events of measurements in flight).
+void attention_tuning_reset();
+// Residency cap and form (1 = workgroup form) the last launch's signature was tuned to; -1 while untuned.
+void attention_tuning_last(int64_t* cap, int64_t* wg);
 // The same contract for the shapes the tiled kernels are not built for (head_dim other than 128 / 256
 // up to 256, block sizes off the 16-token grid); attention_needs_generic says which launches take it.
 bool attention_needs_generic(const int64_t* config, int kv_dtype);

@@ -17,8 +17,11 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <array>
 #include <atomic>
+#include <map>
 #include <mutex>
+#include <vector>
 #include <type_traits>
 
 #include "common.h"
@@ -1278,6 +1281,91 @@ int plan_launch(const int64_t* config, int q_dtype, int kv_dtype, bool have_scal
 }
 }  // namespace
 
+namespace {
+// ---- launch shape by measurement ------------------------------------------------------------
+// How a launch spreads over the CUs depends on how ragged the context lengths are, which the host
+// does not see (they live in device memory).  For every launch signature the first calls therefore
+// time a short list of shapes that all give bit-identical results - residency caps of the
+// partition grid and, where the partition count allows it, the workgroup form - with a pair of
+// events around each call's launches, read back without blocking on later calls; once every
+// candidate has kTuneReps readings the fastest is used from then on.  Calls made while a stream
+// is being captured, and the entry point that allocates nothing, never measure.
+struct TuneCandidate {
+  int cap;      // residency cap of the partition grid (0 = none)
+  bool wg;      // workgroup form
+};
+struct TunePending {
+  int cand;
+  hipEvent_t e0, e1;
+};
+struct TuneState {
+  std::vector<TuneCandidate> cands;
+  std::vector<float> best_us;
+  std::vector<int> issued, done;
+  std::vector<TunePending> pending;
+  int chosen = -1;
+};
+constexpr int kTuneReps = 4;
+typedef std::array<int64_t, 12> TuneKey;
+std::map<TuneKey, TuneState>& tune_table() {
+  static std::map<TuneKey, TuneState> t;
+  return t;
+}
+TuneState* g_last_tuned = nullptr;  // state of the last launch that took part in tuning
+
+void tune_harvest(TuneState& ts) {
+  for (size_t i = 0; i < ts.pending.size();) {
+    TunePending& pd = ts.pending[i];
+    if (hipEventQuery(pd.e1) != hipSuccess) {
+      (void)hipGetLastError();
+      ++i;
+      continue;
+    }
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, pd.e0, pd.e1) == hipSuccess) {
+      ts.best_us[pd.cand] = std::min(ts.best_us[pd.cand], ms * 1e3f);
+      ++ts.done[pd.cand];
+    } else {
+      (void)hipGetLastError();
+      --ts.issued[pd.cand];  // measure it again
+    }
+    (void)hipEventDestroy(pd.e0);
+    (void)hipEventDestroy(pd.e1);
+    ts.pending[i] = ts.pending.back();
+    ts.pending.pop_back();
+  }
+  if (ts.chosen < 0) {
+    bool all = true;
+    for (int d : ts.done) all = all && d >= kTuneReps;
+    if (all) {
+      ts.chosen = 0;
+      for (size_t c = 1; c < ts.cands.size(); ++c)
+        if (ts.best_us[c] < ts.best_us[ts.chosen] * 0.99f) ts.chosen = (int)c;  // a candidate must win by 1 %
+    }
+  }
+}
+}  // namespace
+
+namespace pto_hip {
+void attention_tuning_reset() {
+  for (auto& kv : tune_table())
+    for (TunePending& pd : kv.second.pending) {
+      (void)hipEventDestroy(pd.e0);
+      (void)hipEventDestroy(pd.e1);
+    }
+  tune_table().clear();
+  g_last_tuned = nullptr;
+}
+void attention_tuning_last(int64_t* cap, int64_t* wg) {
+  *cap = *wg = -1;
+  if (!g_last_tuned) return;
+  tune_harvest(*g_last_tuned);  // readings that have arrived since the last launch
+  if (g_last_tuned->chosen < 0) return;
+  *cap = g_last_tuned->cands[g_last_tuned->chosen].cap;
+  *wg = g_last_tuned->cands[g_last_tuned->chosen].wg ? 1 : 0;
+}
+}  // namespace pto_hip
+
 namespace pto_hip {
 int paged_attention(const void* query, const void* key_cache, const void* value_cache,
                     const int32_t* block_table, const int32_t* context_lens, float* out, void* out16,
@@ -1340,8 +1428,44 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   // workgroup from the (sequence, KV head, query tile) pairs alone; "attn_variant" 2 asks for it
   // whenever the partition count allows.
   const int64_t pairs = batch * hkv * p.gtiles;
-  p.wg_merge = !lean && p.n_part > 1 && p.n_part <= wg_max_parts((int)d, gt) &&
-               (cx.attn_variant == 2 || (cx.attn_variant < 0 && pairs >= cx.num_cu));
+  const bool wg_possible = !lean && p.n_part > 1 && p.n_part <= wg_max_parts((int)d, gt);
+  p.wg_merge = wg_possible && (cx.attn_variant == 2 || (cx.attn_variant < 0 && pairs >= cx.num_cu));
+
+  // Launch shape by measurement (see TuneState): only while the caller has not fixed the shape.
+  hipStream_t hs = (hipStream_t)stream;
+  TuneState* ts = nullptr;
+  int measuring = -1;
+  if (cx.attn_autotune != 0 && cx.attn_waves_per_cu == 0 && cx.attn_variant < 0 && !lean) {
+    const TuneKey key = {batch, hq, hkv, d, config[4], config[5], (int64_t)q_dtype, (int64_t)kv_dtype, (int64_t)p.ctx_cap,
+                         (int64_t)p.tpp, (int64_t)gt, (int64_t)(out16 != nullptr)};
+    ts = &tune_table()[key];
+    if (ts->cands.empty()) {
+      ts->cands.push_back({0, p.wg_merge != 0});  // the rule's own choice first
+      if (wg_possible) ts->cands.push_back({0, p.wg_merge == 0});
+      for (int cap : {3, 2, 4}) ts->cands.push_back({cap, false});
+      ts->best_us.assign(ts->cands.size(), 1e30f);
+      ts->issued.assign(ts->cands.size(), 0);
+      ts->done.assign(ts->cands.size(), 0);
+    }
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(hs, &capturing) != hipSuccess) {
+      (void)hipGetLastError();
+      capturing = hipStreamCaptureStatusActive;  // unknown: do not touch events
+    }
+    const bool may_measure = capturing == hipStreamCaptureStatusNone && !fixed_scratch;
+    if (may_measure) tune_harvest(*ts);
+    int use = ts->chosen >= 0 ? ts->chosen : 0;
+    if (ts->chosen < 0 && may_measure) {
+      for (size_t c = 0; c < ts->cands.size(); ++c)
+        if (ts->issued[c] < kTuneReps) {
+          measuring = use = (int)c;
+          break;
+        }
+    }
+    p.resident_cap = ts->cands[use].cap;
+    p.wg_merge = ts->cands[use].wg ? 1 : 0;
+    g_last_tuned = ts;
+  }
   if (p.n_part > 1 && !lean && !p.wg_merge) {
     const size_t rows = (size_t)batch * hq;
     const size_t o_bytes = rows * p.n_part * d * sizeof(float);
@@ -1379,8 +1503,16 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     if (wrote_blocked) *wrote_blocked = p.out16_blocked != 0;
   }
   int rc;
-  hipStream_t hs = (hipStream_t)stream;
   const int nb = (int)batch;
+  hipEvent_t te0 = nullptr, te1 = nullptr;
+  if (measuring >= 0) {
+    if (hipEventCreate(&te0) != hipSuccess || hipEventCreate(&te1) != hipSuccess || hipEventRecord(te0, hs) != hipSuccess) {
+      (void)hipGetLastError();
+      if (te0) (void)hipEventDestroy(te0);
+      if (te1) (void)hipEventDestroy(te1);
+      measuring = -1;
+    }
+  }
   if (d == 128) {
     if (fp8) rc = gt == 1 ? launch<128, true, 1>(p, nb, bf16, hs) : gt == 2 ? launch<128, true, 2>(p, nb, bf16, hs)
                                                                            : launch<128, true, 4>(p, nb, bf16, hs);
@@ -1390,8 +1522,18 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     if (fp8) rc = gt == 1 ? launch<256, true, 1>(p, nb, bf16, hs) : launch<256, true, 2>(p, nb, bf16, hs);
     else rc = gt == 1 ? launch<256, false, 1>(p, nb, bf16, hs) : launch<256, false, 2>(p, nb, bf16, hs);
   }
-  if (rc || !out16 || merged) return rc;
-  return cast_from_f32(out, out16, (size_t)batch * hq * d, q_dtype, (hipStream_t)stream);
+  if (!rc && out16 && !merged) rc = cast_from_f32(out, out16, (size_t)batch * hq * d, q_dtype, (hipStream_t)stream);
+  if (measuring >= 0) {
+    if (!rc && hipEventRecord(te1, hs) == hipSuccess) {
+      ts->pending.push_back({measuring, te0, te1});
+      ++ts->issued[measuring];
+    } else {
+      (void)hipGetLastError();
+      (void)hipEventDestroy(te0);
+      (void)hipEventDestroy(te1);
+    }
+  }
+  return rc;
 }
 }  // namespace pto_hip
 

@@ -863,6 +863,7 @@ int pto_hip_close(void) {
   c.gemm_ws_bytes = 0;
   for (void* old : c.retired) release(old, "hipFree(retired workspace)");
   c.retired.clear();
+  attention_tuning_reset();
   // event pairs of "attn_kernel_timing" that were never read
   for (auto& pr : c.attn_timed) {
     (void)hipEventDestroy(pr.first);
@@ -1060,6 +1061,10 @@ int pto_hip_set_option(const char* name, int64_t value) {
   } else if (!std::strcmp(name, "attn_variant")) {
     PTO_CHECK_ARG(value >= -1 && value <= 2, "attn_variant must be -1, 0, 1 or 2");
     c.attn_variant = value;
+  } else if (!std::strcmp(name, "attn_autotune")) {
+    PTO_CHECK_ARG(value == 0 || value == 1, "attn_autotune must be 0 or 1");
+    c.attn_autotune = value;
+    if (value == 0) attention_tuning_reset();
   } else if (!std::strcmp(name, "attn_kernel_timing")) {
     c.attn_kernel_timing = value != 0;
   } else if (!std::strcmp(name, "attn_waves_per_cu")) {
@@ -1119,6 +1124,12 @@ int pto_hip_get_option(const char* name, int64_t* value) {
     *value = n ? (int64_t)(total_ms * 1e6 / (double)n) : 0;
   }
   else if (!std::strcmp(name, "attn_variant")) *value = c.attn_variant;
+  else if (!std::strcmp(name, "attn_autotune")) *value = c.attn_autotune;
+  else if (!std::strcmp(name, "attn_tuned_waves_per_cu") || !std::strcmp(name, "attn_tuned_workgroup_form")) {
+    int64_t cap = -1, wg = -1;
+    attention_tuning_last(&cap, &wg);
+    *value = !std::strcmp(name, "attn_tuned_waves_per_cu") ? cap : wg;
+  }
   else if (!std::strcmp(name, "attn_group_tiles")) *value = c.attn_group_tiles;
   else if (!std::strcmp(name, "w8a16_wgs_per_cu")) *value = c.w8a16_wgs_per_cu;
   else if (!std::strcmp(name, "w8a16_min_steps")) *value = c.w8a16_min_steps;

@@ -585,7 +585,9 @@ def autotune_attention(worker: ChipWorker, handle: RegistrationHandle, arg_sets:
     for tpp, cap in candidates:
         worker.set_option("attn_tokens_per_partition", tpp)
         worker.set_option("attn_waves_per_cu", cap)
-        prepared.run(max(rounds // 3, 1))
+        # (0, 0) leaves the choice to the library, whose own first calls of a launch signature time
+        # a few shapes: the warm-up is long enough for it to have settled
+        prepared.run(max(rounds, 40))
         timings[(tpp, cap)] = prepared.run(rounds).device_wall_us
     best = min(timings, key=timings.get)
     worker.set_option("attn_tokens_per_partition", best[0])
