@@ -147,7 +147,7 @@ def main() -> int:
 
     from pypto_amd import workloads
     from pypto_amd.runtime import (ChipWorker, PreparedBenchmark, RunConfig, attention_stream_probe,
-                                   autotune_attention, benchmark,
+                                   autotune_attention, benchmark, mfma_only_probe,
                                    decoder_layer_decode, decoder_layer_decode_w16, ffn_block, ffn_block_fp8,
                                    paged_attention,
                                    projection)
@@ -296,6 +296,28 @@ def main() -> int:
             "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
             "bound": "mfma",
         }
+        # Ceiling of the MFMA pipes on this workload's own operand values: the GEMM's instruction, accumulator
+        # tiles and wavefronts per CU, fragments loaded once from x and W_gate, nothing else in the loop.
+        mf = mfma_only_probe(worker, f.x, f.w_gate, iters=1500, warm_rounds=100, rounds=60)
+        result["ffn"]["mfma_only_tflops"] = round(mf["tflops"], 1)
+        result["ffn"]["frac_of_mfma_only"] = round(tflops / mf["tflops"], 4)
+        # The vendor library's two products on the same tensors (no RMSNorm, no SwiGLU): reported, not a target.
+        xg = torch.cat([f.w_gate, f.w_up], dim=1)
+        hv = torch.empty(f.x.shape[0], f.w_down.shape[0], dtype=f.x.dtype, device="cuda").normal_()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        for _ in range(60):
+            torch.matmul(f.x, xg)
+            torch.matmul(hv, f.w_down)
+        ev[0].record()
+        for _ in range(40):
+            torch.matmul(f.x, xg)
+            torch.matmul(hv, f.w_down)
+        ev[1].record()
+        torch.cuda.synchronize()
+        result["ffn"]["vendor_gemm_us"] = round(ev[0].elapsed_time(ev[1]) * 1e3 / 40, 1)
+        result["ffn"]["vendor_gemm_note"] = ("torch.matmul of x[2048,4096] @ [W_gate|W_up][4096,22016] and "
+                                             "h[2048,11008] @ W_down[11008,4096], bf16, back to back")
+        del xg, hv
         if not args.no_ffn_clock_probe:
             result["ffn"]["clock_probe"] = _ffn_clock_probe(worker, ffn_block, fargs[0], (0, 2, 3, 4))
         if cpu:

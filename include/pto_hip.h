@@ -239,6 +239,19 @@ PTO_HIP_API int pto_hip_paged_attention_stream_probe(const void* key_cache, cons
                                                      const int64_t* config, int q_dtype, int kv_dtype, int rounds,
                                                      void* stream, double* mean_ns);
 
+/* Measurement aid with no counterpart in the reference: the rate of the MFMA pipes on the caller's own
+ * operand values with nothing else in the loop.  A kernel with the FFN GEMM's instruction
+ * (v_mfma_f32_32x32x16 of `dtype`), its 4 x 2 accumulator tiles per wavefront and its eight
+ * wavefronts per CU loads a few operand fragments per lane once from a[0 .. a_elems) and
+ * b[0 .. b_elems) (16-bit elements, 16-byte aligned) and then issues `iters` x 32 MFMAs per wavefront
+ * from registers alone.  It is launched warm_rounds + rounds times; *mean_us receives the mean time of
+ * the last `rounds` launches and *flops_per_launch the arithmetic one launch does.  Because the shader
+ * clock under MFMA load depends on the operand bits, the rate on a workload's own tensors - not on
+ * constants - is the ceiling the GEMM's schedule can approach on that workload.  Blocks until done. */
+PTO_HIP_API int pto_hip_mfma_probe(const void* a, int64_t a_elems, const void* b, int64_t b_elems, int dtype, int iters,
+                                   int warm_rounds, int rounds, void* stream, double* mean_us,
+                                   double* flops_per_launch);
+
 /* out[i, :] = src[block_table[idx / bs] * bs + idx % bs, col_offset : col_offset + size]
  * (src/ir/op/tensor_ops/paged_gather.cpp:74-199), bit-exact, asynchronous on the stream.  An index
  * that addresses a block outside block_table or a row outside src is skipped and reported by
@@ -513,6 +526,7 @@ PTO_HIP_API int pto_hip_backend_handler_query(const char* hook, int32_t arg, cha
  *                               under stream capture and pto_hip_paged_attention_noalloc never measure.
  *  "attn_tuned_waves_per_cu"    read only: the cap the last launch's signature settled on (-1 = not yet)
  *  "attn_tuned_workgroup_form"  read only: 1 when it settled on the workgroup form, 0 the grid, -1 = not yet
+ *  "workspace_bytes"            read only: bytes of device memory the library's grow-only scratch areas hold
  *  "attn_kernel_timing"         1 = every paged-attention launch gives its streaming kernel a start and a stop
  *                               HIP event that take the dispatch's own timestamps (results are unaffected;
  *                               not for launches under graph capture)

@@ -651,7 +651,8 @@ extern "C" int pto_hip_gate_up_swiglu_fp8(const void* x8, const float* x_scale, 
   if (m == 0) return PTO_HIP_OK;
   PTO_CHECK_ARG(x8 && x_scale && w_gate8 && w_gate_scale && w_up8 && w_up_scale && h,
                 "gate_up_swiglu_fp8: null tensor pointer");
-  PTO_CHECK_ARG((uintptr_t)w_up8 % 16 == 0, "gate_up_swiglu_fp8: operand pointers must be 16-byte aligned");
+  PTO_CHECK_ARG(((uintptr_t)w_up8 | (uintptr_t)w_gate_scale | (uintptr_t)w_up_scale) % 16 == 0,
+                "gate_up_swiglu_fp8: operand and channel-scale pointers must be 16-byte aligned");
   PTO_CHECK_ARG(h_dtype == PTO_HIP_BF16 || h_dtype == PTO_HIP_FP16, "gate_up_swiglu_fp8: h dtype %s not in {BF16, FP16}",
                 dtype_name(h_dtype));
   gemm8::Params p{};
@@ -681,6 +682,8 @@ extern "C" int pto_hip_projection_fp8(const void* a8, const float* a_scale, cons
   if (rc) return rc;
   if (m == 0) return PTO_HIP_OK;
   PTO_CHECK_ARG(a8 && a_scale && w8 && w_scale && out, "projection_fp8: null tensor pointer");
+  // the split-k finish and the tile epilogue read the channel scales four at a time
+  PTO_CHECK_ARG((uintptr_t)w_scale % 16 == 0, "projection_fp8: the channel scales must be 16-byte aligned");
   gemm8::Params p{};
   p.a = reinterpret_cast<const uint8_t*>(a8);
   p.b0 = reinterpret_cast<const uint8_t*>(w8);
@@ -726,8 +729,13 @@ extern "C" int pto_hip_ffn_swiglu_fp8(const void* x, const float* gamma, const v
     return fail(PTO_HIP_ERR_UNSUPPORTED, "ffn_fp8: hidden %lld and intermediate %lld must be multiples of %d",
                 (long long)hidden, (long long)intermediate, gemm8::BK);
   PTO_CHECK_ARG(((uintptr_t)x | (uintptr_t)gamma | (uintptr_t)w_gate8 | (uintptr_t)w_up8 | (uintptr_t)w_down8 |
-                 (uintptr_t)out) % 16 == 0,
-                "ffn_fp8: operand pointers must be 16-byte aligned");
+                 (uintptr_t)out | (uintptr_t)w_gate_scale | (uintptr_t)w_up_scale | (uintptr_t)w_down_scale) % 16 == 0,
+                "ffn_fp8: operand and channel-scale pointers must be 16-byte aligned");
+  // the row quantiser keeps a whole row in registers: refuse longer rows before anything is queued
+  constexpr int64_t kMaxRow = (int64_t)8 * gemm8::kRowThreads * gemm8::kRowVecs;
+  if (hidden > kMaxRow || intermediate > kMaxRow)
+    return fail(PTO_HIP_ERR_UNSUPPORTED, "ffn_fp8: hidden %lld and intermediate %lld may be at most %lld (the per-row "
+                "quantiser holds a row in registers)", (long long)hidden, (long long)intermediate, (long long)kMaxRow);
   hipStream_t st = (hipStream_t)stream;
 
   auto pad = [](size_t b) { return (b + 255) / 256 * 256; };

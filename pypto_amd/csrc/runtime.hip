@@ -1125,6 +1125,8 @@ int pto_hip_get_option(const char* name, int64_t* value) {
   }
   else if (!std::strcmp(name, "attn_variant")) *value = c.attn_variant;
   else if (!std::strcmp(name, "attn_autotune")) *value = c.attn_autotune;
+  else if (!std::strcmp(name, "workspace_bytes"))  // read only: device memory the three grow-only scratch areas hold
+    *value = (int64_t)(c.workspace_bytes + c.layer_ws_bytes + c.gemm_ws_bytes);
   else if (!std::strcmp(name, "attn_tuned_waves_per_cu") || !std::strcmp(name, "attn_tuned_workgroup_form")) {
     int64_t cap = -1, wg = -1;
     attention_tuning_last(&cap, &wg);

@@ -621,6 +621,27 @@ def attention_stream_probe(worker: ChipWorker, key_cache: torch.Tensor, value_ca
     return mean_ns.value / 1e3
 
 
+def mfma_only_probe(worker: ChipWorker, a: torch.Tensor, b: torch.Tensor, *, iters: int = 1500, warm_rounds: int = 100,
+                    rounds: int = 60, stream: int = 0) -> dict:
+    """Rate of the MFMA pipes on the values of ``a`` and ``b`` with nothing else in the loop.
+
+    Runs the library's register-only MFMA kernel (the FFN GEMM's instruction, accumulator tiles and
+    wavefronts per CU; operand fragments loaded once from the two tensors) and returns
+    ``{"us": mean time per launch, "tflops": rate}``.  The shader clock under MFMA load depends on the
+    operand bits, so this figure for a workload's own tensors is the ceiling its GEMM can approach.
+    """
+    worker._require_ready("mfma_only_probe")
+    for name, t in (("a", a), ("b", b)):
+        if not t.is_cuda or not t.is_contiguous() or t.dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError(f"mfma_only_probe: {name} must be a contiguous 16-bit device tensor")
+    if a.dtype != b.dtype:
+        raise ValueError("mfma_only_probe: a and b must have the same dtype")
+    us, flops = C.c_double(0.0), C.c_double(0.0)
+    _lib.check(worker._lib.pto_hip_mfma_probe(a.data_ptr(), a.numel(), b.data_ptr(), b.numel(), _dtype_code(a.dtype),
+                                              int(iters), int(warm_rounds), int(rounds), stream, C.byref(us), C.byref(flops)))
+    return {"us": us.value, "tflops": flops.value / us.value / 1e6}
+
+
 def benchmark(
     handle: RegistrationHandle,
     arg_sets: Sequence[Sequence[Any]],
@@ -655,7 +676,13 @@ def validate_golden(
     """
     limit = 20
     for name, produced in outputs.items():
-        got, want = produced.detach().cpu().reshape(-1), golden[name].detach().cpu().reshape(-1)
+        got, want = produced.detach().cpu(), golden[name].detach().cpu()
+        # torch.isclose on the tensors as they are fails a shape that does not broadcast (as the
+        # reference's comparison does); two shapes with the same element count must not pass by
+        # being compared in memory order either
+        if got.shape != want.shape:
+            raise AssertionError(f"Output '{name}' has shape {tuple(got.shape)}, golden has {tuple(want.shape)}.")
+        got, want = got.reshape(-1), want.reshape(-1)
         ignored = want.isnan()
         wrong = ~(torch.isclose(got, want, rtol=rtol, atol=atol) | ignored)
         n_wrong = int(wrong.sum())

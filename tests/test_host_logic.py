@@ -53,6 +53,14 @@ def test_validate_golden_nan_is_dont_care():
     validate_golden({"o": actual}, {"o": actual + 1e-3}, rtol=1e-2, atol=1e-2)
 
 
+def test_validate_golden_refuses_a_shape_mismatch():
+    """Same element count, other shape: compared in memory order it could pass; it must not."""
+    got = torch.arange(6, dtype=torch.float32).reshape(2, 3)
+    with pytest.raises(AssertionError, match=r"shape \(2, 3\), golden has \(3, 2\)"):
+        validate_golden({"o": got}, {"o": got.reshape(3, 2)})
+    validate_golden({"o": got}, {"o": got.clone()})
+
+
 def test_argument_count_and_kinds():
     with pytest.raises(ValueError, match="takes 7..9 tensors"):
         runtime._split_args(runtime.paged_attention, [1, 2, 3])
