@@ -126,8 +126,8 @@ namespace pto_hip {
 
 bool gemm_w8_fits(const void* x, const void* wq0, const void* wq1, const void* residual, const void* out, int64_t m,
                   int64_t k, int64_t n, int x_dtype, int out_dtype) {
-  const int64_t from = ctx().w8a16_gemm_rows, variant = ctx().gemm_variant;
-  return from > 0 && m >= from && (variant == 0 || variant >= 4) && k % 8 == 0 && n % 16 == 0 &&
+  const int64_t from = ctx().w8a16_gemm_rows;
+  return from > 0 && m >= from && k % 8 == 0 && n % 16 == 0 &&
          ((uintptr_t)x | (uintptr_t)wq0 | (uintptr_t)wq1 | (uintptr_t)residual | (uintptr_t)out) % 16 == 0 &&
          (x_dtype == PTO_HIP_BF16 || x_dtype == PTO_HIP_FP16) && (out_dtype == PTO_HIP_FP32 || out_dtype == x_dtype);
 }

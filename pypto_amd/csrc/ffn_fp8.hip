@@ -402,10 +402,6 @@ int launch(Params p, hipStream_t st) {
   return PTO_HIP_OK;
 }
 
-// Tile height: 256 rows unless that leaves CUs idle and 128 rows do not.  Eight wavefronts (two per
-// SIMD) by default; "gemm_variant" 1 selects four wavefronts of 128 x 128 on the tall tile, which
-// read a third less from LDS per MFMA but leave a SIMD nothing to issue while its one wavefront
-// waits (LLaMA-7B block: 361 us against 334 us).
 // Sum of the k splits' slabs in split order, times the row and column scales, cast and store.
 template <typename OutT>
 __global__ __launch_bounds__(256) void gemm8_finish_kernel(const float* __restrict__ slabs, int splits,
@@ -429,10 +425,10 @@ __global__ __launch_bounds__(256) void gemm8_finish_kernel(const float* __restri
   }
 }
 
-// Tile height: 256 rows unless that leaves CUs idle and 128 rows do not.  Eight wavefronts (two per
-// SIMD) by default; "gemm_variant" 1 selects four wavefronts of 128 x 128 on the tall tile, which
-// read a third less from LDS per MFMA but leave a SIMD nothing to issue while its one wavefront
-// waits (LLaMA-7B block: 361 us against 334 us).
+// Tile height: 256 rows unless that leaves CUs idle and 128 rows do not; eight wavefronts (two per
+// SIMD).  Four wavefronts of 128 x 128 on the tall tile read a third less from LDS per MFMA but
+// leave a SIMD nothing to issue while its one wavefront waits (LLaMA-7B block: 361 us against 334 us
+// when it was measured; that form is not built any more).
 // A single-operand pass whose tall tiles fill at most half the CUs splits k instead of halving the
 // tile: a k-tile takes a workgroup the same ~1.4 us with 128 rows as with 256 (the tile's arrival,
 // not the MFMAs, sets it), so two workgroups per 256 x 256 tile do the same work in half the k-tiles.
@@ -467,7 +463,6 @@ int launch_any(const Params& p0, hipStream_t st) {
     }
   }
   if (tall < num_cu && p.m > 128) return launch<2, 2, 2, 4, DUAL, OutT>(p, st);
-  if (pto_hip::ctx().gemm_variant == 1) return launch<4, 4, 2, 2, DUAL, OutT>(p, st);
   return launch<4, 2, 2, 4, DUAL, OutT>(p, st);
 }
 

@@ -556,16 +556,16 @@ int launch_variant(GemmParams p, hipStream_t st) {
   // over up to 16 workgroups per tile while CUs would idle, beyond that the 256x256 or the 128x256
   // tile and the k split count with the least estimated time (below).  Splits write fp32 slabs
   // that a second kernel sums in split order.
-  // variants 1-3 keep four wavefronts (one per SIMD): 1 = 256x256 tile, 2 = 128x256 tile,
-  // 3 = 256x256 tile with k split in two.  4 = eight wavefronts, 256x256 tile, k split in two
-  // when CUs would idle.  5 = eight wavefronts, 128x256 tile.  6 = eight wavefronts, 64x256 tile, k split while CUs would idle.
+  // The other values force a tile height (the sweeps behind the estimate, and the tests, use them):
+  // 4 = 256x256 tile, k split in two when CUs would idle; 5 = 128x256 tile; 6 = 64x256 tile, k split
+  // while CUs would idle.
   const int64_t tiles_n = (p.n + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256);
   const int64_t big_tiles = (int64_t)((p.m + 255) / 256) * tiles_n;
   const int64_t small_tiles = (int64_t)((p.m + 127) / 128) * tiles_n;
   const bool few = big_tiles < num_cu;
   int want = 1;
   bool small_tile = variant == 5;
-  if (variant == 3 || (variant == 4 && few)) want = 2;
+  if (variant == 4 && few) want = 2;
   if (variant == 0 && p.m > 64) {
     // Estimated time of each (tile height, k splits) pair, in microseconds, fitted to measured
     // launches: rounds of workgroups over the CUs x the k rows one workgroup walks x the time per
@@ -623,11 +623,7 @@ int launch_variant(GemmParams p, hipStream_t st) {
   int rc;
   if (tiny_tile) rc = launch_gemm<1, 2, 4, DUAL, BF16, OutT, W8>(p, st);
   else if (small_tile) rc = launch_gemm<2, 2, 4, DUAL, BF16, OutT, W8>(p, st);
-  else if (variant == 0 || variant == 4) rc = launch_gemm<4, 2, 4, DUAL, BF16, OutT, W8>(p, st);
-  else if constexpr (W8) return pto_hip::fail(PTO_HIP_ERR_UNSUPPORTED, "gemm_variant %lld has no int8-weight form",
-                                              (long long)variant);
-  else if (variant == 2) rc = launch_gemm<2, 2, 2, DUAL, BF16, OutT>(p, st);
-  else rc = launch_gemm<4, 2, 2, DUAL, BF16, OutT>(p, st);
+  else rc = launch_gemm<4, 2, 4, DUAL, BF16, OutT, W8>(p, st);
   if (rc) return rc;
   if (p.partials_out) {  // a fused consumer sums the slabs (one split: the product is in p.c, scales applied)
     pto_hip::W8Partials& o = *p.partials_out;

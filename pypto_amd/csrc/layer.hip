@@ -139,7 +139,6 @@ extern "C" int pto_hip_decoder_layer_decode(const PtoHipDecoderLayerArgs* a, voi
   const bool w16 = n_scales == 0;
   // int8 codes: the tiled GEMM wants 16-byte aligned matrices, and can be switched off.
   const bool gemm8 = cx.w8a16_gemm_rows > 0 && b >= cx.w8a16_gemm_rows &&
-                     (cx.gemm_variant == 0 || cx.gemm_variant >= 4) &&
                      ((uintptr_t)a->wqkv_q | (uintptr_t)a->wo_q | (uintptr_t)a->wg_q | (uintptr_t)a->wu_q |
                       (uintptr_t)a->wd_q) % 16 == 0;
   if (w16 ? b > kW8MaxM : gemm8) return layer_large_batch(a, rope_w, stream);

@@ -55,7 +55,7 @@ def test_options_round_trip_and_ranges():
     lib = _lib.load()
     knobs = {"attn_tokens_per_partition": 256, "attn_waves_per_cu": 4, "attn_kernel_timing": 1, "attn_variant": 1,
              "attn_group_tiles": 2,
-             "gemm_variant": 2, "gemm_splits": 3, "w8a16_wgs_per_cu": 3, "w8a16_min_steps": 16, "w8a16_wide": 0, "w8a16_gemm_rows": 64}
+             "gemm_variant": 5, "gemm_splits": 3, "w8a16_wgs_per_cu": 3, "w8a16_min_steps": 16, "w8a16_wide": 0, "w8a16_gemm_rows": 64}
     for name, value in knobs.items():
         old = ctypes.c_int64(-99)
         _lib.check(lib.pto_hip_get_option(name.encode(), ctypes.byref(old)))
@@ -65,7 +65,7 @@ def test_options_round_trip_and_ranges():
         assert got.value == value, name
         _lib.check(lib.pto_hip_set_option(name.encode(), old.value))
     for name, bad in (("attn_variant", 3), ("attn_group_tiles", 3), ("attn_waves_per_cu", 17), ("attn_tokens_per_partition", -1),
-                      ("w8a16_wgs_per_cu", 0), ("w8a16_min_steps", 0), ("w8a16_wide", 3), ("gemm_variant", 7), ("gemm_splits", 17)):
+                      ("w8a16_wgs_per_cu", 0), ("w8a16_min_steps", 0), ("w8a16_wide", 3), ("gemm_variant", 7), ("gemm_variant", 2), ("gemm_splits", 17)):
         with pytest.raises(ValueError, match=name):
             _lib.check(lib.pto_hip_set_option(name.encode(), bad))
     with pytest.raises(ValueError, match="unknown option"):

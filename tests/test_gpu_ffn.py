@@ -89,7 +89,7 @@ def test_ffn_reference_example_fp32(worker):
     assert torch.allclose(out, oracle.ffn_swiglu(x, wg, wu, wd), rtol=3e-3, atol=3e-3)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [0, 4, 5, 6])
 def test_ffn_tiny_fp16(worker, variant):
     """x[128,512] fp16, I=1024, weights N(0,0.02), seed 0; max-abs 1e-2 / rel 2e-2."""
     inp = workloads.ffn_tiny(seed=0)
@@ -104,7 +104,7 @@ def test_ffn_tiny_fp16(worker, variant):
     validate_golden({"out": inp.out}, {"out": ref32}, rtol=2e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [0, 4, 5, 6])
 @pytest.mark.parametrize("t,h,i", [(256, 512, 1024), (100, 264, 520), (512, 1024, 2816)])
 def test_ffn_block_bf16(worker, variant, t, h, i):
     """RMSNorm prologue + SwiGLU FFN, bf16, incl. shapes that are not tile multiples."""
@@ -164,7 +164,7 @@ def test_ffn_block_decode_sizes(worker, dtype, t, h, i):
     validate_golden({"out": inp.out.float()}, {"out": ref.float()}, rtol=2e-2, atol=1e-2)
     # the tiled GEMM path computes the same block: the two agree far inside the tolerance
     out_skinny = inp.out.clone()
-    worker.set_option("gemm_variant", 1)
+    worker.set_option("gemm_variant", 6)
     with worker.register(ffn_block) as hd:
         hd(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, inp.out, inp.eps)
     worker.set_option("gemm_variant", 0)
@@ -579,28 +579,6 @@ def test_ffn_block_fp8_llama7b_shape_rows_and_distance_to_16_bit(worker):
     worker.sync()
     rel = ((q.out - f.out).norm() / f.out.norm()).item()
     assert 1e-3 < rel < 0.08, rel
-
-
-def test_ffn_block_fp8_four_wavefront_form_is_bit_identical(worker):
-    """"gemm_variant" 1 runs the tall tile with four wavefronts of 128 x 128 instead of eight of 128 x 64:
-    every accumulator still sums its k-steps in the same order, so the results are the same bits."""
-    from pypto_amd.runtime import ffn_block_fp8
-
-    q, _ = workloads.ffn_fp8_inputs(tokens=2048, hidden=512, intermediate=4096, seed=6, device="cuda")
-    worker.set_option("gemm_splits", 1)   # the eight-wavefront form would split the down pass's k, the other does not
-    try:
-        with worker.register(ffn_block_fp8) as hd:
-            hd(*q.args())
-            worker.sync()
-            first = q.out.clone()
-            q.out.zero_()
-            worker.set_option("gemm_variant", 1)
-            hd(*q.args())
-            worker.sync()
-    finally:
-        worker.set_option("gemm_variant", 0)
-        worker.set_option("gemm_splits", 0)
-    assert first.abs().max().item() > 0 and torch.equal(first, q.out)
 
 
 @pytest.mark.parametrize("m,k,n,splits", [(2048, 11008, 4096, 0),    # the LLaMA-7B down pass: the library's own choice (2)
