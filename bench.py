@@ -181,12 +181,17 @@ def main() -> int:
         args.no_autotune = True
     elif not args.no_autotune:
         tuned = autotune_attention(worker, handle, [p.args() for p in pools])
-    if tuned["tokens_per_partition"] == 0 and tuned["waves_per_cu"] == 0:
-        # the library's own choice: its first calls of this launch signature time a few bit-identical
-        # launch shapes and keep the fastest; let that settle before anything is timed
-        prepared.run(40)
+    if not args.attn_launch:
+        # What the library settles on by itself (its first calls of a launch signature time a few
+        # bit-identical launch shapes and keep the fastest): read back with no option set.
+        best = (tuned["tokens_per_partition"], tuned["waves_per_cu"])
+        worker.set_option("attn_tokens_per_partition", 0)
+        worker.set_option("attn_waves_per_cu", 0)
+        prepared.run(60)
         tuned["library_waves_per_cu"] = worker.get_option("attn_tuned_waves_per_cu")
         tuned["library_workgroup_form"] = worker.get_option("attn_tuned_workgroup_form")
+        worker.set_option("attn_tokens_per_partition", best[0])
+        worker.set_option("attn_waves_per_cu", best[1])
     prepared.run(max(args.warmup, 1))       # W untimed warm-up steps
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -206,7 +211,7 @@ def main() -> int:
     # What the memory system gives this launch shape and access pattern: the library's load-only twin of
     # the kernel (same grid, table walk and loads, nothing computed), over the same rotating pools.
     # (the twin walks the partition grid under the options in force: give it the cap the library settled on)
-    lib_cap = tuned.get("library_waves_per_cu", -1)
+    lib_cap = tuned.get("library_waves_per_cu", -1) if tuned["waves_per_cu"] == 0 else -1
     if lib_cap > 0:
         worker.set_option("attn_waves_per_cu", lib_cap)
     probe = [attention_stream_probe(worker, p.key_cache, p.value_cache, p.block_table, p.context_lens, p.config,
@@ -407,7 +412,7 @@ def main() -> int:
             dargs = [dl.args()]
             dtuned = {"tokens_per_partition": 0, "waves_per_cu": 0}
             if not args.no_autotune:
-                dtuned = autotune_attention(worker, dh, dargs, rounds=15)
+                dtuned = autotune_attention(worker, dh, dargs, rounds=30)
             benchmark(dh, dargs, rounds=5, warmup=0)
             dstats = benchmark(dh, dargs, rounds=20, warmup=0)
         worker.set_option("attn_tokens_per_partition", 0)
