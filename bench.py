@@ -131,6 +131,9 @@ def main() -> int:
     ap.add_argument("--attn-launch", default=None, metavar="TOKENS,WAVES",
                     help="fix attn_tokens_per_partition and attn_waves_per_cu for the small configuration instead of "
                          "measuring (for profiler runs: every traced launch then has the same shape)")
+    ap.add_argument("--no-library-tuning", action="store_true",
+                    help="switch the library's own launch-shape measurement off (\"attn_autotune\" 0): every attention "
+                         "launch of a configuration then has the rule's shape, which profiler runs want")
     ap.add_argument("--ffn-clock-probe", action="store_true",
                     help="run the FFN for about 1.5 s on its random operands and on all-zero operands, reading the "
                          "shader clock (rocm-smi) during each: the gap between the two is the data-dependent clock. "
@@ -157,6 +160,8 @@ def main() -> int:
         return 2
 
     worker = ChipWorker(RunConfig(platform="mi355x", device_id=0))
+    if args.no_library_tuning:
+        worker.set_option("attn_autotune", 0)
     info = worker.device_info()
     cores = torch.get_num_threads()
     cpu = not args.no_cpu_baseline
