@@ -550,7 +550,7 @@ PTO_HIP_API int pto_hip_backend_handler_query(const char* hook, int32_t arg, cha
  *  "gemm_splits"                k splits of the tiled GEMM: 0 = by shape (default), 1..16 = as given
  *                               when k allows (each split at least four 64-row k tiles)
  *  "w8a16_wgs_per_cu"           workgroups per CU the W8A16 k split aims at (default 1)
- *  "w8a16_wide"                 1 = int8 codes of large matrices (>= 150 MB) are read 16 per lane
+ *  "w8a16_wide"                 1 = int8 codes of large matrices (>= 100 MB) are read 16 per lane
  *                               (default), 0 = always 8 per lane, 2 = 16 per lane whenever the
  *                               channel count is a multiple of 16
  *  "w8a16_min_steps"            fewest 32-row steps per wavefront before k is split further

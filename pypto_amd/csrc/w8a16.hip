@@ -437,10 +437,15 @@ int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* w
   p.n = (int)n;
   // int8 codes are read 16 per lane (a 256-channel slab per workgroup, half the requests per byte)
   // for large matrices when rows and base addresses allow 16-byte loads, else 8 per lane like the
-  // 16-bit weights.  Measured: 235 MB of codes 3.6 -> 4.5 TB/s, 525 MB 4.2 -> 4.8 TB/s; but 59 MB
-  // 3.8 -> 3.2 TB/s (half the slabs, so twice the k splits and fewer wavefronts), hence the size bound.
+  // 16-bit weights.  Every workgroup also reads the activations of its k range - 64 bytes per k row
+  // next to 128 bytes of codes with a 128-channel slab - and a CU takes in a bounded number of bytes
+  // per second whatever they are (counters: the decoder layer's gate/up launch requests 177 MB from
+  // L2 for 117 MB of codes, 6.2 TB/s over the chip), so the wider slab moves a sixth less per code.
+  // Measured: 117 MB of codes (two 4096 x 14336 matrices) 28.2 -> 25.6 us, 235 MB 3.6 -> 4.5 TB/s,
+  // 525 MB 4.2 -> 4.8 TB/s; but 59 MB 16.1 -> 17.2 us, 25 MB 10.2 -> 13.0 us (half the slabs, so twice
+  // the k splits or fewer workgroups), hence the size bound.
   const bool wide = !w16 && ctx().w8a16_wide != 0 && n % 16 == 0 && ((uintptr_t)wq0 | (uintptr_t)wq1) % 16 == 0 &&
-                    (ctx().w8a16_wide == 2 || k * n * (wq1 ? 2 : 1) >= (int64_t)150 * 1000 * 1000);
+                    (ctx().w8a16_wide == 2 || k * n * (wq1 ? 2 : 1) >= (int64_t)100 * 1000 * 1000);
   const int slab_cols = wide ? 2 * kSlab : kSlab;
   p.slabs = (int)((n + slab_cols - 1) / slab_cols);
   p.n_mats = wq1 ? 2 : 1;
