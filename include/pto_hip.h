@@ -524,6 +524,11 @@ PTO_HIP_API int pto_hip_backend_handler_query(const char* hook, int32_t arg, cha
  *                               form) with events read back on later calls - nothing blocks - and the
  *                               fastest is used from then on (default); 0 = the fixed rule only.  Calls
  *                               under stream capture and pto_hip_paged_attention_noalloc never measure.
+ *  "attn_lean_siblings"         evenly split form with several query tiles per KV head (more than 64 heads on
+ *                               one KV head, 32 at head_dim 256): 1 = the tiles of a KV head are carried by
+ *                               sibling wavefronts of one workgroup that walk the same chunks side by side,
+ *                               so the second reader of a K/V row finds it in its own L2 (default); 0 =
+ *                               every tile is a stream of its own, placed wherever the list puts it
  *  "attn_tuned_waves_per_cu"    read only: the cap the last launch's signature settled on (-1 = not yet)
  *  "attn_tuned_workgroup_form"  read only: 1 when it settled on the workgroup form, 0 the grid, -1 = not yet
  *  "workspace_bytes"            read only: bytes of device memory the library's grow-only scratch areas hold

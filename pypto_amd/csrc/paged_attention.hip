@@ -58,6 +58,7 @@ struct AttnParams {
   int gt_rows;     // query rows one wavefront covers: 16 x its tile count; gtiles = ceil(group / gt_rows)
   int resident_cap;  // partition grid: wavefronts allowed on a CU at once, 0 = as many as fit
   int wg_merge;    // one workgroup per (sequence, KV head, query tile), merged through LDS: 1, else 0
+  int lean_sib;    // evenly split form: wavefronts of one workgroup that share a run of chunks, one query tile each
   int n_wg;        // evenly split form: resident workgroups (one per CU); 0 = partition grid
   int lean_waves;  // ... and wavefronts in each
   float scale_log2e;
@@ -838,7 +839,12 @@ __global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(A
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, j = lane >> 4;
-  const int hg_count = p.hkv * p.gtiles;
+  // Query tiles of one KV head read the same K and V.  With lean_sib = gtiles the tiles are carried
+  // by sibling wavefronts of one workgroup that walk the same run of chunks side by side: whichever
+  // is behind finds the rows in this XCD's L2, so every cache byte crosses the fabric once.  Then
+  // the item list runs over (sequence, KV head, chunk) only.
+  const int sib = p.lean_sib;
+  const int hg_count = p.hkv * p.gtiles / sib;
   const int max_ctx = p.ctx_cap;
   char* kbuf = lean_lds + wave * KStage<D, FP8>::kBytes;
 
@@ -846,9 +852,9 @@ __global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(A
   // with fewer items than wavefronts only the first `total` wavefronts take part, which keeps
   // every participant's run non-empty (the merge relies on that).
   const long long total = lean_total(p, lane, hg_count);
-  const long long wres = (long long)gridDim.x * (blockDim.x >> 6);
+  const long long wres = (long long)gridDim.x * ((blockDim.x >> 6) / sib);
   const long long wtot = wres < total ? wres : total;
-  const long long w = (long long)wave * gridDim.x + blockIdx.x;
+  const long long w = (long long)(wave / sib) * gridDim.x + blockIdx.x;
   if (w >= wtot) return;
   long long s = (w * total + wtot - 1) / wtot;
   const long long s_end = ((w + 1) * total + wtot - 1) / wtot;
@@ -870,7 +876,8 @@ __global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(A
   while (s < s_end) {  // one iteration per (sequence, head, tile) the run touches
     const long long left = s_end - s;
     const int run = (int)(left < (long long)(chunks - chunk) ? left : (long long)(chunks - chunk));
-    const int h = hg / p.gtiles, gt = hg % p.gtiles;
+    const int hgt = hg * sib + wave % sib;  // (KV head, query tile) of this wavefront
+    const int h = hgt / p.gtiles, gt = hgt % p.gtiles;
     int ctx = p.ctx_lens[b];
     ctx = ctx > max_ctx ? max_ctx : ctx;
     const int tok_first = chunk * kChunk;
@@ -887,7 +894,7 @@ __global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(A
 #pragma unroll
     for (int t = 0; t < GT; ++t) {
       if (g0 + t * 16 + c >= p.group) continue;
-      const size_t slot = ((size_t)((long long)b * hg_count + hg + w)) * (16 * GT) + t * 16 + c;
+      const size_t slot = ((size_t)(((long long)b * hg_count + hg + w) * sib + wave % sib)) * (16 * GT) + t * 16 + c;
       store_rows<D>(p.part_o + slot * D, acc[t], j, v_unit);
       if (j == 0) {
         p.part_ml[slot * 2 + 0] = m_run[t];
@@ -923,7 +930,9 @@ __global__ __launch_bounds__(256) void attn_lean_reduce_kernel(AttnParams p, lon
   const int b = row / p.hq, hqi = row % p.hq;
   const int h = hqi / p.group, g = hqi % p.group;
   const int rows = p.gt_rows;  // rows per partial slot
-  const int hg_count = p.hkv * p.gtiles, hg = h * p.gtiles + g / rows, gi = g % rows;
+  const int sib = p.lean_sib;  // as in the streaming kernel
+  const int hgt = h * p.gtiles + g / rows, gi = g % rows;
+  const int hg_count = p.hkv * p.gtiles / sib, hg = hgt / sib;
 
   // items before sequence b, items in total, chunks of b
   long long total = 0, before = 0;
@@ -951,37 +960,64 @@ __global__ __launch_bounds__(256) void attn_lean_reduce_kernel(AttnParams p, lon
     const long long c0 = before + (long long)hg * chunks, c1 = c0 + chunks;
     const long long w_first = c0 * wtot / total, w_last = (c1 - 1) * wtot / total;
     const int np = (int)(w_last - w_first + 1);
-    const size_t slot0 = ((size_t)((long long)b * hg_count + hg + w_first)) * rows + gi;
+    const size_t slot0 = ((size_t)(((long long)b * hg_count + hg + w_first) * sib + hgt % sib)) * rows + gi;
     const float* ml = p.part_ml + slot0 * 2;   // partial i at ml[i * ml_step], po[i * po_step]
     const float* po = p.part_o + slot0 * D;
-    const size_t ml_step = (size_t)rows * 2, po_step = (size_t)rows * D;
-    float m = kMinMax;
-    for (int i = lane; i < np; i += 64) m = fmaxf(m, ml[(size_t)i * ml_step]);
+    const size_t ml_step = (size_t)sib * rows * 2, po_step = (size_t)sib * rows * D;
+    constexpr int kFew = 4;
+    if (np <= kFew) {
+      // The usual case (a pair's chunks lie in the runs of two to four wavefronts): everything the
+      // row needs is requested at once, one memory round trip after the scan.
+      float pm[kFew], pl[kFew], pv[kFew][D / 64];
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
-    for (int i = lane; i < np; i += 64) l += __builtin_amdgcn_exp2f(ml[(size_t)i * ml_step] - m) * ml[(size_t)i * ml_step + 1];
+      for (int u = 0; u < kFew; ++u) {
+        const size_t i = (size_t)min(u, np - 1);
+        pm[u] = ml[i * ml_step];
+        pl[u] = ml[i * ml_step + 1];
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off);
-    int i = 0;
-    for (; i + 4 <= np; i += 4) {
-      float wv[4], v[4][D / 64];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        wv[u] = ml[(size_t)(i + u) * ml_step];
-#pragma unroll
-        for (int k = 0; k < D / 64; ++k) v[u][k] = po[(size_t)(i + u) * po_step + k * 64 + lane];
+        for (int k = 0; k < D / 64; ++k) pv[u][k] = po[i * po_step + k * 64 + lane];
       }
+      float m = kMinMax;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float wgt = __builtin_amdgcn_exp2f(wv[u] - m);
+      for (int u = 0; u < kFew; ++u) m = u < np ? fmaxf(m, pm[u]) : m;
 #pragma unroll
-        for (int k = 0; k < D / 64; ++k) o[k] += wgt * v[u][k];
+      for (int u = 0; u < kFew; ++u) {
+        const float wgt = __builtin_amdgcn_exp2f(pm[u] - m);
+        if (u < np) {
+          l += wgt * pl[u];
+#pragma unroll
+          for (int k = 0; k < D / 64; ++k) o[k] += wgt * pv[u][k];
+        }
       }
-    }
-    for (; i < np; ++i) {
-      const float wgt = __builtin_amdgcn_exp2f(ml[(size_t)i * ml_step] - m);
+    } else {
+      float m = kMinMax;
+      for (int i = lane; i < np; i += 64) m = fmaxf(m, ml[(size_t)i * ml_step]);
 #pragma unroll
-      for (int k = 0; k < D / 64; ++k) o[k] += wgt * po[(size_t)i * po_step + k * 64 + lane];
+      for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+      for (int i = lane; i < np; i += 64) l += __builtin_amdgcn_exp2f(ml[(size_t)i * ml_step] - m) * ml[(size_t)i * ml_step + 1];
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off);
+      int i = 0;
+      for (; i + 4 <= np; i += 4) {
+        float wv[4], v[4][D / 64];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          wv[u] = ml[(size_t)(i + u) * ml_step];
+#pragma unroll
+          for (int k = 0; k < D / 64; ++k) v[u][k] = po[(size_t)(i + u) * po_step + k * 64 + lane];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const float wgt = __builtin_amdgcn_exp2f(wv[u] - m);
+#pragma unroll
+          for (int k = 0; k < D / 64; ++k) o[k] += wgt * v[u][k];
+        }
+      }
+      for (; i < np; ++i) {
+        const float wgt = __builtin_amdgcn_exp2f(ml[(size_t)i * ml_step] - m);
+#pragma unroll
+        for (int k = 0; k < D / 64; ++k) o[k] += wgt * po[(size_t)i * po_step + k * 64 + lane];
+      }
     }
   }
   const float inv = l > 0.f ? 1.f / l : 0.f;
@@ -1056,7 +1092,7 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
     else rc = go(attn_lean_kernel<D, false, FP8, GT>);
     if (rc) return rc;
     hipLaunchKernelGGL((attn_lean_reduce_kernel<D>), dim3((unsigned)((batch * p.hq + 3) / 4)), dim3(256), 0, stream,
-                       p, (long long)p.n_wg * p.lean_waves);
+                       p, (long long)p.n_wg * (p.lean_waves / p.lean_sib));
     PTO_CHECK_HIP(hipGetLastError());
     return PTO_HIP_OK;
   }
@@ -1252,9 +1288,11 @@ int plan_launch(const int64_t* config, int q_dtype, int kv_dtype, bool have_scal
     const int64_t units = batch * hkv * p.gtiles;
     // With a (sequence, head) pair or more per CU the launch takes the workgroup form (see
     // paged_attention below), where two wavefronts per CU measured best (decoder layer, 32 sequences
-    // of 4096 tokens: 182.5 us a step against 184.0 with four).
+    // of 4096 tokens: 182.5 us a step against 184.0 with four).  A wavefront that carries several
+    // query tiles has that many times the arithmetic per byte and wants a SIMD to itself: four per CU
+    // (256 sequences, 64 heads on one KV head, 2048-4096 tokens: 85 us against 136 with two).
     const bool wg_form = cx.attn_variant == 2 || (cx.attn_variant < 0 && units >= cx.num_cu);
-    const int64_t slots = (int64_t)cx.num_cu * (wg_form ? 2 : 4);
+    const int64_t slots = (int64_t)cx.num_cu * (wg_form && gt == 1 ? 2 : 4);
     int64_t want = (slots + units - 1) / units;
     if (want < 1) want = 1;
     tpp = (max_ctx + want - 1) / want;
@@ -1485,6 +1523,7 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     while (waves > 1 && waves * 32 * kbytes > 160 * 1024) --waves;
     p.n_wg = cx.num_cu;
     p.lean_waves = (int)waves;
+    p.lean_sib = (p.gtiles > 1 && waves % p.gtiles == 0 && cx.attn_lean_siblings != 0) ? p.gtiles : 1;
     // partial slots: one per (sequence, head, tile) plus one per resident wavefront
     const size_t slots = (size_t)batch * hkv * p.gtiles + (size_t)p.n_wg * waves;
     const size_t o_bytes = slots * p.gt_rows * d * sizeof(float), ml_bytes = slots * p.gt_rows * 2 * sizeof(float);
