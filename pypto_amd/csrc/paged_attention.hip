@@ -1344,6 +1344,7 @@ struct TuneState {
   int chosen = -1;
 };
 constexpr int kTuneReps = 4;
+constexpr size_t kTuneMaxSignatures = 512;  // signatures beyond this many run the fixed rule
 typedef std::array<int64_t, 12> TuneKey;
 std::map<TuneKey, TuneState>& tune_table() {
   static std::map<TuneKey, TuneState> t;
@@ -1354,13 +1355,15 @@ TuneState* g_last_tuned = nullptr;  // state of the last launch that took part i
 void tune_harvest(TuneState& ts) {
   for (size_t i = 0; i < ts.pending.size();) {
     TunePending& pd = ts.pending[i];
-    if (hipEventQuery(pd.e1) != hipSuccess) {
+    const hipError_t q = hipEventQuery(pd.e1);
+    if (q == hipErrorNotReady) {
       (void)hipGetLastError();
       ++i;
       continue;
     }
     float ms = 0.f;
-    if (hipEventElapsedTime(&ms, pd.e0, pd.e1) == hipSuccess) {
+    // (a query that fails for any other reason - the stream is gone, say - drops the reading)
+    if (q == hipSuccess && hipEventElapsedTime(&ms, pd.e0, pd.e1) == hipSuccess) {
       ts.best_us[pd.cand] = std::min(ts.best_us[pd.cand], ms * 1e3f);
       ++ts.done[pd.cand];
     } else {
@@ -1476,7 +1479,12 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
   if (cx.attn_autotune != 0 && cx.attn_waves_per_cu == 0 && cx.attn_variant < 0 && !lean) {
     const TuneKey key = {batch, hq, hkv, d, config[4], config[5], (int64_t)q_dtype, (int64_t)kv_dtype, (int64_t)p.ctx_cap,
                          (int64_t)p.tpp, (int64_t)gt, (int64_t)(out16 != nullptr)};
-    ts = &tune_table()[key];
+    auto& table_ = tune_table();
+    auto it = table_.find(key);
+    if (it == table_.end() && table_.size() < kTuneMaxSignatures) it = table_.emplace(key, TuneState{}).first;
+    ts = it == table_.end() ? nullptr : &it->second;
+  }
+  if (ts) {
     if (ts->cands.empty()) {
       ts->cands.push_back({0, p.wg_merge != 0});  // the rule's own choice first
       if (wg_possible) ts->cands.push_back({0, p.wg_merge == 0});
