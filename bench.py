@@ -418,7 +418,7 @@ def main() -> int:
             dtuned = {"tokens_per_partition": 0, "waves_per_cu": 0}
             if not args.no_autotune:
                 dtuned = autotune_attention(worker, dh, dargs, rounds=30)
-            benchmark(dh, dargs, rounds=5, warmup=0)
+            benchmark(dh, dargs, rounds=30, warmup=0)  # past the library's launch-shape measurement
             dstats = benchmark(dh, dargs, rounds=20, warmup=0)
         worker.set_option("attn_tokens_per_partition", 0)
         worker.set_option("attn_waves_per_cu", 0)
@@ -457,7 +457,7 @@ def main() -> int:
         more = {}
         dw = workloads.decoder_layer_inputs(device="cuda", int8_weights=False)
         with worker.register(decoder_layer_decode_w16) as dh:
-            benchmark(dh, [dw.args()], rounds=5, warmup=0)
+            benchmark(dh, [dw.args()], rounds=30, warmup=0)  # past the library's launch-shape measurement
             st = benchmark(dh, [dw.args()], rounds=20, warmup=0)
         more["decoder_layer_w16"] = _hbm_block(
             "decoder-layer decode step with bf16 weights (the reference's layer): H4096 Hq32 Hkv8 D128 I14336 B32 "
@@ -470,7 +470,7 @@ def main() -> int:
                                             intermediate=17408, context=4096, theta=1e6, device="cuda",
                                             int8_weights=False)
         with worker.register(decoder_layer_decode_w16) as dh:
-            benchmark(dh, [dq.args()], rounds=5, warmup=0)
+            benchmark(dh, [dq.args()], rounds=30, warmup=0)  # past the library's launch-shape measurement
             st = benchmark(dh, [dq.args()], rounds=20, warmup=0)
         more["decoder_layer_qwen3_14b"] = _hbm_block(
             "qwen3-14B decoder layer decode step, bf16 weights: H5120 Hq40 Hkv8 D128 I17408 B16 ctx4096 (the shape of "
@@ -484,7 +484,7 @@ def main() -> int:
                                             intermediate=25600, context=4096, block_size=4096, theta=1e6, device="cuda",
                                             int8_weights=False, weight_std=None)
         with worker.register(decoder_layer_decode_w16) as dh:
-            benchmark(dh, [dj.args()], rounds=5, warmup=0)
+            benchmark(dh, [dj.args()], rounds=30, warmup=0)  # past the library's launch-shape measurement
             st = benchmark(dh, [dj.args()], rounds=20, warmup=0)
         more["decoder_layer_qwen3_jit"] = _hbm_block(
             "the reference's qwen3_jit decode model, one layer step, bf16 weights: H8192 Hq64 Hkv8 D128 I25600 B16 "
@@ -516,7 +516,7 @@ def main() -> int:
         mq = workloads.paged_attention_inputs(batch=256, num_heads=64, kv_head_num=1, head_dim=128, block_size=128,
                                               ctx_range=(2048, 4096), seed=0, device="cuda")
         with worker.register(paged_attention) as mh:
-            benchmark(mh, [mq.args()], rounds=5, warmup=0)
+            benchmark(mh, [mq.args()], rounds=30, warmup=0)  # the library's launch-shape measurement ends within these
             st = benchmark(mh, [mq.args()], rounds=20, warmup=0)
         more["attention_mqa64"] = _hbm_block(
             "paged-attention decode, 64 query heads per KV head: B256 Hq64 Hkv1 D128 bs128 ctx~U[2048,4096] bf16 KV; "

@@ -73,3 +73,51 @@ def test_workgroup_form_full_small_configuration(worker):
         got = _run(worker, inp, 2, tpp)
         validate_golden({"out": got}, {"out": ref}, rtol=RTOL, atol=ATOL)
         assert torch.equal(got, _run(worker, inp, 0, tpp))
+
+
+def test_many_sequences_with_64_heads_on_one_kv_head_at_full_size(worker):
+    """256 sequences of 2048-4096 tokens, 64 query heads on one KV head (418 MB of cache): a
+    (sequence, head) pair per CU, so the library's own rule takes the workgroup form, with four
+    wavefronts per pair because each carries four query tiles.  Its result is the partition grid's
+    with the same partitions to the bit; six whole sequences (the shortest and the longest among
+    them) are held to the oracle."""
+    batch, heads, d, bs = 256, 64, 128, 128
+    inp = workloads.paged_attention_inputs(batch=batch, num_heads=heads, kv_head_num=1, head_dim=d, block_size=bs,
+                                           ctx_range=(2048, 4096), seed=3, device="cuda")
+    worker.set_option("attn_autotune", 0)   # the fixed rule, not whatever earlier calls measured
+    try:
+        inp.out.fill_(float("nan"))
+        with worker.register(paged_attention) as h:
+            h(*inp.args())
+        worker.sync()
+        auto = inp.out.clone()
+        for variant in (2, 0):
+            worker.set_option("attn_variant", variant)
+            worker.set_option("attn_tokens_per_partition", 1024)
+            inp.out.fill_(float("nan"))
+            with worker.register(paged_attention) as h:
+                h(*inp.args())
+            worker.sync()
+            assert torch.equal(inp.out, auto), variant
+    finally:
+        worker.set_option("attn_variant", -1)
+        worker.set_option("attn_tokens_per_partition", 0)
+        worker.set_option("attn_autotune", 1)
+    lens = inp.context_lens.cpu()
+    pick = sorted({int(lens.argmin()), int(lens.argmax()), 0, 1, batch // 2, batch - 1})
+    mb = int(inp.config[5])
+    table = inp.block_table.reshape(batch, mb)[pick].cpu().long()
+    used = (lens[pick] + bs - 1) // bs
+    mask = torch.arange(mb).reshape(1, -1) < used.reshape(-1, 1)
+    blocks, inverse = torch.unique(table[mask], return_inverse=True)
+    rows = (blocks.reshape(-1, 1) * bs + torch.arange(bs)).reshape(-1).cuda()
+    sub_table = torch.zeros(len(pick), mb, dtype=torch.int32)
+    sub_table[mask] = inverse.to(torch.int32)
+    cfg = inp.config.clone()
+    cfg[0] = len(pick)
+    q = inp.query.reshape(batch, heads, d)[pick].reshape(-1, d).cpu()
+    ref = oracle.paged_attention_golden(q, inp.key_cache[rows].cpu(), inp.value_cache[rows].cpu(),
+                                        sub_table.reshape(-1), lens[pick].to(torch.int32), cfg)
+    got = auto.reshape(batch, heads, d)[pick].reshape(-1, d).cpu()
+    assert torch.isfinite(auto).all()
+    validate_golden({"out": got}, {"out": ref}, rtol=RTOL, atol=ATOL)
