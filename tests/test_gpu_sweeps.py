@@ -83,6 +83,59 @@ def test_attention_sweep(worker):
             worker.set_option(name, value)
 
 
+def _attention_wide_group_sweep(worker, seed, cases):
+    """More query heads on a KV head than one wavefront carries (several query tiles per KV head), in
+    every launch form: the partition grid, the evenly split form with the tiles on sibling wavefronts
+    or each on its own, the workgroup form."""
+    rng = random.Random(seed)
+    names = ("attn_variant", "attn_tokens_per_partition", "attn_waves_per_cu", "attn_group_tiles", "attn_lean_siblings")
+    try:
+        for case in range(cases):
+            d = rng.choice([128, 128, 256])
+            hkv = rng.choice([1, 1, 2, 3])
+            group = rng.choice([33, 40, 48, 64, 65, 80, 96, 128] if d == 128 else [17, 24, 33, 48, 64, 65, 96])
+            hq = hkv * group
+            fp8 = rng.random() < 0.35
+            bs = rng.choice([32, 64, 128, 256] if fp8 else [16, 32, 48, 64, 128, 256])
+            batch = rng.randint(1, 4)
+            top = rng.choice([40, 300, 1200, 2500])
+            ctxs = [rng.choice([0, 1, bs - 1, bs, bs + 1, rng.randint(1, top), rng.randint(1, top)]) for _ in range(batch)]
+            dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float16
+            mb = (max(max(ctxs), 1) + bs - 1) // bs + rng.choice([0, 0, 3])
+            inp = workloads.paged_attention_inputs(
+                batch=batch, num_heads=hq, kv_head_num=hkv, head_dim=d, block_size=bs, context_lens=ctxs,
+                ctx_range=(1, max(max(ctxs), 1)), dtype=dtype, fp8_kv=fp8, max_num_blocks_per_req=mb,
+                seed=rng.randint(0, 10 ** 6), scale=rng.choice([None, None, 1.0, 0.0884]))
+            align = bs if bs >= 32 else 32
+            variant, tpp, waves, gt, sib = rng.choice([
+                (-1, 0, 0, 0, 1), (0, align * rng.randint(1, 8), 0, 0, 1), (2, align * rng.randint(1, 8), 0, 0, 1),
+                (1, 0, rng.choice([0, 2, 4, 8]), 0, 1), (1, 0, rng.choice([0, 2, 4]), 0, 0), (1, 0, 0, rng.choice([1, 2]), 1),
+                (2, 0, 0, rng.choice([1, 2]), 1)])
+            print(f"wide-group attention case {case} (seed {seed}): B{batch} Hq{hq} Hkv{hkv} D{d} bs{bs} ctx{ctxs} {dtype} "
+                  f"e4m3={fp8} mb={mb} variant={variant} tpp={tpp} waves={waves} tiles={gt} siblings={sib}", flush=True)
+            ref = oracle.paged_attention_golden(inp.query, inp.key_cache, inp.value_cache, inp.block_table,
+                                                inp.context_lens, inp.config, inp.k_scale, inp.v_scale)
+            for name, value in zip(names, (variant, tpp, waves, gt, sib)):
+                worker.set_option(name, value)
+            dev = [t.cuda() if isinstance(t, torch.Tensor) and i != 6 else t for i, t in enumerate(inp.args())]
+            dev[5].fill_(float("nan"))
+            torch.cuda.synchronize()
+            with worker.register(paged_attention) as h:
+                h(*dev)
+            worker.sync()
+            out = dev[5].cpu()
+            assert torch.isfinite(out).all()
+            err = (out - ref).abs().max().item()
+            assert err <= 1e-2 + 2e-2 * ref.abs().max().item(), f"case {case}: max err {err}"
+    finally:
+        for name, value in zip(names, (-1, 0, 0, 0, 1)):
+            worker.set_option(name, value)
+
+
+def test_attention_wide_group_sweep(worker):
+    _attention_wide_group_sweep(worker, 20246, 40)
+
+
 def test_ffn_and_projection_sweep(worker):
     rng = random.Random(20241)
     try:
