@@ -6,7 +6,7 @@
 // examples/models/08_llama_mini.py:384-483; golden
 // tests/st/runtime/framework_and_models/test_qwen3_decode_scope3_mixed.py:255-287), with the
 // projections taking either the reference's 16-bit weights or int8 weights and per-channel scales.  The reference submits one task per
-// tile through its scheduler; here the layer is eleven kernel launches in stream order; each projection is a partial-sum
+// tile through its scheduler; here the layer is ten or eleven kernel launches in stream order; each projection is a partial-sum
 // kernel whose finish is folded into the elementwise step that follows it.
 #include <hip/hip_runtime.h>
 
