@@ -105,11 +105,17 @@ def _ffn_clock_probe(worker, program, fargs, zero_idx) -> dict:
     return out
 
 
+_READ_PROBE_GBPS = None  # rate of the read probe with a stream per wavefront, once it has run
+
+
 def _hbm_block(workload: str, nbytes: int, us: float) -> dict:
     gbps = nbytes / us / 1e3
-    return {"workload": workload, "algorithmic_bytes_per_step": nbytes, "us_per_step": round(us, 1),
-            "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
-            "bound": "hbm"}
+    block = {"workload": workload, "algorithmic_bytes_per_step": nbytes, "us_per_step": round(us, 1),
+             "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
+             "bound": "hbm"}
+    if _READ_PROBE_GBPS:
+        block["frac_of_stream_read_probe"] = round(gbps / _READ_PROBE_GBPS, 4)
+    return block
 
 
 def main() -> int:
@@ -150,7 +156,7 @@ def main() -> int:
 
     from pypto_amd import workloads
     from pypto_amd.runtime import (ChipWorker, PreparedBenchmark, RunConfig, attention_stream_probe,
-                                   autotune_attention, benchmark, mfma_only_probe,
+                                   autotune_attention, benchmark, hbm_read_probe, mfma_only_probe,
                                    decoder_layer_decode, decoder_layer_decode_w16, ffn_block, ffn_block_fp8,
                                    paged_attention,
                                    projection)
@@ -270,6 +276,26 @@ def main() -> int:
             "traffic_source": prof["source"],
         },
     }
+    # What the compute units of this box read per second when they do nothing else: a plain read of
+    # 2 GiB (eight times the last-level cache) by one workgroup per CU, the best of three wavefront
+    # counts - once with all wavefronts sweeping the buffer together (the most the memory system gives)
+    # and once with a contiguous stream per wavefront (independent streams, which is what paged
+    # attention and the projections' column slabs are).  The ceilings of every bandwidth-bound figure
+    # below, next to the published peak.
+    probe_buf = torch.empty(2 << 30, dtype=torch.uint8, device="cuda")
+    probe_buf.zero_()
+    sweep = max(hbm_read_probe(worker, probe_buf, waves_per_cu=w)["gbps"] for w in (4, 8, 16))
+    streams = max(hbm_read_probe(worker, probe_buf, streams=True, waves_per_cu=w)["gbps"] for w in (4, 8, 16))
+    result["roofline"]["read_probe_gbps"] = {"one_sweep": round(sweep, 1), "stream_per_wavefront": round(streams, 1)}
+    result["roofline"]["read_probe_note"] = (
+        f"plain reads of {probe_buf.numel() >> 20} MiB by one workgroup per CU, nothing computed or stored: all wavefronts "
+        f"sweeping the buffer together ({sweep / HBM_PEAK_GBPS:.2f} of the peak) and one contiguous stream per wavefront "
+        f"({streams / HBM_PEAK_GBPS:.2f}); paged attention reads independent (sequence, head) streams")
+    result["roofline"]["frac_of_stream_read_probe"] = round(achieved / streams, 4)
+    global _READ_PROBE_GBPS
+    _READ_PROBE_GBPS = streams
+    del probe_buf
+    torch.cuda.empty_cache()
     if cpu:
         p = pools[0]
         host = [t.cpu() for t in (p.query, p.key_cache, p.value_cache, p.block_table, p.context_lens, p.config)]

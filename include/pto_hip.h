@@ -252,6 +252,19 @@ PTO_HIP_API int pto_hip_mfma_probe(const void* a, int64_t a_elems, const void* b
                                    int warm_rounds, int rounds, void* stream, double* mean_us,
                                    double* flops_per_launch);
 
+/* Measurement aid with no counterpart in the reference: how fast this GPU's compute units read a
+ * buffer when they do nothing else.  One workgroup of waves_per_cu (1..16) wavefronts per CU reads
+ * buf[0 .. bytes) (16-byte aligned; larger than the last-level cache if memory is to be measured) with
+ * eight independent 16-byte loads per lane in flight and stores nothing.  pattern 0: all wavefronts
+ * sweep the buffer together, so the chip reads one contiguous window at a time - the most the memory
+ * system gives; pattern 1: every wavefront streams its own contiguous share - independent streams, as
+ * the (sequence, head) streams of paged attention are - which loads the memory channels less evenly.
+ * The kernel is launched warm_rounds + rounds times; *mean_us receives the mean time of the last
+ * `rounds` launches.  bytes / *mean_us is the ceiling of a bandwidth-bound kernel with that kind of
+ * access on this box.  Blocks until done. */
+PTO_HIP_API int pto_hip_hbm_read_probe(const void* buf, int64_t bytes, int pattern, int waves_per_cu, int warm_rounds,
+                                       int rounds, void* stream, double* mean_us);
+
 /* out[i, :] = src[block_table[idx / bs] * bs + idx % bs, col_offset : col_offset + size]
  * (src/ir/op/tensor_ops/paged_gather.cpp:74-199), bit-exact, asynchronous on the stream.  An index
  * that addresses a block outside block_table or a row outside src is skipped and reported by

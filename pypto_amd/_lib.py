@@ -27,6 +27,7 @@ EXPORTS = (
     "pto_hip_decoder_layer_decode", "pto_hip_select_program", "pto_hip_projection",
     "pto_hip_gate_up_swiglu", "pto_hip_paged_attention_noalloc", "pto_hip_paged_attention_stream_probe",
     "pto_hip_mfma_probe",
+    "pto_hip_hbm_read_probe",
     "pto_hip_ffn_swiglu_fp8", "pto_hip_quantize_rows_fp8", "pto_hip_rms_norm_quantize_fp8",
     "pto_hip_gate_up_swiglu_fp8", "pto_hip_projection_fp8", "pto_hip_llama_mini",
     "pto_hip_write_manifest", "pto_hip_backend_info", "pto_hip_backend_op_name", "pto_hip_backend_op_info",
@@ -121,6 +122,7 @@ def load() -> C.CDLL:
                                                  C.POINTER(C.c_double)],
         "pto_hip_mfma_probe": [vp, i64, vp, i64, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.POINTER(C.c_double),
                                C.POINTER(C.c_double)],
+        "pto_hip_hbm_read_probe": [vp, i64, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.POINTER(C.c_double)],
         "pto_hip_paged_gather": [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, C.c_int, vp],
         "pto_hip_rms_norm": [vp, vp, vp, i64, i64, C.c_float, C.c_int, C.c_int, vp],
         "pto_hip_ffn_swiglu": [vp, vp, vp, vp, vp, vp, i64, i64, i64, C.c_float, C.c_int, C.c_int, vp],

@@ -645,6 +645,23 @@ def mfma_only_probe(worker: ChipWorker, a: torch.Tensor, b: torch.Tensor, *, ite
     return {"us": us.value, "tflops": flops.value / us.value / 1e6}
 
 
+def hbm_read_probe(worker: ChipWorker, buf: torch.Tensor, *, streams: bool = False, waves_per_cu: int = 8,
+                   warm_rounds: int = 3, rounds: int = 10, stream: int = 0) -> dict:
+    """Rate at which the GPU's compute units read ``buf`` (a contiguous device tensor, larger than the
+    last-level cache if memory is to be measured) when they do nothing else.  ``streams=False``: all
+    wavefronts sweep the buffer together (the most the memory system gives); ``streams=True``: every
+    wavefront streams its own contiguous share, as the (sequence, head) streams of paged attention do.
+    Returns ``{"us": mean time per pass, "gbps": rate}``."""
+    worker._require_ready("hbm_read_probe")
+    if not buf.is_cuda or not buf.is_contiguous():
+        raise ValueError("hbm_read_probe: buf must be a contiguous device tensor")
+    nbytes = buf.numel() * buf.element_size()
+    us = C.c_double(0.0)
+    _lib.check(worker._lib.pto_hip_hbm_read_probe(buf.data_ptr(), nbytes, 1 if streams else 0, int(waves_per_cu),
+                                                  int(warm_rounds), int(rounds), stream, C.byref(us)))
+    return {"us": us.value, "gbps": nbytes / us.value / 1e3}
+
+
 def benchmark(
     handle: RegistrationHandle,
     arg_sets: Sequence[Sequence[Any]],
