@@ -542,6 +542,9 @@ PTO_HIP_API int pto_hip_backend_handler_query(const char* hook, int32_t arg, cha
  *                               sibling wavefronts of one workgroup that walk the same chunks side by side,
  *                               so the second reader of a K/V row finds it in its own L2 (default); 0 =
  *                               every tile is a stream of its own, placed wherever the list puts it
+ *  "w8a16_nt"                   skinny projections (up to 32 rows): 1 = the weight rows, read once per call, are
+ *                               loaded with the non-temporal hint so that they do not displace what other
+ *                               kernels keep in the caches (default); 0 = ordinary loads
  *  "attn_tuned_waves_per_cu"    read only: the cap the last launch's signature settled on (-1 = not yet)
  *  "attn_tuned_workgroup_form"  read only: 1 when it settled on the workgroup form, 0 the grid, -1 = not yet
  *  "workspace_bytes"            read only: bytes of device memory the library's grow-only scratch areas hold

@@ -66,6 +66,7 @@ struct Context {
   int64_t attn_group_tiles = 0;  // cap on the query tiles one wavefront carries (0 = by group size)
   int64_t attn_autotune = 1;     // first calls of a launch signature time bit-identical launch shapes and keep the fastest
   int64_t attn_lean_siblings = 1;  // evenly split form: query tiles of one KV head on sibling wavefronts of one workgroup
+  int64_t w8a16_nt = 1;            // skinny projections: weight rows read with non-temporal loads
   int64_t gemm_variant = 0;
   int64_t gemm_splits = 0;       // k splits of the tiled GEMM: 0 = by shape, 1..16 = as given (when k allows)
   int64_t w8a16_wgs_per_cu = 1;  // workgroups of the W8A16 partial kernel aimed at per compute unit

@@ -152,12 +152,23 @@ __device__ __forceinline__ V stream_load(const char* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const V*>(p));
 }
 
-template <int D, bool FP8>
+// ONCE: the launch reads every cache row once (one wavefront per (sequence, KV head) stream).  When
+// several query tiles of a KV head read the same rows from different wavefronts, the later readers
+// want them kept in L2 and the loads are ordinary ones (the reference system tests' head_dim-256
+// shape with two tiles per KV head: 127 us with ordinary loads, 156 us with the hint).  A compile-time
+// choice: given both forms behind a run-time branch the optimiser merges them and drops the hint.
+template <typename V, bool ONCE>
+__device__ __forceinline__ V cache_load(const char* p) {
+  if constexpr (ONCE) return stream_load<V>(p);
+  else return *reinterpret_cast<const V*>(p);
+}
+
+template <int D, bool FP8, bool ONCE>
 __device__ __forceinline__ void load_k(KFrag<D, FP8>& k, const char* base0, const char* base1, int lane) {
 #pragma unroll
   for (int s = 0; s < KStage<D, FP8>::kLoads; ++s) {
-    k.t[0][s] = stream_load<u32x4>(base0 + s * 1024 + lane * 16);
-    k.t[1][s] = stream_load<u32x4>(base1 + s * 1024 + lane * 16);
+    k.t[0][s] = cache_load<u32x4, ONCE>(base0 + s * 1024 + lane * 16);
+    k.t[1][s] = cache_load<u32x4, ONCE>(base1 + s * 1024 + lane * 16);
   }
 }
 
@@ -186,7 +197,7 @@ __device__ __forceinline__ void fetch_k(KFrag<D, FP8>& k, const char* kbuf, int 
   }
 }
 
-template <int D, bool FP8>
+template <int D, bool FP8, bool ONCE>
 __device__ __forceinline__ void load_v(VFrag<D, FP8>& v, const char* base0, const char* base1, uint32_t voff) {
   constexpr int kRow = FP8 ? D : D * 2;        // bytes per token row
   constexpr int kSet = FP8 ? 128 : 256;        // bytes per 128-element set
@@ -197,10 +208,10 @@ __device__ __forceinline__ void load_v(VFrag<D, FP8>& v, const char* base0, cons
       const char* src = (e < 4 ? base0 : base1) + voff + set * kSet + (e & 3) * kRow;
       if constexpr (FP8) {
         typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-        const u32x2 w = stream_load<u32x2>(src);
+        const u32x2 w = cache_load<u32x2, ONCE>(src);
         v.t[set][e] = uint2{w.x, w.y};
       } else {
-        v.t[set][e] = stream_load<u32x4>(src);
+        v.t[set][e] = cache_load<u32x4, ONCE>(src);
       }
     }
 }
@@ -354,7 +365,7 @@ __device__ __forceinline__ void change_unit(f32x4 (&acc)[GT][D / 128][8], float&
 // v_unit, m_run[t] the running maximum (log2 units) and l_run[t] the row sum, both per column and
 // already summed over the wavefront.  tok_first must be a multiple of 32 below tok_end.  Every K
 // and V byte is loaded once and used by all GT tiles.
-template <int D, bool BF16, bool FP8, int GT>
+template <int D, bool BF16, bool FP8, int GT, bool ONCE = true>
 __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, int hq_row0, int g0,
                                              int tok_first, int tok_end, int tok_step, int c, int j,
                                              char* kbuf, int first_window, f32x4 (&acc)[GT][D / 128][8],
@@ -457,8 +468,8 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
       k_mul = p.scale_log2e * scale_k();
       v_unit = scale_v();
     }
-    load_k<D, FP8>(kf, kc + o0, kc + o1, lane);
-    load_v<D, FP8>(vf, vc + o0, vc + o1, voff);
+    load_k<D, FP8, ONCE>(kf, kc + o0, kc + o1, lane);
+    load_v<D, FP8, ONCE>(vf, vc + o0, vc + o1, voff);
     stage_k<D, FP8>(kf, kbuf, lane);
 
     for (int tok = tok_first; tok < tok_end; tok += tok_step) {
@@ -472,7 +483,7 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
       fetch_k<D, FP8>(kf, kbuf, c, j);
 #pragma unroll
       for (int t = 0; t < GT; ++t) qk_scores<D, BF16, FP8>(kf, qf[t], s0[t], s1[t]);
-      load_k<D, FP8>(kf, kc + o0, kc + o1, lane);  // next chunk, into the registers QK^T just released
+      load_k<D, FP8, ONCE>(kf, kc + o0, kc + o1, lane);  // next chunk, into the registers QK^T just released
       u32x4 pf[GT];
 #pragma unroll
       for (int t = 0; t < GT; ++t)
@@ -483,7 +494,7 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
         change_unit<D, GT>(acc, v_unit, v_next);
         k_mul = k_next;
       }
-      load_v<D, FP8>(vf, vc + o0, vc + o1, voff);  // next chunk, into the registers PV just released
+      load_v<D, FP8, ONCE>(vf, vc + o0, vc + o1, voff);  // next chunk, into the registers PV just released
       stage_k<D, FP8>(kf, kbuf, lane);
     }
   }
@@ -497,7 +508,7 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
   }
 }
 
-template <int D, bool BF16, bool FP8, int GT>
+template <int D, bool BF16, bool FP8, int GT, bool ONCE = true>
 __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   const int lane = threadIdx.x;
   const int c = lane & 15;   // MFMA row / column index of this lane
@@ -542,7 +553,7 @@ __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   __shared__ __attribute__((aligned(16))) char k_lds[KStage<D, FP8>::kBytes];
   f32x4 acc[GT][D / 128][8];
   float m_run[GT], l_run[GT], v_unit;
-  attend_range<D, BF16, FP8, GT>(p, b, h, hq_row0, g0, tok_begin, tok_end, kChunk, c, j, k_lds, first_window, acc,
+  attend_range<D, BF16, FP8, GT, ONCE>(p, b, h, hq_row0, g0, tok_begin, tok_end, kChunk, c, j, k_lds, first_window, acc,
                                  m_run, l_run, v_unit);
 
 #pragma unroll
@@ -693,7 +704,7 @@ constexpr int wg_region_bytes() {
 // as many wavefronts as the register file allows at the tile count (see lean_max_waves)
 constexpr int wg_max_parts(int d, int gt) { return d == 128 && gt == 1 ? 8 : 4; }
 
-template <int D, bool BF16, bool FP8, int GT>
+template <int D, bool BF16, bool FP8, int GT, bool ONCE = true>
 __global__ __launch_bounds__(wg_max_parts(D, GT) * 64) void attn_wg_kernel(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char wg_lds[];
   constexpr int kRegion = wg_region_bytes<D, FP8, GT>();
@@ -720,7 +731,7 @@ __global__ __launch_bounds__(wg_max_parts(D, GT) * 64) void attn_wg_kernel(AttnP
   if (tok_begin < tok_end) {
     f32x4 acc[GT][D / 128][8];
     float m_run[GT], l_run[GT], v_unit;
-    attend_range<D, BF16, FP8, GT>(p, b, h, hq_row0, g0, tok_begin, tok_end, kChunk, c, j,
+    attend_range<D, BF16, FP8, GT, ONCE>(p, b, h, hq_row0, g0, tok_begin, tok_end, kChunk, c, j,
                                    reinterpret_cast<char*>(region), first_window, acc, m_run, l_run, v_unit);
     // the K stage is dead (LDS operations of one wavefront complete in order): the partial takes its place
 #pragma unroll
@@ -849,7 +860,7 @@ __device__ __forceinline__ void lean_locate(const AttnParams& p, int lane, int h
 // wavefront: four wavefronts (one per SIMD) there.
 constexpr int lean_max_waves(int d, int gt) { return d == 128 && gt == 1 ? kLeanMaxWaves : 4; }
 
-template <int D, bool BF16, bool FP8, int GT>
+template <int D, bool BF16, bool FP8, int GT, bool ONCE = true>
 __global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char lean_lds[];
   const int lane = threadIdx.x & 63;
@@ -905,7 +916,7 @@ __global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(A
     float m_run[GT], l_run[GT], v_unit;
     const int first_window =
         p.block_table[(size_t)b * p.max_blocks + min(tok_first / p.bs + lane, p.max_blocks - 1)];
-    attend_range<D, BF16, FP8, GT>(p, b, h, hq_row0, g0, tok_first, tok_end, kChunk, c, j, kbuf, first_window,
+    attend_range<D, BF16, FP8, GT, ONCE>(p, b, h, hq_row0, g0, tok_first, tok_end, kChunk, c, j, kbuf, first_window,
                                    acc, m_run, l_run, v_unit);
 #pragma unroll
     for (int t = 0; t < GT; ++t) {
@@ -1082,6 +1093,11 @@ inline size_t lds_share(int cap) { return cap > 0 ? (size_t)((163840 - 8192) / c
 template <int D, bool FP8, int GT>
 int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   dim3 grid((unsigned)(p.n_part * p.hkv * p.gtiles * batch));
+  // Several query tiles per KV head - the shapes whose groups are wider than a wavefront carries, i.e.
+  // the widest tile count of each head size - read the cache rows from several wavefronts: ordinary
+  // loads there, the non-temporal hint everywhere else (see load_k).
+  constexpr bool kWidest = (D == 128 && GT == 4) || (D == 256 && GT == 2);
+  const bool shared_rows = kWidest && p.gtiles > 1;
   // Unused dynamic LDS caps the wavefronts resident per CU so that the dispatcher spreads the
   // grid over all CUs instead of filling some to their register limit.
   // (the kernel's own K stage counts against the same 160 KB, so the request is what is left of a
@@ -1104,8 +1120,12 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
       return launch_streaming(kern, lgrid, lblock, lean_lds, stream, p);
     };
     int rc = PTO_HIP_OK;
-    if (bf16) rc = go(attn_lean_kernel<D, true, FP8, GT>);
-    else rc = go(attn_lean_kernel<D, false, FP8, GT>);
+    if constexpr (kWidest) {
+      if (shared_rows) rc = bf16 ? go(attn_lean_kernel<D, true, FP8, GT, false>) : go(attn_lean_kernel<D, false, FP8, GT, false>);
+      else rc = bf16 ? go(attn_lean_kernel<D, true, FP8, GT>) : go(attn_lean_kernel<D, false, FP8, GT>);
+    } else {
+      rc = bf16 ? go(attn_lean_kernel<D, true, FP8, GT>) : go(attn_lean_kernel<D, false, FP8, GT>);
+    }
     if (rc) return rc;
     hipLaunchKernelGGL((attn_lean_reduce_kernel<D>), dim3((unsigned)((batch * p.hq + 3) / 4)), dim3(256), 0, stream,
                        p, (long long)p.n_wg * (p.lean_waves / p.lean_sib));
@@ -1129,12 +1149,25 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
       }
       return launch_streaming(kern, dim3((unsigned)pairs), dim3((unsigned)p.n_part * 64), wg_lds_bytes, stream, p);
     };
+    if constexpr (kWidest) {
+      if (shared_rows) return bf16 ? go(attn_wg_kernel<D, true, FP8, GT, false>) : go(attn_wg_kernel<D, false, FP8, GT, false>);
+    }
     if (bf16) return go(attn_wg_kernel<D, true, FP8, GT>);
     return go(attn_wg_kernel<D, false, FP8, GT>);
   }
   int rc;
-  if (bf16) rc = launch_streaming(attn_partition_kernel<D, true, FP8, GT>, grid, dim3(64), lds, stream, p);
-  else rc = launch_streaming(attn_partition_kernel<D, false, FP8, GT>, grid, dim3(64), lds, stream, p);
+  bool launched = false;
+  if constexpr (kWidest) {
+    if (shared_rows) {
+      if (bf16) rc = launch_streaming(attn_partition_kernel<D, true, FP8, GT, false>, grid, dim3(64), lds, stream, p);
+      else rc = launch_streaming(attn_partition_kernel<D, false, FP8, GT, false>, grid, dim3(64), lds, stream, p);
+      launched = true;
+    }
+  }
+  if (!launched) {
+    if (bf16) rc = launch_streaming(attn_partition_kernel<D, true, FP8, GT>, grid, dim3(64), lds, stream, p);
+    else rc = launch_streaming(attn_partition_kernel<D, false, FP8, GT>, grid, dim3(64), lds, stream, p);
+  }
   if (rc) return rc;
   if (p.n_part > 1) {
     hipLaunchKernelGGL((attn_reduce_kernel<D>), dim3((unsigned)((batch * p.hq + 3) / 4)), dim3(256), 0,
@@ -1194,8 +1227,8 @@ __global__ __launch_bounds__(64) void attn_stream_probe_kernel(AttnParams p) {
   uint32_t fold = 0;
   auto request = [&](int slot, int tok) {
     const size_t o1 = tile_offset(tok + 16), o0 = tile_offset(tok);
-    load_k<D, FP8>(kf[slot], kc + o0, kc + o1, lane);
-    load_v<D, FP8>(vf[slot], vc + o0, vc + o1, voff);
+    load_k<D, FP8, true>(kf[slot], kc + o0, kc + o1, lane);
+    load_v<D, FP8, true>(vf[slot], vc + o0, vc + o1, voff);
   };
   auto consume = [&](int slot) {
 #pragma unroll

@@ -1065,6 +1065,9 @@ int pto_hip_set_option(const char* name, int64_t value) {
     PTO_CHECK_ARG(value == 0 || value == 1, "attn_autotune must be 0 or 1");
     c.attn_autotune = value;
     if (value == 0) attention_tuning_reset();
+  } else if (!std::strcmp(name, "w8a16_nt")) {
+    PTO_CHECK_ARG(value == 0 || value == 1, "w8a16_nt must be 0 or 1");
+    c.w8a16_nt = value;
   } else if (!std::strcmp(name, "attn_lean_siblings")) {
     PTO_CHECK_ARG(value == 0 || value == 1, "attn_lean_siblings must be 0 or 1");
     c.attn_lean_siblings = value;
@@ -1129,6 +1132,7 @@ int pto_hip_get_option(const char* name, int64_t* value) {
   else if (!std::strcmp(name, "attn_variant")) *value = c.attn_variant;
   else if (!std::strcmp(name, "attn_autotune")) *value = c.attn_autotune;
   else if (!std::strcmp(name, "attn_lean_siblings")) *value = c.attn_lean_siblings;
+  else if (!std::strcmp(name, "w8a16_nt")) *value = c.w8a16_nt;
   else if (!std::strcmp(name, "workspace_bytes"))  // read only: device memory the three grow-only scratch areas hold
     *value = (int64_t)(c.workspace_bytes + c.layer_ws_bytes + c.gemm_ws_bytes);
   else if (!std::strcmp(name, "attn_tuned_waves_per_cu") || !std::strcmp(name, "attn_tuned_workgroup_form")) {

@@ -81,7 +81,7 @@ struct Stage {
 
 // kWaves wavefronts per workgroup, kStages register stages per wavefront (kStages - 1 in flight),
 // kOcc wavefronts per SIMD the register budget is cut for.
-template <bool BF16, bool W8, int kCols, int kWaves, int kStages, int kOcc>
+template <bool BF16, bool W8, int kCols, int kWaves, int kStages, int kOcc, bool NT = false>
 __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOcc, kOcc))) void w8a16_partial_kernel(
     GemvParams p) {
   static_assert(kCols == 8 || (W8 && kCols == 16), "16 channels per lane only with int8 codes");
@@ -134,7 +134,8 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(kOc
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const char* row = wbase + (size_t)(kstep + e) * p.n * kWBytes;  // uniform
-      s.w[e] = *reinterpret_cast<const wvec_t*>(row + (size_t)lane_off * kWBytes);
+      if constexpr (NT) s.w[e] = __builtin_nontemporal_load(reinterpret_cast<const wvec_t*>(row + (size_t)lane_off * kWBytes));
+      else s.w[e] = *reinterpret_cast<const wvec_t*>(row + (size_t)lane_off * kWBytes);
     }
   };
   auto compute = [&](const Stage<W8, kCols>& s, int step) {
@@ -462,17 +463,19 @@ int w8a16_partials(const void* x, bool x_blocked, const void* wq0, const void* w
   // with 2-4 stages (more requests in flight per CU only lengthened the memory queueing delay).
   const dim3 block((unsigned)kWavesPerWg * 64);
   const bool bf = x_dtype == PTO_HIP_BF16;
+  const bool nt = ctx().w8a16_nt != 0;
+  auto go = [&](auto plain, auto streamed) { hipLaunchKernelGGL(nt ? streamed : plain, grid, block, 0, st, p); };
   if (w16) {  // twice the bytes per stage: three wavefronts per SIMD
-    if (bf) hipLaunchKernelGGL((w8a16_partial_kernel<true, false, 8, kWavesPerWg, 2, 3>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((w8a16_partial_kernel<false, false, 8, kWavesPerWg, 2, 3>), grid, block, 0, st, p);
+    if (bf) go(w8a16_partial_kernel<true, false, 8, kWavesPerWg, 2, 3>, w8a16_partial_kernel<true, false, 8, kWavesPerWg, 2, 3, true>);
+    else go(w8a16_partial_kernel<false, false, 8, kWavesPerWg, 2, 3>, w8a16_partial_kernel<false, false, 8, kWavesPerWg, 2, 3, true>);
   } else if (wide) {  // 32 accumulators per lane: two wavefronts per SIMD
-    if (bf) hipLaunchKernelGGL((w8a16_partial_kernel<true, true, 16, kWavesPerWg, 2, 2>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((w8a16_partial_kernel<false, true, 16, kWavesPerWg, 2, 2>), grid, block, 0, st, p);
+    if (bf) go(w8a16_partial_kernel<true, true, 16, kWavesPerWg, 2, 2>, w8a16_partial_kernel<true, true, 16, kWavesPerWg, 2, 2, true>);
+    else go(w8a16_partial_kernel<false, true, 16, kWavesPerWg, 2, 2>, w8a16_partial_kernel<false, true, 16, kWavesPerWg, 2, 2, true>);
   } else {
     // register budget of three wavefronts per SIMD: with four (128 registers) one value spilled to
     // scratch memory (decoder layer 183.0 -> 181.3 us a step)
-    if (bf) hipLaunchKernelGGL((w8a16_partial_kernel<true, true, 8, kWavesPerWg, 2, 3>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((w8a16_partial_kernel<false, true, 8, kWavesPerWg, 2, 3>), grid, block, 0, st, p);
+    if (bf) go(w8a16_partial_kernel<true, true, 8, kWavesPerWg, 2, 3>, w8a16_partial_kernel<true, true, 8, kWavesPerWg, 2, 3, true>);
+    else go(w8a16_partial_kernel<false, true, 8, kWavesPerWg, 2, 3>, w8a16_partial_kernel<false, true, 8, kWavesPerWg, 2, 3, true>);
   }
   PTO_CHECK_HIP(hipGetLastError());
   out->part[0] = p.part[0];

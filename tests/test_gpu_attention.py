@@ -387,7 +387,10 @@ def test_autotune_attention_picks_a_launch_shape_and_results_stay_correct(worker
         with worker.register(paged_attention) as h:
             best = autotune_attention(worker, h, [dev], rounds=5, candidates=[(0, 0), (0, 3), (512, 2), (2048, 0)])
             assert (best["tokens_per_partition"], best["waves_per_cu"]) in best["timings"]
-            assert best["us"] == min(best["timings"].values()) and best["default_us"] == best["timings"][(0, 0)]
+            # the library's own choice (0, 0) stays unless a candidate beats it by more than 1 %
+            assert best["default_us"] == best["timings"][(0, 0)]
+            assert best["us"] == best["timings"][(best["tokens_per_partition"], best["waves_per_cu"])]
+            assert best["us"] <= best["default_us"] and best["us"] <= min(best["timings"].values()) / 0.99 + 1e-9
             assert worker.get_option("attn_tokens_per_partition") == best["tokens_per_partition"]
             assert worker.get_option("attn_waves_per_cu") == best["waves_per_cu"]
             for tpp, cap in best["timings"]:
