@@ -62,9 +62,12 @@ __global__ __launch_bounds__(256) void paged_gather_kernel(GatherParams p, int l
     uint8_t* d = p.out + row * p.out_row_bytes;
     const int64_t nb = p.out_row_bytes;
     if ((((uintptr_t)s | (uintptr_t)d | (uintptr_t)nb) & 15) == 0) {
-      const uint4* s4 = reinterpret_cast<const uint4*>(s);
-      uint4* d4 = reinterpret_cast<uint4*>(d);
-      for (int64_t i = sub; i < nb / 16; i += lanes_per_row) d4[i] = s4[i];
+      // every row is read once and written once: both sides with the non-temporal hint
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      const u32x4* s4 = reinterpret_cast<const u32x4*>(s);
+      u32x4* d4 = reinterpret_cast<u32x4*>(d);
+      for (int64_t i = sub; i < nb / 16; i += lanes_per_row)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(s4 + i), d4 + i);
     } else {
       for (int64_t i = sub; i < nb; i += lanes_per_row) d[i] = s[i];
     }
