@@ -176,6 +176,21 @@ def main() -> int:
 
     # ---- paged-attention decode, small configuration ------------------------------------
     pools = [workloads.attention_small(seed=0, device="cuda") for _ in range(KV_POOLS)]
+    # The inputs of the other bandwidth-bound configurations are built now, so that no block's memory
+    # placement depends on what an earlier block has freed.  (Their step times come in two modes 3-4 %
+    # apart from one process to the next - same box, same tensors at the same addresses - and are
+    # stable within a process.)
+    want_layer = not args.no_extra and not args.no_layer
+    want_long = not args.no_extra and not args.no_long
+    if want_layer:
+        # Two layers with weights of their own, taken in turn: 218 MB of int8 weights would otherwise stay in
+        # the 256 MB last-level cache from one step to the next (the K/V rows pass through it without
+        # settling), which no model with more than one layer offers.
+        dl = workloads.decoder_layer_inputs(device="cuda")
+        dl_other = workloads.decoder_layer_inputs(device="cuda", seed=1)
+    if want_long:
+        lf = workloads.attention_long_fp8(seed=0, device="cuda")
+    probe_buf = torch.zeros(2 << 30, dtype=torch.uint8, device="cuda")
     torch.cuda.synchronize()
     step_bytes = pools[0].algorithmic_bytes()
     handle = worker.register(paged_attention)
@@ -282,8 +297,6 @@ def main() -> int:
     # and once with a contiguous stream per wavefront (independent streams, which is what paged
     # attention and the projections' column slabs are).  The ceilings of every bandwidth-bound figure
     # below, next to the published peak.
-    probe_buf = torch.empty(2 << 30, dtype=torch.uint8, device="cuda")
-    probe_buf.zero_()
     sweep = max(hbm_read_probe(worker, probe_buf, waves_per_cu=w)["gbps"] for w in (4, 8, 16))
     streams = max(hbm_read_probe(worker, probe_buf, streams=True, waves_per_cu=w)["gbps"] for w in (4, 8, 16))
     result["roofline"]["read_probe_gbps"] = {"one_sweep": round(sweep, 1), "stream_per_wavefront": round(streams, 1)}
@@ -309,6 +322,79 @@ def main() -> int:
     del pools, prepared
     worker.set_option("attn_tokens_per_partition", 0)
     worker.set_option("attn_waves_per_cu", 0)
+
+    # ---- the path's other configurations --------------------------------------------------------
+    if want_layer:
+        with worker.register(decoder_layer_decode) as dh:
+            dargs = [dl.args(), dl_other.args()]
+            dtuned = {"tokens_per_partition": 0, "waves_per_cu": 0}
+            if not args.no_autotune:
+                dtuned = autotune_attention(worker, dh, dargs, rounds=30)
+            benchmark(dh, dargs, rounds=300, warmup=0)  # ~50 ms: past the library's launch-shape measurement and the
+            dstats = benchmark(dh, dargs, rounds=60, warmup=0)   # clock ramp after the idle time of the CPU timings above
+        worker.set_option("attn_tokens_per_partition", 0)
+        worker.set_option("attn_waves_per_cu", 0)
+        dbytes = dl.algorithmic_bytes()
+        result["decoder_layer"] = _hbm_block(
+            "decoder-layer decode step: H4096 Hq32 Hkv8 D128 I14336 B32 ctx4096, int8 weights with per-channel "
+            "scales, bf16 activations and paged KV; two layers (weights and caches of their own) in turn, so that every "
+            "step's weights come from HBM", dbytes, dstats.device_wall_us)
+        result["decoder_layer"]["attn_tokens_per_partition"] = dtuned["tokens_per_partition"]
+        result["decoder_layer"]["attn_waves_per_cu"] = dtuned["waves_per_cu"]
+        if cpu:
+            # four of the 32 sequences: their blocks in a compact pool; the weights are the full ones
+            seqs = [0, 9, 18, 27]
+            mb, hkv, bs = dl.max_num_blocks_per_req, dl.kv_head_num, dl.block_size
+            blocks = dl.block_table.reshape(-1, mb)[seqs].reshape(-1).long()
+            rows = (blocks[:, None] * (hkv * bs) + torch.arange(hkv * bs, device="cuda")[None, :]).reshape(-1)
+            hw = [t.cpu() for name in ("qkv", "o", "gate", "up", "down") for t in dl.weights[name]]
+            hargs = (dl.hidden[seqs].cpu(), dl.seq_lens[seqs].cpu(), torch.arange(len(seqs) * mb, dtype=torch.int32),
+                     dl.key_cache[rows].cpu(), dl.value_cache[rows].cpu(), dl.rope_cos.cpu(), dl.rope_sin.cpu(),
+                     dl.gamma_in.cpu(), dl.gamma_post.cpu(), *hw)
+            kw = dict(num_heads=dl.num_heads, kv_head_num=hkv, head_dim=dl.head_dim, block_size=bs,
+                      max_num_blocks_per_req=mb, eps=dl.eps)
+            med, n = _time_cpu(lambda: oracle.decoder_layer_decode(*hargs, **kw), 6.0, min_runs=2)
+            wbytes = sum(c.numel() * c.element_size() for c, _ in dl.weights.values())
+            sub_bytes = wbytes + (dbytes - wbytes) * len(seqs) // dl.hidden.shape[0]
+            result["decoder_layer"]["cpu_baseline"] = {
+                "value": round(sub_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+                "sample": f"{len(seqs)} of the 32 sequences through the oracle's decoder_layer_decode with the full "
+                          f"weights (bytes = all weights + those sequences' K/V): median of {n} runs, "
+                          f"{med * 1e3:.0f} ms per run"}
+            del hw, hargs
+        del dl, dl_other, dargs
+        torch.cuda.empty_cache()
+
+    if want_long:
+        with worker.register(paged_attention) as lh:
+            largs = [lf.args()]
+            benchmark(lh, largs, rounds=100, warmup=0)  # ~45 ms: the GPU has idled during the CPU timings above
+            lstats = benchmark(lh, largs, rounds=30, warmup=0)
+        result["attention_long_fp8"] = _hbm_block(
+            "paged-attention decode long: B64 Hq64 Hkv8 D128 bs128 ctx~U[8192,32768], e4m3 KV with one fp32 scale per "
+            "(block, KV head), dequantised in-kernel", lf.algorithmic_bytes(), lstats.device_wall_us)
+        if cpu:
+            # one whole sequence of the batch: its blocks gathered into a compact pool with an identity table
+            cfg = lf.config.tolist()
+            b, hq, hkv, d, bs, mb = cfg[:6]
+            seq = 0
+            ctx = int(lf.context_lens[seq])
+            nblk = (ctx + bs - 1) // bs
+            blocks = lf.block_table.reshape(b, mb)[seq, :nblk].long()
+            rows = (blocks[:, None] * (hkv * bs) + torch.arange(hkv * bs, device="cuda")[None, :]).reshape(-1)
+            sub = (lf.query[seq * hq:(seq + 1) * hq].cpu(), lf.key_cache[rows].cpu(), lf.value_cache[rows].cpu(),
+                   torch.arange(nblk, dtype=torch.int32), lf.context_lens[seq:seq + 1].cpu(),
+                   torch.tensor([1, hq, hkv, d, bs, nblk, cfg[6]], dtype=torch.int64),
+                   lf.k_scale[blocks].cpu(), lf.v_scale[blocks].cpu())
+            med, n = _time_cpu(lambda: oracle.paged_attention_golden(*sub), 5.0)
+            sub_bytes = ctx * hkv * d * 2 + nblk * hkv * 8 + hq * d * 6
+            result["attention_long_fp8"]["cpu_baseline"] = {
+                "value": round(sub_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+                "sample": f"one of the 64 sequences (context {ctx}) through the torch block-loop golden, codes "
+                          f"dequantised on the host: median of {n} runs, {med * 1e3:.0f} ms per run"}
+            del sub
+        del lf, largs
+        torch.cuda.empty_cache()
 
     # ---- FFN block at LLaMA-7B shape (second half of the metric) ------------------------------
     if not args.no_ffn:
@@ -400,87 +486,6 @@ def main() -> int:
                           f"median of {n} runs, {med * 1e3:.0f} ms per run"}
             del hq_args, hx
         del f, q, qargs, bf16_out
-        torch.cuda.empty_cache()
-
-    # ---- the path's other configurations --------------------------------------------------------
-    if not args.no_extra and not args.no_long:
-        lf = workloads.attention_long_fp8(seed=0, device="cuda")
-        torch.cuda.synchronize()
-        with worker.register(paged_attention) as lh:
-            largs = [lf.args()]
-            benchmark(lh, largs, rounds=3, warmup=0)
-            lstats = benchmark(lh, largs, rounds=10, warmup=0)
-        result["attention_long_fp8"] = _hbm_block(
-            "paged-attention decode long: B64 Hq64 Hkv8 D128 bs128 ctx~U[8192,32768], e4m3 KV with one fp32 scale per "
-            "(block, KV head), dequantised in-kernel", lf.algorithmic_bytes(), lstats.device_wall_us)
-        if cpu:
-            # one whole sequence of the batch: its blocks gathered into a compact pool with an identity table
-            cfg = lf.config.tolist()
-            b, hq, hkv, d, bs, mb = cfg[:6]
-            seq = 0
-            ctx = int(lf.context_lens[seq])
-            nblk = (ctx + bs - 1) // bs
-            blocks = lf.block_table.reshape(b, mb)[seq, :nblk].long()
-            rows = (blocks[:, None] * (hkv * bs) + torch.arange(hkv * bs, device="cuda")[None, :]).reshape(-1)
-            sub = (lf.query[seq * hq:(seq + 1) * hq].cpu(), lf.key_cache[rows].cpu(), lf.value_cache[rows].cpu(),
-                   torch.arange(nblk, dtype=torch.int32), lf.context_lens[seq:seq + 1].cpu(),
-                   torch.tensor([1, hq, hkv, d, bs, nblk, cfg[6]], dtype=torch.int64),
-                   lf.k_scale[blocks].cpu(), lf.v_scale[blocks].cpu())
-            med, n = _time_cpu(lambda: oracle.paged_attention_golden(*sub), 5.0)
-            sub_bytes = ctx * hkv * d * 2 + nblk * hkv * 8 + hq * d * 6
-            result["attention_long_fp8"]["cpu_baseline"] = {
-                "value": round(sub_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-                "sample": f"one of the 64 sequences (context {ctx}) through the torch block-loop golden, codes "
-                          f"dequantised on the host: median of {n} runs, {med * 1e3:.0f} ms per run"}
-            del sub
-        del lf, largs
-        torch.cuda.empty_cache()
-
-    if not args.no_extra and not args.no_layer:
-        # Two layers with weights of their own, taken in turn: 218 MB of int8 weights would otherwise stay in
-        # the 256 MB last-level cache from one step to the next (the K/V rows pass through it without
-        # settling), which no model with more than one layer offers.
-        dl = workloads.decoder_layer_inputs(device="cuda")
-        dl_other = workloads.decoder_layer_inputs(device="cuda", seed=1)
-        torch.cuda.synchronize()
-        with worker.register(decoder_layer_decode) as dh:
-            dargs = [dl.args(), dl_other.args()]
-            dtuned = {"tokens_per_partition": 0, "waves_per_cu": 0}
-            if not args.no_autotune:
-                dtuned = autotune_attention(worker, dh, dargs, rounds=30)
-            benchmark(dh, dargs, rounds=30, warmup=0)  # past the library's launch-shape measurement
-            dstats = benchmark(dh, dargs, rounds=20, warmup=0)
-        worker.set_option("attn_tokens_per_partition", 0)
-        worker.set_option("attn_waves_per_cu", 0)
-        dbytes = dl.algorithmic_bytes()
-        result["decoder_layer"] = _hbm_block(
-            "decoder-layer decode step: H4096 Hq32 Hkv8 D128 I14336 B32 ctx4096, int8 weights with per-channel "
-            "scales, bf16 activations and paged KV; two layers (weights and caches of their own) in turn, so that every "
-            "step's weights come from HBM", dbytes, dstats.device_wall_us)
-        result["decoder_layer"]["attn_tokens_per_partition"] = dtuned["tokens_per_partition"]
-        result["decoder_layer"]["attn_waves_per_cu"] = dtuned["waves_per_cu"]
-        if cpu:
-            # four of the 32 sequences: their blocks in a compact pool; the weights are the full ones
-            seqs = [0, 9, 18, 27]
-            mb, hkv, bs = dl.max_num_blocks_per_req, dl.kv_head_num, dl.block_size
-            blocks = dl.block_table.reshape(-1, mb)[seqs].reshape(-1).long()
-            rows = (blocks[:, None] * (hkv * bs) + torch.arange(hkv * bs, device="cuda")[None, :]).reshape(-1)
-            hw = [t.cpu() for name in ("qkv", "o", "gate", "up", "down") for t in dl.weights[name]]
-            hargs = (dl.hidden[seqs].cpu(), dl.seq_lens[seqs].cpu(), torch.arange(len(seqs) * mb, dtype=torch.int32),
-                     dl.key_cache[rows].cpu(), dl.value_cache[rows].cpu(), dl.rope_cos.cpu(), dl.rope_sin.cpu(),
-                     dl.gamma_in.cpu(), dl.gamma_post.cpu(), *hw)
-            kw = dict(num_heads=dl.num_heads, kv_head_num=hkv, head_dim=dl.head_dim, block_size=bs,
-                      max_num_blocks_per_req=mb, eps=dl.eps)
-            med, n = _time_cpu(lambda: oracle.decoder_layer_decode(*hargs, **kw), 6.0, min_runs=2)
-            wbytes = sum(c.numel() * c.element_size() for c, _ in dl.weights.values())
-            sub_bytes = wbytes + (dbytes - wbytes) * len(seqs) // dl.hidden.shape[0]
-            result["decoder_layer"]["cpu_baseline"] = {
-                "value": round(sub_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-                "sample": f"{len(seqs)} of the 32 sequences through the oracle's decoder_layer_decode with the full "
-                          f"weights (bytes = all weights + those sequences' K/V): median of {n} runs, "
-                          f"{med * 1e3:.0f} ms per run"}
-            del hw, hargs
-        del dl, dl_other, dargs
         torch.cuda.empty_cache()
 
     # ---- shapes outside the benchmark configurations (on request) ---------------------------------
