@@ -34,7 +34,7 @@ MFMA_FP8_PEAK_TFLOPS = 5000.0   # MI355X dense fp8
 KV_POOLS = 4                   # 4 x 537 MB of K+V, cycled
 ROOT = Path(__file__).resolve().parent
 PROFILE = ROOT / "profiles" / "bench_attention_small_ffn_llama7b.json"
-DOMINANT_KERNEL = "attn_partition_kernel<128, true, false, 1>"
+DOMINANT_KERNEL = "attn_partition_kernel<128, true, false, 1, true>"
 
 
 def _profile_figures() -> dict:
