@@ -539,9 +539,10 @@ PTO_HIP_API int pto_hip_backend_handler_query(const char* hook, int32_t arg, cha
  *                               under stream capture and pto_hip_paged_attention_noalloc never measure.
  *  "attn_lean_siblings"         evenly split form with several query tiles per KV head (more than 64 heads on
  *                               one KV head, 32 at head_dim 256): 1 = the tiles of a KV head are carried by
- *                               sibling wavefronts of one workgroup that walk the same chunks side by side,
- *                               so the second reader of a K/V row finds it in its own L2 (default); 0 =
- *                               every tile is a stream of its own, placed wherever the list puts it
+ *                               sibling wavefronts that walk the same chunks side by side; two tiles over a
+ *                               16-bit cache run as a pair that reads every cache row once and shares it
+ *                               through LDS (default); 2 = sibling wavefronts that each read the rows (the
+ *                               second finds them in L2); 0 = every tile is a stream of its own
  *  "w8a16_nt"                   skinny projections (up to 32 rows): 1 = the weight rows, read once per call, are
  *                               loaded with the non-temporal hint so that they do not displace what other
  *                               kernels keep in the caches (default); 0 = ordinary loads

@@ -59,6 +59,7 @@ struct AttnParams {
   int resident_cap;  // partition grid: wavefronts allowed on a CU at once, 0 = as many as fit
   int wg_merge;    // one workgroup per (sequence, KV head, query tile), merged through LDS: 1, else 0
   int lean_sib;    // evenly split form: wavefronts of one workgroup that share a run of chunks, one query tile each
+  int lean_pair;   // ... as workgroups of one pair of siblings that share the cache rows through LDS
   int n_wg;        // evenly split form: resident workgroups (one per CU); 0 = partition grid
   int lean_waves;  // ... and wavefronts in each
   float scale_log2e;
@@ -508,6 +509,145 @@ __device__ __forceinline__ void attend_range(const AttnParams& p, int b, int h, 
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Two query tiles of one KV head on a pair of wavefronts that read every cache row once between
+// them (16-bit caches).  With more query heads on a KV head than one wavefront carries, the tiles'
+// wavefronts each used to read all of K and V, the second time from L2 - twice the bytes through
+// the CU's L1, which is what bounds such launches.  Here the pair forms a workgroup of its own and
+// shares both operands through LDS: of every 32-token chunk wavefront r requests K tile r and V
+// rows 16 r .. 16 r + 15 (coalesced, 1 KB per instruction, non-temporal), parks them in a stage
+// both read - K back in operand order as in attend_range, V in the order pv_chunk's transposes
+// expect - and one barrier per chunk separates the writes of a stage from its reads; two stages
+// alternate, so the requests of chunk n + 1 are in flight during all of chunk n's arithmetic.
+// Arguments and results as attend_range; pair_lds is the workgroup's LDS, r the wavefront's index
+// in the pair.  Both wavefronts must call it with the same range.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+struct PairStage {
+  typedef KStage<D, false> K;
+  static constexpr int kVPitch = K::kRowBytes + 16;
+  static constexpr int kVBytes = 32 * kVPitch;
+  static constexpr int kBytes = K::kBytes + kVBytes;  // one of the two alternating stages
+  static constexpr int kLoads = K::kLoads;            // 16-byte loads per lane for 16 rows
+};
+
+// LDS writes of this wavefront done, then the workgroup's barrier - without the wait for the global
+// loads in flight that a full fence (__syncthreads) would add.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int D, bool BF16, int GT>
+__device__ __forceinline__ void attend_range_pair(const AttnParams& p, int b, int h, int hq_row0, int g0, int tok_first,
+                                                  int tok_end, int c, int j, int r, char* pair_lds, int first_window,
+                                                  f32x4 (&acc)[GT][D / 128][8], float (&m_run)[GT],
+                                                  float (&l_run)[GT], float& v_unit) {
+  typedef PairStage<D> S;
+  typedef KStage<D, false> KS;
+  const int lane = j * 16 + c;
+  u32x4 qf[GT][D / 32];
+#pragma unroll
+  for (int t = 0; t < GT; ++t) {
+    const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + (size_t)(hq_row0 + t * 16 + c) * D;
+    const bool g_valid = g0 + t * 16 + c < p.group;
+#pragma unroll
+    for (int s = 0; s < D / 32; ++s) {
+      u32x4 z = {0u, 0u, 0u, 0u};
+      qf[t][s] = g_valid ? *reinterpret_cast<const u32x4*>(qrow + (s * 4 + j) * 8) : z;
+    }
+  }
+  const char* kc = reinterpret_cast<const char*>(p.kc);
+  const char* vc = reinterpret_cast<const char*>(p.vc);
+  const int32_t* table = p.block_table + (size_t)b * p.max_blocks;
+
+  int win_base = 0, win_blk = 0;
+  bool bad_entry = false;
+  auto load_window = [&](int first_block, bool preloaded) {
+    win_base = first_block;
+    const int idx = min(first_block + lane, p.max_blocks - 1);
+    win_blk = preloaded ? first_window : table[idx];
+    if (p.pool_blocks > 0 && (unsigned)win_blk >= (unsigned)p.pool_blocks) {
+      bad_entry |= (first_block + lane) * p.bs < tok_end;
+      win_blk = 0;
+    }
+    if (!preloaded) asm volatile("" : "+v"(win_blk));  // keeps the wait for a refill on its own branch
+  };
+  load_window(tok_first / p.bs, true);
+  // byte offset of this wavefront's 16-token tile of the chunk starting at `tok`
+  auto tile_offset = [&](int tok) -> size_t {
+    tok += r * 16;
+    if (tok >= tok_end) tok = tok_first;
+    const int lb = tok / p.bs;
+    if (lb < win_base || lb >= win_base + 64) load_window(lb, false);
+    const int blk = __builtin_amdgcn_readlane(win_blk, lb - win_base);
+    return ((size_t)(blk * p.hkv + h) * p.bs + (tok % p.bs)) * (D * 2);
+  };
+
+#pragma unroll
+  for (int t = 0; t < GT; ++t) {
+#pragma unroll
+    for (int set = 0; set < D / 128; ++set)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[t][set][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m_run[t] = kMinMax;
+    l_run[t] = 0.f;
+  }
+  v_unit = 1.f;
+
+  u32x4 kh[S::kLoads], vh[S::kLoads];  // this wavefront's 16 rows of K and of V, memory order
+  auto request = [&](int tok) {
+    const size_t o = tile_offset(tok);
+#pragma unroll
+    for (int s = 0; s < S::kLoads; ++s) {
+      kh[s] = stream_load<u32x4>(kc + o + s * 1024 + lane * 16);
+      vh[s] = stream_load<u32x4>(vc + o + s * 1024 + lane * 16);
+    }
+  };
+  auto park = [&](char* stage) {  // registers -> the stage's K tile r and V rows 16 r ..
+#pragma unroll
+    for (int s = 0; s < S::kLoads; ++s) {
+      const int off = s * 1024 + lane * 16;
+      const int row = off / KS::kRowBytes, col = off % KS::kRowBytes;
+      *reinterpret_cast<u32x4*>(stage + r * KS::kTileBytes + row * KS::kPitch + col) = kh[s];
+      *reinterpret_cast<u32x4*>(stage + KS::kBytes + (r * 16 + row) * S::kVPitch + col) = vh[s];
+    }
+  };
+
+  request(tok_first);
+  park(pair_lds);
+  lds_barrier();
+  int cur = 0;
+  for (int tok = tok_first; tok < tok_end; tok += kChunk) {
+    char* stage = pair_lds + cur * S::kBytes;
+    KFrag<D, false> kf;
+    fetch_k<D, false>(kf, stage, c, j);
+    request(tok + kChunk);  // the next chunk, in flight during this one's arithmetic
+    f32x4 s0[GT], s1[GT];
+#pragma unroll
+    for (int t = 0; t < GT; ++t) qk_scores<D, BF16, false>(kf, qf[t], s0[t], s1[t]);
+    u32x4 pf[GT];
+#pragma unroll
+    for (int t = 0; t < GT; ++t)
+      pf[t] = softmax_chunk<D, BF16>(s0[t], s1[t], tok, tok_end, j, p.scale_log2e, acc[t], m_run[t], l_run[t]);
+    VFrag<D, false> vf;
+#pragma unroll
+    for (int set = 0; set < D / 128; ++set)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int t_row = (e >> 2) * 16 + j * 4 + (e & 3);
+        vf.t[set][e] = *reinterpret_cast<const u32x4*>(stage + KS::kBytes + t_row * S::kVPitch + (set * 16 + c) * 16);
+      }
+    pv_chunk<D, BF16, false, GT>(vf, pf, tok, tok_end, j, acc);
+    cur ^= 1;
+    park(pair_lds + cur * S::kBytes);
+    lds_barrier();
+  }
+  if (bad_entry) *p.error_flag = 1;
+#pragma unroll
+  for (int t = 0; t < GT; ++t) {
+    l_run[t] += __shfl_xor(l_run[t], 16);
+    l_run[t] += __shfl_xor(l_run[t], 32);
+  }
+}
+
 template <int D, bool BF16, bool FP8, int GT, bool ONCE = true>
 __global__ __launch_bounds__(64) void attn_partition_kernel(AttnParams p) {
   const int lane = threadIdx.x;
@@ -860,16 +1000,18 @@ __device__ __forceinline__ void lean_locate(const AttnParams& p, int lane, int h
 // wavefront: four wavefronts (one per SIMD) there.
 constexpr int lean_max_waves(int d, int gt) { return d == 128 && gt == 1 ? kLeanMaxWaves : 4; }
 
-template <int D, bool BF16, bool FP8, int GT, bool ONCE = true>
-__global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(AttnParams p) {
+// PAIR: workgroups of exactly two sibling wavefronts that share the cache rows through LDS
+// (attend_range_pair); 16-bit caches, two query tiles per KV head.
+template <int D, bool BF16, bool FP8, int GT, bool ONCE = true, bool PAIR = false>
+__global__ __launch_bounds__(PAIR ? 128 : lean_max_waves(D, GT) * 64) void attn_lean_kernel(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char lean_lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, j = lane >> 4;
   // Query tiles of one KV head read the same K and V.  With lean_sib = gtiles the tiles are carried
   // by sibling wavefronts of one workgroup that walk the same run of chunks side by side: whichever
-  // is behind finds the rows in this XCD's L2, so every cache byte crosses the fabric once.  Then
-  // the item list runs over (sequence, KV head, chunk) only.
+  // is behind finds the rows in this XCD's L2, so every cache byte crosses the fabric once (and, in
+  // the PAIR form, the CU's L1 once).  Then the item list runs over (sequence, KV head, chunk) only.
   const int sib = p.lean_sib;
   const int hg_count = p.hkv * p.gtiles / sib;
   const int max_ctx = p.ctx_cap;
@@ -916,8 +1058,14 @@ __global__ __launch_bounds__(lean_max_waves(D, GT) * 64) void attn_lean_kernel(A
     float m_run[GT], l_run[GT], v_unit;
     const int first_window =
         p.block_table[(size_t)b * p.max_blocks + min(tok_first / p.bs + lane, p.max_blocks - 1)];
-    attend_range<D, BF16, FP8, GT, ONCE>(p, b, h, hq_row0, g0, tok_first, tok_end, kChunk, c, j, kbuf, first_window,
-                                   acc, m_run, l_run, v_unit);
+    if constexpr (PAIR) {
+      static_assert(!FP8, "the pair form is built for 16-bit caches");
+      attend_range_pair<D, BF16, GT>(p, b, h, hq_row0, g0, tok_first, tok_end, c, j, wave, lean_lds, first_window, acc,
+                                     m_run, l_run, v_unit);
+    } else {
+      attend_range<D, BF16, FP8, GT, ONCE>(p, b, h, hq_row0, g0, tok_first, tok_end, kChunk, c, j, kbuf, first_window,
+                                           acc, m_run, l_run, v_unit);
+    }
 #pragma unroll
     for (int t = 0; t < GT; ++t) {
       if (g0 + t * 16 + c >= p.group) continue;
@@ -1107,7 +1255,10 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
   if (p.n_wg > 0) {
     // Evenly split form: one workgroup of lean_waves wavefronts per CU.  The LDS request (K stages
     // of the wavefronts, padded past half of the CU's LDS) keeps a second workgroup off the CU.
-    const size_t lean_lds = std::max<size_t>((size_t)p.lean_waves * KStage<D, FP8>::kBytes, 84 * 1024);
+    size_t lean_lds = std::max<size_t>((size_t)p.lean_waves * KStage<D, FP8>::kBytes, 84 * 1024);
+    if constexpr (!FP8) {
+      if (p.lean_pair) lean_lds = 2 * (size_t)PairStage<D>::kBytes;  // two alternating stages; two workgroups fit a CU
+    }
     dim3 lgrid(p.n_wg), lblock(p.lean_waves * 64);
     auto go = [&](auto kern) -> int {
       // per instantiation; setting the attribute twice from two threads is harmless
@@ -1121,6 +1272,16 @@ int launch(const AttnParams& p, int batch, bool bf16, hipStream_t stream) {
     };
     int rc = PTO_HIP_OK;
     if constexpr (kWidest) {
+      if constexpr (!FP8) {
+        if (p.lean_pair) {
+          rc = bf16 ? go(attn_lean_kernel<D, true, FP8, GT, true, true>) : go(attn_lean_kernel<D, false, FP8, GT, true, true>);
+          if (rc) return rc;
+          hipLaunchKernelGGL((attn_lean_reduce_kernel<D>), dim3((unsigned)((batch * p.hq + 3) / 4)), dim3(256), 0, stream,
+                             p, (long long)p.n_wg * (p.lean_waves / p.lean_sib));
+          PTO_CHECK_HIP(hipGetLastError());
+          return PTO_HIP_OK;
+        }
+      }
       if (shared_rows) rc = bf16 ? go(attn_lean_kernel<D, true, FP8, GT, false>) : go(attn_lean_kernel<D, false, FP8, GT, false>);
       else rc = bf16 ? go(attn_lean_kernel<D, true, FP8, GT>) : go(attn_lean_kernel<D, false, FP8, GT>);
     } else {
@@ -1581,6 +1742,14 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     p.n_wg = cx.num_cu;
     p.lean_waves = (int)waves;
     p.lean_sib = (p.gtiles > 1 && waves % p.gtiles == 0 && cx.attn_lean_siblings != 0) ? p.gtiles : 1;
+    const bool widest = (d == 128 && gt == 4) || (d == 256 && gt == 2);
+    if (p.lean_sib == 2 && !fp8 && widest && cx.attn_lean_siblings == 1) {
+      // one workgroup per pair of siblings, waves / 2 of them per CU
+      p.lean_pair = 1;
+      p.n_wg = cx.num_cu * (int)(waves / 2);
+      p.lean_waves = 2;
+      waves = 2;
+    }
     // partial slots: one per (sequence, head, tile) plus one per resident wavefront
     const size_t slots = (size_t)batch * hkv * p.gtiles + (size_t)p.n_wg * waves;
     const size_t o_bytes = slots * p.gt_rows * d * sizeof(float), ml_bytes = slots * p.gt_rows * 2 * sizeof(float);

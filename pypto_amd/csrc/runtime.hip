@@ -1069,7 +1069,7 @@ int pto_hip_set_option(const char* name, int64_t value) {
     PTO_CHECK_ARG(value == 0 || value == 1, "w8a16_nt must be 0 or 1");
     c.w8a16_nt = value;
   } else if (!std::strcmp(name, "attn_lean_siblings")) {
-    PTO_CHECK_ARG(value == 0 || value == 1, "attn_lean_siblings must be 0 or 1");
+    PTO_CHECK_ARG(value >= 0 && value <= 2, "attn_lean_siblings must be 0, 1 or 2");
     c.attn_lean_siblings = value;
   } else if (!std::strcmp(name, "attn_kernel_timing")) {
     c.attn_kernel_timing = value != 0;

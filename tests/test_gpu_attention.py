@@ -510,15 +510,16 @@ def test_launch_shape_settles_by_measurement_and_never_changes_a_bit(worker):
 def test_evenly_split_form_with_several_query_tiles_per_kv_head(worker, hq, hkv, d, fp8):
     """More query heads on a KV head than one wavefront carries (64, or 32 at head_dim 256): in the
     evenly split form the tiles of a KV head ride on sibling wavefronts of one workgroup and walk
-    the same run of chunks (`attn_lean_siblings`, default) - or, with 4 wavefronts and 3 tiles, each
-    tile is a stream of its own.  Ragged lengths incl. an empty sequence, both layouts against the
-    golden, and the two against each other."""
+    the same run of chunks (`attn_lean_siblings`; two tiles over a 16-bit cache as a pair that shares the
+    rows through LDS, the default, or each reading them, 2) - or, with 4 wavefronts and 3 tiles, each
+    tile is a stream of its own.  Ragged lengths incl. an empty sequence, every layout against the
+    golden, and all against each other."""
     inp = workloads.paged_attention_inputs(batch=6, num_heads=hq, kv_head_num=hkv, head_dim=d, block_size=64,
                                            context_lens=[0, 1, 700, 3000, 1500, 33], ctx_range=(1, 3000),
                                            fp8_kv=fp8, seed=21)
     ref = _golden(inp)
     outs = []
-    for sib in (1, 0):
+    for sib in (1, 2, 0):
         worker.set_option("attn_lean_siblings", sib)
         try:
             for waves in (-4, -2):

@@ -109,7 +109,8 @@ def _attention_wide_group_sweep(worker, seed, cases):
             align = bs if bs >= 32 else 32
             variant, tpp, waves, gt, sib = rng.choice([
                 (-1, 0, 0, 0, 1), (0, align * rng.randint(1, 8), 0, 0, 1), (2, align * rng.randint(1, 8), 0, 0, 1),
-                (1, 0, rng.choice([0, 2, 4, 8]), 0, 1), (1, 0, rng.choice([0, 2, 4]), 0, 0), (1, 0, 0, rng.choice([1, 2]), 1),
+                (1, 0, rng.choice([0, 2, 4, 8]), 0, 1), (1, 0, rng.choice([0, 2, 4]), 0, 0), (1, 0, rng.choice([0, 2, 4]), 0, 2),
+                (1, 0, 0, rng.choice([1, 2]), 1),
                 (2, 0, 0, rng.choice([1, 2]), 1)])
             print(f"wide-group attention case {case} (seed {seed}): B{batch} Hq{hq} Hkv{hkv} D{d} bs{bs} ctx{ctxs} {dtype} "
                   f"e4m3={fp8} mb={mb} variant={variant} tpp={tpp} waves={waves} tiles={gt} siblings={sib}", flush=True)
