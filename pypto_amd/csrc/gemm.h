@@ -472,6 +472,265 @@ int launch_gemm(GemmParams p, hipStream_t st) {
   return launch_gemm_e<MT, WM, WN, DUAL, BF16, 0, OutT, W8>(p, st);
 }
 
+// ---- four wavefronts, one per SIMD ---------------------------------------------------------------
+// The 256 x 256 tile as 2 x 2 wavefronts that own 128 x 128 each (4 x 4 accumulators, 256 accumulator
+// registers): a k-step's fragments are 8 KB per wavefront for 16 MFMAs where the eight-wavefront form
+// reads 6 KB for 8, a third less LDS traffic per MFMA.  A SIMD then has a single instruction stream
+// and a wavefront issues at most one instruction every four clocks, eight per MFMA, so the loop must
+// be lean and nothing may stall it:
+//  - the tiles are cut into stages of 32 k (16 KB of A + 16 KB of B) and five stages (all of a CU's
+//    LDS) rotate - one computed on, the next complete and being read for its first fragments, the
+//    third landing, the last two requested - so that the barrier at the end of an iteration waits
+//    for data requested three iterations earlier and the first fragments of the next stage are
+//    already in registers when it falls;
+//  - the loop is unrolled over the five stages, so every LDS address is a loop-invariant register
+//    plus an immediate and every request is one scalar add into m0 plus the load.
+// Operands go global -> LDS directly, as in the eight-wavefront form; with four 16-byte chunks to an
+// A row the swizzle key is (row / 4) % 4 (16 consecutive rows of a fragment read then cover all 16
+// slots of four rows' worth of banks), B keeps 64-byte group g ^ (k-row % 8).  Built for 16-bit
+// weights with m, n and every k range multiples of the tile.
+constexpr int QK = 32;   // k extent of a stage
+constexpr int QST = 5;   // stages
+constexpr int kQuadStageBytes = (256 * QK + QK * BN) * 2;  // A rows, then B rows
+typedef __attribute__((address_space(3))) const char lds_cchar;
+typedef __attribute__((address_space(3))) const u32x4 lds_cu32x4;
+template <int N>
+struct QuadConst {
+  static constexpr int value = N;
+};
+
+// One direct request: 16 bytes per lane from `src` to the KB of LDS at lds_w + OFF (wave-uniform).
+template <int OFF>
+__device__ __forceinline__ void quad_to_lds(const char* src, uint32_t lds_w) {
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // m0 is named as clobbered on purpose
+  asm volatile("s_add_u32 m0, %1, %2\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_w), "n"(OFF) : "memory", "m0", "scc");
+#pragma clang diagnostic pop
+}
+
+template <bool DUAL, bool BF16, typename OutT>
+__global__ __launch_bounds__(256) void gemm_quad_kernel(GemmParams p) {
+  constexpr int MT = 4, NT = 4;
+  constexpr int A_BYTES = 256 * QK * 2;
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  lds_cchar* lds0 = (lds_cchar*)smem;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+
+  const int ntiles = p.tiles_m * p.tiles_n;
+  const int logical = xcd_remap(blockIdx.x, ntiles * p.splits);
+  const int split = logical / ntiles, tile = logical % ntiles;
+  const int tm = tile % p.tiles_m, tn = tile / p.tiles_m;
+  const int k_begin = split * p.k_per_split;
+  const int klen = min(p.k, k_begin + p.k_per_split) - k_begin;
+  const int m0 = tm * 256;
+  const int n0 = tn * (DUAL ? BN / 2 : BN);
+  const int nk = klen / QK;
+
+  // Requests.  A: instruction e brings rows 64 e + 16 wave + lane / 4, the lane's bytes land in slot
+  // lane % 4 of its row.  B: instruction e brings k-rows 8 e + 2 wave + lane / 32, slot lane % 32.
+  // Either way a wavefront's instruction e fills the KB at e * 4 KB + wave * 1 KB of its operand's
+  // half of the stage.
+  const int a_chunk = (lane & 3) ^ ((lane >> 4) & 3);
+  const int b_krow = 2 * wave + (lane >> 5);
+  const int b_chunk = ((((lane & 31) >> 2) ^ (b_krow & 7)) << 2) | (lane & 3);
+  const uint16_t* bsrc = p.b0;
+  int b_col = n0 + b_chunk * 8;
+  if (DUAL) {
+    bsrc = b_chunk < 16 ? p.b0 : p.b1;
+    b_col = n0 + (b_chunk & 15) * 8;
+  }
+  const char* ga[4];  // this lane's source of request e, for the stage requested next
+  const char* gb[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    ga[e] = reinterpret_cast<const char*>(p.a + (int64_t)(m0 + 64 * e + 16 * wave + (lane >> 2)) * p.lda + k_begin + a_chunk * 8);
+    gb[e] = reinterpret_cast<const char*>(bsrc + (int64_t)(k_begin + 8 * e + b_krow) * p.ldb + b_col);
+  }
+  const int64_t a_adv = QK * 2, b_adv = (int64_t)QK * p.ldb * 2;  // bytes from one stage to the next
+  const uint32_t lds_w = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds0 + wave * 1024);
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int jn = 0; jn < NT; ++jn)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][jn][r] = 0.f;
+
+  // Fragments (see gemm_kernel): A row lane % 32 of fragment r, k-chunk 2 ks + lane / 32 in slot
+  // chunk ^ ((row / 4) % 4); B as two transposing reads per fragment.  An LDS instruction reaches
+  // 64 KB past its address register, two stages: one register per pair of stages.
+  const int a_key = ((lane & 31) >> 2) & 3;
+  const int grp = lane >> 4, sub = lane & 15;
+  lds_cchar* a_base[3][2];
+  lds_cchar* b_base[3][NT][2];
+#pragma unroll
+  for (int h = 0; h < 3; ++h) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+      a_base[h][ks] = lds0 + h * 2 * kQuadStageBytes + ((wm * 128 + (lane & 31)) * QK + (((2 * ks) | (lane >> 5)) ^ a_key) * 8) * 2;
+#pragma unroll
+    for (int jn = 0; jn < NT; ++jn) {
+      const int col = DUAL ? ((jn / 2) * (BN / 2) + wn * 64 + (jn % 2) * 32) : (wn * 128 + jn * 32);
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+        b_base[h][jn][half] = lds0 + h * 2 * kQuadStageBytes + A_BYTES +
+                              (((grp >> 1) * 8 + half * 4 + (sub >> 2)) * BN + (((col >> 5) ^ (half * 4 + (sub >> 2))) << 5) +
+                               (grp & 1) * 16 + (sub & 3) * 4) * 2;
+    }
+  }
+  u32x4 fa[2][MT], fb[2][NT];
+  auto read_one = [&](auto st_c, int ks, int set, int r) {
+    constexpr int ST = decltype(st_c)::value;
+    constexpr int kOff = (ST % 2) * kQuadStageBytes;
+    if (r < MT) {
+      fa[set][r] = *reinterpret_cast<lds_cu32x4*>(a_base[ST / 2][ks] + kOff + r * 32 * QK * 2);
+    } else {
+      const int jn = (r - MT) >> 1, half = (r - MT) & 1;
+      lds_cchar* src = b_base[ST / 2][jn][half] + kOff + ks * 16 * BN * 2;
+      const uint2 v = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)src));
+      fb[set][jn][half * 2 + 0] = v.x;
+      fb[set][jn][half * 2 + 1] = v.y;
+    }
+  };
+  constexpr int kReads = MT + 2 * NT;  // 12 LDS reads per k-step
+  constexpr int kSlots = MT * NT;      // 16 MFMAs per k-step
+  constexpr int kInFlight = 8 * (QST - 3);  // every wait leaves the requests of the newest QST - 3 stages outstanding
+
+  // request e (0-3: A, 4-7: B) of the stage the pointers stand at, into buffer ST
+  auto request = [&](auto st_c, int e) {
+    constexpr int ST = decltype(st_c)::value;
+    if (e == 0) quad_to_lds<ST * kQuadStageBytes + 0 * 4096>(ga[0], lds_w);
+    if (e == 1) quad_to_lds<ST * kQuadStageBytes + 1 * 4096>(ga[1], lds_w);
+    if (e == 2) quad_to_lds<ST * kQuadStageBytes + 2 * 4096>(ga[2], lds_w);
+    if (e == 3) quad_to_lds<ST * kQuadStageBytes + 3 * 4096>(ga[3], lds_w);
+    if (e == 4) quad_to_lds<ST * kQuadStageBytes + 4 * 4096>(gb[0], lds_w);
+    if (e == 5) quad_to_lds<ST * kQuadStageBytes + 5 * 4096>(gb[1], lds_w);
+    if (e == 6) quad_to_lds<ST * kQuadStageBytes + 6 * 4096>(gb[2], lds_w);
+    if (e == 7) quad_to_lds<ST * kQuadStageBytes + 7 * 4096>(gb[3], lds_w);
+  };
+  // moves the pointers on to stage `next` unless that is past the end (then the last stage is requested again)
+  auto advance = [&](int next) {
+    const int64_t da = next < nk ? a_adv : 0, db = next < nk ? b_adv : 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      ga[e] += da;
+      gb[e] += db;
+    }
+  };
+  auto prologue_stage = [&](auto st_c) {
+    constexpr int ST = decltype(st_c)::value;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) request(st_c, e);
+    advance(ST + 1);
+  };
+  prologue_stage(QuadConst<0>{});
+  prologue_stage(QuadConst<1>{});
+  prologue_stage(QuadConst<2>{});
+  prologue_stage(QuadConst<3>{});
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kInFlight) : "memory");  // stages 0 and 1 have landed
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < kReads; ++r) read_one(QuadConst<0>{}, 0, 0, r);
+
+  // iteration t on buffer ST = t % QST
+  auto iteration = [&](auto st_c, int t) {
+    constexpr int ST = decltype(st_c)::value;
+    // k-step 0: fragments of k-step 1 and the requests of stage t + QST - 1 (its buffer was last read in iteration t - 1)
+#pragma unroll
+    for (int q = 0; q < kSlots; ++q) {
+      acc[q / NT][q % NT] = mfma32<BF16>(fa[0][q / NT], fb[0][q % NT], acc[q / NT][q % NT]);
+      if (q < kReads) read_one(st_c, 1, 1, q);
+      if ((q & 1) == 0) request(QuadConst<(ST + QST - 1) % QST>{}, q >> 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    advance(t + QST);
+    // k-step 1: first fragments of stage t + 1, complete since the last barrier
+#pragma unroll
+    for (int q = 0; q < kSlots; ++q) {
+      acc[q / NT][q % NT] = mfma32<BF16>(fa[1][q / NT], fb[1][q % NT], acc[q / NT][q % NT]);
+      if (q < kReads) read_one(QuadConst<(ST + 1) % QST>{}, 0, 0, q);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kInFlight) : "memory");  // this wavefront's part of stage t + 2 has landed
+    __syncthreads();
+  };
+  const int rounds = nk / QST;
+  int t = 0;
+  for (int round = 0; round < rounds; ++round, t += QST) {
+    iteration(QuadConst<0>{}, t);
+    iteration(QuadConst<1>{}, t + 1);
+    iteration(QuadConst<2>{}, t + 2);
+    iteration(QuadConst<3>{}, t + 3);
+    iteration(QuadConst<4>{}, t + 4);
+  }
+  if (t < nk) iteration(QuadConst<0>{}, t);
+  if (t + 1 < nk) iteration(QuadConst<1>{}, t + 1);
+  if (t + 2 < nk) iteration(QuadConst<2>{}, t + 2);
+  if (t + 3 < nk) iteration(QuadConst<3>{}, t + 3);
+
+  // ---- epilogue (row = m0 + wm*128 + i*32 + (r/4)*8 + (lane/32)*4 + r%4, column lane%32 + ...) ----
+  OutT* c = reinterpret_cast<OutT*>(p.c);
+  const int row_base = m0 + wm * 128 + (lane >> 5) * 4;
+  const int col0 = (DUAL ? n0 + wn * 64 : n0 + wn * 128) + (lane & 31);
+  const int64_t mn = (int64_t)p.m * p.n;
+  constexpr int JN = DUAL ? NT / 2 : NT;
+  if (p.splits > 1) {
+    float* lane_s = p.slabs + (int64_t)split * (DUAL ? 2 : 1) * mn + (int64_t)row_base * p.n + col0;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float* s = lane_s + (int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * p.n;
+#pragma unroll
+        for (int jn = 0; jn < JN; ++jn) {
+          s[jn * 32] = acc[i][jn][r];
+          if constexpr (DUAL) s[mn + jn * 32] = acc[i][jn + NT / 2][r];
+        }
+      }
+    }
+    return;
+  }
+  OutT* lane_c = c + (int64_t)row_base * p.ldc + col0;
+  const int64_t lane_res = (int64_t)row_base * p.n + col0;
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int rr = i * 32 + (r >> 2) * 8 + (r & 3);
+      OutT* dst = lane_c + (int64_t)rr * p.ldc;
+#pragma unroll
+      for (int jn = 0; jn < JN; ++jn) {
+        if constexpr (DUAL) {
+          store_out<OutT>(dst + jn * 32, silu(acc[i][jn][r]) * acc[i][jn + NT / 2][r]);
+        } else {
+          float v = acc[i][jn][r];
+          if (p.residual) v += load_residual(p.residual, p.res_dtype, lane_res + (int64_t)rr * p.n + jn * 32);
+          store_out<OutT>(dst + jn * 32, v);
+        }
+      }
+    }
+  }
+}
+
+template <bool DUAL, bool BF16, typename OutT>
+int launch_quad(GemmParams p, hipStream_t st) {
+  p.tiles_m = p.m / 256;
+  p.tiles_n = p.n / (DUAL ? BN / 2 : BN);
+  const size_t smem = (size_t)QST * kQuadStageBytes;
+  auto kern = gemm_quad_kernel<DUAL, BF16, OutT>;
+  static std::atomic<bool> attr_set{false};  // per instantiation; callers hold the dispatch lock
+  if (!attr_set.load(std::memory_order_acquire)) {
+    PTO_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    attr_set.store(true, std::memory_order_release);
+  }
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(256), smem, st, p);
+  PTO_CHECK_HIP(hipGetLastError());
+  return PTO_HIP_OK;
+}
+
 // Sum of the split-K slabs in split order (so the result does not depend on which workgroup
 // finished first), then SwiGLU for the gate/up pass, cast and store.  n is a multiple of 4.
 constexpr int kMaxSplits = 16;
@@ -558,14 +817,14 @@ int launch_variant(GemmParams p, hipStream_t st) {
   // that a second kernel sums in split order.
   // The other values force a tile height (the sweeps behind the estimate, and the tests, use them):
   // 4 = 256x256 tile, k split in two when CUs would idle; 5 = 128x256 tile; 6 = 64x256 tile, k split
-  // while CUs would idle.
+  // while CUs would idle; 7 = as 4 with four wavefronts per workgroup (16-bit weights, whole tiles).
   const int64_t tiles_n = (p.n + (DUAL ? 127 : 255)) / (DUAL ? 128 : 256);
   const int64_t big_tiles = (int64_t)((p.m + 255) / 256) * tiles_n;
   const int64_t small_tiles = (int64_t)((p.m + 127) / 128) * tiles_n;
   const bool few = big_tiles < num_cu;
   int want = 1;
   bool small_tile = variant == 5;
-  if (variant == 4 && few) want = 2;
+  if ((variant == 4 || variant == 7) && few) want = 2;
   if (variant == 0 && p.m > 64) {
     // Estimated time of each (tile height, k splits) pair, in microseconds, fitted to measured
     // launches: rounds of workgroups over the CUs x the k rows one workgroup walks x the time per
@@ -620,10 +879,25 @@ int launch_variant(GemmParams p, hipStream_t st) {
       p.slabs = reinterpret_cast<float*>(ws);
     }
   }
-  int rc;
-  if (tiny_tile) rc = launch_gemm<1, 2, 4, DUAL, BF16, OutT, W8>(p, st);
-  else if (small_tile) rc = launch_gemm<2, 2, 4, DUAL, BF16, OutT, W8>(p, st);
-  else rc = launch_gemm<4, 2, 4, DUAL, BF16, OutT, W8>(p, st);
+  int rc = PTO_HIP_OK;
+  // The four-wavefront form of the tall tile (bit-identical to the eight-wavefront one): measured
+  // ahead by 3-6 % where a workgroup walks a long k range and the launch is a few rounds of
+  // workgroups (2048 tokens of the LLaMA-7B block 496 -> 482 us, 1024 tokens at hidden 8192
+  // 1231 -> 1159 us), behind by 1-3 % on many rounds or short k (8192 tokens 2189 -> 2256 us,
+  // hidden 2048 370 -> 378 us).  "gemm_variant" 7 asks for it wherever it is built.
+  bool quad = false;
+  if constexpr (!W8) {
+    const bool fits = !tiny_tile && !small_tile && p.m % 256 == 0 && p.n % (DUAL ? BN / 2 : BN) == 0 &&
+                      p.k % QK == 0 && p.k_per_split % QK == 0;
+    const int64_t rounds = (big_tiles * p.splits + num_cu - 1) / num_cu;
+    quad = fits && (variant == 7 || (variant == 0 && rounds <= 4 && p.k_per_split >= 4096));
+    if (quad) rc = launch_quad<DUAL, BF16, OutT>(p, st);
+  }
+  if (!quad) {
+    if (tiny_tile) rc = launch_gemm<1, 2, 4, DUAL, BF16, OutT, W8>(p, st);
+    else if (small_tile) rc = launch_gemm<2, 2, 4, DUAL, BF16, OutT, W8>(p, st);
+    else rc = launch_gemm<4, 2, 4, DUAL, BF16, OutT, W8>(p, st);
+  }
   if (rc) return rc;
   if (p.partials_out) {  // a fused consumer sums the slabs (one split: the product is in p.c, scales applied)
     pto_hip::W8Partials& o = *p.partials_out;

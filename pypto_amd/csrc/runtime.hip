@@ -1050,7 +1050,7 @@ int pto_hip_set_option(const char* name, int64_t value) {
     PTO_CHECK_ARG(value >= 0, "attn_tokens_per_partition must be >= 0");
     c.attn_tokens_per_partition = value;
   } else if (!std::strcmp(name, "gemm_variant")) {
-    PTO_CHECK_ARG(value == 0 || (value >= 4 && value <= 6), "gemm_variant must be 0, 4, 5 or 6");
+    PTO_CHECK_ARG(value == 0 || (value >= 4 && value <= 7), "gemm_variant must be 0, 4, 5, 6 or 7");
     c.gemm_variant = value;
   } else if (!std::strcmp(name, "gemm_splits")) {
     PTO_CHECK_ARG(value >= 0 && value <= 16, "gemm_splits must be in [0, 16]");

@@ -65,7 +65,7 @@ def test_options_round_trip_and_ranges():
         assert got.value == value, name
         _lib.check(lib.pto_hip_set_option(name.encode(), old.value))
     for name, bad in (("attn_variant", 3), ("attn_group_tiles", 3), ("attn_lean_siblings", 3), ("w8a16_nt", 2), ("attn_autotune", 2), ("attn_waves_per_cu", 17), ("attn_tokens_per_partition", -1),
-                      ("w8a16_wgs_per_cu", 0), ("w8a16_min_steps", 0), ("w8a16_wide", 3), ("gemm_variant", 7), ("gemm_variant", 2), ("gemm_splits", 17)):
+                      ("w8a16_wgs_per_cu", 0), ("w8a16_min_steps", 0), ("w8a16_wide", 3), ("gemm_variant", 8), ("gemm_variant", 2), ("gemm_splits", 17)):
         with pytest.raises(ValueError, match=name):
             _lib.check(lib.pto_hip_set_option(name.encode(), bad))
     with pytest.raises(ValueError, match="unknown option"):

@@ -104,7 +104,7 @@ def test_ffn_tiny_fp16(worker, variant):
     validate_golden({"out": inp.out}, {"out": ref32}, rtol=2e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("variant", [0, 4, 5, 6])
+@pytest.mark.parametrize("variant", [0, 4, 5, 6, 7])
 @pytest.mark.parametrize("t,h,i", [(256, 512, 1024), (100, 264, 520), (512, 1024, 2816)])
 def test_ffn_block_bf16(worker, variant, t, h, i):
     """RMSNorm prologue + SwiGLU FFN, bf16, incl. shapes that are not tile multiples."""
@@ -255,6 +255,45 @@ def test_every_tile_height_and_split_count_gives_the_same_product(worker, varian
     validate_golden({"out": out}, {"out": oracle.projection(x, w)}, rtol=2e-3, atol=2e-3)
     want = oracle.swiglu(oracle.projection(x, w), oracle.projection(x, wu)).to(torch.bfloat16)
     validate_golden({"out": out16.float()}, {"out": want.float()}, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,k,n,splits", [(256, 32, 256, 0), (256, 64, 512, 0), (512, 96, 256, 0), (256, 128, 256, 0),
+                                          (256, 160, 256, 0), (256, 192, 512, 0), (512, 352, 768, 0), (256, 4096, 256, 0),
+                                          (256, 4096, 512, 3), (768, 1024, 256, 2), (256, 11008, 256, 0)])
+def test_four_wavefront_tile_form_gives_the_bits_of_the_eight_wavefront_form(worker, dtype, m, k, n, splits):
+    """The 256-row tile as four wavefronts (one per SIMD, five rotating 32-k stages) walks k in the same
+    16-wide steps into the same accumulators as the eight-wavefront form: identical bits for the plain
+    product, the residual + cast form and the gate/up pair, over k extents that end the five-stage
+    rotation at every position (1, 2, 3, 4, 5, 6, 11, 128 stages), with and without k splits; and the
+    product itself against the oracle."""
+    from pypto_amd.runtime import gate_up_swiglu, projection, projection_residual
+    g = torch.Generator().manual_seed(m + k + n)
+    x = (torch.randn(m, k, generator=g) / k ** 0.5).to(dtype)
+    w = torch.randn(k, n, generator=g).to(dtype)
+    wu = torch.randn(k, n // 2, generator=g).to(dtype)
+    res = torch.randn(m, n, generator=g)
+    got = {}
+    worker.set_option("gemm_splits", splits)
+    try:
+        for variant in (4, 7):
+            worker.set_option("gemm_variant", variant)
+            out, out16, h16 = torch.zeros(m, n), torch.zeros(m, n, dtype=dtype), torch.zeros(m, n // 2, dtype=dtype)
+            with worker.register(projection) as h:
+                h(x, w, out)
+            with worker.register(projection_residual) as h:
+                h(x, w, res, out16)
+            with worker.register(gate_up_swiglu) as h:
+                h(x, w[:, : n // 2].contiguous(), wu, h16)
+            got[variant] = (out, out16, h16)
+    finally:
+        worker.set_option("gemm_variant", 0)
+        worker.set_option("gemm_splits", 0)
+    for a, b in zip(got[4], got[7]):
+        assert torch.equal(a, b)
+    validate_golden({"out": got[7][0]}, {"out": oracle.projection(x, w)}, rtol=2e-3, atol=2e-3)
+    want = oracle.swiglu(oracle.projection(x, w[:, : n // 2].contiguous()), oracle.projection(x, wu)).to(dtype)
+    validate_golden({"out": got[7][2].float()}, {"out": want.float()}, rtol=1e-2, atol=1e-2)
 
 
 def test_projection_argument_rules(worker):
