@@ -428,7 +428,10 @@ __global__ __launch_bounds__(256) void gemm8_finish_kernel(const float* __restri
 // Tile height: 256 rows unless that leaves CUs idle and 128 rows do not; eight wavefronts (two per
 // SIMD).  Four wavefronts of 128 x 128 on the tall tile read a third less from LDS per MFMA but
 // leave a SIMD nothing to issue while its one wavefront waits (LLaMA-7B block: 361 us against 334 us
-// when it was measured; that form is not built any more).
+// when it was measured; rebuilt as the 16-bit GEMM's four-wavefront form is - five rotating stages of
+// 64 codes, requests three iterations ahead, a loop of loop-invariant addresses plus immediates -
+// it gave the same bits in 309 us against 293: with 64-byte rows the tiles cost twice the L2
+// requests and the wavefronts wait on them for 63 % of their cycles.  That form is not built).
 // A single-operand pass whose tall tiles fill at most half the CUs splits k instead of halving the
 // tile: a k-tile takes a workgroup the same ~1.4 us with 128 rows as with 256 (the tile's arrival,
 // not the MFMAs, sets it), so two workgroups per 256 x 256 tile do the same work in half the k-tiles.
