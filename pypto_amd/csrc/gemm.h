@@ -669,6 +669,7 @@ __global__ __launch_bounds__(256) void gemm_quad_kernel(GemmParams p) {
   if (t + 1 < nk) iteration(QuadConst<1>{}, t + 1);
   if (t + 2 < nk) iteration(QuadConst<2>{}, t + 2);
   if (t + 3 < nk) iteration(QuadConst<3>{}, t + 3);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land in LDS after the workgroup has gone
 
   // ---- epilogue (row = m0 + wm*128 + i*32 + (r/4)*8 + (lane/32)*4 + r%4, column lane%32 + ...) ----
   OutT* c = reinterpret_cast<OutT*>(p.c);
