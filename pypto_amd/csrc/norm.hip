@@ -71,12 +71,15 @@ __global__ __launch_bounds__(kThreads) void rms_norm_vec_kernel(const TI* __rest
   constexpr int kOutStride = BLOCKED ? 32 : 1;  // vec8 units between consecutive 8-element groups
   const int nvec = (int)(hidden / 8);
   vec8i v[kVecPerThread];
+  float4 g0[kVecPerThread], g1[kVecPerThread];  // requested with the row, so that the second pass waits for nothing
   float ss = 0.f;
 #pragma unroll
   for (int u = 0; u < kVecPerThread; ++u) {
     const int i = threadIdx.x + u * kThreads;
     if (i < nvec) {
       v[u] = xr[i];
+      g0[u] = gamma ? reinterpret_cast<const float4*>(gamma)[2 * i] : float4{1.f, 1.f, 1.f, 1.f};
+      g1[u] = gamma ? reinterpret_cast<const float4*>(gamma)[2 * i + 1] : float4{1.f, 1.f, 1.f, 1.f};
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float f = (float)v[u][e];
@@ -98,9 +101,7 @@ __global__ __launch_bounds__(kThreads) void rms_norm_vec_kernel(const TI* __rest
     const int i = threadIdx.x + u * kThreads;
     if (i < nvec) {
       vec8 o;
-      const float4 g0 = gamma ? reinterpret_cast<const float4*>(gamma)[2 * i] : float4{1.f, 1.f, 1.f, 1.f};
-      const float4 g1 = gamma ? reinterpret_cast<const float4*>(gamma)[2 * i + 1] : float4{1.f, 1.f, 1.f, 1.f};
-      const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+      const float g[8] = {g0[u].x, g0[u].y, g0[u].z, g0[u].w, g1[u].x, g1[u].y, g1[u].z, g1[u].w};
 #pragma unroll
       for (int e = 0; e < 8; ++e) o[e] = (T)((float)v[u][e] * inv * g[e]);
       orow[(size_t)i * kOutStride] = o;

@@ -340,11 +340,13 @@ struct FinishNormParams {
 __global__ __launch_bounds__(kNormThreads) void w8a16_finish_norm_kernel(FinishNormParams p) {
   const int m = blockIdx.x;
   float4 v[kNormVec];
+  float4 g[kNormVec];  // requested with the row, so that the second pass waits for nothing
   float ss = 0.f;
 #pragma unroll
   for (int u = 0; u < kNormVec; ++u) {
     const int n = (threadIdx.x + u * kNormThreads) * 4;
     if (n < p.n) {
+      g[u] = *reinterpret_cast<const float4*>(p.gamma + n);
       float4 a = sum_splits(p.part, p.scale, p.splits, (size_t)p.stride, m, n, p.n);
       const float4 r = load4_as_f32(p.residual, (size_t)m * p.n + n, p.res_dtype);
       a.x += r.x; a.y += r.y; a.z += r.z; a.w += r.w;
@@ -366,8 +368,7 @@ __global__ __launch_bounds__(kNormThreads) void w8a16_finish_norm_kernel(FinishN
   for (int u = 0; u < kNormVec; ++u) {
     const int n = (threadIdx.x + u * kNormThreads) * 4;
     if (n < p.n) {
-      const float4 g = *reinterpret_cast<const float4*>(p.gamma + n);
-      const float4 y = {v[u].x * inv * g.x, v[u].y * inv * g.y, v[u].z * inv * g.z, v[u].w * inv * g.w};
+      const float4 y = {v[u].x * inv * g[u].x, v[u].y * inv * g[u].y, v[u].z * inv * g[u].z, v[u].w * inv * g[u].w};
       store4_from_f32(p.normed_out, p.out_blocked ? blocked_index(m, n) : (size_t)m * p.n + n, p.out_dtype, y);
     }
   }
