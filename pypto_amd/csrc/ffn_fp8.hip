@@ -141,7 +141,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm8_kernel(Params p) {
   const int ntiles = p.tiles_m * p.tiles_n;
   const int logical = xcd_remap(blockIdx.x, ntiles * p.splits);
   const int split = logical / ntiles, tile = logical % ntiles;
-  const int tm = tile % p.tiles_m, tn = tile / p.tiles_m;
+  // bands of eight row tiles, rows first: an XCD's 32 consecutive ids are 8 row tiles x 4 column tiles
+  // whatever the height of the problem (walking whole columns would pull all of A through its L2 per column tile)
+  const int per_band = 8 * p.tiles_n;
+  const int band = tile / per_band, idx = tile - band * per_band;
+  const int band_rows = min(8, p.tiles_m - band * 8);
+  const int tn = idx / band_rows, tm = band * 8 + (idx - tn * band_rows);
   const int k_begin = split * p.k_per_split;  // this workgroup's k range: [k_begin, k_begin + nk * BK)
   const int m0 = tm * BM;
   const int n0 = tn * (DUAL ? BN / 2 : BN);
@@ -432,9 +437,11 @@ __global__ __launch_bounds__(256) void gemm8_finish_kernel(const float* __restri
 // 64 codes, requests three iterations ahead, a loop of loop-invariant addresses plus immediates -
 // it gave the same bits in 309 us against 293: with 64-byte rows the tiles cost twice the L2
 // requests and the wavefronts wait on them for 63 % of their cycles.  That form is not built).
-// A single-operand pass whose tall tiles fill at most half the CUs splits k instead of halving the
+// A single-operand pass whose tall tiles fill less than half the CUs splits k instead of halving the
 // tile: a k-tile takes a workgroup the same ~1.4 us with 128 rows as with 256 (the tile's arrival,
 // not the MFMAs, sets it), so two workgroups per 256 x 256 tile do the same work in half the k-tiles.
+// At exactly half (the LLaMA-7B down pass at 2048 tokens: 128 tall tiles on 256 CUs) the 128-row
+// tiles fill every CU in one round and need neither slabs nor a finish launch: block 293 -> 279 us.
 template <bool DUAL, typename OutT>
 int launch_any(const Params& p0, hipStream_t st) {
   Params p = p0;
@@ -446,7 +453,9 @@ int launch_any(const Params& p0, hipStream_t st) {
   const int64_t tall = (int64_t)((p.m + 255) / 256) * tiles_n;
   if constexpr (!DUAL) {
     const int nk = p.k / BK;
-    int64_t want = pto_hip::ctx().gemm_splits > 0 ? pto_hip::ctx().gemm_splits : std::min<int64_t>(num_cu / tall, 4);
+    // by default only where even 128-row tiles would leave CUs idle (see above)
+    const int64_t forced = pto_hip::ctx().gemm_splits;
+    const int64_t want = forced > 0 ? forced : (2 * tall < num_cu ? std::min<int64_t>(num_cu / tall, 4) : 1);
     if (pto_hip::ctx().gemm_variant == 0 && p.m > 128 && want >= 2 && nk >= 8 * want && p.n % 4 == 0 && p.ldc % 4 == 0) {
       const int per = (int)((nk + want - 1) / want);
       p.k_per_split = per * BK;

@@ -86,6 +86,20 @@ __device__ __forceinline__ int xcd_remap(int pid, int nwg) {
   return base + local;
 }
 
+// Tile id -> (row tile, column tile).  Ids walk bands of eight row tiles, down the rows first and then
+// across the columns, so that the 32 consecutive ids an XCD works on at a time (xcd_remap) are eight row
+// tiles by four column tiles whatever the height of the problem: 12 operand tiles for 32 output tiles.
+// Walking whole columns of a tall problem instead would give an XCD 32 row tiles of one column tile, and
+// every column tile would pull all of A through that XCD's L2 again.
+__device__ __forceinline__ void tile_coords(int tile, int tiles_m, int tiles_n, int& tm, int& tn) {
+  constexpr int kBand = 8;
+  const int per_band = kBand * tiles_n;
+  const int band = tile / per_band, idx = tile - band * per_band;
+  const int rows = min(kBand, tiles_m - band * kBand);  // the last band may be shorter
+  tn = idx / rows;
+  tm = band * kBand + (idx - tn * rows);
+}
+
 // EDGE = 0 assumes m, n, k are multiples of the tile.  EDGE = 1: only m is ragged - the A row
 // pointers are clamped once, the loop is the same.  EDGE = 2 clamps every address into the
 // operands (so all loads stay unconditional) and zeroes the A chunks that lie past k.
@@ -134,7 +148,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
   const int ntiles = p.tiles_m * p.tiles_n;
   const int logical = xcd_remap(blockIdx.x, ntiles * p.splits);
   const int split = logical / ntiles, tile = logical % ntiles;
-  const int tm = tile % p.tiles_m, tn = tile / p.tiles_m;
+  int tm, tn;
+  tile_coords(tile, p.tiles_m, p.tiles_n, tm, tn);
   const int k_begin = split * p.k_per_split;
   const int klen = min(p.k, k_begin + p.k_per_split) - k_begin;  // this workgroup's k extent
   const int m0 = tm * BM;
@@ -521,7 +536,8 @@ __global__ __launch_bounds__(256) void gemm_quad_kernel(GemmParams p) {
   const int ntiles = p.tiles_m * p.tiles_n;
   const int logical = xcd_remap(blockIdx.x, ntiles * p.splits);
   const int split = logical / ntiles, tile = logical % ntiles;
-  const int tm = tile % p.tiles_m, tn = tile / p.tiles_m;
+  int tm, tn;
+  tile_coords(tile, p.tiles_m, p.tiles_n, tm, tn);
   const int k_begin = split * p.k_per_split;
   const int klen = min(p.k, k_begin + p.k_per_split) - k_begin;
   const int m0 = tm * 256;
@@ -851,8 +867,7 @@ int launch_variant(GemmParams p, hipStream_t st) {
             (tall ? 18.1 + 9.4 * load : 11.0 + 6.5 * load) + (W8 && rounds > 1 ? (tall ? 2.5 : 4.5) : 0.0);
         const double slab_mb = (double)real * p.m * p.n * mats * 4.0 / 1e6;  // written, then read back
         // where the tall tile runs as four wavefronts (see below) it measured about 5 % faster
-        const bool as_quad = !W8 && tall && rounds <= 4 && kps >= 4096 && p.m % 256 == 0 && p.n % (DUAL ? BN / 2 : BN) == 0 &&
-                             p.k % QK == 0;
+        const bool as_quad = !W8 && tall && p.m % 256 == 0 && p.n % (DUAL ? BN / 2 : BN) == 0 && p.k % QK == 0;
         const double t = std::max((double)rounds * (double)kps * ns_row * (as_quad ? 0.95 : 1.0) * 1e-3, stream_us) +
                          (real > 1 ? 7.0 + 2.0 * slab_mb / (slab_mb <= 128.0 ? 8.0 : 4.0) : 0.0);
         if (t < best) {
@@ -884,17 +899,15 @@ int launch_variant(GemmParams p, hipStream_t st) {
     }
   }
   int rc = PTO_HIP_OK;
-  // The four-wavefront form of the tall tile (bit-identical to the eight-wavefront one): measured
-  // ahead by 3-6 % where a workgroup walks a long k range and the launch is a few rounds of
-  // workgroups (2048 tokens of the LLaMA-7B block 496 -> 482 us, 1024 tokens at hidden 8192
-  // 1231 -> 1159 us), behind by 1-3 % on many rounds or short k (8192 tokens 2189 -> 2256 us,
-  // hidden 2048 370 -> 378 us).  "gemm_variant" 7 asks for it wherever it is built.
+  // The four-wavefront form of the tall tile (bit-identical to the eight-wavefront one) wherever it
+  // is built: measured ahead by 1-6 % on every shape tried (LLaMA-7B block at 1024 / 2048 / 4096 / 8192
+  // tokens 346 -> 335, 510 -> 490, 956 -> 936, 1831 -> 1795 us on one box; hidden 8192 at 1024 tokens
+  // 1280 -> 1200; hidden 2048 at 4096 tokens 383 -> 380).  "gemm_variant" 4 keeps eight wavefronts.
   bool quad = false;
   if constexpr (!W8) {
     const bool fits = !tiny_tile && !small_tile && p.m % 256 == 0 && p.n % (DUAL ? BN / 2 : BN) == 0 &&
                       p.k % QK == 0 && p.k_per_split % QK == 0;
-    const int64_t rounds = (big_tiles * p.splits + num_cu - 1) / num_cu;
-    quad = fits && (variant == 7 || (variant == 0 && rounds <= 4 && p.k_per_split >= 4096));
+    quad = fits && (variant == 7 || variant == 0);
     if (quad) rc = launch_quad<DUAL, BF16, OutT>(p, st);
   }
   if (!quad) {

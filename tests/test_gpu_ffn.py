@@ -620,10 +620,11 @@ def test_ffn_block_fp8_llama7b_shape_rows_and_distance_to_16_bit(worker):
     assert 1e-3 < rel < 0.08, rel
 
 
-@pytest.mark.parametrize("m,k,n,splits", [(2048, 11008, 4096, 0),    # the LLaMA-7B down pass: the library's own choice (2)
+@pytest.mark.parametrize("m,k,n,splits", [(2048, 11008, 4096, 2),    # the LLaMA-7B down pass, split in two
+                                          (1024, 11008, 4096, 0),    # ... at 1024 tokens: the library's own choice (4)
                                           (300, 4096, 520, 3), (257, 4096, 256, 4), (1000, 2048, 1024, 2)])
 def test_projection_fp8_k_split_sums_the_same_products(worker, m, k, n, splits):
-    """A single-operand pass whose 256-row tiles fill at most half the CUs splits k over 2-4 workgroups per
+    """A single-operand pass whose 256-row tiles fill less than half the CUs splits k over 2-4 workgroups per
     tile; a finish kernel sums their fp32 slabs and applies the scales.  Small-integer operands with
     power-of-two scales make every sum exact: identical to the unsplit pass and to the product itself."""
     _lib, lib, code = _fp8_stage_lib()
