@@ -566,12 +566,12 @@ PTO_HIP_API int pto_hip_backend_handler_query(const char* hook, int32_t arg, cha
  *  "gemm_variant"               FFN GEMM tiling: 0 = default choice (64-row tile up to 64 rows, else the
  *                               256- or 128-row tile and k split count with the least estimated time,
  *                               eight wavefronts, two per SIMD; the 256-row tile with four wavefronts,
- *                               one per SIMD, where that measured ahead: 16-bit weights, whole tiles,
- *                               k ranges of 4096 or more, at most four rounds of workgroups; skinny
- *                               projections up to 32 tokens); 4 = 256-row tile, k split in two when
- *                               CUs would idle, 5 = 128-row tile, 6 = 64-row tile, k split while CUs
- *                               would idle, 7 = as 4 with four wavefronts wherever that form is built
- *                               (forced forms, for sweeps and tests; 4 and 7 give identical bits)
+ *                               one per SIMD, wherever that form is built: 16-bit weights, whole
+ *                               tiles; skinny projections up to 32 tokens); 4 = 256-row tile with
+ *                               eight wavefronts, k split in two when CUs would idle, 5 = 128-row
+ *                               tile, 6 = 64-row tile, k split while CUs would idle, 7 = as 4 with
+ *                               four wavefronts wherever that form is built (forced forms, for sweeps
+ *                               and tests; 4 and 7 give identical bits)
  *  "gemm_splits"                k splits of the tiled GEMM: 0 = by shape (default), 1..16 = as given
  *                               when k allows (each split at least four 64-row k tiles)
  *  "w8a16_wgs_per_cu"           workgroups per CU the W8A16 k split aims at (default 1)
