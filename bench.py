@@ -176,10 +176,11 @@ def main() -> int:
 
     # ---- paged-attention decode, small configuration ------------------------------------
     pools = [workloads.attention_small(seed=0, device="cuda") for _ in range(KV_POOLS)]
-    # The inputs of the other bandwidth-bound configurations are built now, so that no block's memory
-    # placement depends on what an earlier block has freed.  (Their step times come in two modes 3-4 %
-    # apart from one process to the next - same box, same tensors at the same addresses - and are
-    # stable within a process.)
+    # The decoder layer's inputs are built now, the long configuration's only when its turn comes, after
+    # the layer's have been freed: what else lives in device memory moves the bandwidth-bound step times
+    # by 3-4 % (same box, same kernels: the layer 163 us on its own, 168 us with the long configuration's
+    # 2.8 GB allocated next to it; the long configuration 414 us in a process of its own, 435-441 us after
+    # or next to the layer's tensors), and this order measured best for both.
     want_layer = not args.no_extra and not args.no_layer
     want_long = not args.no_extra and not args.no_long
     if want_layer:
@@ -188,8 +189,6 @@ def main() -> int:
         # settling), which no model with more than one layer offers.
         dl = workloads.decoder_layer_inputs(device="cuda")
         dl_other = workloads.decoder_layer_inputs(device="cuda", seed=1)
-    if want_long:
-        lf = workloads.attention_long_fp8(seed=0, device="cuda")
     probe_buf = torch.zeros(2 << 30, dtype=torch.uint8, device="cuda")
     torch.cuda.synchronize()
     step_bytes = pools[0].algorithmic_bytes()
@@ -332,6 +331,8 @@ def main() -> int:
                 dtuned = autotune_attention(worker, dh, dargs, rounds=30)
             benchmark(dh, dargs, rounds=300, warmup=0)  # ~50 ms: past the library's launch-shape measurement and the
             dstats = benchmark(dh, dargs, rounds=60, warmup=0)   # clock ramp after the idle time of the CPU timings above
+            dchoice = {"waves_per_cu": worker.get_option("attn_tuned_waves_per_cu"),
+                       "workgroup_form": worker.get_option("attn_tuned_workgroup_form")}
         worker.set_option("attn_tokens_per_partition", 0)
         worker.set_option("attn_waves_per_cu", 0)
         dbytes = dl.algorithmic_bytes()
@@ -341,6 +342,7 @@ def main() -> int:
             "step's weights come from HBM", dbytes, dstats.device_wall_us)
         result["decoder_layer"]["attn_tokens_per_partition"] = dtuned["tokens_per_partition"]
         result["decoder_layer"]["attn_waves_per_cu"] = dtuned["waves_per_cu"]
+        result["decoder_layer"]["attn_library_choice"] = dchoice  # what the library's own timing of launch shapes settled on
         if cpu:
             # four of the 32 sequences: their blocks in a compact pool; the weights are the full ones
             seqs = [0, 9, 18, 27]
@@ -366,6 +368,8 @@ def main() -> int:
         torch.cuda.empty_cache()
 
     if want_long:
+        lf = workloads.attention_long_fp8(seed=0, device="cuda")
+        torch.cuda.synchronize()
         with worker.register(paged_attention) as lh:
             largs = [lf.args()]
             benchmark(lh, largs, rounds=100, warmup=0)  # ~45 ms: the GPU has idled during the CPU timings above

@@ -1712,10 +1712,14 @@ int paged_attention(const void* query, const void* key_cache, const void* value_
     if (may_measure) tune_harvest(*ts);
     int use = ts->chosen >= 0 ? ts->chosen : 0;
     if (ts->chosen < 0 && may_measure) {
+      // the candidate measured least so far: the readings of every candidate are spread over the
+      // first calls alike (the clocks ramp up during them; a block of early calls per candidate
+      // would favour whichever comes last)
+      int least = kTuneReps;
       for (size_t c = 0; c < ts->cands.size(); ++c)
-        if (ts->issued[c] < kTuneReps) {
+        if (ts->issued[c] < least) {
+          least = ts->issued[c];
           measuring = use = (int)c;
-          break;
         }
     }
     p.resident_cap = ts->cands[use].cap;
