@@ -176,11 +176,11 @@ def main() -> int:
 
     # ---- paged-attention decode, small configuration ------------------------------------
     pools = [workloads.attention_small(seed=0, device="cuda") for _ in range(KV_POOLS)]
-    # The decoder layer's inputs are built now, the long configuration's only when its turn comes, after
-    # the layer's have been freed: what else lives in device memory moves the bandwidth-bound step times
-    # by 3-4 % (same box, same kernels: the layer 163 us on its own, 168 us with the long configuration's
-    # 2.8 GB allocated next to it; the long configuration 414 us in a process of its own, 435-441 us after
-    # or next to the layer's tensors), and this order measured best for both.
+    # The decoder layer's inputs are built now, the long configuration's only when its turn comes.  Freed
+    # tensors stay with torch's allocator for the next block to reuse: whenever GB-sized blocks went back to
+    # the driver between the blocks (torch.cuda.empty_cache()), what ran afterwards streamed 3-6 % slower on
+    # the same box - the layer 168 us instead of 163, the long configuration 435-446 us instead of 413,
+    # both FFN blocks 1-2 % - with the same kernels and the same read-probe rate.
     want_layer = not args.no_extra and not args.no_layer
     want_long = not args.no_extra and not args.no_long
     if want_layer:
@@ -307,7 +307,6 @@ def main() -> int:
     global _READ_PROBE_GBPS
     _READ_PROBE_GBPS = streams
     del probe_buf
-    torch.cuda.empty_cache()
     if cpu:
         p = pools[0]
         host = [t.cpu() for t in (p.query, p.key_cache, p.value_cache, p.block_table, p.context_lens, p.config)]
@@ -365,7 +364,6 @@ def main() -> int:
                           f"{med * 1e3:.0f} ms per run"}
             del hw, hargs
         del dl, dl_other, dargs
-        torch.cuda.empty_cache()
 
     if want_long:
         lf = workloads.attention_long_fp8(seed=0, device="cuda")
@@ -398,7 +396,6 @@ def main() -> int:
                           f"dequantised on the host: median of {n} runs, {med * 1e3:.0f} ms per run"}
             del sub
         del lf, largs
-        torch.cuda.empty_cache()
 
     # ---- FFN block at LLaMA-7B shape (second half of the metric) ------------------------------
     if not args.no_ffn:
