@@ -487,7 +487,6 @@ def main() -> int:
                           f"median of {n} runs, {med * 1e3:.0f} ms per run"}
             del hq_args, hx
         del f, q, qargs, bf16_out
-        torch.cuda.empty_cache()
 
     # ---- shapes outside the benchmark configurations (on request) ---------------------------------
     if args.more:
@@ -500,7 +499,6 @@ def main() -> int:
             "decoder-layer decode step with bf16 weights (the reference's layer): H4096 Hq32 Hkv8 D128 I14336 B32 "
             "ctx4096", dw.algorithmic_bytes(), st.device_wall_us)
         del dw
-        torch.cuda.empty_cache()
         # the reference's CI perf-guard workload: one qwen3-14B decoder layer, batch 16, sequences at
         # max_seq 4096 (.github/perf_baselines/qwen3_14b_decode.json: 1016.66 us on its own hardware)
         dq = workloads.decoder_layer_inputs(batch=16, hidden=5120, num_heads=40, kv_head_num=8, head_dim=128,
@@ -514,7 +512,6 @@ def main() -> int:
             "the reference's CI perf guard, 1016.66 us there on other hardware)", dq.algorithmic_bytes(),
             st.device_wall_us)
         del dq
-        torch.cuda.empty_cache()
         # the reference's own decode model (examples/models/qwen3_jit/config.py:16-29) in its own cache layout:
         # one block of MAX_SEQ tokens per sequence
         dj = workloads.decoder_layer_inputs(batch=16, hidden=8192, num_heads=64, kv_head_num=8, head_dim=128,
@@ -527,7 +524,6 @@ def main() -> int:
             "the reference's qwen3_jit decode model, one layer step, bf16 weights: H8192 Hq64 Hkv8 D128 I25600 B16 "
             "ctx4096, one 4096-token block per sequence", dj.algorithmic_bytes(), st.device_wall_us)
         del dj
-        torch.cuda.empty_cache()
         fd = [workloads.ffn_inputs(tokens=16, hidden=4096, intermediate=11008, seed=s, device="cuda") for s in (0, 1)]
         with worker.register(ffn_block) as fh:
             fdargs = [(f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.out, f.eps) for f in fd]
@@ -537,7 +533,6 @@ def main() -> int:
             "FFN LLaMA-7B at 16 tokens: H4096 I11008 bf16 weights streamed once, RMSNorm prologue, SwiGLU",
             3 * 4096 * 11008 * 2 + 2 * 16 * 4096 * 2, st.device_wall_us)
         del fd, fdargs
-        torch.cuda.empty_cache()
         lm_m, lm_k, lm_n = 16, 5120, 151936
         lx = (torch.randn(lm_m, lm_k, device="cuda") / lm_k ** 0.5).to(torch.bfloat16)
         lw = torch.randn(lm_k, lm_n, device="cuda").to(torch.bfloat16)
@@ -549,7 +544,6 @@ def main() -> int:
             "projection x[16,5120] @ W[5120,151936] bf16 -> fp32 (qwen3-14B vocabulary projection), weights streamed "
             "once", lm_k * lm_n * 2 + lm_m * lm_k * 2 + lm_m * lm_n * 4, st.device_wall_us)
         del lx, lw, lo
-        torch.cuda.empty_cache()
         mq = workloads.paged_attention_inputs(batch=256, num_heads=64, kv_head_num=1, head_dim=128, block_size=128,
                                               ctx_range=(2048, 4096), seed=0, device="cuda")
         with worker.register(paged_attention) as mh:
@@ -559,7 +553,6 @@ def main() -> int:
             "paged-attention decode, 64 query heads per KV head: B256 Hq64 Hkv1 D128 bs128 ctx~U[2048,4096] bf16 KV; "
             "the cache is counted once", mq.algorithmic_bytes(), st.device_wall_us)
         del mq
-        torch.cuda.empty_cache()
         result["more"] = more
 
     if args.calibrate_copy:
