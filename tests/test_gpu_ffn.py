@@ -296,6 +296,33 @@ def test_four_wavefront_tile_form_gives_the_bits_of_the_eight_wavefront_form(wor
     validate_golden({"out": got[7][2].float()}, {"out": want.float()}, rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("variant", [0, 4, 5, 6, 7])
+@pytest.mark.parametrize("m", [2304, 2560, 4352])
+def test_tall_problems_walk_their_row_tiles_in_bands_of_eight(worker, variant, m):
+    """More than eight row tiles: tile ids walk bands of eight row tiles (a last band of 1, 2 or fewer
+    rows of tiles included), for every tile height and both wavefront forms; every output row and
+    column of the product and of the gate/up pair is written exactly once and right."""
+    from pypto_amd.runtime import gate_up_swiglu, projection
+    k, n = 256, 768
+    g = torch.Generator().manual_seed(m + variant)
+    x = (torch.randn(m, k, generator=g) / k ** 0.5).to(torch.bfloat16)
+    w = torch.randn(k, n, generator=g).to(torch.bfloat16)
+    wu = torch.randn(k, n, generator=g).to(torch.bfloat16)
+    out = torch.full((m, n), float("nan"))
+    h16 = torch.full((m, n), float("nan"), dtype=torch.bfloat16)
+    worker.set_option("gemm_variant", variant)
+    try:
+        with worker.register(projection) as h:
+            h(x, w, out)
+        with worker.register(gate_up_swiglu) as h:
+            h(x, w, wu, h16)
+    finally:
+        worker.set_option("gemm_variant", 0)
+    validate_golden({"out": out}, {"out": oracle.projection(x, w)}, rtol=2e-3, atol=2e-3)
+    want = oracle.swiglu(oracle.projection(x, w), oracle.projection(x, wu)).to(torch.bfloat16)
+    validate_golden({"out": h16.float()}, {"out": want.float()}, rtol=1e-2, atol=1e-2)
+
+
 def test_projection_argument_rules(worker):
     from pypto_amd.runtime import projection
     x = torch.zeros(4, 64, dtype=torch.bfloat16)
