@@ -195,6 +195,60 @@ def test_ffn_and_projection_sweep(worker):
         worker.set_option("gemm_splits", 0)
 
 
+def test_ffn_whole_tile_sweep(worker):
+    """Shapes made of whole 256-row tiles, where the tall tile runs as four wavefronts by default: blocks,
+    products and gate/up pairs against the oracle, and the four-wavefront form against the eight-wavefront
+    form bit for bit, with the library's split counts and forced ones."""
+    rng = random.Random(20247)
+    try:
+        for case in range(24):
+            t = 256 * rng.choice([1, 2, 3, 4, 9])
+            h = 256 * rng.randint(1, 6)
+            i = 256 * rng.randint(1, 10)
+            dtype = rng.choice([torch.bfloat16, torch.float16])
+            splits = rng.choice([0, 0, 2, 3])
+            kind = rng.choice(["ffn_block", "projection", "projection_residual", "gate_up"])
+            seed = rng.randint(0, 10 ** 6)
+            print(f"whole-tile case {case}: {kind} T{t} H{h} I{i} {dtype} splits={splits} seed={seed}", flush=True)
+            worker.set_option("gemm_splits", splits)
+            g = torch.Generator().manual_seed(seed)
+            outs = {}
+            if kind == "ffn_block":
+                inp = workloads.ffn_inputs(tokens=t, hidden=h, intermediate=i, seed=seed, dtype=dtype)
+                ref = oracle.ffn_block(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, inp.eps)
+            else:
+                x = (torch.randn(t, h, generator=g) / h ** 0.5).to(dtype)
+                wa = torch.randn(h, i, generator=g).to(dtype)
+                wb = torch.randn(h, i, generator=g).to(dtype)
+                res = torch.randn(t, i, generator=g)
+                ref = (oracle.swiglu(oracle.projection(x, wa), oracle.projection(x, wb)).to(dtype) if kind == "gate_up"
+                       else oracle.projection(x, wa, res if kind == "projection_residual" else None))
+            for variant in (0, 4, 7):
+                worker.set_option("gemm_variant", variant)
+                if kind == "ffn_block":
+                    out = torch.zeros(t, h, dtype=torch.float32)
+                    with worker.register(ffn_block) as hd:
+                        hd(inp.x, inp.gamma, inp.w_gate, inp.w_up, inp.w_down, out, inp.eps)
+                elif kind == "gate_up":
+                    out = torch.zeros(t, i, dtype=dtype)
+                    with worker.register(gate_up_swiglu) as hd:
+                        hd(x, wa, wb, out)
+                elif kind == "projection":
+                    out = torch.zeros(t, i, dtype=torch.float32)
+                    with worker.register(projection) as hd:
+                        hd(x, wa, out)
+                else:
+                    out = torch.zeros(t, i, dtype=dtype)
+                    with worker.register(projection_residual) as hd:
+                        hd(x, wa, res, out)
+                outs[variant] = out
+                _close(f"case {case} variant {variant}", out, ref.to(out.dtype), 2e-2, 1e-2)
+            assert torch.equal(outs[4], outs[7]), f"case {case}: four- and eight-wavefront forms differ"
+    finally:
+        worker.set_option("gemm_variant", 0)
+        worker.set_option("gemm_splits", 0)
+
+
 def test_w8a16_sweep(worker):
     rng = random.Random(20242)
     try:
