@@ -403,9 +403,9 @@ def main() -> int:
         torch.cuda.synchronize()
         with worker.register(ffn_block) as fh:
             fargs = [(f.x, f.gamma, f.w_gate, f.w_up, f.w_down, f.out, f.eps)]
-            # the clocks need some tens of milliseconds of MFMA load to settle: the first rounds of a
-            # process run ~10 % slower than the steady state
-            benchmark(fh, fargs, rounds=100, warmup=0)
+            # the clocks need a few hundred milliseconds of MFMA load to settle after the GPU has idled (as it
+            # does during the CPU timings above)
+            benchmark(fh, fargs, rounds=800, warmup=0)
             fstats = benchmark(fh, fargs, rounds=60, warmup=0)
         bf16_out = f.out.clone()  # kept for the distance of the e4m3 block below (the clock probe overwrites f.out)
         tflops = f.flops() / fstats.device_wall_us / 1e6
@@ -461,7 +461,7 @@ def main() -> int:
         torch.cuda.synchronize()
         with worker.register(ffn_block_fp8) as qh:
             qargs = [q.args()]
-            benchmark(qh, qargs, rounds=60, warmup=0)
+            benchmark(qh, qargs, rounds=800, warmup=0)
             qstats = benchmark(qh, qargs, rounds=max(20, args.steps // 2), warmup=0)
         q_tflops = q.flops() / qstats.device_wall_us / 1e6
         rel = float(((q.out - bf16_out).norm() / bf16_out.norm()).item())
