@@ -503,7 +503,7 @@ int launch_gemm(GemmParams p, hipStream_t st) {
 // Operands go global -> LDS directly, as in the eight-wavefront form; with four 16-byte chunks to an
 // A row the swizzle key is (row / 4) % 4 (16 consecutive rows of a fragment read then cover all 16
 // slots of four rows' worth of banks), B keeps 64-byte group g ^ (k-row % 8).  Built for 16-bit
-// weights with m, n and every k range multiples of the tile.
+// weights with n and every k range multiples of the tile (EDGE_M: any number of rows).
 constexpr int QK = 32;   // k extent of a stage
 constexpr int QST = 5;   // stages
 constexpr int kQuadStageBytes = (256 * QK + QK * BN) * 2;  // A rows, then B rows
@@ -523,7 +523,7 @@ __device__ __forceinline__ void quad_to_lds(const char* src, uint32_t lds_w) {
 #pragma clang diagnostic pop
 }
 
-template <bool DUAL, bool BF16, typename OutT>
+template <bool DUAL, bool BF16, typename OutT, bool EDGE_M>
 __global__ __launch_bounds__(256) void gemm_quad_kernel(GemmParams p) {
   constexpr int MT = 4, NT = 4;
   constexpr int A_BYTES = 256 * QK * 2;
@@ -561,7 +561,9 @@ __global__ __launch_bounds__(256) void gemm_quad_kernel(GemmParams p) {
   const char* gb[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    ga[e] = reinterpret_cast<const char*>(p.a + (int64_t)(m0 + 64 * e + 16 * wave + (lane >> 2)) * p.lda + k_begin + a_chunk * 8);
+    int a_row = m0 + 64 * e + 16 * wave + (lane >> 2);
+    if (EDGE_M) a_row = min(a_row, p.m - 1);  // rows past the end read the last row; their products are not stored
+    ga[e] = reinterpret_cast<const char*>(p.a + (int64_t)a_row * p.lda + k_begin + a_chunk * 8);
     gb[e] = reinterpret_cast<const char*>(bsrc + (int64_t)(k_begin + 8 * e + b_krow) * p.ldb + b_col);
   }
   const int64_t a_adv = QK * 2, b_adv = (int64_t)QK * p.ldb * 2;  // bytes from one stage to the next
@@ -688,55 +690,65 @@ __global__ __launch_bounds__(256) void gemm_quad_kernel(GemmParams p) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land in LDS after the workgroup has gone
 
   // ---- epilogue (row = m0 + wm*128 + i*32 + (r/4)*8 + (lane/32)*4 + r%4, column lane%32 + ...) ----
+  // Only the last row tile of a ragged problem checks its rows: the checks keep the stores of a tile
+  // from being issued as one batch, which every other tile should not pay for.
   OutT* c = reinterpret_cast<OutT*>(p.c);
   const int row_base = m0 + wm * 128 + (lane >> 5) * 4;
   const int col0 = (DUAL ? n0 + wn * 64 : n0 + wn * 128) + (lane & 31);
   const int64_t mn = (int64_t)p.m * p.n;
   constexpr int JN = DUAL ? NT / 2 : NT;
-  if (p.splits > 1) {
-    float* lane_s = p.slabs + (int64_t)split * (DUAL ? 2 : 1) * mn + (int64_t)row_base * p.n + col0;
+  auto epilogue = [&](auto guard_c) {
+    constexpr bool GUARD = decltype(guard_c)::value != 0;
+    if (p.splits > 1) {
+      float* lane_s = p.slabs + (int64_t)split * (DUAL ? 2 : 1) * mn + (int64_t)row_base * p.n + col0;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int rr = i * 32 + (r >> 2) * 8 + (r & 3);
+          if (GUARD && row_base + rr >= p.m) continue;
+          float* s = lane_s + (int64_t)rr * p.n;
+#pragma unroll
+          for (int jn = 0; jn < JN; ++jn) {
+            s[jn * 32] = acc[i][jn][r];
+            if constexpr (DUAL) s[mn + jn * 32] = acc[i][jn + NT / 2][r];
+          }
+        }
+      }
+      return;
+    }
+    OutT* lane_c = c + (int64_t)row_base * p.ldc + col0;
+    const int64_t lane_res = (int64_t)row_base * p.n + col0;
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        float* s = lane_s + (int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * p.n;
+        const int rr = i * 32 + (r >> 2) * 8 + (r & 3);
+        if (GUARD && row_base + rr >= p.m) continue;
+        OutT* dst = lane_c + (int64_t)rr * p.ldc;
 #pragma unroll
         for (int jn = 0; jn < JN; ++jn) {
-          s[jn * 32] = acc[i][jn][r];
-          if constexpr (DUAL) s[mn + jn * 32] = acc[i][jn + NT / 2][r];
+          if constexpr (DUAL) {
+            store_out<OutT>(dst + jn * 32, silu(acc[i][jn][r]) * acc[i][jn + NT / 2][r]);
+          } else {
+            float v = acc[i][jn][r];
+            if (p.residual) v += load_residual(p.residual, p.res_dtype, lane_res + (int64_t)rr * p.n + jn * 32);
+            store_out<OutT>(dst + jn * 32, v);
+          }
         }
       }
     }
-    return;
-  }
-  OutT* lane_c = c + (int64_t)row_base * p.ldc + col0;
-  const int64_t lane_res = (int64_t)row_base * p.n + col0;
-#pragma unroll
-  for (int i = 0; i < MT; ++i) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int rr = i * 32 + (r >> 2) * 8 + (r & 3);
-      OutT* dst = lane_c + (int64_t)rr * p.ldc;
-#pragma unroll
-      for (int jn = 0; jn < JN; ++jn) {
-        if constexpr (DUAL) {
-          store_out<OutT>(dst + jn * 32, silu(acc[i][jn][r]) * acc[i][jn + NT / 2][r]);
-        } else {
-          float v = acc[i][jn][r];
-          if (p.residual) v += load_residual(p.residual, p.res_dtype, lane_res + (int64_t)rr * p.n + jn * 32);
-          store_out<OutT>(dst + jn * 32, v);
-        }
-      }
-    }
-  }
+  };
+  if (EDGE_M && m0 + 256 > p.m) epilogue(QuadConst<1>{});
+  else epilogue(QuadConst<0>{});
 }
 
-template <bool DUAL, bool BF16, typename OutT>
-int launch_quad(GemmParams p, hipStream_t st) {
-  p.tiles_m = p.m / 256;
+template <bool DUAL, bool BF16, typename OutT, bool EDGE_M>
+int launch_quad_e(GemmParams p, hipStream_t st) {
+  p.tiles_m = (p.m + 255) / 256;
   p.tiles_n = p.n / (DUAL ? BN / 2 : BN);
   const size_t smem = (size_t)QST * kQuadStageBytes;
-  auto kern = gemm_quad_kernel<DUAL, BF16, OutT>;
+  auto kern = gemm_quad_kernel<DUAL, BF16, OutT, EDGE_M>;
   static std::atomic<bool> attr_set{false};  // per instantiation; callers hold the dispatch lock
   if (!attr_set.load(std::memory_order_acquire)) {
     PTO_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -746,6 +758,12 @@ int launch_quad(GemmParams p, hipStream_t st) {
   hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.splits), dim3(256), smem, st, p);
   PTO_CHECK_HIP(hipGetLastError());
   return PTO_HIP_OK;
+}
+
+// m ragged: the same loop with the A row pointers clamped once and the stores of the missing rows skipped
+template <bool DUAL, bool BF16, typename OutT>
+int launch_quad(const GemmParams& p, hipStream_t st) {
+  return p.m % 256 == 0 ? launch_quad_e<DUAL, BF16, OutT, false>(p, st) : launch_quad_e<DUAL, BF16, OutT, true>(p, st);
 }
 
 // Sum of the split-K slabs in split order (so the result does not depend on which workgroup
@@ -867,7 +885,7 @@ int launch_variant(GemmParams p, hipStream_t st) {
             (tall ? 18.1 + 9.4 * load : 11.0 + 6.5 * load) + (W8 && rounds > 1 ? (tall ? 2.5 : 4.5) : 0.0);
         const double slab_mb = (double)real * p.m * p.n * mats * 4.0 / 1e6;  // written, then read back
         // where the tall tile runs as four wavefronts (see below) it measured about 5 % faster
-        const bool as_quad = !W8 && tall && p.m % 256 == 0 && p.n % (DUAL ? BN / 2 : BN) == 0 && p.k % QK == 0;
+        const bool as_quad = !W8 && tall && p.n % (DUAL ? BN / 2 : BN) == 0 && p.k % QK == 0;
         const double t = std::max((double)rounds * (double)kps * ns_row * (as_quad ? 0.95 : 1.0) * 1e-3, stream_us) +
                          (real > 1 ? 7.0 + 2.0 * slab_mb / (slab_mb <= 128.0 ? 8.0 : 4.0) : 0.0);
         if (t < best) {
@@ -905,8 +923,8 @@ int launch_variant(GemmParams p, hipStream_t st) {
   // 1280 -> 1200; hidden 2048 at 4096 tokens 383 -> 380).  "gemm_variant" 4 keeps eight wavefronts.
   bool quad = false;
   if constexpr (!W8) {
-    const bool fits = !tiny_tile && !small_tile && p.m % 256 == 0 && p.n % (DUAL ? BN / 2 : BN) == 0 &&
-                      p.k % QK == 0 && p.k_per_split % QK == 0;
+    const bool fits = !tiny_tile && !small_tile && p.n % (DUAL ? BN / 2 : BN) == 0 && p.k % QK == 0 &&
+                      p.k_per_split % QK == 0;
     quad = fits && (variant == 7 || variant == 0);
     if (quad) rc = launch_quad<DUAL, BF16, OutT>(p, st);
   }

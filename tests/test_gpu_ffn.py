@@ -260,13 +260,14 @@ def test_every_tile_height_and_split_count_gives_the_same_product(worker, varian
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("m,k,n,splits", [(256, 32, 256, 0), (256, 64, 512, 0), (512, 96, 256, 0), (256, 128, 256, 0),
                                           (256, 160, 256, 0), (256, 192, 512, 0), (512, 352, 768, 0), (256, 4096, 256, 0),
-                                          (256, 4096, 512, 3), (768, 1024, 256, 2), (256, 11008, 256, 0)])
+                                          (256, 4096, 512, 3), (768, 1024, 256, 2), (256, 11008, 256, 0),
+                                          (300, 512, 256, 0), (1000, 1024, 512, 2), (257, 4096, 256, 0), (65, 256, 512, 0)])
 def test_four_wavefront_tile_form_gives_the_bits_of_the_eight_wavefront_form(worker, dtype, m, k, n, splits):
     """The 256-row tile as four wavefronts (one per SIMD, five rotating 32-k stages) walks k in the same
     16-wide steps into the same accumulators as the eight-wavefront form: identical bits for the plain
     product, the residual + cast form and the gate/up pair, over k extents that end the five-stage
-    rotation at every position (1, 2, 3, 4, 5, 6, 11, 128 stages), with and without k splits; and the
-    product itself against the oracle."""
+    rotation at every position (1, 2, 3, 4, 5, 6, 11, 128 stages), with and without k splits, whole row tiles
+    and ragged ones; and the product itself against the oracle."""
     from pypto_amd.runtime import gate_up_swiglu, projection, projection_residual
     g = torch.Generator().manual_seed(m + k + n)
     x = (torch.randn(m, k, generator=g) / k ** 0.5).to(dtype)
