@@ -566,8 +566,8 @@ PTO_HIP_API int pto_hip_backend_handler_query(const char* hook, int32_t arg, cha
  *  "gemm_variant"               FFN GEMM tiling: 0 = default choice (64-row tile up to 64 rows, else the
  *                               256- or 128-row tile and k split count with the least estimated time,
  *                               eight wavefronts, two per SIMD; the 256-row tile with four wavefronts,
- *                               one per SIMD, wherever that form is built: 16-bit weights, whole
- *                               tiles; skinny projections up to 32 tokens); 4 = 256-row tile with
+ *                               one per SIMD, wherever that form is built: 16-bit weights, columns
+ *                               and k in whole tiles; skinny projections up to 32 tokens); 4 = 256-row tile with
  *                               eight wavefronts, k split in two when CUs would idle, 5 = 128-row
  *                               tile, 6 = 64-row tile, k split while CUs would idle, 7 = as 4 with
  *                               four wavefronts wherever that form is built (forced forms, for sweeps
